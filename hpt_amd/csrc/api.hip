@@ -1,0 +1,618 @@
+// C ABI of libhpt_hip (see include/hpt_hip.h): argument validation, the device
+// caching allocator, per-stream scratch, and dispatch into the kernel tables.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <list>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "common.hpp"
+#include "norm_entry.hpp"
+#include "reduce_entry.hpp"
+
+namespace hpt {
+
+// ---- error transport ---------------------------------------------------------
+
+static thread_local std::string g_last_error;
+
+template <class F> static int32_t guarded(F&& f) {
+    try {
+        f();
+        return HPT_OK;
+    } catch (const Error& e) {
+        g_last_error = e.msg;
+        return e.code;
+    } catch (const std::bad_alloc&) {
+        g_last_error = "host allocation failed";
+        return HPT_ERR_MEMORY;
+    } catch (...) {
+        g_last_error = "unknown error";
+        return HPT_ERR_KERNEL;
+    }
+}
+
+static void hip_check(hipError_t e, int code, const char* what) {
+    if (e != hipSuccess) fail(code, "%s: %s", what, hipGetErrorString(e));
+}
+
+static void use_device(int dev) {
+    int n = 0;
+    hip_check(hipGetDeviceCount(&n), HPT_ERR_DEVICE, "hipGetDeviceCount");
+    if (dev < 0 || dev >= n) fail(HPT_ERR_DEVICE, "device %d does not exist (%d visible)", dev, n);
+    hip_check(hipSetDevice(dev), HPT_ERR_DEVICE, "hipSetDevice");
+}
+
+// ---- device caching allocator ------------------------------------------------
+// Same policy as the reference's CudaAllocator
+// (hpt-allocator/src/allocators/cuda.rs:41-322, utils/allocate.rs:15-130,
+// utils/deallocate.rs:11-32): blocks are keyed by their exact (size, align)
+// layout; a freed block is kept in an LRU cache of layouts; evicting a layout
+// releases all of its blocks; when the device is out of memory, layouts are
+// evicted least-recently-used first and the allocation is retried.
+
+struct LayoutKey {
+    size_t bytes, align;
+    bool operator<(const LayoutKey& o) const {
+        return bytes != o.bytes ? bytes < o.bytes : align < o.align;
+    }
+};
+
+struct DeviceAllocator {
+    std::mutex mu;
+    size_t capacity = 100;  // cached layouts; the CPU allocator's default (allocators/cpu.rs:22)
+    std::list<LayoutKey> lru;  // front = most recently used
+    std::map<LayoutKey, std::pair<std::list<LayoutKey>::iterator, std::vector<void*>>> cache;
+    std::unordered_map<void*, LayoutKey> live;
+    uint64_t device_mallocs = 0;
+
+    size_t cached_blocks() const {
+        size_t n = 0;
+        for (auto& kv : cache) n += kv.second.second.size();
+        return n;
+    }
+    void evict_one() {  // requires a non-empty cache
+        LayoutKey k = lru.back();
+        auto it = cache.find(k);
+        for (void* p : it->second.second) (void)hipFree(p);
+        cache.erase(it);
+        lru.pop_back();
+    }
+    void* allocate(size_t bytes, size_t align) {
+        LayoutKey k{bytes, align};
+        auto it = cache.find(k);
+        if (it != cache.end() && !it->second.second.empty()) {
+            void* p = it->second.second.back();
+            it->second.second.pop_back();
+            lru.splice(lru.begin(), lru, it->second.first);
+            if (it->second.second.empty()) {
+                lru.erase(it->second.first);
+                cache.erase(it);
+            }
+            live[p] = k;
+            return p;
+        }
+        void* p = nullptr;
+        for (;;) {
+            hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+            if (e == hipSuccess) break;
+            (void)hipGetLastError();  // clear the sticky error before retrying
+            if (cache.empty())
+                fail(HPT_ERR_MEMORY, "Failed to allocate %zu bytes on device: %s", bytes,
+                     hipGetErrorString(e));
+            evict_one();
+        }
+        ++device_mallocs;
+        if (align > 1 && ((uintptr_t)p % align) != 0) {
+            (void)hipFree(p);
+            fail(HPT_ERR_MEMORY, "device allocation cannot satisfy alignment %zu", align);
+        }
+        live[p] = k;
+        return p;
+    }
+    void deallocate(void* p, size_t bytes, size_t align) {
+        auto it = live.find(p);
+        if (it == live.end()) fail(HPT_ERR_MEMORY, "pointer %p was not allocated by hpt_hip_alloc", p);
+        if (it->second.bytes != bytes || it->second.align != align)
+            fail(HPT_ERR_MEMORY, "layout mismatch on free: allocated (%zu, %zu), freed as (%zu, %zu)",
+                 it->second.bytes, it->second.align, bytes, align);
+        LayoutKey k = it->second;
+        live.erase(it);
+        if (capacity == 0) {
+            (void)hipFree(p);
+            return;
+        }
+        auto c = cache.find(k);
+        if (c == cache.end()) {
+            lru.push_front(k);
+            cache[k] = {lru.begin(), {p}};
+            while (cache.size() > capacity) evict_one();
+        } else {
+            c->second.second.push_back(p);
+            lru.splice(lru.begin(), lru, c->second.first);
+        }
+    }
+    void clear() {
+        while (!cache.empty()) evict_one();
+    }
+};
+
+static std::mutex g_alloc_table_mu;
+static std::map<int, DeviceAllocator*> g_allocators;
+
+static DeviceAllocator& allocator_of(int dev) {
+    std::lock_guard<std::mutex> g(g_alloc_table_mu);
+    auto it = g_allocators.find(dev);
+    if (it == g_allocators.end()) it = g_allocators.emplace(dev, new DeviceAllocator()).first;
+    return *it->second;
+}
+
+// ---- scratch of the multi-workgroup reductions -----------------------------------
+
+struct StreamScratch {
+    void* partial = nullptr;
+    size_t partial_bytes = 0;
+    unsigned* counters = nullptr;
+    size_t n_counters = 0;
+};
+
+static std::mutex g_scratch_mu;  // held from lookup to launch
+static std::map<std::pair<int, hipStream_t>, StreamScratch> g_scratch;
+
+// Requires g_scratch_mu. Grows the scratch of (dev, stream); growing frees the
+// old buffers, which waits for the device to go idle first.
+static ReduceScratch scratch_for(int dev, hipStream_t st, size_t partial_bytes, size_t counters) {
+    StreamScratch& s = g_scratch[{dev, st}];
+    if (partial_bytes > s.partial_bytes) {
+        if (s.partial) hip_check(hipFree(s.partial), HPT_ERR_MEMORY, "hipFree(scratch)");
+        s.partial = nullptr;
+        s.partial_bytes = 0;
+        size_t want = std::max<size_t>(partial_bytes, 1u << 20);
+        hip_check(hipMalloc(&s.partial, want), HPT_ERR_MEMORY, "hipMalloc(scratch)");
+        s.partial_bytes = want;
+    }
+    if (counters > s.n_counters) {
+        if (s.counters) hip_check(hipFree(s.counters), HPT_ERR_MEMORY, "hipFree(counters)");
+        s.counters = nullptr;
+        s.n_counters = 0;
+        size_t want = std::max<size_t>(counters, 4096);
+        hip_check(hipMalloc((void**)&s.counters, want * sizeof(unsigned)), HPT_ERR_MEMORY,
+                  "hipMalloc(counters)");
+        hip_check(hipMemset(s.counters, 0, want * sizeof(unsigned)), HPT_ERR_MEMORY,
+                  "hipMemset(counters)");
+        s.n_counters = want;
+    }
+    ReduceScratch r;
+    r.partial = s.partial;
+    r.counters = s.counters;
+    return r;
+}
+
+void scratch_need(const ReducePlan& p, size_t acc_size, size_t* partial_bytes, size_t* counters) {
+    *partial_bytes = 0;
+    *counters = 0;
+    if (p.split <= 1) return;
+    *partial_bytes = (size_t)p.K * p.split * acc_size;
+    if (p.kind == ReduceKind::Row) {
+        *counters = (size_t)p.K;
+    } else {
+        int64_t kv = p.K / p.vec;
+        *counters = (size_t)((kv + p.bx - 1) / p.bx);
+    }
+}
+
+// ---- dispatch tables -----------------------------------------------------------
+
+const ReduceEntry& reduce_entry_for(int e) {
+    switch (e) {
+        case 0: return reduce_entry<0>();
+        case 1: return reduce_entry<1>();
+        case 2: return reduce_entry<2>();
+        case 3: return reduce_entry<3>();
+        case 4: return reduce_entry<4>();
+        case 5: return reduce_entry<5>();
+        case 6: return reduce_entry<6>();
+        case 7: return reduce_entry<7>();
+        case 8: return reduce_entry<8>();
+        case 9: return reduce_entry<9>();
+        case 10: return reduce_entry<10>();
+        case 11: return reduce_entry<11>();
+        case 12: return reduce_entry<12>();
+        case 13: return reduce_entry<13>();
+        case 14: return reduce_entry<14>();
+        case 15: return reduce_entry<15>();
+        default: fail(HPT_ERR_PARAM, "invalid reduce op %d", e);
+    }
+}
+
+NormLaunchFn norm_launcher_for(int kind, int dtype) {
+    switch (kind) {
+        case NORM_SOFTMAX: return norm_launcher<NORM_SOFTMAX>(dtype);
+        case NORM_LOGSOFTMAX: return norm_launcher<NORM_LOGSOFTMAX>(dtype);
+        case NORM_LAYERNORM: return norm_launcher<NORM_LAYERNORM>(dtype);
+        default: return nullptr;
+    }
+}
+
+// ---- view validation -------------------------------------------------------------
+
+static void check_view(const hpt_view* v, const char* name, bool need_data) {
+    if (!v) fail(HPT_ERR_PARAM, "%s: view is null", name);
+    if (v->dtype < 0 || v->dtype >= HPT_DTYPE_COUNT)
+        fail(HPT_ERR_DTYPE, "%s: invalid dtype %d", name, v->dtype);
+    if (v->ndim < 0 || v->ndim > kMaxRank)
+        fail(HPT_ERR_SHAPE, "%s: ndim %d outside 0..%d", name, v->ndim, kMaxRank);
+    if (v->ndim > 0 && (!v->shape || !v->strides))
+        fail(HPT_ERR_PARAM, "%s: shape/strides are null", name);
+    int64_t n = 1;
+    for (int i = 0; i < v->ndim; ++i) {
+        if (v->shape[i] < 0) fail(HPT_ERR_SHAPE, "%s: negative dim %lld", name, (long long)v->shape[i]);
+        n *= v->shape[i];
+    }
+    if (need_data && n > 0 && !v->data) fail(HPT_ERR_PARAM, "%s: data pointer is null", name);
+}
+
+static int64_t view_size(const hpt_view* v) {
+    int64_t n = 1;
+    for (int i = 0; i < v->ndim; ++i) n *= v->shape[i];
+    return n;
+}
+
+// Layout::is_contiguous (hpt-common/src/layout/layout_utils.rs:363-375), with
+// size-1 dims allowed any stride.
+static bool view_contiguous(const hpt_view* v) {
+    int64_t expect = 1;
+    for (int i = v->ndim - 1; i >= 0; --i) {
+        if (v->shape[i] == 0) return true;
+        if (v->shape[i] == 1) continue;
+        if (v->strides[i] != expect) return false;
+        expect *= v->shape[i];
+    }
+    return true;
+}
+
+static void check_out(const hpt_view* out, int dtype, int64_t count, const char* name) {
+    check_view(out, name, true);
+    if (out->dtype != dtype)
+        fail(HPT_ERR_DTYPE, "%s: dtype is %s, expected %s", name, dtype_name(out->dtype),
+             dtype_name(dtype));
+    if (!view_contiguous(out)) fail(HPT_ERR_SHAPE, "%s: output tensor must be contiguous", name);
+    if (view_size(out) != count)
+        fail(HPT_ERR_SHAPE, "%s: Size mismatch: expected %lld, got %lld", name, (long long)count,
+             (long long)view_size(out));
+}
+
+static void check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) fail(HPT_ERR_KERNEL, "%s: kernel launch failed: %s", what, hipGetErrorString(e));
+}
+
+struct ReduceCall {
+    ReducePlan plan;
+    const ReduceEntry* entry;
+    int out_dtype;
+};
+
+static ReduceCall prepare_reduce(int entry_id, const hpt_view* in, const int64_t* axes, int naxes) {
+    check_view(in, "reduce input", false);
+    if (naxes < 0 || naxes > kMaxRank || (naxes > 0 && !axes))
+        fail(HPT_ERR_PARAM, "reduce: bad axes argument");
+    int64_t norm[kMaxRank];
+    process_axes(axes, naxes, in->ndim, norm);
+    if (in->ndim == 0) naxes = 0;
+    ReduceCall c;
+    c.entry = &reduce_entry_for(entry_id);
+    c.out_dtype = entry_id < HPT_REDUCE_OP_COUNT ? reduce_out_dtype(entry_id, in->dtype) : HPT_I64;
+    c.plan = plan_reduce(in->data, in->shape, in->strides, in->ndim, norm, naxes,
+                         dtype_size(in->dtype), c.entry->acc_size[in->dtype]);
+    return c;
+}
+
+static void run_reduce(int dev, void* stream, int entry_id, const hpt_view* in, const int64_t* axes,
+                       int naxes, int init_out, hpt_view* out) {
+    ReduceCall c = prepare_reduce(entry_id, in, axes, naxes);
+    check_out(out, c.out_dtype, c.plan.K, "reduce output");
+    if (c.plan.kind == ReduceKind::Empty) return;
+    if (!in->data && c.plan.kind != ReduceKind::Identity)
+        fail(HPT_ERR_PARAM, "reduce input: data pointer is null");
+    if (!init_out && !(entry_id == HPT_SUM || entry_id == HPT_NANSUM))
+        fail(HPT_ERR_PARAM, "init_out = 0 (accumulate into out) is only defined for sum and nansum");
+    use_device(dev);
+    hipStream_t st = (hipStream_t)stream;
+    ReduceLaunchFn fn = c.entry->launch[in->dtype];
+    size_t pbytes, ncount;
+    scratch_need(c.plan, c.entry->acc_size[in->dtype], &pbytes, &ncount);
+    if (pbytes) {
+        std::lock_guard<std::mutex> g(g_scratch_mu);
+        ReduceScratch sc = scratch_for(dev, st, pbytes, ncount);
+        fn(c.plan, in->data, out->data, sc, st, init_out);
+        check_launch("reduce");
+    } else {
+        fn(c.plan, in->data, out->data, ReduceScratch{}, st, init_out);
+        check_launch("reduce");
+    }
+}
+
+struct NormCall {
+    NormPlan plan;
+    NormArgs args;
+};
+
+static NormCall prepare_norm(const hpt_view* in, const void* out_data, int64_t axis, int n_norm_dims) {
+    check_view(in, "normalize input", false);
+    if (!is_float_dtype(in->dtype))
+        fail(HPT_ERR_DTYPE, "softmax/log_softmax/layernorm need a float dtype, got %s",
+             dtype_name(in->dtype));
+    if (in->ndim == 0) fail(HPT_ERR_SHAPE, "normalize: input has no dimensions");
+    if (n_norm_dims <= 0) {
+        int64_t a = axis;
+        int64_t na;
+        process_axes(&a, 1, in->ndim, &na);
+        axis = na;
+    } else if (n_norm_dims > in->ndim) {
+        fail(HPT_ERR_SHAPE, "layernorm: %d normalized dims but input has %d", n_norm_dims, in->ndim);
+    }
+    NormCall c;
+    c.plan = plan_normalize(in->data, out_data, in->shape, in->strides, in->ndim, axis, n_norm_dims,
+                            dtype_size(in->dtype));
+    NormArgs& a = c.args;
+    memset(&a, 0, sizeof a);
+    a.in = in->data;
+    a.out = const_cast<void*>(out_data);
+    a.kept_in = c.plan.kept_in;
+    a.kept_out = c.plan.kept_out;
+    a.norm_in = c.plan.norm_in;
+    a.rows = c.plan.rows;
+    a.cols = c.plan.cols;
+    a.sa = c.plan.norm_in.n == 1 ? c.plan.norm_in.stride[0] : 0;
+    a.out_axis_stride = c.plan.out_axis_stride;
+    return c;
+}
+
+}  // namespace hpt
+
+using namespace hpt;
+
+extern "C" {
+
+const char* hpt_hip_last_error(void) { return g_last_error.c_str(); }
+
+size_t hpt_hip_dtype_size(int32_t dtype) { return dtype_size(dtype); }
+
+int32_t hpt_hip_device_count(int32_t* n) {
+    return guarded([&] {
+        if (!n) fail(HPT_ERR_PARAM, "device_count: null output");
+        int c = 0;
+        hip_check(hipGetDeviceCount(&c), HPT_ERR_DEVICE, "hipGetDeviceCount");
+        *n = c;
+    });
+}
+
+int32_t hpt_hip_alloc(int32_t dev, size_t bytes, size_t align, int32_t zeroed, void** out) {
+    return guarded([&] {
+        if (!out) fail(HPT_ERR_PARAM, "alloc: null output");
+        if (align == 0 || (align & (align - 1))) fail(HPT_ERR_PARAM, "alloc: align %zu is not a power of two", align);
+        use_device(dev);
+        DeviceAllocator& a = allocator_of(dev);
+        std::lock_guard<std::mutex> g(a.mu);
+        void* p = a.allocate(bytes, align);
+        if (zeroed && bytes) {
+            hipError_t e = hipMemset(p, 0, bytes);
+            if (e != hipSuccess) {
+                a.deallocate(p, bytes, align);
+                hip_check(e, HPT_ERR_MEMORY, "hipMemset");
+            }
+        }
+        *out = p;
+    });
+}
+
+int32_t hpt_hip_free(int32_t dev, void* p, size_t bytes, size_t align) {
+    return guarded([&] {
+        if (!p) return;
+        use_device(dev);
+        DeviceAllocator& a = allocator_of(dev);
+        std::lock_guard<std::mutex> g(a.mu);
+        a.deallocate(p, bytes, align);
+    });
+}
+
+int32_t hpt_hip_cache_resize(int32_t dev, size_t entries) {
+    return guarded([&] {
+        use_device(dev);
+        DeviceAllocator& a = allocator_of(dev);
+        std::lock_guard<std::mutex> g(a.mu);
+        a.capacity = entries;
+        while (a.cache.size() > a.capacity) a.evict_one();
+    });
+}
+
+int32_t hpt_hip_cache_clear(int32_t dev) {
+    return guarded([&] {
+        use_device(dev);
+        DeviceAllocator& a = allocator_of(dev);
+        std::lock_guard<std::mutex> g(a.mu);
+        a.clear();
+    });
+}
+
+int32_t hpt_hip_alloc_stats(int32_t dev, uint64_t* live_blocks, uint64_t* cached_blocks,
+                            uint64_t* device_mallocs) {
+    return guarded([&] {
+        DeviceAllocator& a = allocator_of(dev);
+        std::lock_guard<std::mutex> g(a.mu);
+        if (live_blocks) *live_blocks = a.live.size();
+        if (cached_blocks) *cached_blocks = a.cached_blocks();
+        if (device_mallocs) *device_mallocs = a.device_mallocs;
+    });
+}
+
+int32_t hpt_hip_memcpy_h2d_sync(int32_t dev, void* dst, const void* src, size_t bytes) {
+    return guarded([&] {
+        if (!bytes) return;
+        if (!dst || !src) fail(HPT_ERR_PARAM, "memcpy: null pointer");
+        use_device(dev);
+        hip_check(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice), HPT_ERR_DEVICE, "hipMemcpy(h2d)");
+    });
+}
+
+int32_t hpt_hip_memcpy_d2h_sync(int32_t dev, void* dst, const void* src, size_t bytes) {
+    return guarded([&] {
+        if (!bytes) return;
+        if (!dst || !src) fail(HPT_ERR_PARAM, "memcpy: null pointer");
+        use_device(dev);
+        hip_check(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost), HPT_ERR_DEVICE, "hipMemcpy(d2h)");
+    });
+}
+
+int32_t hpt_hip_memcpy_d2d_sync(int32_t dev, void* dst, const void* src, size_t bytes) {
+    return guarded([&] {
+        if (!bytes) return;
+        if (!dst || !src) fail(HPT_ERR_PARAM, "memcpy: null pointer");
+        use_device(dev);
+        hip_check(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToDevice), HPT_ERR_DEVICE, "hipMemcpy(d2d)");
+    });
+}
+
+int32_t hpt_hip_stream_synchronize(int32_t dev, void* stream) {
+    return guarded([&] {
+        use_device(dev);
+        hip_check(hipStreamSynchronize((hipStream_t)stream), HPT_ERR_KERNEL, "hipStreamSynchronize");
+    });
+}
+
+int32_t hpt_hip_process_axes(const int64_t* axes, int32_t naxes, int32_t ndim, int64_t* out) {
+    return guarded([&] {
+        if (naxes < 0 || (naxes > 0 && (!axes || !out))) fail(HPT_ERR_PARAM, "process_axes: bad arguments");
+        process_axes(axes, naxes, ndim, out);
+    });
+}
+
+int32_t hpt_hip_reduce_shape(const int64_t* shape, int32_t ndim, const int64_t* axes, int32_t naxes,
+                             int32_t keep_dims, int64_t* out_shape, int32_t* out_ndim) {
+    return guarded([&] {
+        if (ndim < 0 || ndim > kMaxRank || naxes < 0 || naxes > kMaxRank || !out_shape || !out_ndim)
+            fail(HPT_ERR_PARAM, "reduce_shape: bad arguments");
+        int64_t norm[kMaxRank];
+        process_axes(axes, naxes, ndim, norm);
+        bool red[kMaxRank] = {};
+        if (ndim > 0)
+            for (int i = 0; i < naxes; ++i) red[norm[i]] = true;
+        int n = 0;
+        for (int i = 0; i < ndim; ++i) {
+            if (red[i]) {
+                if (keep_dims) out_shape[n++] = 1;
+            } else {
+                out_shape[n++] = shape[i];
+            }
+        }
+        if (n == 0) out_shape[n++] = 1;
+        *out_ndim = n;
+    });
+}
+
+int32_t hpt_hip_reduce_out_dtype(int32_t op, int32_t in_dtype, int32_t* out_dtype) {
+    return guarded([&] {
+        if (!out_dtype) fail(HPT_ERR_PARAM, "reduce_out_dtype: null output");
+        if (op < 0 || op >= HPT_REDUCE_OP_COUNT) fail(HPT_ERR_PARAM, "invalid reduce op %d", op);
+        *out_dtype = reduce_out_dtype(op, in_dtype);
+    });
+}
+
+int32_t hpt_hip_reduce_plan(int32_t op, const hpt_view* in, const int64_t* axes, int32_t naxes,
+                            char* buf, size_t buflen) {
+    return guarded([&] {
+        if (!buf || !buflen) fail(HPT_ERR_PARAM, "reduce_plan: no buffer");
+        if (op < 0 || op >= kReduceEntryCount) fail(HPT_ERR_PARAM, "invalid reduce op %d", op);
+        ReduceCall c = prepare_reduce(op, in, axes, naxes);
+        snprintf(buf, buflen, "%s", describe(c.plan).c_str());
+    });
+}
+
+int32_t hpt_hip_normalize_plan(const hpt_view* in, int64_t axis, int32_t n_norm_dims, char* buf,
+                               size_t buflen) {
+    return guarded([&] {
+        if (!buf || !buflen) fail(HPT_ERR_PARAM, "normalize_plan: no buffer");
+        NormCall c = prepare_norm(in, nullptr, axis, n_norm_dims);
+        snprintf(buf, buflen, "%s", describe(c.plan).c_str());
+    });
+}
+
+int32_t hpt_hip_reduce(int32_t dev, void* stream, int32_t op, const hpt_view* in, const int64_t* axes,
+                       int32_t naxes, int32_t init_out, hpt_view* out) {
+    return guarded([&] {
+        if (op < 0 || op >= HPT_REDUCE_OP_COUNT) fail(HPT_ERR_PARAM, "invalid reduce op %d", op);
+        run_reduce(dev, stream, op, in, axes, naxes, init_out, out);
+    });
+}
+
+int32_t hpt_hip_argreduce(int32_t dev, void* stream, int32_t is_max, const hpt_view* in, int64_t axis,
+                          hpt_view* out) {
+    return guarded([&] {
+        check_view(in, "argreduce input", false);
+        if (in->ndim == 0) fail(HPT_ERR_SHAPE, "argreduce: input has no dimensions");
+        int64_t na;
+        process_axes(&axis, 1, in->ndim, &na);
+        if (in->shape[na] > INT32_MAX)
+            fail(HPT_ERR_SHAPE, "argreduce: axis of %lld elements exceeds 2^31-1", (long long)in->shape[na]);
+        run_reduce(dev, stream, is_max ? kArgMaxEntry : kArgMinEntry, in, &na, 1, 1, out);
+    });
+}
+
+int32_t hpt_hip_softmax(int32_t dev, void* stream, int32_t log, const hpt_view* in, int64_t axis,
+                        hpt_view* out) {
+    return guarded([&] {
+        check_view(in, "softmax input", true);
+        check_out(out, in->dtype, view_size(in), "softmax output");
+        NormCall c = prepare_norm(in, out->data, axis, 0);
+        if (c.plan.kind == NormKind::Empty) return;
+        NormLaunchFn fn = norm_launcher_for(log ? NORM_LOGSOFTMAX : NORM_SOFTMAX, in->dtype);
+        if (!fn) fail(HPT_ERR_DTYPE, "softmax: unsupported dtype %s", dtype_name(in->dtype));
+        use_device(dev);
+        fn(c.plan, c.args, (hipStream_t)stream);
+        check_launch("softmax");
+    });
+}
+
+int32_t hpt_hip_layernorm(int32_t dev, void* stream, const hpt_view* in, int32_t n_norm_dims,
+                          const hpt_view* gamma, const hpt_view* beta, double eps, hpt_view* out) {
+    return guarded([&] {
+        check_view(in, "layernorm input", true);
+        if (n_norm_dims <= 0) fail(HPT_ERR_SHAPE, "layernorm: normalized_shape must not be empty");
+        check_out(out, in->dtype, view_size(in), "layernorm output");
+        NormCall c = prepare_norm(in, out->data, 0, n_norm_dims);
+        const hpt_view* gb[2] = {gamma, beta};
+        const char* names[2] = {"layernorm gamma", "layernorm beta"};
+        for (int k = 0; k < 2; ++k) {
+            if (!gb[k]) continue;
+            check_view(gb[k], names[k], true);
+            if (gb[k]->dtype != in->dtype)
+                fail(HPT_ERR_DTYPE, "%s: dtype is %s, expected %s", names[k], dtype_name(gb[k]->dtype),
+                     dtype_name(in->dtype));
+            if (!view_contiguous(gb[k])) fail(HPT_ERR_SHAPE, "%s: must be contiguous", names[k]);
+            // shape must equal the normalised dims (leading 1s aside)
+            if (view_size(gb[k]) != c.plan.cols && c.plan.kind != NormKind::Empty)
+                fail(HPT_ERR_SHAPE, "%s: Size mismatch: expected %lld, got %lld", names[k],
+                     (long long)c.plan.cols, (long long)view_size(gb[k]));
+        }
+        if (c.plan.kind == NormKind::Empty) return;
+        c.args.gamma = gamma ? gamma->data : nullptr;
+        c.args.beta = beta ? beta->data : nullptr;
+        c.args.eps = eps;
+        // vector loads of gamma/beta need 16-byte alignment too
+        if (c.plan.vec > 1 && (((uintptr_t)c.args.gamma | (uintptr_t)c.args.beta) % 16) != 0) {
+            c.plan.vec = 1;
+            if (c.plan.kind == NormKind::RowReg) c.plan.kind = NormKind::Generic;
+        }
+        NormLaunchFn fn = norm_launcher_for(NORM_LAYERNORM, in->dtype);
+        if (!fn) fail(HPT_ERR_DTYPE, "layernorm: unsupported dtype %s", dtype_name(in->dtype));
+        use_device(dev);
+        fn(c.plan, c.args, (hipStream_t)stream);
+        check_launch("layernorm");
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,138 @@
+// Shared host-side declarations of libhpt_hip: error transport, coalesced
+// dimension lists, and the plans the host logic hands to the kernel launchers.
+#pragma once
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "hpt_hip.h"
+
+namespace hpt {
+
+constexpr int kMaxDims = 8;   // coalesced dims per group (kept / reduced) a kernel can walk
+constexpr int kMaxRank = 32;  // rank of a view accepted at the ABI
+
+// Thrown by host logic and launchers; the C ABI wrappers turn it into a status
+// code plus the thread-local message.
+struct Error {
+    int code;
+    std::string msg;
+};
+
+[[noreturn]] inline void fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    throw Error{code, buf};
+}
+
+// A list of (size, stride) pairs, outermost first. Strides are in elements of
+// the view they came from and may be negative (reversed slices) or zero.
+struct Dims {
+    int n = 0;
+    int64_t size[kMaxDims] = {};
+    int64_t stride[kMaxDims] = {};
+    int64_t count() const {
+        int64_t c = 1;
+        for (int i = 0; i < n; ++i) c *= size[i];
+        return c;
+    }
+};
+
+inline size_t dtype_size(int dt) {
+    switch (dt) {
+        case HPT_BOOL: case HPT_I8: case HPT_U8: return 1;
+        case HPT_I16: case HPT_U16: case HPT_F16: case HPT_BF16: return 2;
+        case HPT_I32: case HPT_U32: case HPT_F32: return 4;
+        case HPT_I64: case HPT_U64: case HPT_F64: return 8;
+        default: return 0;
+    }
+}
+
+inline const char* dtype_name(int dt) {
+    static const char* names[] = {"bool", "i8", "i16", "i32", "i64", "u8", "u16",
+                                  "u32", "u64", "f16", "bf16", "f32", "f64"};
+    return (dt >= 0 && dt < HPT_DTYPE_COUNT) ? names[dt] : "?";
+}
+
+inline bool is_float_dtype(int dt) {
+    return dt == HPT_F16 || dt == HPT_BF16 || dt == HPT_F32 || dt == HPT_F64;
+}
+
+// ---- host shape logic (layout.cpp) ---------------------------------------
+
+// process_axes of the reference: wrap negatives, reject out-of-range and
+// duplicates. Returns normalised axes in the caller's order.
+void process_axes(const int64_t* axes, int naxes, int ndim, int64_t* out);
+
+// Output dtype of reduce op `op` on input dtype `in`.
+int reduce_out_dtype(int op, int in);
+
+enum class ReduceKind {
+    Empty,     // no output elements: nothing to launch
+    Identity,  // outputs exist but nothing is reduced into them (a reduced dim has size 0)
+    Row,       // lanes walk the reduced index space (the reduced group owns the smallest stride)
+    Col        // lanes walk the outputs (a kept dim owns the smallest stride)
+};
+
+struct ReducePlan {
+    ReduceKind kind = ReduceKind::Empty;
+    int64_t K = 0;  // number of outputs
+    int64_t R = 0;  // number of elements reduced into each output
+    Dims kept;      // kept dims, logical order, coalesced
+    Dims red;       // reduced dims, sorted by |stride| descending, coalesced
+    // launch shape
+    int vec = 1;     // elements per vector load
+    int tpr = 1;     // Row: threads cooperating on one output (power of two)
+    int rpb = 1;     // Row: outputs per block
+    int bx = 1;      // Col: lanes along the outputs
+    int by = 1;      // Col: thread rows that split the reduced range inside a block
+    int split = 1;   // blocks that share one output (second stage combines them)
+    int split_q = 1; // Row: how `split` divides the outer reduced dims ...
+    int split_i = 1; // ... and the innermost reduced dim (split = split_q * split_i)
+    int64_t chunk = 0;  // Col: reduced indices per split
+};
+
+// Build the plan for reducing `axes` (already normalised) of a view.
+// `elem_size` and `data` decide whether 128-bit loads are legal; `acc_size` is
+// the size of one accumulator (bounds the LDS a column kernel may use).
+ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* strides, int ndim,
+                       const int64_t* axes, int naxes, size_t elem_size, size_t acc_size);
+
+std::string describe(const ReducePlan& p);
+
+enum class NormKind {
+    Empty,
+    RowReg,     // a row sits in the registers of `tpr` threads; one HBM read, one write
+    RowStream,  // rows too long for registers: statistics pass, then a second read
+    Col,        // the normalised axis is strided in input and output alike; lanes walk the inner dim
+    Transposed, // input contiguous along the rows, output along the axis: statistics + LDS tile transpose
+    Generic     // anything else: one block per row, per-element offset arithmetic
+};
+
+struct NormPlan {
+    NormKind kind = NormKind::Empty;
+    int64_t rows = 0, cols = 0;
+    Dims kept_in;        // input strides of the row dims (logical order, coalesced with the output)
+    Dims kept_out;       // output strides of the same dims
+    Dims norm_in;        // input (size, stride) of the normalised dims, logical order, coalesced
+    int64_t out_axis_stride = 1;  // output stride between consecutive elements of a row
+    int vec = 1;
+    int tpr = 1;      // threads per row (RowReg / RowStream / Generic)
+    int rpb = 1;      // rows per block
+    int nchunk = 1;   // RowReg: vectors held per thread
+    int64_t inner = 1;  // Col: size of the contiguous inner dim the lanes walk
+};
+
+// axis >= 0: softmax-style single axis; n_norm_dims > 0: trailing dims (layernorm).
+NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t* shape,
+                        const int64_t* strides, int ndim, int64_t axis, int n_norm_dims,
+                        size_t elem_size);
+
+std::string describe(const NormPlan& p);
+
+}  // namespace hpt

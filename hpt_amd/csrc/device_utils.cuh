@@ -1,0 +1,187 @@
+// Device-side building blocks shared by every kernel of libhpt_hip (gfx950):
+// element types, 128-bit vector access, index arithmetic over coalesced
+// dimension lists, and wavefront-64 / workgroup combines.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "common.hpp"
+
+namespace hpt {
+
+// ---- element types --------------------------------------------------------
+
+struct bool8 { uint8_t v; };
+struct bf16_t { uint16_t bits; };
+using f16_t = _Float16;
+
+template <int DT> struct DType;
+template <> struct DType<HPT_BOOL> { using type = bool8; };
+template <> struct DType<HPT_I8> { using type = int8_t; };
+template <> struct DType<HPT_I16> { using type = int16_t; };
+template <> struct DType<HPT_I32> { using type = int32_t; };
+template <> struct DType<HPT_I64> { using type = int64_t; };
+template <> struct DType<HPT_U8> { using type = uint8_t; };
+template <> struct DType<HPT_U16> { using type = uint16_t; };
+template <> struct DType<HPT_U32> { using type = uint32_t; };
+template <> struct DType<HPT_U64> { using type = uint64_t; };
+template <> struct DType<HPT_F16> { using type = f16_t; };
+template <> struct DType<HPT_BF16> { using type = bf16_t; };
+template <> struct DType<HPT_F32> { using type = float; };
+template <> struct DType<HPT_F64> { using type = double; };
+
+__device__ __forceinline__ float bf16_to_float(bf16_t h) {
+    return __uint_as_float((uint32_t)h.bits << 16);
+}
+// round-to-nearest-even, NaN stays a quiet NaN
+__device__ __forceinline__ bf16_t float_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    bf16_t r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        r.bits = (uint16_t)((u >> 16) | 0x0040u);
+    } else {
+        u += 0x7fffu + ((u >> 16) & 1u);
+        r.bits = (uint16_t)(u >> 16);
+    }
+    return r;
+}
+
+// Per element type: the type arithmetic is carried out in (`Wide`), the type
+// order comparisons are carried out in (`Cmp`), and conversions.
+//   floats  : f16/bf16/f32 compute in float, f64 in double
+//   integers: two's-complement wrapping arithmetic, done on unsigned words
+//             (hpt-types/src/scalars/impls.rs:31-48 uses wrapping_add/mul)
+template <class T> struct Elem;
+
+#define HPT_INT_ELEM(T, W, C, SIGNED)                                                    \
+    template <> struct Elem<T> {                                                         \
+        using Wide = W;                                                                  \
+        using Cmp = C;                                                                   \
+        static constexpr bool is_float = false;                                          \
+        static constexpr bool is_signed = SIGNED;                                        \
+        static constexpr bool is_bool = false;                                           \
+        __device__ static __forceinline__ W widen(T x) { return (W)(C)x; }               \
+        __device__ static __forceinline__ T narrow(W x) { return (T)x; }                 \
+        __device__ static __forceinline__ C cmp(T x) { return (C)x; }                    \
+        __device__ static __forceinline__ T from_cmp(C x) { return (T)x; }               \
+        __device__ static __forceinline__ bool is_nan(T) { return false; }               \
+        __device__ static __forceinline__ bool truthy(T x) { return x != 0; }            \
+    };
+HPT_INT_ELEM(int8_t, uint32_t, int32_t, true)
+HPT_INT_ELEM(int16_t, uint32_t, int32_t, true)
+HPT_INT_ELEM(int32_t, uint32_t, int32_t, true)
+HPT_INT_ELEM(int64_t, uint64_t, int64_t, true)
+HPT_INT_ELEM(uint8_t, uint32_t, uint32_t, false)
+HPT_INT_ELEM(uint16_t, uint32_t, uint32_t, false)
+HPT_INT_ELEM(uint32_t, uint32_t, uint32_t, false)
+HPT_INT_ELEM(uint64_t, uint64_t, uint64_t, false)
+#undef HPT_INT_ELEM
+
+template <> struct Elem<bool8> {
+    using Wide = uint32_t;
+    using Cmp = uint32_t;
+    static constexpr bool is_float = false;
+    static constexpr bool is_signed = false;
+    static constexpr bool is_bool = true;
+    __device__ static __forceinline__ uint32_t widen(bool8 x) { return x.v != 0; }
+    __device__ static __forceinline__ bool8 narrow(uint32_t x) { return bool8{(uint8_t)(x != 0)}; }
+    __device__ static __forceinline__ uint32_t cmp(bool8 x) { return x.v != 0; }
+    __device__ static __forceinline__ bool8 from_cmp(uint32_t x) { return bool8{(uint8_t)(x != 0)}; }
+    __device__ static __forceinline__ bool is_nan(bool8) { return false; }
+    __device__ static __forceinline__ bool truthy(bool8 x) { return x.v != 0; }
+};
+
+#define HPT_FLOAT_ELEM(T, W, TOW, FROMW)                                                 \
+    template <> struct Elem<T> {                                                         \
+        using Wide = W;                                                                  \
+        using Cmp = W;                                                                   \
+        static constexpr bool is_float = true;                                           \
+        static constexpr bool is_signed = true;                                          \
+        static constexpr bool is_bool = false;                                           \
+        __device__ static __forceinline__ W widen(T x) { return TOW; }                   \
+        __device__ static __forceinline__ T narrow(W x) { return FROMW; }                \
+        __device__ static __forceinline__ W cmp(T x) { return widen(x); }                \
+        __device__ static __forceinline__ T from_cmp(W x) { return narrow(x); }          \
+        __device__ static __forceinline__ bool is_nan(T x) { W w = widen(x); return w != w; } \
+        __device__ static __forceinline__ bool truthy(T x) { return widen(x) != (W)0; }  \
+    };
+HPT_FLOAT_ELEM(f16_t, float, (float)x, (f16_t)x)
+HPT_FLOAT_ELEM(bf16_t, float, bf16_to_float(x), float_to_bf16(x))
+HPT_FLOAT_ELEM(float, float, x, x)
+HPT_FLOAT_ELEM(double, double, x, x)
+#undef HPT_FLOAT_ELEM
+
+// ---- vector access -----------------------------------------------------------
+
+template <class T, int N> struct alignas(sizeof(T) * N) Pack { T v[N]; };
+
+template <class T, int N>
+__device__ __forceinline__ Pack<T, N> load_pack(const T* p) {
+    return *reinterpret_cast<const Pack<T, N>*>(p);
+}
+template <class T, int N>
+__device__ __forceinline__ void store_pack(T* p, const Pack<T, N>& v) {
+    *reinterpret_cast<Pack<T, N>*>(p) = v;
+}
+
+// ---- index arithmetic -----------------------------------------------------
+
+// Offset (in elements) of linear index `idx` over dims `d`, outermost first.
+__device__ __forceinline__ int64_t offset_of(const Dims& d, int64_t idx) {
+    int64_t off = 0;
+    if (((uint64_t)idx >> 32) == 0) {
+        uint32_t i32 = (uint32_t)idx;
+        for (int i = d.n - 1; i > 0; --i) {
+            uint32_t s = (uint32_t)d.size[i];
+            uint32_t q = i32 / s;
+            off += (int64_t)(i32 - q * s) * d.stride[i];
+            i32 = q;
+        }
+        if (d.n > 0) off += (int64_t)i32 * d.stride[0];
+    } else {
+        for (int i = d.n - 1; i > 0; --i) {
+            int64_t s = d.size[i];
+            int64_t q = idx / s;
+            off += (idx - q * s) * d.stride[i];
+            idx = q;
+        }
+        if (d.n > 0) off += idx * d.stride[0];
+    }
+    return off;
+}
+
+// ---- wavefront / workgroup combines ---------------------------------------
+
+template <class A> __device__ __forceinline__ A shfl_xor_any(A v, int mask) {
+    static_assert(sizeof(A) % 4 == 0, "shuffle works on 32-bit words");
+    constexpr int W = sizeof(A) / 4;
+    union { A a; int w[W]; } in, out;
+    in.a = v;
+#pragma unroll
+    for (int i = 0; i < W; ++i) out.w[i] = __shfl_xor(in.w[i], mask, 64);
+    return out.a;
+}
+
+// All-reduce over aligned groups of `width` consecutive lanes (power of two, <= 64).
+template <class Op, class A> __device__ __forceinline__ A group_reduce(A v, int width) {
+    for (int m = width >> 1; m > 0; m >>= 1) v = Op::comb(v, shfl_xor_any(v, m));
+    return v;
+}
+
+// All-reduce over the whole workgroup (blockDim.x * blockDim.y threads, a
+// multiple of 64). `smem` must hold one A per wavefront (<= 16).
+template <class Op, class A> __device__ __forceinline__ A block_reduce(A v, A* smem) {
+    const int tid = threadIdx.y * blockDim.x + threadIdx.x;
+    const int nwaves = (blockDim.x * blockDim.y) >> 6;
+    v = group_reduce<Op>(v, 64);
+    __syncthreads();  // protect smem from a previous use
+    if ((tid & 63) == 0) smem[tid >> 6] = v;
+    __syncthreads();
+    A r = smem[0];
+    for (int w = 1; w < nwaves; ++w) r = Op::comb(r, smem[w]);
+    return r;
+}
+
+}  // namespace hpt

@@ -1,0 +1,382 @@
+// Host-side shape logic: axis normalisation, dimension coalescing and the
+// choice of kernel family and launch shape for reductions and normalisations.
+//
+// The reference prepares a reduction by coalescing dims, grouping them by
+// "reduced or kept" and permuting the reduced axes last
+// (hpt/src/backends/cpu/utils/reduce/reduce_template.rs:165-253,
+// hpt/src/backends/common/reduce.rs:44-96,
+// hpt/src/backends/cpu/utils/reduce/reduce_utils.rs:23-56) and then splits on
+// "does a reduced axis have stride 1" (hpt/src/backends/common/reduce.rs:24-33).
+// The same preparation is done here, generalised to any strides: whichever
+// group (kept or reduced) owns the smallest stride decides which way the lanes
+// of a wavefront run, so that they always walk memory in address order.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+
+#include "common.hpp"
+
+namespace hpt {
+
+void process_axes(const int64_t* axes, int naxes, int ndim, int64_t* out) {
+    for (int i = 0; i < naxes; ++i) {
+        int64_t a = axes[i];
+        for (int j = 0; j < i; ++j)
+            if (axes[j] == a) fail(HPT_ERR_PARAM, "Axis %lld is duplicated", (long long)a);
+        int64_t v = a < 0 ? a + ndim : a;
+        if (ndim > 0 && (v < 0 || v >= ndim))
+            fail(HPT_ERR_SHAPE, "Dimension out of range: expected in 0..%d, got %lld", ndim,
+                 (long long)v);
+        out[i] = v;
+    }
+    // Two spellings of one axis (-1 and ndim-1) are the same axis.
+    for (int i = 0; i < naxes; ++i)
+        for (int j = 0; j < i; ++j)
+            if (out[j] == out[i]) fail(HPT_ERR_PARAM, "Axis %lld is duplicated", (long long)axes[i]);
+}
+
+int reduce_out_dtype(int op, int in) {
+    if (in < 0 || in >= HPT_DTYPE_COUNT) fail(HPT_ERR_DTYPE, "invalid dtype %d", in);
+    switch (op) {
+        case HPT_SUM: case HPT_PROD: case HPT_MAX: case HPT_MIN: case HPT_NANSUM:
+        case HPT_NANPROD: case HPT_REDUCEL1: case HPT_SUM_SQUARE:
+            return in;
+        case HPT_ALL: case HPT_ANY:
+            return HPT_BOOL;
+        case HPT_MEAN: case HPT_REDUCEL2: case HPT_REDUCEL3: case HPT_LOGSUMEXP:
+            // FloatBinaryType<T>: hpt-types/src/promotion/normal_promote/_*.rs
+            switch (in) {
+                case HPT_BOOL: case HPT_I8: case HPT_I16: case HPT_U8: case HPT_U16: case HPT_F16:
+                    return HPT_F16;
+                case HPT_I32: case HPT_U32: case HPT_F32: return HPT_F32;
+                case HPT_BF16: return HPT_BF16;
+                default: return HPT_F64;
+            }
+        default:
+            fail(HPT_ERR_PARAM, "invalid reduce op %d", op);
+    }
+}
+
+static int64_t iabs(int64_t v) { return v < 0 ? -v : v; }
+
+static int pow2_floor(int64_t v) {
+    int p = 1;
+    while ((int64_t)p * 2 <= v) p *= 2;
+    return p;
+}
+static int pow2_ceil(int64_t v) {
+    int p = 1;
+    while (p < v) p *= 2;
+    return p;
+}
+
+// Append (size, stride) to `d`, merging with the previous entry when the two
+// are one dense run: prev.stride == stride * size.
+static void push_merged(Dims& d, int64_t size, int64_t stride) {
+    if (size == 1) return;
+    if (d.n > 0 && d.stride[d.n - 1] == stride * size) {
+        d.size[d.n - 1] *= size;
+        d.stride[d.n - 1] = stride;
+        return;
+    }
+    if (d.n == kMaxDims)
+        fail(HPT_ERR_SHAPE, "view has more than %d non-mergeable dims in one group", kMaxDims);
+    d.size[d.n] = size;
+    d.stride[d.n] = stride;
+    ++d.n;
+}
+
+// Largest power-of-two vector width (in elements, at most 16 bytes) that every
+// access of the form data + sum(idx_i * stride_i) + inner*1 can use: the base
+// address, every other stride and the inner length must be multiples of it.
+// Kernels are built for two widths only: the full 16-byte vector or one element.
+static int legal_vec(const void* data, size_t elem_size, int64_t inner_len, const Dims& a,
+                     const Dims& b, int skip_a_last, int skip_b_last) {
+    const int v = (int)(16 / elem_size);
+    if (v <= 1) return 1;
+    bool ok = ((uintptr_t)data % 16) == 0 && inner_len % v == 0;
+    for (int i = 0; ok && i < a.n - skip_a_last; ++i) ok = a.stride[i] % v == 0;
+    for (int i = 0; ok && i < b.n - skip_b_last; ++i) ok = b.stride[i] % v == 0;
+    return ok ? v : 1;
+}
+
+// How many blocks of 256 threads keep an MI355X busy: 256 CUs, each able to
+// hold 8 such blocks.
+constexpr int64_t kBlocksToFill = 2048;
+
+ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* strides, int ndim,
+                       const int64_t* axes, int naxes, size_t elem_size, size_t acc_size) {
+    ReducePlan p;
+    bool is_red[kMaxRank] = {};
+    for (int i = 0; i < naxes; ++i) is_red[axes[i]] = true;
+
+    p.K = 1;
+    p.R = 1;
+    for (int i = 0; i < ndim; ++i) (is_red[i] ? p.R : p.K) *= shape[i];
+    if (p.K == 0) {
+        p.kind = ReduceKind::Empty;
+        return p;
+    }
+    if (p.R == 0) {
+        p.kind = ReduceKind::Identity;
+        return p;
+    }
+
+    // kept dims keep their logical order (the output is contiguous in it)
+    for (int i = 0; i < ndim; ++i)
+        if (!is_red[i]) push_merged(p.kept, shape[i], strides[i]);
+    // reduced dims may be visited in any order: sort by |stride| descending
+    int order[kMaxRank], nr = 0;
+    for (int i = 0; i < ndim; ++i)
+        if (is_red[i] && shape[i] != 1) order[nr++] = i;
+    std::stable_sort(order, order + nr,
+                     [&](int a, int b) { return iabs(strides[a]) > iabs(strides[b]); });
+    for (int i = 0; i < nr; ++i) push_merged(p.red, shape[order[i]], strides[order[i]]);
+
+    int64_t sr = p.red.n ? iabs(p.red.stride[p.red.n - 1]) : INT64_MAX;
+    int64_t sk = p.kept.n ? iabs(p.kept.stride[p.kept.n - 1]) : INT64_MAX;
+
+    if (p.red.n > 0 && (p.kept.n == 0 || sr <= sk)) {
+        // ---- Row: lanes walk the reduced index space ---------------------
+        p.kind = ReduceKind::Row;
+        int64_t rin = p.red.size[p.red.n - 1];
+        p.vec = 1;
+        if (p.red.stride[p.red.n - 1] == 1)
+            p.vec = legal_vec(data, elem_size, rin, p.kept, p.red, 0, 1);
+        int64_t nv = p.R / p.vec;  // vector loads per output
+        // aim at about 8 loads per thread before widening the group
+        p.tpr = (int)std::min<int64_t>(1024, pow2_ceil((nv + 7) / 8));
+        if (p.tpr > 64 && p.tpr < 256) p.tpr = 256;  // above a wave, whole blocks only
+        int block = std::max(256, p.tpr);
+        p.rpb = block / p.tpr;
+        int64_t blocks = (p.K + p.rpb - 1) / p.rpb;
+        p.split = p.split_q = p.split_i = 1;
+        if (blocks < kBlocksToFill / 2) {
+            // too few outputs to fill the chip: several blocks of 256 threads per
+            // output, each with at least 8 vector loads per thread
+            int64_t want = (kBlocksToFill * 2 + p.K - 1) / p.K;
+            int64_t can = nv / (256 * 8);
+            int64_t split = std::min<int64_t>(std::min(want, can), 4096);
+            if (split > 1) {
+                p.tpr = 256;
+                p.rpb = 1;
+                int64_t rout = p.R / rin;
+                int64_t sq = std::min(split, rout);
+                int64_t si = std::max<int64_t>(1, split / sq);
+                int64_t can_i = std::max<int64_t>(1, (rin / p.vec) / p.tpr);
+                si = std::min(si, can_i);
+                p.split_q = (int)sq;
+                p.split_i = (int)si;
+                p.split = (int)(sq * si);
+            }
+        }
+    } else {
+        // ---- Col: lanes walk the outputs -----------------------------------
+        p.kind = ReduceKind::Col;
+        int64_t kin = p.kept.n ? p.kept.size[p.kept.n - 1] : 1;
+        p.vec = 1;
+        if (p.kept.n && p.kept.stride[p.kept.n - 1] == 1)
+            p.vec = legal_vec(data, elem_size, kin, p.kept, p.red, 1, 0);
+        int64_t kv = p.K / p.vec;  // vector columns
+        p.bx = (int)std::min<int64_t>(64, pow2_ceil(kv));
+        int64_t xblocks = (kv + p.bx - 1) / p.bx;
+        // split the reduced range over thread rows while each keeps >= 8 loads
+        int by = 256 / p.bx;
+        int64_t waves_x = xblocks * std::max(1, p.bx / 64);
+        int want_by = pow2_ceil((kBlocksToFill * 4 + waves_x - 1) / waves_x);
+        int can_by = pow2_floor(std::max<int64_t>(1, p.R / 8));
+        by = std::max(by, std::min(16 * 64 / p.bx, want_by));
+        by = std::min(by, std::max(1, can_by));
+        by = std::min(by, 1024 / p.bx);
+        // the thread rows meet in LDS: keep bx*by*vec accumulators within 64 KiB
+        while (by > 1 && (size_t)p.bx * by * p.vec * acc_size > (64u << 10)) by /= 2;
+        p.by = std::max(1, by);
+        p.split = 1;
+        int64_t blocks = xblocks;
+        int64_t per_thread = p.R / p.by;
+        if (blocks * p.by * p.bx / 256 < kBlocksToFill / 2 && per_thread > 32) {
+            int64_t want = (kBlocksToFill * 256 / ((int64_t)p.bx * p.by) + blocks - 1) / blocks;
+            int64_t can = per_thread / 16;
+            // bound the partial buffer: K * split accumulators of 16 bytes <= 64 MiB
+            int64_t cap = std::max<int64_t>(1, (64ll << 20) / 16 / p.K);
+            p.split = (int)std::max<int64_t>(1, std::min(std::min(want, can), std::min<int64_t>(cap, 1024)));
+        }
+        p.chunk = (p.R + p.split - 1) / p.split;
+    }
+    return p;
+}
+
+static void describe_dims(std::string& s, const char* name, const Dims& d) {
+    s += name;
+    s += "=[";
+    char buf[64];
+    for (int i = 0; i < d.n; ++i) {
+        snprintf(buf, sizeof buf, "%s%lld:%lld", i ? "," : "", (long long)d.size[i],
+                 (long long)d.stride[i]);
+        s += buf;
+    }
+    s += "]";
+}
+
+std::string describe(const ReducePlan& p) {
+    char buf[256];
+    std::string s;
+    switch (p.kind) {
+        case ReduceKind::Empty: return "empty";
+        case ReduceKind::Identity: return "identity";
+        case ReduceKind::Row:
+            snprintf(buf, sizeof buf, "row vec=%d tpr=%d rpb=%d rows=%lld cols=%lld split=%d(%dx%d) ",
+                     p.vec, p.tpr, p.rpb, (long long)p.K, (long long)p.R, p.split, p.split_q,
+                     p.split_i);
+            break;
+        case ReduceKind::Col:
+            snprintf(buf, sizeof buf, "col vec=%d bx=%d by=%d outs=%lld red=%lld split=%d ", p.vec,
+                     p.bx, p.by, (long long)p.K, (long long)p.R, p.split);
+            break;
+    }
+    s = buf;
+    describe_dims(s, "kept", p.kept);
+    s += " ";
+    describe_dims(s, "red", p.red);
+    return s;
+}
+
+// ---- normalisation ---------------------------------------------------------
+
+NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t* shape,
+                        const int64_t* strides, int ndim, int64_t axis, int n_norm_dims,
+                        size_t elem_size) {
+    NormPlan p;
+    int64_t total = 1;
+    for (int i = 0; i < ndim; ++i) total *= shape[i];
+    if (total == 0 || ndim == 0) {
+        p.kind = NormKind::Empty;
+        return p;
+    }
+    // contiguous output strides
+    int64_t ostr[kMaxRank];
+    {
+        int64_t s = 1;
+        for (int i = ndim - 1; i >= 0; --i) {
+            ostr[i] = s;
+            s *= shape[i];
+        }
+    }
+    bool is_norm[kMaxRank] = {};
+    if (n_norm_dims > 0)
+        for (int i = ndim - n_norm_dims; i < ndim; ++i) is_norm[i] = true;
+    else
+        is_norm[axis] = true;
+
+    // Row dims: merged only where input AND output are both one dense run.
+    p.rows = 1;
+    for (int i = 0; i < ndim; ++i) {
+        if (is_norm[i]) continue;
+        p.rows *= shape[i];
+        if (shape[i] == 1) continue;
+        int n = p.kept_in.n;
+        if (n > 0 && p.kept_in.stride[n - 1] == strides[i] * shape[i] &&
+            p.kept_out.stride[n - 1] == ostr[i] * shape[i]) {
+            p.kept_in.size[n - 1] *= shape[i];
+            p.kept_in.stride[n - 1] = strides[i];
+            p.kept_out.size[n - 1] *= shape[i];
+            p.kept_out.stride[n - 1] = ostr[i];
+        } else {
+            if (n == kMaxDims)
+                fail(HPT_ERR_SHAPE, "view has more than %d non-mergeable row dims", kMaxDims);
+            p.kept_in.size[n] = p.kept_out.size[n] = shape[i];
+            p.kept_in.stride[n] = strides[i];
+            p.kept_out.stride[n] = ostr[i];
+            p.kept_in.n = p.kept_out.n = n + 1;
+        }
+    }
+    // Normalised dims keep their logical order (gamma/beta and the output index by it).
+    p.cols = 1;
+    for (int i = 0; i < ndim; ++i) {
+        if (!is_norm[i]) continue;
+        p.cols *= shape[i];
+        push_merged(p.norm_in, shape[i], strides[i]);
+    }
+    // Output stride along the (flattened) normalised index.
+    p.out_axis_stride = 1;
+    if (n_norm_dims <= 0) p.out_axis_stride = ostr[axis];
+    if (p.cols == 1) {
+        // one element per row: still a legal call; the generic kernel handles it
+        p.norm_in.n = 1;
+        p.norm_in.size[0] = 1;
+        p.norm_in.stride[0] = 1;
+    }
+
+    const int64_t sa = p.norm_in.n == 1 ? p.norm_in.stride[0] : 0;  // input stride along the row
+    const int max_vec = (int)(16 / elem_size);
+
+    // default: one group of lanes per row, striding along the row
+    p.kind = NormKind::Generic;
+    p.vec = 1;
+    p.tpr = (int)std::min<int64_t>(1024, pow2_ceil((p.cols + 3) / 4));
+    if (p.tpr > 64 && p.tpr < 256) p.tpr = 256;
+    p.rpb = std::max(1, 256 / p.tpr);
+
+    if (p.norm_in.n == 1 && p.out_axis_stride == 1) {
+        // rows are contiguous in the output
+        bool transposed = sa != 1 && p.kept_in.n >= 1 && p.kept_in.stride[p.kept_in.n - 1] == 1 &&
+                          p.kept_in.size[p.kept_in.n - 1] >= 64 && p.cols >= 64 && sa > 0;
+        if (transposed) {
+            p.kind = NormKind::Transposed;
+            return p;
+        }
+        if (sa >= 1 && sa <= 4) {
+            // vector width: input and output must both allow it
+            int v = 1;
+            if (sa == 1) {
+                Dims none;
+                int vi = legal_vec(in_data, elem_size, p.cols, p.kept_in, none, 0, 0);
+                int vo = legal_vec(out_data, elem_size, p.cols, p.kept_out, none, 0, 0);
+                v = std::min(std::min(vi, vo), max_vec);
+            }
+            p.vec = v;
+            int64_t nv = p.cols / v;
+            if (nv <= 8192) {
+                p.kind = NormKind::RowReg;
+                p.tpr = (int)std::min<int64_t>(1024, pow2_ceil((nv + 3) / 4));
+                if (p.tpr > 64 && p.tpr < 256) p.tpr = 256;
+                int64_t nc = (nv + p.tpr - 1) / p.tpr;
+                p.nchunk = std::max(1, pow2_ceil(nc));
+                int block = std::max(256, p.tpr);
+                p.rpb = block / p.tpr;
+            } else {
+                p.kind = NormKind::RowStream;
+                p.tpr = 1024;
+                p.rpb = 1;
+            }
+            return p;
+        }
+    }
+    if (p.norm_in.n == 1 && p.out_axis_stride > 1) {
+        // normalised axis is not the last one: lanes walk the trailing dims
+        p.kind = NormKind::Col;
+        p.inner = p.out_axis_stride;
+        if (p.rows >= 1024) {
+            // every lane owns one row; neighbouring lanes are neighbours in memory
+            p.tpr = 1;
+            p.rpb = 256;
+        }
+        return p;
+    }
+    return p;
+}
+
+std::string describe(const NormPlan& p) {
+    static const char* names[] = {"empty", "rowreg", "rowstream", "col", "transposed", "generic"};
+    char buf[256];
+    snprintf(buf, sizeof buf, "%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
+             names[(int)p.kind], (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             p.nchunk, (long long)p.out_axis_stride);
+    std::string s = buf;
+    describe_dims(s, "rows_in", p.kept_in);
+    s += " ";
+    describe_dims(s, "norm_in", p.norm_in);
+    return s;
+}
+
+}  // namespace hpt

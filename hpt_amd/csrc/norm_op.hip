@@ -1,0 +1,61 @@
+// One normalisation kind (softmax, log_softmax or layernorm) for the four
+// float dtypes. Compiled once per kind with -DHPT_NORM_KIND=<0|1|2>.
+#include "norm_kernels.cuh"
+
+#ifndef HPT_NORM_KIND
+#error "compile with -DHPT_NORM_KIND=<kind>"
+#endif
+
+namespace hpt {
+
+namespace {
+
+constexpr int KIND = HPT_NORM_KIND;
+
+inline int ilog2(int v) {
+    int l = 0;
+    while ((1 << l) < v) ++l;
+    return l;
+}
+
+template <class T, int VEC>
+void launch_row_reg(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block, hipStream_t st) {
+    switch (p.nchunk) {
+        case 1: row_reg_kernel<KIND, T, VEC, 1><<<grid, block, 0, st>>>(a); break;
+        case 2: row_reg_kernel<KIND, T, VEC, 2><<<grid, block, 0, st>>>(a); break;
+        case 4: row_reg_kernel<KIND, T, VEC, 4><<<grid, block, 0, st>>>(a); break;
+        case 8: row_reg_kernel<KIND, T, VEC, 8><<<grid, block, 0, st>>>(a); break;
+        default: fail(HPT_ERR_KERNEL, "row_reg: unsupported chunk count %d", p.nchunk);
+    }
+}
+
+template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) {
+    constexpr int FULL = 16 / sizeof(T);
+    if (p.kind == NormKind::Empty) return;
+    a.tpr = p.tpr;
+    a.tpr_log2 = ilog2(p.tpr);
+    a.rpb = p.rpb;
+    dim3 grid((unsigned)((p.rows + p.rpb - 1) / p.rpb));
+    dim3 block((unsigned)(p.tpr * p.rpb));
+    if (p.kind == NormKind::RowReg) {
+        if (p.vec == FULL) launch_row_reg<T, FULL>(p, a, grid, block, st);
+        else launch_row_reg<T, 1>(p, a, grid, block, st);
+        return;
+    }
+    if (p.vec == FULL) row_stream_kernel<KIND, T, FULL><<<grid, block, 0, st>>>(a);
+    else row_stream_kernel<KIND, T, 1><<<grid, block, 0, st>>>(a);
+}
+
+}  // namespace
+
+template <> NormLaunchFn norm_launcher<HPT_NORM_KIND>(int dtype) {
+    switch (dtype) {
+        case HPT_F16: return &launch_t<f16_t>;
+        case HPT_BF16: return &launch_t<bf16_t>;
+        case HPT_F32: return &launch_t<float>;
+        case HPT_F64: return &launch_t<double>;
+        default: return nullptr;
+    }
+}
+
+}  // namespace hpt

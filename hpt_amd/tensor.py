@@ -1,0 +1,475 @@
+"""Host-side mirror of Hpt's tensor API for the reduction / normalisation path.
+
+`Tensor` plays the role of `hpt::Tensor<T, B, DEVICE>` (hpt/src/tensor.rs:31-37):
+a shape + element strides + an already-offset data pointer over shared storage.
+Two backends exist here:
+
+  * "cpu": a host tensor over a numpy buffer. It only carries data; like the
+    reference's `to_cuda` (hpt/src/backends/cpu/tensor_impls.rs:295-313) the way
+    onto the device is `to_hip()`. No operator runs on it in this package.
+  * "hip": device memory obtained from the caching allocator of libhpt_hip.so.
+    The reduce / normalisation traits of the reference
+    (hpt-traits/src/ops/reduce.rs:6-358, hpt-traits/src/ops/normalization.rs:6-64)
+    are methods of the same names with the same arguments, and every one of them
+    is a call into the C ABI: there is no other execution path.
+
+Views (`permute`, `transpose`, `slice`, `__getitem__`) share storage and follow
+hpt/src/backends/common/shape_manipulate.rs:144-167 and hpt-common/src/slice.rs:41-120.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Iterable, Optional, Sequence
+
+import numpy as np
+
+from . import _ffi
+from ._ffi import ParamError, ShapeError, check, make_view
+
+ALIGN = 64  # every tensor's mem_layout alignment (hpt/src/lib.rs:560)
+
+
+class DType:
+    """hpt_dtype values and their numpy carriers (bf16 travels as uint16 bit patterns)."""
+
+    def __init__(self, code: int, name: str, np_dtype, size: int):
+        self.code, self.name, self.np_dtype, self.size = code, name, np.dtype(np_dtype), size
+
+    def __repr__(self):
+        return f"hpt.{self.name}"
+
+
+bool_ = DType(0, "bool", np.bool_, 1)
+i8 = DType(1, "i8", np.int8, 1)
+i16 = DType(2, "i16", np.int16, 2)
+i32 = DType(3, "i32", np.int32, 4)
+i64 = DType(4, "i64", np.int64, 8)
+u8 = DType(5, "u8", np.uint8, 1)
+u16 = DType(6, "u16", np.uint16, 2)
+u32 = DType(7, "u32", np.uint32, 4)
+u64 = DType(8, "u64", np.uint64, 8)
+f16 = DType(9, "f16", np.float16, 2)
+bf16 = DType(10, "bf16", np.uint16, 2)
+f32 = DType(11, "f32", np.float32, 4)
+f64 = DType(12, "f64", np.float64, 8)
+DTYPES = [bool_, i8, i16, i32, i64, u8, u16, u32, u64, f16, bf16, f32, f64]
+_BY_NP = {d.np_dtype: d for d in DTYPES if d is not bf16}
+
+# hpt_reduce_op
+SUM, PROD, MAX, MIN, MEAN, NANSUM, NANPROD, REDUCEL1, REDUCEL2, REDUCEL3, SUM_SQUARE, LOGSUMEXP, ALL, ANY = range(14)
+
+
+def f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
+    """Round float32 to bfloat16 (nearest even, NaN quieted); returns uint16 bit patterns."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = ((u + (0x7FFF + ((u >> 16) & 1))) >> 16).astype(np.uint16)
+    r[nan] = ((u[nan] >> 16) | 0x0040).astype(np.uint16)
+    return r
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+class _HostStorage:
+    def __init__(self, arr: np.ndarray):
+        self.arr = arr  # C-contiguous 1-D view keeps the buffer alive
+        self.ptr = arr.ctypes.data
+
+
+class _DeviceStorage:
+    """A block owned through the library's caching allocator (hpt-allocator's Backend<B>)."""
+
+    def __init__(self, device: int, nbytes: int, zeroed: bool = False):
+        p = C.c_void_p()
+        check(_ffi.lib().hpt_hip_alloc(device, nbytes, ALIGN, int(zeroed), C.byref(p)))
+        self.ptr = p.value or 0
+        self.nbytes, self.device = nbytes, device
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                _ffi.lib().hpt_hip_free(self.device, C.c_void_p(self.ptr), self.nbytes, ALIGN)
+                self.ptr = 0
+        except Exception:
+            pass
+
+
+def _contiguous_strides(shape: Sequence[int]):
+    st, s = [0] * len(shape), 1
+    for i in range(len(shape) - 1, -1, -1):
+        st[i] = s
+        s *= shape[i]
+    return st
+
+
+def _tdiv(a: int, b: int) -> int:
+    """Integer division truncating toward zero (Rust's `/`)."""
+    q = abs(a) // abs(b)
+    return q if (a < 0) == (b < 0) else -q
+
+
+def _as_axes(axes) -> list:
+    if isinstance(axes, (int, np.integer)):
+        return [int(axes)]
+    return [int(a) for a in axes]
+
+
+class Tensor:
+    def __init__(self, storage, ptr: int, shape, strides, dtype: DType, backend: str, device: int,
+                 parent: Optional[int] = None):
+        self._storage = storage
+        self.ptr = ptr                      # already-offset element pointer (Pointer<T>)
+        self.shape = [int(s) for s in shape]
+        self.strides = [int(s) for s in strides]  # in elements
+        self.dtype = dtype
+        self.backend = backend
+        self.device = device
+        self.parent = parent                # set on views, as _Tensor.parent is
+
+    # ---- construction / transfer --------------------------------------------
+    @classmethod
+    def from_numpy(cls, arr: np.ndarray, dtype: Optional[DType] = None) -> "Tensor":
+        """A host ("cpu") tensor over a copy of `arr`. Pass dtype=bf16 with uint16 bit patterns."""
+        arr = np.ascontiguousarray(arr)
+        if dtype is None:
+            dtype = _BY_NP.get(arr.dtype)
+            if dtype is None:
+                raise _ffi.DTypeError(_ffi.ERR_DTYPE, f"unsupported numpy dtype {arr.dtype}")
+        if arr.dtype != dtype.np_dtype:
+            raise _ffi.DTypeError(_ffi.ERR_DTYPE, f"{dtype} is carried by {dtype.np_dtype}, got {arr.dtype}")
+        flat = arr.reshape(-1).copy()
+        st = _HostStorage(flat)
+        return cls(st, st.ptr, arr.shape, _contiguous_strides(arr.shape), dtype, "cpu", 0)
+
+    @classmethod
+    def empty(cls, shape, dtype: DType, device: int = 0, zeroed: bool = False) -> "Tensor":
+        """TensorCreator::empty for the Hip backend (cuda/tensor_internal/normal_creation.rs:34-69)."""
+        shape = [int(s) for s in shape]
+        n = int(np.prod(shape, dtype=np.int64)) if shape else 1
+        st = _DeviceStorage(device, n * dtype.size, zeroed)
+        return cls(st, st.ptr, shape, _contiguous_strides(shape), dtype, "hip", device)
+
+    def size(self) -> int:
+        return int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
+
+    @property
+    def ndim(self) -> int:
+        return len(self.shape)
+
+    def is_contiguous(self) -> bool:
+        """Layout::is_contiguous (hpt-common/src/layout/layout_utils.rs:363-375)."""
+        expected = 1
+        for d, s in zip(reversed(self.shape), reversed(self.strides)):
+            if d == 0:
+                continue
+            if s != expected:
+                return False
+            expected *= d
+        return True
+
+    def to_hip(self, device: int = 0) -> "Tensor":
+        """to_cuda's twin: allocate on the device, make contiguous if needed, synchronous copy."""
+        if self.backend != "cpu":
+            raise ParamError(_ffi.ERR_PARAM, "to_hip expects a cpu tensor")
+        host = self.numpy()
+        out = Tensor.empty(self.shape, self.dtype, device)
+        check(_ffi.lib().hpt_hip_memcpy_h2d_sync(device, C.c_void_p(out.ptr), C.c_void_p(host.ctypes.data),
+                                                 host.nbytes))
+        return out
+
+    def to_cpu(self) -> "Tensor":
+        """to_cpu (hpt/src/backends/cuda/tensor_impls.rs:142-169): contiguous copy back to the host."""
+        if self.backend != "hip":
+            raise ParamError(_ffi.ERR_PARAM, "to_cpu expects a hip tensor")
+        return Tensor.from_numpy(self.numpy(), self.dtype)
+
+    def numpy(self) -> np.ndarray:
+        """Contiguous numpy copy of this (possibly strided) tensor; bf16 comes back as uint16 bits."""
+        if not self.size():
+            return np.empty(self.shape, self.dtype.np_dtype)
+        st = self._storage
+        if self.backend == "cpu":
+            base = st.arr
+        else:
+            # device: copy the whole allocation once, then gather through the strides
+            raw = np.empty(st.nbytes, np.uint8)
+            check(_ffi.lib().hpt_hip_stream_synchronize(self.device, None))
+            check(_ffi.lib().hpt_hip_memcpy_d2h_sync(self.device, C.c_void_p(raw.ctypes.data),
+                                                     C.c_void_p(st.ptr), st.nbytes))
+            base = raw.view(self.dtype.np_dtype)
+        off = (self.ptr - st.ptr) // self.dtype.size
+        if self.is_contiguous():
+            return base[off:off + self.size()].reshape(self.shape).copy()
+        idx = np.full(self.shape, off, dtype=np.int64)
+        for ax, (d, stride) in enumerate(zip(self.shape, self.strides)):
+            sh = [1] * self.ndim
+            sh[ax] = d
+            idx = idx + (np.arange(d, dtype=np.int64) * stride).reshape(sh)
+        return base[idx]
+
+    # ---- views -----------------------------------------------------------------
+    def _view(self, ptr, shape, strides) -> "Tensor":
+        return Tensor(self._storage, ptr, shape, strides, self.dtype, self.backend, self.device,
+                      parent=self.parent if self.parent is not None else self.ptr)
+
+    def permute(self, axes) -> "Tensor":
+        axes = _as_axes(axes)
+        if sorted(a % max(1, self.ndim) for a in axes) != list(range(self.ndim)):
+            raise ShapeError(_ffi.ERR_SHAPE, f"permute: axes {axes} are not a permutation of 0..{self.ndim}")
+        axes = [a % self.ndim for a in axes]
+        t = Tensor(self._storage, self.ptr, [self.shape[a] for a in axes], [self.strides[a] for a in axes],
+                   self.dtype, self.backend, self.device, parent=self.parent)
+        return t
+
+    def transpose(self, a: int, b: int) -> "Tensor":
+        axes = list(range(self.ndim))
+        axes[a], axes[b] = axes[b], axes[a]
+        return self.permute(axes)
+
+    def t(self) -> "Tensor":
+        return self.permute(list(range(self.ndim))[::-1])
+
+    def slice(self, index: Sequence) -> "Tensor":
+        """slice_process (hpt-common/src/slice.rs:41-120). `index` holds (start, end, step)
+        triples, one per leading dim; end=None means "to the end"."""
+        BIG = 0x7FFFFFFFFFFFFFFF
+        shape, strides, ptr_off = list(self.shape), list(self.strides), 0
+        if len(index) > self.ndim:
+            raise ShapeError(_ffi.ERR_SHAPE, f"index length is greater than the shape length, shape: {self.shape}")
+        for d, (start, end, step) in enumerate(index):
+            dim = self.shape[d]
+            end = dim if end is None or end == BIG else end
+            start = start if start >= 0 else start + dim
+            end = end if end >= 0 else end + dim
+            if start >= dim:
+                start = dim - 1
+            if end > dim:
+                end = dim
+            if step > 0:
+                length = _tdiv(end - start + step - 1, step)
+            elif step < 0:
+                length = _tdiv(end - start + step + 1, step)
+            else:
+                length = 0
+            if length > 0:
+                shape[d] = length
+                ptr_off += start * strides[d]
+                strides[d] *= step
+            else:
+                shape[d] = 0
+        keep = [i for i, s in enumerate(shape) if s != 0]
+        return self._view(self.ptr + ptr_off * self.dtype.size, [shape[i] for i in keep],
+                          [strides[i] for i in keep])
+
+    def __getitem__(self, key) -> "Tensor":
+        if not isinstance(key, tuple):
+            key = (key,)
+        index = []
+        for d, k in enumerate(key):
+            if not isinstance(k, slice):
+                raise ParamError(_ffi.ERR_PARAM, "only slices are supported in __getitem__")
+            step = 1 if k.step is None else k.step
+            if step > 0:
+                start = 0 if k.start is None else k.start
+                end = None if k.stop is None else k.stop
+            else:
+                start = self.shape[d] - 1 if k.start is None else k.start
+                end = -self.shape[d] - 1 if k.stop is None else k.stop
+            index.append((start, end, step))
+        return self.slice(index)
+
+    # ---- ABI plumbing ------------------------------------------------------------
+    def _require_hip(self, what: str):
+        if self.backend != "hip":
+            raise NotImplementedError(
+                f"{what}: this package implements the Hip backend only; move the tensor with to_hip()")
+
+    def _c_view(self):
+        return make_view(self.ptr, self.shape, self.strides, self.dtype.code)
+
+    def _reduce_shape(self, axes, keep_dims: bool):
+        l = _ffi.lib()
+        sh = _ffi.i64_array(self.shape)
+        ax = _ffi.i64_array(axes)
+        out = (C.c_int64 * max(1, self.ndim))()
+        n = C.c_int32()
+        check(l.hpt_hip_reduce_shape(sh, self.ndim, ax, len(axes), int(keep_dims), out, C.byref(n)))
+        return [out[i] for i in range(n.value)]
+
+    def _reduce(self, op: int, axes, keep_dims: bool, init_out: bool = True, out: "Tensor" = None,
+                stream=None) -> "Tensor":
+        self._require_hip("reduce")
+        l = _ffi.lib()
+        axes = _as_axes(axes)
+        od = C.c_int32()
+        check(l.hpt_hip_reduce_out_dtype(op, self.dtype.code, C.byref(od)))
+        out_dtype = DTYPES[od.value]
+        flat_shape = self._reduce_shape(axes, False)
+        final_shape = self._reduce_shape(axes, keep_dims)
+        if out is None:
+            res = Tensor.empty(flat_shape, out_dtype, self.device)
+        else:
+            if not out.is_contiguous():
+                raise ShapeError(_ffi.ERR_SHAPE, "out tensor must be contiguous")
+            res = Tensor(out._storage, out.ptr, flat_shape, _contiguous_strides(flat_shape), out.dtype,
+                         out.backend, out.device)
+            if out.size() != res.size():
+                raise ShapeError(_ffi.ERR_SHAPE,
+                                 f"Size mismatch: expected {res.size()}, got {out.size()}")
+        vin, k1 = self._c_view()
+        vout, k2 = res._c_view()
+        ax = _ffi.i64_array(axes)
+        check(l.hpt_hip_reduce(self.device, stream, op, C.byref(vin), ax, len(axes), int(init_out), C.byref(vout)))
+        del k1, k2
+        return Tensor(res._storage, res.ptr, final_shape, _contiguous_strides(final_shape), res.dtype, "hip",
+                      self.device)
+
+    def _argreduce(self, is_max: bool, axis, keep_dims: bool, stream=None) -> "Tensor":
+        self._require_hip("argreduce")
+        l = _ffi.lib()
+        axes = _as_axes(axis)
+        if len(axes) != 1:
+            raise ParamError(_ffi.ERR_PARAM, "argmax/argmin reduce exactly one axis")
+        flat_shape = self._reduce_shape(axes, False)
+        final_shape = self._reduce_shape(axes, keep_dims)
+        res = Tensor.empty(flat_shape, i64, self.device)
+        vin, k1 = self._c_view()
+        vout, k2 = res._c_view()
+        check(l.hpt_hip_argreduce(self.device, stream, int(is_max), C.byref(vin), axes[0], C.byref(vout)))
+        del k1, k2
+        return Tensor(res._storage, res.ptr, final_shape, _contiguous_strides(final_shape), i64, "hip", self.device)
+
+    # ---- NormalReduce (hpt-traits/src/ops/reduce.rs:45-176) ----------------------
+    def sum(self, axes, keep_dims: bool = False, **kw):
+        return self._reduce(SUM, axes, keep_dims, **kw)
+
+    def sum_(self, axes, keep_dims: bool, init_out: bool, out: "Tensor", **kw):
+        return self._reduce(SUM, axes, keep_dims, init_out=init_out, out=out, **kw)
+
+    def prod(self, axis, keep_dims: bool = False, **kw):
+        return self._reduce(PROD, axis, keep_dims, **kw)
+
+    def min(self, axis, keep_dims: bool = False, **kw):
+        return self._reduce(MIN, axis, keep_dims, **kw)
+
+    def max(self, axis, keep_dims: bool = False, **kw):
+        return self._reduce(MAX, axis, keep_dims, **kw)
+
+    def reducel1(self, axis, keep_dims: bool = False, **kw):
+        return self._reduce(REDUCEL1, axis, keep_dims, **kw)
+
+    def sum_square(self, axis, keep_dims: bool = False, **kw):
+        return self._reduce(SUM_SQUARE, axis, keep_dims, **kw)
+
+    # ---- EvalReduce / NormalEvalReduce (reduce.rs:179-277) -----------------------
+    def all(self, axis, keep_dims: bool = False, **kw):
+        return self._reduce(ALL, axis, keep_dims, **kw)
+
+    def any(self, axis, keep_dims: bool = False, **kw):
+        return self._reduce(ANY, axis, keep_dims, **kw)
+
+    def nansum(self, axes, keep_dims: bool = False, **kw):
+        return self._reduce(NANSUM, axes, keep_dims, **kw)
+
+    def nansum_(self, axes, keep_dims: bool, init_out: bool, out: "Tensor", **kw):
+        return self._reduce(NANSUM, axes, keep_dims, init_out=init_out, out=out, **kw)
+
+    def nanprod(self, axis, keep_dims: bool = False, **kw):
+        return self._reduce(NANPROD, axis, keep_dims, **kw)
+
+    # ---- FloatReduce (reduce.rs:280-358) -----------------------------------------
+    def mean(self, axis, keep_dims: bool = False, **kw):
+        return self._reduce(MEAN, axis, keep_dims, **kw)
+
+    def reducel2(self, axis, keep_dims: bool = False, **kw):
+        return self._reduce(REDUCEL2, axis, keep_dims, **kw)
+
+    def reducel3(self, axis, keep_dims: bool = False, **kw):
+        return self._reduce(REDUCEL3, axis, keep_dims, **kw)
+
+    def logsumexp(self, axis, keep_dims: bool = False, **kw):
+        return self._reduce(LOGSUMEXP, axis, keep_dims, **kw)
+
+    # ---- IndexReduce (reduce.rs:6-42) --------------------------------------------
+    def argmax(self, axis, keep_dims: bool = False, **kw):
+        return self._argreduce(True, axis, keep_dims, **kw)
+
+    def argmin(self, axis, keep_dims: bool = False, **kw):
+        return self._argreduce(False, axis, keep_dims, **kw)
+
+    # ---- NormalizationOps (hpt-traits/src/ops/normalization.rs:6-64) ------------
+    def _softmax(self, log: bool, axis: int, stream=None) -> "Tensor":
+        self._require_hip("softmax")
+        res = Tensor.empty(self.shape, self.dtype, self.device)
+        vin, k1 = self._c_view()
+        vout, k2 = res._c_view()
+        check(_ffi.lib().hpt_hip_softmax(self.device, stream, int(log), C.byref(vin), int(axis), C.byref(vout)))
+        del k1, k2
+        return res
+
+    def softmax(self, axis: int, **kw) -> "Tensor":
+        return self._softmax(False, axis, **kw)
+
+    def log_softmax(self, axis: int, **kw) -> "Tensor":
+        return self._softmax(True, axis, **kw)
+
+    def layernorm(self, normalized_shape, gamma: Optional["Tensor"] = None, beta: Optional["Tensor"] = None,
+                  eps: float = 1e-5, stream=None) -> "Tensor":
+        self._require_hip("layernorm")
+        ns = [int(s) for s in (normalized_shape if isinstance(normalized_shape, Iterable) else [normalized_shape])]
+        if len(ns) > self.ndim or (ns and self.shape[self.ndim - len(ns):] != ns) or not ns:
+            # the reference panics with this text (cpu/tensor_internal/normalization.rs:68-70)
+            raise ShapeError(_ffi.ERR_SHAPE,
+                             "normalized dims must match last dims of input tensor, "
+                             f"shape: {self.shape}, normalized_shape: {ns}")
+        res = Tensor.empty(self.shape, self.dtype, self.device)
+        vin, k1 = self._c_view()
+        vout, k2 = res._c_view()
+        keep = [k1, k2]
+        gv = bv = None
+        if gamma is not None:
+            gamma._require_hip("layernorm gamma")
+            gv, k = gamma._c_view()
+            keep.append(k)
+        if beta is not None:
+            beta._require_hip("layernorm beta")
+            bv, k = beta._c_view()
+            keep.append(k)
+        check(_ffi.lib().hpt_hip_layernorm(self.device, stream, C.byref(vin), len(ns),
+                                           C.byref(gv) if gv is not None else None,
+                                           C.byref(bv) if bv is not None else None, float(eps), C.byref(vout)))
+        del keep
+        return res
+
+    def __repr__(self):
+        return f"Tensor<{self.dtype.name}, {self.backend}, {self.device}>(shape={self.shape}, strides={self.strides})"
+
+
+def reduce_plan(t: Tensor, op: int, axes) -> str:
+    """The kernel family and launch shape the library would use (no device needed)."""
+    axes = _as_axes(axes)
+    v, k = t._c_view()
+    buf = C.create_string_buffer(512)
+    check(_ffi.lib().hpt_hip_reduce_plan(op, C.byref(v), _ffi.i64_array(axes), len(axes), buf, 512))
+    del k
+    return buf.value.decode()
+
+
+def normalize_plan(t: Tensor, axis: int = 0, n_norm_dims: int = 0) -> str:
+    v, k = t._c_view()
+    buf = C.create_string_buffer(512)
+    check(_ffi.lib().hpt_hip_normalize_plan(C.byref(v), int(axis), int(n_norm_dims), buf, 512))
+    del k
+    return buf.value.decode()
+
+
+def synchronize(device: int = 0, stream=None) -> None:
+    check(_ffi.lib().hpt_hip_stream_synchronize(device, stream))
+
+
+def device_count() -> int:
+    n = C.c_int32()
+    check(_ffi.lib().hpt_hip_device_count(C.byref(n)))
+    return n.value

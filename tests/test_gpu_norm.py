@@ -1,0 +1,169 @@
+"""GPU parity of softmax / log_softmax / layernorm against the CPU oracle, through the C ABI.
+
+Mirrors hpt-tests/src/hpt/cpu/softmax.rs:30-87 (random 1-2-D shapes, gamma/beta, eps 1e-5) and
+hpt-tests/src/hpt/cuda/normalization.rs:39-53 (one shape per kernel size class, both axes),
+extended to the four layouts and the half types.
+"""
+import numpy as np
+import pytest
+
+from conftest import assert_close
+from util import F32_ATOL, F32_RTOL, HALF_RTOL, half_atol, layouts_for, upload
+
+pytestmark = pytest.mark.gpu
+
+SIZE_CLASS_SHAPES = [[1, 13], [2, 1024], [3, 1123], [3, 4096], [3, 5551]]
+
+
+@pytest.mark.parametrize("log", [False, True])
+def test_softmax_f32_size_classes_both_axes(hpt, orc, dev, log):
+    rng = np.random.default_rng(200)
+    for shape in SIZE_CLASS_SHAPES + [[5, 40000], [2, 70001], [300, 7], [1, 1]]:
+        base = rng.uniform(-10, 10, shape).astype(np.float32)
+        t, a = upload(hpt, base, dev=dev)
+        for axis in (0, 1, -1):
+            got = (t.log_softmax(axis) if log else t.softmax(axis)).numpy()
+            want = orc.softmax(a, axis, log=log, acc=orc.ACC_F64)
+            assert_close(got, want, F32_RTOL, F32_ATOL, f"softmax log={log} {shape} axis={axis}")
+
+
+@pytest.mark.parametrize("log", [False, True])
+def test_softmax_random_shapes_layouts(hpt, orc, dev, log):
+    rng = np.random.default_rng(201)
+    for case in range(20):
+        nd = int(rng.integers(1, 4))
+        shape = [int(rng.integers(1, 40)) for _ in range(nd)]
+        for npdt in (np.float32, np.float64):
+            base = (rng.standard_normal(shape) * 3).astype(npdt)
+            for lname, ops in layouts_for(shape, rng):
+                t, a = upload(hpt, base, ops, dev=dev)
+                if a.size == 0:
+                    continue
+                for axis in range(a.ndim):
+                    got = (t.log_softmax(axis) if log else t.softmax(axis)).numpy()
+                    want = orc.softmax(a, axis, log=log, acc=orc.ACC_F64)
+                    assert_close(got, want, F32_RTOL, F32_ATOL, f"softmax log={log} {npdt.__name__} {shape} {lname} axis={axis}")
+                    if not log:
+                        assert_close(got.sum(axis), np.ones_like(got.sum(axis)), 1e-5, 0, "rows sum to 1")
+
+
+def test_softmax_masked_rows(hpt, orc, dev):
+    """-inf entries (a causal mask is data): one finite entry -> exactly one-hot / (0, -inf);
+    an all -inf row -> NaN, as x - max = -inf - -inf on the CPU."""
+    x = np.full((4, 300), -np.inf, np.float32)
+    x[0, 0] = 1.5
+    x[1, :7] = np.arange(7)
+    x[2, 299] = -3.0
+    t, a = upload(hpt, x, dev=dev)
+    s = t.softmax(1).numpy()
+    assert s[0, 0] == 1.0 and np.all(s[0, 1:] == 0)
+    assert s[2, 299] == 1.0 and np.all(s[2, :299] == 0)
+    assert_close(s[1], orc.softmax(a, 1, acc=orc.ACC_F64)[1], F32_RTOL, F32_ATOL, "partly masked row")
+    assert np.all(np.isnan(s[3]))
+    ls = t.log_softmax(1).numpy()
+    assert ls[0, 0] == 0.0 and np.all(np.isneginf(ls[0, 1:]))
+
+
+@pytest.mark.parametrize("name", ["f16", "bf16"])
+@pytest.mark.parametrize("log", [False, True])
+def test_softmax_half_types(hpt, orc, dev, name, log):
+    rng = np.random.default_rng(202)
+    for shape in ([7, 2048], [5, 333], [64, 64], [3, 9000]):
+        x = (rng.standard_normal(shape) * 3).astype(np.float32)
+        if name == "f16":
+            base, dt, odt, bits, tof = x.astype(np.float16), None, None, 11, lambda v: v.astype(np.float32)
+        else:
+            base, dt, odt, bits, tof = hpt.f32_to_bf16_bits(x), hpt.bf16, orc.BF16, 8, hpt.bf16_bits_to_f32
+        for lname, ops in layouts_for(shape, rng):
+            t, a = upload(hpt, base, ops, dtype=dt, dev=dev)
+            for axis in range(a.ndim):
+                got = tof((t.log_softmax(axis) if log else t.softmax(axis)).numpy())
+                want = tof(orc.softmax(a, axis, log=log, acc=orc.ACC_F32, dtype=odt))
+                # floor: f16 results below its smallest normal lose bits; half an ulp of the scale otherwise
+                atol = max(half_atol(want, bits), 6.2e-5 * 2.0 ** -bits if name == "f16" else 0.0)
+                if name == "f16" and not log:
+                    atol = max(atol, 6e-8)
+                assert_close(got, want, HALF_RTOL, atol, f"softmax {name} log={log} {shape} {lname} axis={axis}")
+
+
+def test_layernorm_f32_random_shapes(hpt, orc, dev):
+    rng = np.random.default_rng(203)
+    for case in range(40):
+        nd = int(rng.integers(1, 3))
+        shape = [int(rng.integers(1, 10)) for _ in range(nd)]
+        base = rng.standard_normal(shape).astype(np.float32)
+        n = shape[-1]
+        g = np.arange(n, dtype=np.float32)
+        b = np.arange(n, dtype=np.float32)
+        t, a = upload(hpt, base, dev=dev)
+        tg, tb = hpt.Tensor.from_numpy(g).to_hip(dev), hpt.Tensor.from_numpy(b).to_hip(dev)
+        got = t.layernorm([n], tg, tb, 1e-5).numpy()
+        want = orc.layernorm(a, 1, g, b, 1e-5, acc=orc.ACC_F64)
+        assert_close(got, want, 1e-5, 1e-5, f"layernorm {shape}")
+
+
+def test_layernorm_sizes_layouts_affine_variants(hpt, orc, dev):
+    rng = np.random.default_rng(204)
+    for shape, nn in (([6, 13], 1), ([5, 1024], 1), ([3, 1123], 1), ([4, 4096], 1), ([2, 5551], 1),
+                      ([3, 40000], 1), ([2, 70001], 1), ([4, 6, 32], 2), ([2, 3, 4, 5], 3), ([7, 5], 2)):
+        for npdt in (np.float32, np.float64):
+            base = (rng.standard_normal(shape) + rng.uniform(-5, 5, shape[:1] + [1] * (len(shape) - 1))).astype(npdt)
+            for lname, ops in layouts_for(shape, rng):
+                t, a = upload(hpt, base, ops, dev=dev)
+                if a.size == 0:
+                    continue
+                ns = list(a.shape[a.ndim - nn:])
+                g = rng.normal(1, 0.1, ns).astype(npdt)
+                b = rng.normal(0, 0.1, ns).astype(npdt)
+                tg, tb = hpt.Tensor.from_numpy(g).to_hip(dev), hpt.Tensor.from_numpy(b).to_hip(dev)
+                for gg, bb, tgg, tbb in ((g, b, tg, tb), (g, None, tg, None), (None, b, None, tb), (None, None, None, None)):
+                    got = t.layernorm(ns, tgg, tbb, 1e-5).numpy()
+                    want = orc.layernorm(a, nn, gg, bb, 1e-5, acc=orc.ACC_F64)
+                    assert_close(got, want, F32_RTOL, 2e-6, f"layernorm {npdt.__name__} {shape} {lname} g={gg is not None} b={bb is not None}")
+
+
+def test_layernorm_closed_forms(hpt, dev):
+    # constant rows: x - mean = 0 -> output = beta
+    x = np.full((3, 257), 7.25, np.float32)
+    g = np.linspace(0.5, 2, 257).astype(np.float32)
+    b = np.linspace(-1, 1, 257).astype(np.float32)
+    t = hpt.Tensor.from_numpy(x).to_hip(dev)
+    out = t.layernorm([257], hpt.Tensor.from_numpy(g).to_hip(dev), hpt.Tensor.from_numpy(b).to_hip(dev), 1e-5).numpy()
+    assert np.array_equal(out, np.broadcast_to(b, out.shape))
+    # two-element rows: +-1/sqrt(1 + eps/var)
+    x2 = np.array([[1.0, 3.0], [-2.0, 6.0]], np.float32)
+    out2 = hpt.Tensor.from_numpy(x2).to_hip(dev).layernorm([2], None, None, 1e-5).numpy()
+    var = np.array([1.0, 16.0])
+    want = np.stack([-1 / np.sqrt(1 + 1e-5 / var), 1 / np.sqrt(1 + 1e-5 / var)], 1)
+    assert_close(out2, want, 1e-6, 1e-7, "2-element rows")
+    with pytest.raises(hpt.ShapeError, match="normalized dims must match last dims"):
+        hpt.Tensor.from_numpy(x2).to_hip(dev).layernorm([3])
+
+
+@pytest.mark.parametrize("name", ["f16", "bf16"])
+def test_layernorm_half_types(hpt, orc, dev, name):
+    rng = np.random.default_rng(205)
+    for shape in ([9, 4096], [5, 333], [130, 64]):
+        x = (rng.standard_normal(shape) * 2).astype(np.float32)
+        n = shape[-1]
+        gf, bf = rng.normal(1, 0.1, n).astype(np.float32), rng.normal(0, 0.1, n).astype(np.float32)
+        if name == "f16":
+            cv, dt, odt, bits, tof = (lambda v: v.astype(np.float16)), None, None, 11, (lambda v: v.astype(np.float32))
+        else:
+            cv, dt, odt, bits, tof = hpt.f32_to_bf16_bits, hpt.bf16, orc.BF16, 8, hpt.bf16_bits_to_f32
+        base, g, b = cv(x), cv(gf), cv(bf)
+        tg, tb = hpt.Tensor.from_numpy(g, dt).to_hip(dev), hpt.Tensor.from_numpy(b, dt).to_hip(dev)
+        for lname, ops in layouts_for(shape, rng):
+            if lname != "contiguous" and ops and ops[0][0] == "permute":
+                continue  # the normalised size changes under a permutation; covered by the f32 test
+            t, a = upload(hpt, base, ops, dtype=dt, dev=dev)
+            m = a.shape[-1]
+            got = tof(t.layernorm([m], tg[:m] if m != n else tg, tb[:m] if m != n else tb, 1e-5).numpy()) if m == n else None
+            if got is None:
+                g2, b2 = np.ascontiguousarray(g[:m]), np.ascontiguousarray(b[:m])
+                tg2, tb2 = hpt.Tensor.from_numpy(g2, dt).to_hip(dev), hpt.Tensor.from_numpy(b2, dt).to_hip(dev)
+                got = tof(t.layernorm([m], tg2, tb2, 1e-5).numpy())
+                want = tof(orc.layernorm(a, 1, g2, b2, 1e-5, acc=orc.ACC_F32, dtype=odt))
+            else:
+                want = tof(orc.layernorm(a, 1, g, b, 1e-5, acc=orc.ACC_F32, dtype=odt))
+            assert_close(got, want, HALF_RTOL, half_atol(want, bits), f"layernorm {name} {shape} {lname}")

@@ -1,0 +1,232 @@
+"""GPU parity of the axis reductions against the CPU oracle, through the C ABI.
+
+Mirrors the reference's reduce tests (hpt-tests/src/hpt/cpu/reduce.rs:63-650,
+hpt-tests/src/hpt/cuda/reduce.rs:17-206, 1421-1612): random shapes, every axis
+subset, keep_dims, the four layouts (contiguous / permuted / sliced / stepped),
+integer inputs compared exactly, arg-reductions with ties.
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+from conftest import assert_close
+from util import F32_ATOL, F32_RTOL, HALF_RTOL, half_atol, layouts_for, upload
+
+pytestmark = pytest.mark.gpu
+
+
+def axis_subsets(nd):
+    for r in range(1, nd + 1):
+        for c in itertools.combinations(range(nd), r):
+            yield list(c)
+
+
+def test_sum_f32_random_shapes_all_axis_subsets_all_layouts(hpt, orc, dev):
+    rng = np.random.default_rng(100)
+    for case in range(24):
+        nd = int(rng.integers(1, 4))
+        shape = [int(rng.integers(1, 33)) for _ in range(nd)]
+        base = rng.standard_normal(shape).astype(np.float32)
+        for lname, ops in layouts_for(shape, rng):
+            t, a = upload(hpt, base, ops, dev=dev)
+            if a.size == 0:
+                continue
+            for axes in axis_subsets(a.ndim):
+                for keep in (False, True):
+                    got = t.sum(axes, keep).numpy()
+                    want = orc.reduce(orc.SUM, a, axes, keep, acc=orc.ACC_F64)
+                    assert_close(got, want, F32_RTOL, F32_ATOL, f"sum {shape} {lname} axes={axes} keep={keep}")
+
+
+@pytest.mark.parametrize("op", ["sum", "prod", "max", "min", "mean", "nansum", "nanprod", "reducel1",
+                                "reducel2", "reducel3", "sum_square", "logsumexp"])
+def test_float_ops_f32_f64(hpt, orc, dev, op):
+    rng = np.random.default_rng(101)
+    code = getattr(orc, op.upper())
+    for npdt in (np.float32, np.float64):
+        for shape in ([2, 5, 10], [7, 33], [129], [3, 4, 5, 6]):
+            base = (rng.standard_normal(shape) * (0.5 if op in ("prod", "nanprod") else 1.0) +
+                    (1.0 if op in ("prod", "nanprod") else 0.0)).astype(npdt)
+            if op.startswith("nan"):
+                base.reshape(-1)[::7] = np.nan
+            for lname, ops in layouts_for(shape, rng):
+                t, a = upload(hpt, base, ops, dev=dev)
+                for axes in ([0], [a.ndim - 1], list(range(a.ndim))):
+                    got = getattr(t, op)(axes).numpy()
+                    want = orc.reduce(code, a, axes, acc=orc.ACC_F64)
+                    if op in ("max", "min"):
+                        assert np.array_equal(got, want), f"{op} {shape} {lname} {axes}"
+                    else:
+                        assert_close(got, want, F32_RTOL, F32_ATOL, f"{op} {npdt.__name__} {shape} {lname} {axes}")
+
+
+INT_DTYPES = [np.int8, np.int16, np.int32, np.int64, np.uint8, np.uint16, np.uint32, np.uint64]
+
+
+@pytest.mark.parametrize("npdt", INT_DTYPES)
+def test_integer_ops_bit_exact(hpt, orc, dev, npdt):
+    """Integer sums/products wrap (hpt-types/src/scalars/impls.rs:31-48): bit-exact, any layout."""
+    rng = np.random.default_rng(102)
+    info = np.iinfo(npdt)
+    lo, hi = max(info.min, -1000), min(info.max, 1000)
+    for shape in ([6, 40, 9], [300, 17], [5000]):
+        base = rng.integers(lo, hi + 1, shape).astype(npdt)
+        for lname, ops in layouts_for(shape, rng):
+            t, a = upload(hpt, base, ops, dev=dev)
+            for axes in ([0], [a.ndim - 1], list(range(a.ndim))):
+                for op in ("sum", "prod", "max", "min", "reducel1", "sum_square"):
+                    got = getattr(t, op)(axes).numpy()
+                    want = orc.reduce(getattr(orc, op.upper()), a, axes)
+                    assert got.dtype == want.dtype
+                    assert np.array_equal(got, want), f"{op} {npdt.__name__} {shape} {lname} {axes}"
+                # and the closed form: numpy's wrap-around sum in the same dtype
+                assert np.array_equal(t.sum(axes).numpy().reshape(-1),
+                                      np.asarray(a.sum(axis=tuple(axes), dtype=npdt)).reshape(-1))
+                # mean of integers is computed in FloatBinaryType<T>
+                gm = t.mean(axes).numpy()
+                wm = orc.reduce(orc.MEAN, a, axes, acc=orc.ACC_F64)
+                assert gm.dtype == wm.dtype
+                tol = 1e-3 if gm.dtype == np.float16 else 1e-5
+                assert_close(gm, wm, tol, tol, f"mean {npdt.__name__} {shape} {lname} {axes}")
+
+
+def test_bool_and_all_any(hpt, orc, dev):
+    rng = np.random.default_rng(103)
+    base = rng.random((9, 31, 5)) < 0.9
+    for lname, ops in layouts_for(list(base.shape), rng):
+        t, a = upload(hpt, base, ops, dev=dev)
+        for axes in ([0], [1], [2], [0, 1, 2]):
+            for op in ("sum", "prod", "max", "min", "all", "any"):
+                got = getattr(t, op)(axes).numpy()
+                want = orc.reduce(getattr(orc, op.upper()), a, axes)
+                assert np.array_equal(got, want), f"{op} bool {lname} {axes}"
+    f = rng.standard_normal((17, 65)).astype(np.float32)
+    f[f < -1.5] = 0.0
+    t, a = upload(hpt, f, dev=dev)
+    assert np.array_equal(t.all([1]).numpy(), (a != 0).all(1))
+    assert np.array_equal(t.any([0]).numpy(), (a != 0).any(0))
+
+
+@pytest.mark.parametrize("npdt", [np.int32, np.int64, np.float32, np.float64, np.int8, np.uint16, np.float16])
+def test_argmax_argmin_ties_resolve_to_lowest_index(hpt, orc, dev, npdt):
+    rng = np.random.default_rng(104)
+    for shape in ([7, 128, 33], [64, 300], [1000], [4, 5, 6, 3]):
+        # few distinct values => many ties
+        base = rng.integers(-3, 4, shape).astype(npdt)
+        for lname, ops in layouts_for(shape, rng):
+            t, a = upload(hpt, base, ops, dev=dev)
+            for axis in range(a.ndim):
+                for keep in (False, True):
+                    gmax = t.argmax(axis, keep).numpy()
+                    gmin = t.argmin(axis, keep).numpy()
+                    assert gmax.dtype == np.int64
+                    assert np.array_equal(gmax, orc.argreduce(True, a, axis, keep)), f"argmax {shape} {lname} {axis}"
+                    assert np.array_equal(gmin, orc.argreduce(False, a, axis, keep)), f"argmin {shape} {lname} {axis}"
+                    assert np.array_equal(gmax.reshape(-1), a.argmax(axis).reshape(-1))
+                    assert np.array_equal(gmin.reshape(-1), a.argmin(axis).reshape(-1))
+
+
+def test_argmax_docstring_kat_and_nan(hpt, dev):
+    # hpt-traits/src/ops/reduce.rs:21-39
+    t = hpt.Tensor.from_numpy(np.array([10.0, 3.0, 2.0], np.float32)).to_hip(dev)
+    assert t.argmax(0).numpy().tolist() == [0]
+    assert t.argmin(0).numpy().tolist() == [2]
+    # NaN never wins (strict compares): argreduce_kernels.rs:13-21
+    t = hpt.Tensor.from_numpy(np.array([[np.nan, 1.0, 5.0, 5.0], [np.nan, np.nan, -np.inf, -np.inf]], np.float32)).to_hip(dev)
+    assert t.argmax(1).numpy().tolist() == [2, 0]
+    assert t.argmin(1).numpy().tolist() == [1, 2]
+
+
+def test_docstring_kats(hpt, dev):
+    # hpt-traits/src/ops/reduce.rs:58-62, 146-149, 166-168, 294-297, 328-331, 347-350
+    a = hpt.Tensor.from_numpy(np.array([[1.0, 2.0], [3.0, 4.0]], np.float32)).to_hip(dev)
+    assert a.sum([0, 1]).numpy().tolist() == [10.0]
+    assert a.sum([0, 1], True).numpy().tolist() == [[10.0]]
+    assert a.mean([0, 1]).numpy().tolist() == [2.5]
+    assert a.sum_square([0, 1]).numpy().tolist() == [30.0]
+    assert a.reducel1([0, 1]).numpy().tolist() == [10.0]
+    assert a.prod([0, 1]).numpy().tolist() == [24.0]
+    c = hpt.Tensor.from_numpy(np.array([[1.0, 2.0], [2.0, 3.0]], np.float32)).to_hip(dev)
+    assert abs(c.reducel2([0, 1], True).numpy()[0, 0] - 4.2426405) < 1e-5   # "sqrt(1+4+4+9) ~ 4.24"
+    assert abs(c.reducel3([0, 1], True).numpy()[0, 0] - 3.5303483) < 1e-5   # "[[3.5303]]"
+    assert abs(a.logsumexp([0, 1]).numpy()[0] - 4.4401898) < 1e-5
+    assert a.max([0]).numpy().tolist() == [3.0, 4.0]
+    assert a.min([1]).numpy().tolist() == [1.0, 3.0]
+
+
+@pytest.mark.parametrize("name", ["f16", "bf16"])
+def test_half_types_f32_accumulate(hpt, orc, dev, name):
+    rng = np.random.default_rng(105)
+    for shape in ([33, 1000], [64, 8, 24], [4096]):
+        x = rng.standard_normal(shape).astype(np.float32) * 2
+        if name == "f16":
+            base, dt, odt, bits = x.astype(np.float16), None, None, 11
+            tof = lambda v: v.astype(np.float32)
+        else:
+            base, dt, odt, bits = hpt.f32_to_bf16_bits(x), hpt.bf16, orc.BF16, 8
+            tof = hpt.bf16_bits_to_f32
+        for lname, ops in layouts_for(shape, rng):
+            t, a = upload(hpt, base, ops, dtype=dt, dev=dev)
+            for axes in ([0], [a.ndim - 1], list(range(a.ndim))):
+                for op in ("sum", "mean", "max", "min", "sum_square", "reducel2"):
+                    got = tof(getattr(t, op)(axes).numpy())
+                    want = tof(orc.reduce(getattr(orc, op.upper()), a, axes, acc=orc.ACC_F32, dtype=odt))
+                    if op in ("max", "min"):
+                        assert np.array_equal(got, want)
+                    else:
+                        assert_close(got, want, HALF_RTOL, half_atol(want, bits), f"{op} {name} {shape} {lname} {axes}")
+
+
+def test_multi_stage_and_large_shapes(hpt, orc, dev):
+    """Shapes that take the several-workgroups-per-output paths (row and column) and run twice
+    to check that the arrival counters were reset."""
+    rng = np.random.default_rng(106)
+    cases = [((3, 1 << 20), [1]), ((1 << 21,), [0]), ((1 << 16, 40), [0]), ((2, 70000, 3), [1]),
+             ((64, 128, 56, 56), [1]), ((700, 3, 900), [0, 2])]
+    for shape, axes in cases:
+        base = rng.standard_normal(shape).astype(np.float32)
+        t, a = upload(hpt, base, dev=dev)
+        want = orc.reduce(orc.SUM, a, axes, acc=orc.ACC_F64)
+        for rep in range(2):
+            got = t.sum(axes).numpy()
+            assert_close(got, want, F32_RTOL, F32_ATOL, f"sum {shape} axes={axes} rep={rep}")
+        gi = t.argmax(axes[0]).numpy() if len(axes) == 1 else None
+        if gi is not None:
+            assert np.array_equal(gi, orc.argreduce(True, a, axes[0]))
+        ib = rng.integers(-1000, 1001, shape).astype(np.int32)
+        ti, ai = upload(hpt, ib, dev=dev)
+        assert np.array_equal(ti.sum(axes).numpy(), orc.reduce(orc.SUM, ai, axes))
+        # run-to-run determinism of the multi-stage float path
+        assert np.array_equal(t.sum(axes).numpy().view(np.uint32), t.sum(axes).numpy().view(np.uint32))
+
+
+def test_sum_inplace_out_and_accumulate(hpt, orc, dev):
+    """sum_ with init_out: true overwrites, false adds to what `out` holds (reduce.rs:84-92)."""
+    rng = np.random.default_rng(107)
+    base = rng.standard_normal((40, 50)).astype(np.float32)
+    t, a = upload(hpt, base, dev=dev)
+    out = hpt.Tensor.from_numpy(np.full((40,), 5.0, np.float32)).to_hip(dev)
+    r = t.sum_([1], False, True, out)
+    assert_close(r.numpy(), a.astype(np.float64).sum(1), F32_RTOL, F32_ATOL, "sum_ init_out")
+    assert_close(out.numpy(), a.astype(np.float64).sum(1), F32_RTOL, F32_ATOL, "sum_ writes into out")
+    out2 = hpt.Tensor.from_numpy(np.full((40,), 5.0, np.float32)).to_hip(dev)
+    t.sum_([1], False, False, out2)
+    assert_close(out2.numpy(), a.astype(np.float64).sum(1) + 5.0, F32_RTOL, F32_ATOL, "sum_ accumulate")
+    with pytest.raises(hpt.ShapeError):
+        t.sum_([1], False, True, hpt.Tensor.empty([41], hpt.f32, dev))
+
+
+def test_empty_and_degenerate(hpt, orc, dev):
+    z = hpt.Tensor.from_numpy(np.zeros((4, 0, 3), np.float32)).to_hip(dev)
+    assert z.sum([1]).numpy().tolist() == np.zeros((4, 3)).tolist()          # reduced dim empty -> identity
+    assert z.prod([1]).numpy().tolist() == np.ones((4, 3)).tolist()
+    assert np.all(np.isneginf(z.max([1]).numpy()))
+    assert z.sum([0]).numpy().shape == (0, 3)                                 # no outputs
+    one = hpt.Tensor.from_numpy(np.arange(6, dtype=np.float32).reshape(1, 6, 1)).to_hip(dev)
+    assert one.sum([0, 2]).numpy().tolist() == [0, 1, 2, 3, 4, 5]              # only size-1 axes reduced
+    assert one.argmax(0).numpy().tolist() == [[0]] * 6
+    with pytest.raises(hpt.ShapeError, match=r"Dimension out of range: expected in 0\.\.3, got 3"):
+        one.sum([3])
+    with pytest.raises(hpt.ParamError, match="Axis 1 is duplicated"):
+        one.sum([1, 1])
