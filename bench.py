@@ -1,0 +1,333 @@
+#!/usr/bin/env python3
+"""bench.py — throughput of the reduction / softmax / layernorm path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|headline] [--no-cpu]
+
+A "step" is one pass of the hot path over one batch of synthetic input. The headline
+workload is the configuration the metric is quoted on: LayerNorm over the last axis of an
+f32 [8192, 4096] tensor with gamma and beta (eps 1e-5). Inputs are resident in HBM before
+the timed region starts; successive steps rotate over several input/output buffer pairs so
+that the working set is far larger than the 256 MB Infinity Cache and every step streams
+from HBM.
+
+Prints ONE JSON line. `value` is algorithmic GB/s (every logical input element read once +
+every output element written once + gamma/beta once, per step) over the wall-clock time of
+exactly K steps. `roofline.achieved` uses the same bytes over the kernel's average duration
+measured with HIP events on the launch stream. `ops` lists the same measurement for every
+op of the five benchmark configurations. `cpu_baseline` is the CPU restatement of Hpt's
+layernorm (oracle/, test infrastructure) timed on the host cores of this box.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+
+
+# ---- HIP events on the launch stream (the null stream: the library is called with stream=NULL) ----
+class HipEvents:
+    def __init__(self):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.hip.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.hip.hipDeviceSynchronize.argtypes = []
+
+    def event(self):
+        e = C.c_void_p()
+        assert self.hip.hipEventCreate(C.byref(e)) == 0
+        return e
+
+    def record(self, e, stream=None):
+        assert self.hip.hipEventRecord(e, stream) == 0
+
+    def elapsed_ms(self, a, b):
+        assert self.hip.hipEventSynchronize(b) == 0
+        ms = C.c_float()
+        assert self.hip.hipEventElapsedTime(C.byref(ms), a, b) == 0
+        return float(ms.value)
+
+    def sync(self):
+        assert self.hip.hipDeviceSynchronize() == 0
+
+
+def gen_c2(seed=1):
+    """f32 [8192,4096]: N(0,1) + per-row offset U(-5,5); gamma ~ N(1,0.1), beta ~ N(0,0.1)."""
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((8192, 4096), dtype=np.float32)
+    x += rng.uniform(-5, 5, (8192, 1)).astype(np.float32)
+    g = rng.normal(1, 0.1, 4096).astype(np.float32)
+    b = rng.normal(0, 0.1, 4096).astype(np.float32)
+    return x, g, b
+
+
+class Case:
+    """One op on one configuration: `run(i)` enqueues one step on buffer set i % nbuf."""
+
+    def __init__(self, name, cfg, dtype, rows, algo_bytes, run, nbuf, check=None):
+        self.name, self.cfg, self.dtype, self.rows = name, cfg, dtype, rows
+        self.bytes, self.run, self.nbuf, self.check = algo_bytes, run, nbuf, check
+
+
+def time_case(ev: HipEvents, case: Case, steps: int, warmup: int):
+    import hpt_amd as hpt
+    for i in range(warmup):
+        case.run(i)
+    hpt.synchronize(0)
+    e0, e1 = ev.event(), ev.event()
+    t0 = time.perf_counter()
+    ev.record(e0)
+    for i in range(steps):
+        case.run(i)
+    ev.record(e1)
+    hpt.synchronize(0)
+    wall = time.perf_counter() - t0
+    dev_ms = ev.elapsed_ms(e0, e1)
+    return wall, dev_ms
+
+
+class Prepared:
+    """Views and rotating output tensors built once, so that a step is one C-ABI call
+    (a few microseconds of host time) and nothing else."""
+
+    def __init__(self):
+        import hpt_amd as hpt
+        from hpt_amd import _ffi
+        self.hpt, self.ffi, self.l = hpt, _ffi, hpt.lib()
+        self.keep = []
+
+    def view(self, t):
+        v, k = t._c_view()
+        self.keep.append((t, v, k))
+        return C.byref(v)
+
+    def norm(self, ins, kind, axis=1, n_norm=0, gamma=None, beta=None, eps=1e-5):
+        hpt, l, check = self.hpt, self.l, self.ffi.check
+        outs = [hpt.Tensor.empty(t.shape, t.dtype, 0) for t in ins]
+        vi, vo = [self.view(t) for t in ins], [self.view(t) for t in outs]
+        n = len(ins)
+        if kind == "layernorm":
+            vg, vb = self.view(gamma), self.view(beta)
+            return lambda i: check(l.hpt_hip_layernorm(0, None, vi[i % n], n_norm, vg, vb, eps, vo[i % n])), outs
+        log = int(kind == "log_softmax")
+        return lambda i: check(l.hpt_hip_softmax(0, None, log, vi[i % n], axis, vo[i % n])), outs
+
+    def reduce(self, ins, op, axes, arg=None):
+        hpt, l, check = self.hpt, self.l, self.ffi.check
+        outs = []
+        for t in ins:
+            outs.append(getattr(t, op)(axes) if arg is None else (t.argmax(axes) if arg else t.argmin(axes)))
+        vi, vo = [self.view(t) for t in ins], [self.view(t) for t in outs]
+        n = len(ins)
+        if arg is not None:
+            return lambda i: check(l.hpt_hip_argreduce(0, None, int(arg), vi[i % n], axes, vo[i % n])), outs
+        code = getattr(hpt, op.upper())
+        ax = self.ffi.i64_array(axes)
+        self.keep.append(ax)
+        na = len(axes)
+        return lambda i: check(l.hpt_hip_reduce(0, None, code, vi[i % n], ax, na, 1, vo[i % n])), outs
+
+
+def build_cases(which: str):
+    """Synthetic inputs of the five configurations, uploaded once; outputs preallocated."""
+    import hpt_amd as hpt
+    P = Prepared()
+    cases = []
+
+    # ---- C2: LayerNorm / log_softmax, f32 [8192, 4096] (headline) ----
+    x, g, b = gen_c2()
+    nbuf = 4
+    xs = [hpt.Tensor.from_numpy(np.roll(x, k, axis=0)).to_hip(0) for k in range(nbuf)]
+    tg, tb = hpt.Tensor.from_numpy(g).to_hip(0), hpt.Tensor.from_numpy(b).to_hip(0)
+    ln_bytes = 2 * x.nbytes + g.nbytes + b.nbytes
+    run, ln_outs = P.norm(xs, "layernorm", n_norm=1, gamma=tg, beta=tb)
+    cases.append(Case("layernorm", "C2 f32 [8192,4096] gamma,beta eps=1e-5", "f32", 8192, ln_bytes, run, nbuf))
+    head_out = ln_outs[0]
+    if which == "headline":
+        return cases, P, (x, g, b, head_out)
+    run, _ = P.norm(xs, "log_softmax", axis=1)
+    cases.append(Case("log_softmax", "C2 f32 [8192,4096] axis=1", "f32", 8192, 2 * x.nbytes, run, nbuf))
+
+    # ---- C1: f32 [1024,1024] U(-10,10) ----
+    rng = np.random.default_rng(0)
+    c1 = rng.uniform(-10, 10, (1024, 1024)).astype(np.float32)
+    c1s = [hpt.Tensor.from_numpy(np.roll(c1, k, 0)).to_hip(0) for k in range(64)]
+    run, _ = P.norm(c1s, "softmax", axis=1)
+    cases.append(Case("softmax", "C1 f32 [1024,1024] axis=1", "f32", 1024, 2 * c1.nbytes, run, 64))
+    run, _ = P.reduce(c1s, "sum", [1])
+    cases.append(Case("sum(axis=1)", "C1 f32 [1024,1024]", "f32", 1024, c1.nbytes + 4096, run, 64))
+    run, _ = P.reduce(c1s, "max", [1])
+    cases.append(Case("max(axis=1)", "C1 f32 [1024,1024]", "f32", 1024, c1.nbytes + 4096, run, 64))
+
+    # ---- C3: f32 / i32 [64,128,56,56] ----
+    rng = np.random.default_rng(2)
+    c3 = rng.standard_normal((64, 128, 56, 56), dtype=np.float32)
+    c3s = [hpt.Tensor.from_numpy(np.roll(c3, k, 0)).to_hip(0) for k in range(6)]
+    rng = np.random.default_rng(3)
+    c3i = rng.integers(-1000, 1001, (64, 128, 56, 56)).astype(np.int32)
+    c3is = [hpt.Tensor.from_numpy(np.roll(c3i, k, 0)).to_hip(0) for k in range(6)]
+    nb = c3.nbytes
+    for name, op, axes, rows, outb in (("sum([2,3])", "sum", [2, 3], 8192, 8192 * 4),
+                                       ("mean([2,3])", "mean", [2, 3], 8192, 8192 * 4),
+                                       ("max(axis=1)", "max", [1], 200704, 200704 * 4),
+                                       ("sum(all)", "sum", [0, 1, 2, 3], 1, 4)):
+        run, _ = P.reduce(c3s, op, axes)
+        cases.append(Case(name, "C3 f32 [64,128,56,56]", "f32", rows, nb + outb, run, 6))
+    run, _ = P.reduce(c3is, "sum", [1])
+    cases.append(Case("sum(axis=1)", "C3 i32 [64,128,56,56]", "i32", 200704, nb + 200704 * 4, run, 6))
+    run, _ = P.reduce(c3is, "argmax", 1, arg=True)
+    cases.append(Case("argmax(axis=1)", "C3 i32 [64,128,56,56]", "i32", 200704, nb + 200704 * 8, run, 6))
+
+    # ---- C4: bf16 [65536, 2048] causal-masked logits ----
+    rng = np.random.default_rng(4)
+    c4 = rng.standard_normal((65536, 2048), dtype=np.float32) * 3
+    q = (np.arange(65536) % 2048)[:, None]
+    c4[np.arange(2048)[None, :] > q] = -np.inf
+    c4b = hpt.f32_to_bf16_bits(c4)
+    del c4
+    c4s = [hpt.Tensor.from_numpy(c4b, hpt.bf16).to_hip(0),
+           hpt.Tensor.from_numpy(np.roll(c4b, 2048, 0), hpt.bf16).to_hip(0)]
+    run, _ = P.norm(c4s, "softmax", axis=1)
+    cases.append(Case("softmax", "C4 bf16 [65536,2048] causal mask as data, axis=1", "bf16", 65536,
+                      2 * c4b.nbytes, run, 2))
+
+    # ---- C5: f16 base [4096,8192]: transposed view and [:, ::2] view ----
+    rng = np.random.default_rng(5)
+    c5 = (rng.standard_normal((4096, 8192), dtype=np.float32) * 2).astype(np.float16)
+    c5s = [hpt.Tensor.from_numpy(np.roll(c5, k, 0)).to_hip(0) for k in range(6)]
+    g5 = rng.normal(1, 0.1, 4096).astype(np.float16)
+    b5 = rng.normal(0, 0.1, 4096).astype(np.float16)
+    tg5, tb5 = hpt.Tensor.from_numpy(g5).to_hip(0), hpt.Tensor.from_numpy(b5).to_hip(0)
+    n5 = c5.nbytes
+    c5t = [t.permute([1, 0]) for t in c5s]
+    c5h = [t[:, ::2] for t in c5s]
+    run, _ = P.norm(c5t, "layernorm", n_norm=1, gamma=tg5, beta=tb5)
+    cases.append(Case("layernorm", "C5a f16 [4096,8192].permute(1,0) -> [8192,4096]", "f16", 8192, 2 * n5 + 16384, run, 6))
+    run, _ = P.norm(c5t, "softmax", axis=1)
+    cases.append(Case("softmax", "C5a f16 [4096,8192].permute(1,0) axis=1", "f16", 8192, 2 * n5, run, 6))
+    run, _ = P.reduce(c5t, "sum", [0])
+    cases.append(Case("sum(axis=0)", "C5a f16 [4096,8192].permute(1,0)", "f16", 4096, n5 + 8192, run, 6))
+    run, _ = P.norm(c5h, "layernorm", n_norm=1, gamma=tg5, beta=tb5)
+    cases.append(Case("layernorm", "C5b f16 [4096,8192][:, ::2] -> [4096,4096]", "f16", 4096, n5 + 16384, run, 6))
+    run, _ = P.norm(c5h, "softmax", axis=1)
+    cases.append(Case("softmax", "C5b f16 [4096,8192][:, ::2] axis=1", "f16", 4096, n5, run, 6))
+    run, _ = P.reduce(c5h, "sum", [0])
+    cases.append(Case("sum(axis=0)", "C5b f16 [4096,8192][:, ::2]", "f16", 4096, n5 // 2 + 8192, run, 6))
+    return cases, P, (x, g, b, head_out)
+
+
+def cpu_baseline(x, g, b, gpu_out, budget_s=15.0):
+    """The restated Hpt CPU layernorm (three scalar passes per row + the affine pass, rows split
+    over the physical cores as Hpt's pools are) on the same input, timed on this host."""
+    from oracle import oracle as orc
+    cores = orc.physical_cores()
+    out = np.empty_like(x)
+    orc.mt_layernorm_f32(x, g, b, 1e-5, cores, out)  # warm-up, also the check below
+    port_err = None
+    if gpu_out is not None:
+        # checker: the f64-accumulating oracle on a sample of rows. The f32 port itself carries
+        # the summation error of 4096 sequential f32 adds (about 1e-5 absolute on this input),
+        # so it is reported against the same truth rather than used as the yardstick.
+        rows = slice(0, 512)
+        truth = orc.layernorm(x[rows], 1, g, b, 1e-5, acc=orc.ACC_F64).astype(np.float64)
+        err = np.abs(gpu_out[rows].astype(np.float64) - truth)
+        assert (err <= 2e-6 + 1e-5 * np.abs(truth)).all(), \
+            f"GPU layernorm differs from the f64 oracle (max err {err.max():g})"
+        port_err = float(np.abs(out[rows].astype(np.float64) - truth).max())
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
+        t0 = time.perf_counter()
+        orc.mt_layernorm_f32(x, g, b, 1e-5, cores, out)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    nbytes = 2 * x.nbytes + g.nbytes + b.nbytes
+    return {"value": round(nbytes / med / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"{len(times)} passes of the full f32 [8192,4096] layernorm (median {med * 1e3:.1f} ms/pass, "
+                      f"{8192 / med:.0f} rows/s)",
+            "rows_per_s": round(8192 / med, 1), "port_max_abs_err_vs_f64_oracle": port_err}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--ops", choices=["all", "headline"], default="all")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU form (every op but a full "
+              "reduction is independent per row). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import hpt_amd as hpt
+    from hpt_amd import _ffi, build
+    if not _ffi.LIB_PATH.exists():
+        build.build()
+    assert hpt.device_count() >= 1, "no HIP device visible"
+    ev = HipEvents()
+
+    cases, prepared, (x, g, b, head_out) = build_cases(args.ops)
+    head = cases[0]
+    wall, dev_ms = time_case(ev, head, args.steps, args.warmup)
+    ms_per_step = wall * 1e3 / args.steps
+    value = head.bytes * args.steps / wall / 1e9
+    kernel_us = dev_ms * 1e3 / args.steps
+    achieved = head.bytes / (dev_ms / args.steps * 1e-3) / 1e9
+
+    ops = []
+    for c in cases:
+        if c is head:
+            w, d = wall, dev_ms
+            n = args.steps
+        else:
+            n = max(20, min(args.steps, 100))
+            w, d = time_case(ev, c, n, min(args.warmup, 10))
+        ops.append({"config": c.cfg, "op": c.name, "dtype": c.dtype, "algorithmic_bytes": c.bytes,
+                    "us_per_launch": round(d * 1e3 / n, 2),
+                    "GBps": round(c.bytes / (d / n * 1e-3) / 1e9, 1),
+                    "pct_of_hbm_peak": round(100 * c.bytes / (d / n * 1e-3) / 1e9 / HBM_PEAK_GBS, 1),
+                    "rows_per_s": round(c.rows / (d / n * 1e-3), 1)})
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(x, g, b, head_out.numpy())
+
+    line = {
+        "metric": "achieved HBM GB/s (% of MI355X peak) + rows/s for softmax/layernorm/reduce",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "LayerNorm over the last axis, f32 [8192,4096] ~N(0,1)+row offset U(-5,5), "
+                               "gamma~N(1,0.1), beta~N(0,0.1), eps=1e-5 (BASELINE.json configs[1])",
+                   "rows": 8192, "cols": 4096, "algorithmic_bytes_per_step": head.bytes,
+                   "buffers_rotated": head.nbuf},
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1),
+        "rows_per_s": round(8192 * args.steps / wall, 1),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "row_reg_kernel<LAYERNORM, float, 4, 4>", "kernel_us": round(kernel_us, 2)},
+        "cpu_baseline": cpu,
+        "ops": ops,
+    }
+    for o in ops:
+        print(f"  {o['config']:<58} {o['op']:<16} {o['us_per_launch']:>9.2f} us  {o['GBps']:>8.1f} GB/s "
+              f"{o['pct_of_hbm_peak']:>5.1f}%  {o['rows_per_s']:.3g} rows/s", file=sys.stderr)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

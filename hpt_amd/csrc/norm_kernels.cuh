@@ -59,6 +59,11 @@ template <class CT> __device__ __forceinline__ CT neg_inf() {
     else return -__builtin_huge_valf();
 }
 
+// type the layernorm row statistics are accumulated in
+template <class T> struct StatType { using type = float; };
+template <> struct StatType<float> { using type = double; };
+template <> struct StatType<double> { using type = double; };
+
 template <class Op, class CT>
 __device__ __forceinline__ CT row_all_reduce(CT v, int tpr, CT* smem) {
     if (tpr <= 64) return group_reduce<Op>(v, tpr);
@@ -69,7 +74,8 @@ __device__ __forceinline__ CT row_all_reduce(CT v, int tpr, CT* smem) {
 template <int KIND, class T, int VEC, int NCHUNK>
 __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     using CT = typename Elem<T>::Wide;
-    __shared__ CT smem[16];
+    __shared__ __align__(8) unsigned char smem_stat[16 * sizeof(double)];
+    CT* smem = reinterpret_cast<CT*>(smem_stat);
     const int tpr = a.tpr;
     const int tx = threadIdx.x & (tpr - 1);
     const int ty = threadIdx.x >> a.tpr_log2;
@@ -123,26 +129,31 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) x[c][j] = KIND == NORM_SOFTMAX ? x[c][j] * k : x[c][j] - k;
     } else {
-        CT s = 0;
+        // Row statistics of f32 (and f64) rows are taken in f64: x - mean is then
+        // exact before it is rounded, so rows whose spread is small against
+        // their offset keep full f32 accuracy. Half types use f32.
+        using ST = typename StatType<T>::type;
+        ST* ssmem = reinterpret_cast<ST*>(smem_stat);
+        ST s = 0;
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) s += x[c][j];
-        s = row_all_reduce<SumC<CT>>(s, tpr, smem);
-        const CT mean = s / (CT)a.cols;
-        CT q = 0;
+            for (int j = 0; j < VEC; ++j) s += (ST)x[c][j];
+        s = row_all_reduce<SumC<ST>>(s, tpr, ssmem);
+        const ST mean = s / (ST)a.cols;
+        ST q = 0;
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const bool in_row_c = ((int64_t)c * tpr + tx) < nv;
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
-                CT d = in_row_c ? x[c][j] - mean : (CT)0;
-                x[c][j] = d;
+                const ST d = in_row_c ? (ST)x[c][j] - mean : (ST)0;
+                x[c][j] = (CT)d;
                 q += d * d;
             }
         }
-        q = row_all_reduce<SumC<CT>>(q, tpr, smem);
-        const CT rstd = rsqrt_ct(q / (CT)a.cols + (CT)a.eps);
+        q = row_all_reduce<SumC<ST>>(q, tpr, ssmem);
+        const CT rstd = (CT)rsqrt_ct(q / (ST)a.cols + (ST)a.eps);
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int64_t iv = (int64_t)c * tpr + tx;
@@ -300,30 +311,46 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
             store(iv, x);
         }
     } else {
-        MomentStat<CT> st{(CT)0, (CT)0, (CT)0};
+        using ST = typename StatType<T>::type;
+        MomentStat<ST> st{(ST)0, (ST)0, (ST)0};
         if (valid) {
+            // Per thread: sums of (x - k) and (x - k)^2 around the first element k
+            // it sees (no division per element, no cancellation against a far
+            // origin), turned into (count, mean, M2) once at the end.
+            ST k = 0, s1 = 0, s2 = 0, n = 0;
+            bool first = true;
             for (int64_t iv = tx; iv < nv; iv += tpr) {
                 CT x[VEC];
                 load(iv, x);
+                if (first) {
+                    k = (ST)x[0];
+                    first = false;
+                }
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
-                    st.n += (CT)1;
-                    const CT d = x[j] - st.mean;
-                    st.mean += d / st.n;
-                    st.m2 += d * (x[j] - st.mean);
+                    const ST d = (ST)x[j] - k;
+                    s1 += d;
+                    s2 += d * d;
                 }
+                n += (ST)VEC;
+            }
+            if (n > (ST)0) {
+                st.n = n;
+                st.mean = k + s1 / n;
+                st.m2 = s2 - s1 * s1 / n;
+                if (st.m2 < (ST)0) st.m2 = 0;
             }
         }
-        st = stat_all_reduce<MomentStatOp<CT>>(st, tpr, (MomentStat<CT>*)smem_raw);
+        st = stat_all_reduce<MomentStatOp<ST>>(st, tpr, (MomentStat<ST>*)smem_raw);
         if (!valid) return;
-        const CT mean = st.mean;
-        const CT rstd = rsqrt_ct(st.m2 / (CT)a.cols + (CT)a.eps);
+        const ST mean = st.mean;
+        const CT rstd = (CT)rsqrt_ct(st.m2 / (ST)a.cols + (ST)a.eps);
         for (int64_t iv = tx; iv < nv; iv += tpr) {
             CT x[VEC];
             load(iv, x);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
-                CT y = (x[j] - mean) * rstd;
+                CT y = (CT)((ST)x[j] - mean) * rstd;
                 const int64_t col = iv * VEC + j;
                 if (a.gamma) y *= Elem<T>::widen(((const T*)a.gamma)[col]);
                 if (a.beta) y += Elem<T>::widen(((const T*)a.beta)[col]);

@@ -141,9 +141,11 @@ __global__ void __launch_bounds__(1024) row_reduce_kernel(const RowArgs a) {
 
     // several workgroups per output: one output per workgroup here (rpb == 1)
     Acc* part = (Acc*)a.partial + row * split;
-    if (threadIdx.x == 0) part[blockIdx.y] = acc;
-    __threadfence();
+    // Only the thread that wrote the partial releases it: a device-scope fence
+    // writes back the L2 of this XCD, so it must not run once per wavefront.
     if (threadIdx.x == 0) {
+        part[blockIdx.y] = acc;
+        __threadfence();
         unsigned prev = atomicAdd(&a.counters[row], 1u);
         s_last = (prev == (unsigned)(split - 1));
     }
@@ -246,7 +248,7 @@ __global__ void __launch_bounds__(1024) col_reduce_kernel(const ColArgs a) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) part[(int64_t)blockIdx.y * a.K + o0 + j] = acc[j];
     }
-    __threadfence();
+    if (ty == 0) __threadfence();  // the writers release their partials
     __syncthreads();
     if (tx == 0 && ty == 0) {
         unsigned prev = atomicAdd(&a.counters[blockIdx.x], 1u);
