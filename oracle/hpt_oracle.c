@@ -113,14 +113,6 @@ uint16_t orc_f32_to_bf16(float f) {
     return (uint16_t)(u >> 16);
 }
 
-static int dt_size(int dt) {
-    switch (dt) {
-        case ORC_BOOL: case ORC_I8: case ORC_U8: return 1;
-        case ORC_I16: case ORC_U16: case ORC_F16: case ORC_BF16: return 2;
-        case ORC_I32: case ORC_U32: case ORC_F32: return 4;
-        default: return 8;
-    }
-}
 static int dt_is_float(int dt) { return dt >= ORC_F16; }
 static int dt_is_signed_int(int dt) { return dt >= ORC_I8 && dt <= ORC_I64; }
 

@@ -1,0 +1,162 @@
+"""Host logic of libhpt_hip.so that needs no GPU: the library loads, exports every symbol the
+header declares, and its shape logic / planner agree with the oracle and the reference's KATs."""
+import ctypes as C
+import itertools
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def test_library_exports_every_declared_symbol(hpt):
+    header = (ROOT / "include" / "hpt_hip.h").read_text()
+    declared = set(re.findall(r"\b(hpt_hip_\w+)\s*\(", header))
+    assert len(declared) >= 20
+    from hpt_amd import _ffi
+    assert declared == set(_ffi.SIGNATURES), "binding table and header disagree"
+    l = hpt.lib()
+    for name in declared:
+        assert getattr(l, name) is not None
+
+
+def test_dtype_sizes(hpt):
+    l = hpt.lib()
+    for d in hpt.DTYPES:
+        assert l.hpt_hip_dtype_size(d.code) == d.size == d.np_dtype.itemsize
+    assert l.hpt_hip_dtype_size(99) == 0
+
+
+def test_process_axes_through_the_abi(hpt, orc):
+    from hpt_amd import _ffi
+    l = hpt.lib()
+
+    def pa(axes, ndim):
+        out = _ffi.i64_array([0] * len(axes))
+        _ffi.check(l.hpt_hip_process_axes(_ffi.i64_array(axes), len(axes), ndim, out))
+        return [out[i] for i in range(len(axes))]
+
+    # hpt-tests/src/hpt_common/axis.rs:6-50
+    with pytest.raises(hpt.ShapeError, match=r"Dimension out of range: expected in 0\.\.2, got 10"):
+        pa([10], 2)
+    with pytest.raises(hpt.ShapeError, match=r"Dimension out of range: expected in 0\.\.2, got -1"):
+        pa([-3], 2)
+    assert pa([-1], 2) == [1]
+    with pytest.raises(hpt.ParamError, match="Axis 2 is duplicated"):
+        pa([2, 2], 3)
+    with pytest.raises(hpt.ParamError, match="duplicated"):
+        pa([-1, 2], 3)      # two spellings of one axis
+    for ndim in range(1, 5):
+        for r in range(1, ndim + 1):
+            for axes in itertools.permutations(range(-ndim, ndim), r):
+                try:
+                    want = orc.process_axes(list(axes), ndim)
+                except ValueError:
+                    continue
+                if len(set(want)) != len(want):
+                    continue
+                assert pa(list(axes), ndim) == want
+
+
+def test_reduce_shape_and_out_dtype_match_the_oracle(hpt, orc):
+    t = hpt.Tensor.from_numpy(np.zeros((2, 3, 4, 5), np.float32))
+    for r in range(1, 5):
+        for axes in itertools.combinations(range(4), r):
+            for keep in (False, True):
+                assert t._reduce_shape(list(axes), keep) == orc.reduce_shape([2, 3, 4, 5], list(axes), keep)
+    l = hpt.lib()
+    for op in range(14):
+        for d in hpt.DTYPES:
+            od = C.c_int32()
+            assert l.hpt_hip_reduce_out_dtype(op, d.code, C.byref(od)) == 0
+            assert od.value == orc.reduce_out_dtype(op, d.code)
+
+
+def test_plans_for_the_benchmark_configurations(hpt):
+    """Which kernel family and launch shape each benchmark op gets (no device needed)."""
+    f32 = lambda *s: hpt.Tensor.from_numpy(np.zeros(s, np.float32))
+    c3 = f32(64, 128, 56, 56)
+    p = hpt.reduce_plan(c3, hpt.SUM, [2, 3])
+    assert p.startswith("row vec=4") and "rows=8192 cols=3136" in p and "kept=[8192:3136] red=[3136:1]" in p
+    p = hpt.reduce_plan(c3, hpt.MAX, [1])
+    assert p.startswith("col vec=4") and "outs=200704 red=128" in p and "red=[128:3136]" in p
+    p = hpt.reduce_plan(c3, hpt.SUM, [0, 1, 2, 3])
+    assert p.startswith("row vec=4") and "rows=1 cols=25690112" in p and "split=1(" not in p
+    c1 = f32(1024, 1024)
+    assert hpt.reduce_plan(c1, hpt.SUM, [1]).startswith("row vec=4")
+    assert hpt.normalize_plan(c1, 1).startswith("rowreg rows=1024 cols=1024 vec=4")
+    c2 = f32(8192, 4096)
+    assert hpt.normalize_plan(c2, 0, 1).startswith("rowreg rows=8192 cols=4096 vec=4 tpr=256 rpb=1 nchunk=4")
+    c4 = hpt.Tensor.from_numpy(np.zeros((64, 2048), np.uint16), hpt.bf16)
+    assert hpt.normalize_plan(c4, 1).startswith("rowreg rows=64 cols=2048 vec=8 tpr=64 rpb=4 nchunk=4")
+    c5 = hpt.Tensor.from_numpy(np.zeros((64, 128), np.float16))
+    assert hpt.normalize_plan(c5.permute([1, 0]), 1).startswith("transposed rows=128 cols=64")
+    assert hpt.reduce_plan(c5.permute([1, 0]), hpt.SUM, [0]).startswith("row vec=8")
+    assert "norm_in=[64:2]" in hpt.normalize_plan(c5[:, ::2], 1)
+    assert hpt.reduce_plan(c5[:, ::2], hpt.SUM, [0]).startswith("col vec=1")
+    # misaligned base pointer or odd row length: scalar loads
+    assert hpt.reduce_plan(f32(7, 1023), hpt.SUM, [1]).startswith("row vec=1")
+    assert hpt.reduce_plan(f32(8, 1024)[:, 1:], hpt.SUM, [1]).startswith("row vec=1")
+
+
+def test_coalescing_matches_brute_force_offsets(hpt):
+    """The planner's (kept, reduced) dim lists must address exactly the elements of the view."""
+    rng = np.random.default_rng(11)
+    base = hpt.Tensor.from_numpy(np.zeros((4, 6, 5, 8), np.float32))
+    for _ in range(60):
+        t = base.permute(list(rng.permutation(4)))
+        if rng.random() < 0.5:
+            t = t[:, ::2]
+        axes = sorted(rng.choice(4, int(rng.integers(1, 4)), replace=False).tolist())
+        plan = hpt.reduce_plan(t, hpt.SUM, axes)
+        dims = {}
+        for name in ("kept", "red"):
+            m = re.search(name + r"=\[([^\]]*)\]", plan)
+            dims[name] = [tuple(int(x) for x in d.split(":")) for d in m.group(1).split(",") if d]
+        offs = lambda ds: [sum(i * st for i, (_, st) in zip(ix, ds)) for ix in itertools.product(*[range(n) for n, _ in ds])]
+        want_kept = [sum(i * t.strides[a] for i, a in zip(ix, [a for a in range(4) if a not in axes]))
+                     for ix in itertools.product(*[range(t.shape[a]) for a in range(4) if a not in axes])]
+        want_red = sorted(sum(i * t.strides[a] for i, a in zip(ix, axes))
+                          for ix in itertools.product(*[range(t.shape[a]) for a in axes]))
+        assert offs(dims["kept"]) == want_kept
+        assert sorted(offs(dims["red"])) == want_red
+
+
+def test_argument_errors_without_a_device(hpt):
+    t = hpt.Tensor.from_numpy(np.zeros((3, 4), np.float32))
+    with pytest.raises(hpt.ShapeError):
+        hpt.reduce_plan(t, hpt.SUM, [5])
+    with pytest.raises(hpt.ParamError):
+        hpt.reduce_plan(t, 99, [0])
+    with pytest.raises(hpt.DTypeError):
+        hpt.normalize_plan(hpt.Tensor.from_numpy(np.zeros((3, 4), np.int32)), 1)
+    with pytest.raises(NotImplementedError, match="Hip backend only"):
+        t.sum([0])
+    with pytest.raises(NotImplementedError):
+        t.softmax(1)
+
+
+def test_views_follow_the_reference_slice_rules(hpt, orc):
+    BIG = 0x7FFFFFFFFFFFFFFF
+    a = np.arange(3 * 4 * 5, dtype=np.float32).reshape(3, 4, 5)
+    t = hpt.Tensor.from_numpy(a)
+    v = t.slice([(1, BIG, 1), (0, 3, 1), (0, BIG, 2)])   # hpt-common/src/slice.rs:30-38
+    assert (v.shape, v.strides, (v.ptr - t.ptr) // 4) == ([2, 3, 3], [20, 5, 2], 20)
+    assert np.array_equal(v.numpy(), a[1:, 0:3, ::2])
+    rng = np.random.default_rng(12)
+    for _ in range(100):
+        idx = []
+        for d in a.shape:
+            step = int(rng.integers(1, 4))
+            start = int(rng.integers(0, d))
+            idx.append((start, int(rng.integers(start + 1, d + 1)), step))
+        v = t.slice(idx)
+        shape, strides, off = orc.slice_process([3, 4, 5], [20, 5, 1], idx)
+        assert (v.shape, v.strides, (v.ptr - t.ptr) // 4) == (shape, strides, off)
+        assert np.array_equal(v.numpy(), a[tuple(slice(*i) for i in idx)])
+    p = t.permute([2, 0, 1])
+    assert p.shape == [5, 3, 4] and p.strides == [1, 20, 5] and not p.is_contiguous()
+    assert np.array_equal(p[:, ::2].numpy(), a.transpose(2, 0, 1)[:, ::2])
+    assert np.array_equal(t[::-1].numpy(), a[::-1])
