@@ -140,38 +140,41 @@ class Prepared:
         return lambda i: check(l.hpt_hip_reduce(0, None, code, vi[i % n], ax, na, 1, vo[i % n])), outs
 
 
-def build_cases(which: str):
-    """Synthetic inputs of the five configurations, uploaded once; outputs preallocated."""
+def cases_c2(P, headline_only):
+    """C2: LayerNorm / log_softmax, f32 [8192, 4096] (the headline)."""
     import hpt_amd as hpt
-    P = Prepared()
-    cases = []
-
-    # ---- C2: LayerNorm / log_softmax, f32 [8192, 4096] (headline) ----
     x, g, b = gen_c2()
     nbuf = 4
     xs = [hpt.Tensor.from_numpy(np.roll(x, k, axis=0)).to_hip(0) for k in range(nbuf)]
     tg, tb = hpt.Tensor.from_numpy(g).to_hip(0), hpt.Tensor.from_numpy(b).to_hip(0)
     ln_bytes = 2 * x.nbytes + g.nbytes + b.nbytes
     run, ln_outs = P.norm(xs, "layernorm", n_norm=1, gamma=tg, beta=tb)
-    cases.append(Case("layernorm", "C2 f32 [8192,4096] gamma,beta eps=1e-5", "f32", 8192, ln_bytes, run, nbuf))
-    head_out = ln_outs[0]
-    if which == "headline":
-        return cases, P, (x, g, b, head_out)
-    run, _ = P.norm(xs, "log_softmax", axis=1)
-    cases.append(Case("log_softmax", "C2 f32 [8192,4096] axis=1", "f32", 8192, 2 * x.nbytes, run, nbuf))
+    cases = [Case("layernorm", "C2 f32 [8192,4096] gamma,beta eps=1e-5", "f32", 8192, ln_bytes, run, nbuf)]
+    if not headline_only:
+        run, _ = P.norm(xs, "log_softmax", axis=1)
+        cases.append(Case("log_softmax", "C2 f32 [8192,4096] axis=1", "f32", 8192, 2 * x.nbytes, run, nbuf))
+    return cases, (x, g, b, ln_outs[0])
 
-    # ---- C1: f32 [1024,1024] U(-10,10) ----
+
+def cases_c1(P):
+    """C1: f32 [1024,1024] U(-10,10): softmax, sum, max over axis 1 (launch-bound: 4-8 MB)."""
+    import hpt_amd as hpt
     rng = np.random.default_rng(0)
     c1 = rng.uniform(-10, 10, (1024, 1024)).astype(np.float32)
     c1s = [hpt.Tensor.from_numpy(np.roll(c1, k, 0)).to_hip(0) for k in range(64)]
+    cases = []
     run, _ = P.norm(c1s, "softmax", axis=1)
     cases.append(Case("softmax", "C1 f32 [1024,1024] axis=1", "f32", 1024, 2 * c1.nbytes, run, 64))
     run, _ = P.reduce(c1s, "sum", [1])
     cases.append(Case("sum(axis=1)", "C1 f32 [1024,1024]", "f32", 1024, c1.nbytes + 4096, run, 64))
     run, _ = P.reduce(c1s, "max", [1])
     cases.append(Case("max(axis=1)", "C1 f32 [1024,1024]", "f32", 1024, c1.nbytes + 4096, run, 64))
+    return cases
 
-    # ---- C3: f32 / i32 [64,128,56,56] ----
+
+def cases_c3(P):
+    """C3: f32 / i32 [64,128,56,56]: axis reductions."""
+    import hpt_amd as hpt
     rng = np.random.default_rng(2)
     c3 = rng.standard_normal((64, 128, 56, 56), dtype=np.float32)
     c3s = [hpt.Tensor.from_numpy(np.roll(c3, k, 0)).to_hip(0) for k in range(6)]
@@ -179,6 +182,7 @@ def build_cases(which: str):
     c3i = rng.integers(-1000, 1001, (64, 128, 56, 56)).astype(np.int32)
     c3is = [hpt.Tensor.from_numpy(np.roll(c3i, k, 0)).to_hip(0) for k in range(6)]
     nb = c3.nbytes
+    cases = []
     for name, op, axes, rows, outb in (("sum([2,3])", "sum", [2, 3], 8192, 8192 * 4),
                                        ("mean([2,3])", "mean", [2, 3], 8192, 8192 * 4),
                                        ("max(axis=1)", "max", [1], 200704, 200704 * 4),
@@ -189,8 +193,12 @@ def build_cases(which: str):
     cases.append(Case("sum(axis=1)", "C3 i32 [64,128,56,56]", "i32", 200704, nb + 200704 * 4, run, 6))
     run, _ = P.reduce(c3is, "argmax", 1, arg=True)
     cases.append(Case("argmax(axis=1)", "C3 i32 [64,128,56,56]", "i32", 200704, nb + 200704 * 8, run, 6))
+    return cases
 
-    # ---- C4: bf16 [65536, 2048] causal-masked logits ----
+
+def cases_c4(P):
+    """C4: bf16 [65536, 2048] logits with the causal mask as data (-inf above the diagonal)."""
+    import hpt_amd as hpt
     rng = np.random.default_rng(4)
     c4 = rng.standard_normal((65536, 2048), dtype=np.float32) * 3
     q = (np.arange(65536) % 2048)[:, None]
@@ -200,10 +208,13 @@ def build_cases(which: str):
     c4s = [hpt.Tensor.from_numpy(c4b, hpt.bf16).to_hip(0),
            hpt.Tensor.from_numpy(np.roll(c4b, 2048, 0), hpt.bf16).to_hip(0)]
     run, _ = P.norm(c4s, "softmax", axis=1)
-    cases.append(Case("softmax", "C4 bf16 [65536,2048] causal mask as data, axis=1", "bf16", 65536,
-                      2 * c4b.nbytes, run, 2))
+    return [Case("softmax", "C4 bf16 [65536,2048] causal mask as data, axis=1", "bf16", 65536,
+                 2 * c4b.nbytes, run, 2)]
 
-    # ---- C5: f16 base [4096,8192]: transposed view and [:, ::2] view ----
+
+def cases_c5(P):
+    """C5: f16 base [4096,8192]: the transposed view and the [:, ::2] view."""
+    import hpt_amd as hpt
     rng = np.random.default_rng(5)
     c5 = (rng.standard_normal((4096, 8192), dtype=np.float32) * 2).astype(np.float16)
     c5s = [hpt.Tensor.from_numpy(np.roll(c5, k, 0)).to_hip(0) for k in range(6)]
@@ -213,6 +224,7 @@ def build_cases(which: str):
     n5 = c5.nbytes
     c5t = [t.permute([1, 0]) for t in c5s]
     c5h = [t[:, ::2] for t in c5s]
+    cases = []
     run, _ = P.norm(c5t, "layernorm", n_norm=1, gamma=tg5, beta=tb5)
     cases.append(Case("layernorm", "C5a f16 [4096,8192].permute(1,0) -> [8192,4096]", "f16", 8192, 2 * n5 + 16384, run, 6))
     run, _ = P.norm(c5t, "softmax", axis=1)
@@ -225,7 +237,19 @@ def build_cases(which: str):
     cases.append(Case("softmax", "C5b f16 [4096,8192][:, ::2] axis=1", "f16", 4096, n5, run, 6))
     run, _ = P.reduce(c5h, "sum", [0])
     cases.append(Case("sum(axis=0)", "C5b f16 [4096,8192][:, ::2]", "f16", 4096, n5 // 2 + 8192, run, 6))
-    return cases, P, (x, g, b, head_out)
+    return cases
+
+
+def build_cases(which: str, configs=None):
+    """Synthetic inputs of the benchmark configurations, uploaded once; outputs preallocated.
+    The headline (C2 layernorm) is always first; `configs` limits the others (e.g. {"c3"})."""
+    P = Prepared()
+    cases, head = cases_c2(P, which == "headline")
+    if which != "headline":
+        for name, fn in (("c1", cases_c1), ("c3", cases_c3), ("c4", cases_c4), ("c5", cases_c5)):
+            if configs is None or name in configs:
+                cases += fn(P)
+    return cases, P, head
 
 
 def cpu_baseline(x, g, b, gpu_out, budget_s=15.0):
@@ -267,6 +291,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--ops", choices=["all", "headline"], default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--configs", default="", help="comma list of c1,c3,c4,c5 to measure besides the headline")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU form (every op but a full "
@@ -280,7 +305,8 @@ def main():
     assert hpt.device_count() >= 1, "no HIP device visible"
     ev = HipEvents()
 
-    cases, prepared, (x, g, b, head_out) = build_cases(args.ops)
+    configs = set(args.configs.split(",")) if args.configs else None
+    cases, prepared, (x, g, b, head_out) = build_cases(args.ops, configs)
     head = cases[0]
     wall, dev_ms = time_case(ev, head, args.steps, args.warmup)
     ms_per_step = wall * 1e3 / args.steps

@@ -192,16 +192,8 @@ static ReduceScratch scratch_for(int dev, hipStream_t st, size_t partial_bytes, 
 }
 
 void scratch_need(const ReducePlan& p, size_t acc_size, size_t* partial_bytes, size_t* counters) {
-    *partial_bytes = 0;
     *counters = 0;
-    if (p.split <= 1) return;
-    *partial_bytes = (size_t)p.K * p.split * acc_size;
-    if (p.kind == ReduceKind::Row) {
-        *counters = (size_t)p.K;
-    } else {
-        int64_t kv = p.K / p.vec;
-        *counters = (size_t)((kv + p.bx - 1) / p.bx);
-    }
+    *partial_bytes = p.split > 1 ? (size_t)p.K * p.split * acc_size : 0;
 }
 
 // ---- dispatch tables -----------------------------------------------------------

@@ -95,6 +95,7 @@ struct ReducePlan {
     int split_q = 1; // Row: how `split` divides the outer reduced dims ...
     int split_i = 1; // ... and the innermost reduced dim (split = split_q * split_i)
     int64_t chunk = 0;  // Col: reduced indices per split
+    bool lean = false;  // the layout fits the lean kernels (one reduced dim, <= 2 kept dims, 32-bit extents)
 };
 
 // Build the plan for reducing `axes` (already normalised) of a view.
@@ -125,6 +126,7 @@ struct NormPlan {
     int tpr = 1;      // threads per row (RowReg / RowStream / Generic)
     int rpb = 1;      // rows per block
     int nchunk = 1;   // RowReg: vectors held per thread
+    int max_blocks = 4096;  // RowReg layernorm: workgroups launched at most (they walk the rows)
     int64_t inner = 1;  // Col: size of the contiguous inner dim the lanes walk
 };
 

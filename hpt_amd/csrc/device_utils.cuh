@@ -126,6 +126,44 @@ __device__ __forceinline__ void store_pack(T* p, const Pack<T, N>& v) {
     *reinterpret_cast<Pack<T, N>*>(p) = v;
 }
 
+// Streaming (non-temporal) forms for data that is touched exactly once: the
+// access is marked so that it does not displace reusable lines from the caches.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+#ifndef HPT_STREAMING_ACCESS
+#define HPT_STREAMING_ACCESS 1
+#endif
+template <class T, int N>
+__device__ __forceinline__ Pack<T, N> load_pack_stream(const T* p) {
+#if HPT_STREAMING_ACCESS
+    if constexpr (sizeof(T) * N == 16) {
+        union { u32x4 u; Pack<T, N> v; } c;
+        c.u = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+        return c.v;
+    } else if constexpr (sizeof(T) * N == 8) {
+        union { u32x2 u; Pack<T, N> v; } c;
+        c.u = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+        return c.v;
+    } else
+#endif
+        return load_pack<T, N>(p);
+}
+template <class T, int N>
+__device__ __forceinline__ void store_pack_stream(T* p, const Pack<T, N>& v) {
+#if HPT_STREAMING_ACCESS
+    if constexpr (sizeof(T) * N == 16) {
+        union { u32x4 u; Pack<T, N> v; } c;
+        c.v = v;
+        __builtin_nontemporal_store(c.u, reinterpret_cast<u32x4*>(p));
+    } else if constexpr (sizeof(T) * N == 8) {
+        union { u32x2 u; Pack<T, N> v; } c;
+        c.v = v;
+        __builtin_nontemporal_store(c.u, reinterpret_cast<u32x2*>(p));
+    } else
+#endif
+        store_pack<T, N>(p, v);
+}
+
 // ---- index arithmetic -----------------------------------------------------
 
 // Offset (in elements) of linear index `idx` over dims `d`, outermost first.

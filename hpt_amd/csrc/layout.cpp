@@ -136,6 +136,7 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
     int64_t sr = p.red.n ? iabs(p.red.stride[p.red.n - 1]) : INT64_MAX;
     int64_t sk = p.kept.n ? iabs(p.kept.stride[p.kept.n - 1]) : INT64_MAX;
 
+    const int64_t kI32 = 0x7fffffff;
     if (p.red.n > 0 && (p.kept.n == 0 || sr <= sk)) {
         // ---- Row: lanes walk the reduced index space ---------------------
         p.kind = ReduceKind::Row;
@@ -143,19 +144,24 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
         p.vec = 1;
         if (p.red.stride[p.red.n - 1] == 1)
             p.vec = legal_vec(data, elem_size, rin, p.kept, p.red, 0, 1);
+        p.lean = p.red.n == 1 && p.kept.n <= 1 && p.K <= kI32 && rin <= kI32 &&
+                 iabs(p.red.stride[0]) <= kI32;
         int64_t nv = p.R / p.vec;  // vector loads per output
-        // aim at about 8 loads per thread before widening the group
-        p.tpr = (int)std::min<int64_t>(1024, pow2_ceil((nv + 7) / 8));
-        if (p.tpr > 64 && p.tpr < 256) p.tpr = 256;  // above a wave, whole blocks only
+        // About 8 vector loads per lane; groups of one or two wavefronts per row
+        // stream best (each wavefront walks its own long run of the row), and
+        // only very long rows get a whole workgroup.
+        p.tpr = (int)std::min<int64_t>(128, pow2_ceil((nv + 7) / 8));
+        if (nv >= 128 * 64) p.tpr = nv >= 1024 * 32 ? 1024 : 256;
         int block = std::max(256, p.tpr);
         p.rpb = block / p.tpr;
         int64_t blocks = (p.K + p.rpb - 1) / p.rpb;
         p.split = p.split_q = p.split_i = 1;
-        if (blocks < kBlocksToFill / 2) {
-            // too few outputs to fill the chip: several blocks of 256 threads per
-            // output, each with at least 8 vector loads per thread
-            int64_t want = (kBlocksToFill * 2 + p.K - 1) / p.K;
-            int64_t can = nv / (256 * 8);
+        if (blocks < kBlocksToFill / 4) {
+            // Too few outputs to fill the chip: several workgroups of 256 threads
+            // per output, each with a long contiguous share (>= 16 loads per
+            // thread); about 1024 workgroups in all is the measured sweet spot.
+            int64_t want = (1024 + p.K - 1) / p.K;
+            int64_t can = nv / (256 * 16);
             int64_t split = std::min<int64_t>(std::min(want, can), 4096);
             if (split > 1) {
                 p.tpr = 256;
@@ -173,32 +179,35 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
     } else {
         // ---- Col: lanes walk the outputs -----------------------------------
         p.kind = ReduceKind::Col;
-        int64_t kin = p.kept.n ? p.kept.size[p.kept.n - 1] : 1;
+        const int nk = p.kept.n;
+        int64_t kin = nk ? p.kept.size[nk - 1] : 1;
         p.vec = 1;
-        if (p.kept.n && p.kept.stride[p.kept.n - 1] == 1)
+        if (nk && p.kept.stride[nk - 1] == 1)
             p.vec = legal_vec(data, elem_size, kin, p.kept, p.red, 1, 0);
-        int64_t kv = p.K / p.vec;  // vector columns
+        const int64_t outer = nk > 1 ? p.kept.size[0] : 1;
+        p.lean = p.red.n <= 1 && nk <= 2 && outer <= 65535 && kin <= kI32 && p.R <= kI32 &&
+                 (nk == 0 || iabs(p.kept.stride[nk - 1]) <= kI32);
+        int64_t kv = (p.lean ? kin : p.K) / p.vec;  // vector columns the lanes spread over
         p.bx = (int)std::min<int64_t>(64, pow2_ceil(kv));
-        int64_t xblocks = (kv + p.bx - 1) / p.bx;
-        // split the reduced range over thread rows while each keeps >= 8 loads
-        int by = 256 / p.bx;
-        int64_t waves_x = xblocks * std::max(1, p.bx / 64);
-        int want_by = pow2_ceil((kBlocksToFill * 4 + waves_x - 1) / waves_x);
-        int can_by = pow2_floor(std::max<int64_t>(1, p.R / 8));
-        by = std::max(by, std::min(16 * 64 / p.bx, want_by));
-        by = std::min(by, std::max(1, can_by));
-        by = std::min(by, 1024 / p.bx);
+        int64_t xblocks = (kv + p.bx - 1) / p.bx * (p.lean ? outer : 1);
+        // One wavefront per 64 vector columns streams best when there are enough
+        // columns (measured: 832 wavefronts with 128 loads each reach 5.9 TB/s);
+        // with fewer, thread rows and then workgroups split the reduced range.
+        const int base_by = 64 / p.bx;  // a workgroup is at least one wavefront
+        const int64_t kWavesWanted = 768;
+        int by = base_by;
+        while (xblocks * (by / base_by) < kWavesWanted && by * p.bx < 1024 && p.R / (by * 2) >= 8) by *= 2;
         // the thread rows meet in LDS: keep bx*by*vec accumulators within 64 KiB
         while (by > 1 && (size_t)p.bx * by * p.vec * acc_size > (64u << 10)) by /= 2;
         p.by = std::max(1, by);
         p.split = 1;
-        int64_t blocks = xblocks;
+        int64_t waves = xblocks * std::max(1, p.by / base_by);
         int64_t per_thread = p.R / p.by;
-        if (blocks * p.by * p.bx / 256 < kBlocksToFill / 2 && per_thread > 32) {
-            int64_t want = (kBlocksToFill * 256 / ((int64_t)p.bx * p.by) + blocks - 1) / blocks;
-            int64_t can = per_thread / 16;
-            // bound the partial buffer: K * split accumulators of 16 bytes <= 64 MiB
-            int64_t cap = std::max<int64_t>(1, (64ll << 20) / 16 / p.K);
+        if (waves < kWavesWanted && per_thread >= 64) {
+            int64_t want = (kWavesWanted + waves - 1) / waves;
+            int64_t can = per_thread / 32;
+            // bound the partial buffer: K * split accumulators <= 64 MiB
+            int64_t cap = std::max<int64_t>(1, (int64_t)((64ll << 20) / acc_size) / p.K);
             p.split = (int)std::max<int64_t>(1, std::min(std::min(want, can), std::min<int64_t>(cap, 1024)));
         }
         p.chunk = (p.R + p.split - 1) / p.split;
@@ -225,13 +234,13 @@ std::string describe(const ReducePlan& p) {
         case ReduceKind::Empty: return "empty";
         case ReduceKind::Identity: return "identity";
         case ReduceKind::Row:
-            snprintf(buf, sizeof buf, "row vec=%d tpr=%d rpb=%d rows=%lld cols=%lld split=%d(%dx%d) ",
-                     p.vec, p.tpr, p.rpb, (long long)p.K, (long long)p.R, p.split, p.split_q,
-                     p.split_i);
+            snprintf(buf, sizeof buf, "row%s vec=%d tpr=%d rpb=%d rows=%lld cols=%lld split=%d(%dx%d) ",
+                     p.lean ? "" : "-general", p.vec, p.tpr, p.rpb, (long long)p.K, (long long)p.R,
+                     p.split, p.split_q, p.split_i);
             break;
         case ReduceKind::Col:
-            snprintf(buf, sizeof buf, "col vec=%d bx=%d by=%d outs=%lld red=%lld split=%d ", p.vec,
-                     p.bx, p.by, (long long)p.K, (long long)p.R, p.split);
+            snprintf(buf, sizeof buf, "col%s vec=%d bx=%d by=%d outs=%lld red=%lld split=%d ",
+                     p.lean ? "" : "-general", p.vec, p.bx, p.by, (long long)p.K, (long long)p.R, p.split);
             break;
     }
     s = buf;

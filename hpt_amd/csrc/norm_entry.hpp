@@ -22,6 +22,7 @@ struct NormArgs {
     int64_t sa;               // input stride along the row when norm_in.n == 1
     int64_t out_axis_stride;  // output stride along the row
     double eps;
+    double inv_cols;  // 1 / cols
     int tpr, tpr_log2, rpb;
 };
 

@@ -51,6 +51,8 @@ template <class T> __device__ __forceinline__ float log_ct(float x) {
     else return logf(x);
 }
 template <class T> __device__ __forceinline__ double log_ct(double x) { return log(x); }
+__device__ __forceinline__ float fma_ct(float a, float b, float c) { return fmaf(a, b, c); }
+__device__ __forceinline__ double fma_ct(double a, double b, double c) { return fma(a, b, c); }
 __device__ __forceinline__ float rsqrt_ct(float x) { return 1.0f / sqrtf(x); }
 __device__ __forceinline__ double rsqrt_ct(double x) { return 1.0 / sqrt(x); }
 
@@ -59,141 +61,169 @@ template <class CT> __device__ __forceinline__ CT neg_inf() {
     else return -__builtin_huge_valf();
 }
 
-// type the layernorm row statistics are accumulated in
+// Type the layernorm row statistics are combined in ACROSS lanes. Each lane sums
+// its own (few) elements in the compute type; f32 rows then combine the lane
+// sums in f64 and carry the mean as an f32 (hi, lo) pair, so that x - mean is
+// accurate to an ulp of the difference even when the row's offset dwarfs its
+// spread. No per-element f64 arithmetic is involved.
 template <class T> struct StatType { using type = float; };
 template <> struct StatType<float> { using type = double; };
 template <> struct StatType<double> { using type = double; };
 
-template <class Op, class CT>
-__device__ __forceinline__ CT row_all_reduce(CT v, int tpr, CT* smem) {
-    if (tpr <= 64) return group_reduce<Op>(v, tpr);
-    return block_reduce<Op>(v, smem);
+// All-reduce over the `tpr` lanes that share a row: shuffles inside a wavefront,
+// LDS across the wavefronts of the row. Every thread of the workgroup must call it.
+template <class Op, class A>
+__device__ __forceinline__ A row_all_reduce(A v, int tpr, int ty, A* smem) {
+    v = group_reduce<Op>(v, tpr < 64 ? tpr : 64);
+    if (tpr > 64) {
+        const int wpr = tpr >> 6;
+        __syncthreads();
+        if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = v;
+        __syncthreads();
+        A r = smem[ty * wpr];
+        for (int w = 1; w < wpr; ++w) r = Op::comb(r, smem[ty * wpr + w]);
+        v = r;
+    }
+    return v;
 }
 
 // ---- rows held in registers ---------------------------------------------------
+// grid.x workgroups walk the rows in steps of gridDim.x * rpb, so that gamma and
+// beta are fetched once per thread (they index by column, and a thread keeps its
+// columns) instead of once per row, and the launch prologue is paid once.
 template <int KIND, class T, int VEC, int NCHUNK>
 __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     using CT = typename Elem<T>::Wide;
+    using ST = typename StatType<T>::type;
     __shared__ __align__(8) unsigned char smem_stat[16 * sizeof(double)];
     CT* smem = reinterpret_cast<CT*>(smem_stat);
+    ST* ssmem = reinterpret_cast<ST*>(smem_stat);
     const int tpr = a.tpr;
     const int tx = threadIdx.x & (tpr - 1);
     const int ty = threadIdx.x >> a.tpr_log2;
-    const int64_t row = (int64_t)blockIdx.x * a.rpb + ty;
-    const bool valid = row < a.rows;
-    const int64_t nv = a.cols / VEC;
-    const T* in_row = (const T*)a.in + (valid ? offset_of(a.kept_in, row) : 0);
-    T* out_row = (T*)a.out + (valid ? row * a.cols : 0);
-
-    CT x[NCHUNK][VEC];
+    const int nv = (int)(a.cols / VEC);
     constexpr bool kSoft = KIND != NORM_LAYERNORM;
     const CT fill = kSoft ? neg_inf<CT>() : (CT)0;
-#pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) {
-        const int64_t iv = (int64_t)c * tpr + tx;
-        if (valid && iv < nv) {
-            if constexpr (VEC > 1) {
-                Pack<T, VEC> v = load_pack<T, VEC>(in_row + iv * VEC);
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) x[c][j] = Elem<T>::widen(v.v[j]);
-            } else {
-                x[c][0] = Elem<T>::widen(in_row[iv * a.sa]);
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) x[c][j] = fill;
-        }
-    }
 
-    if constexpr (kSoft) {
-        CT m = neg_inf<CT>();
-#pragma unroll
-        for (int c = 0; c < NCHUNK; ++c)
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, x[c][j]);
-        m = row_all_reduce<MaxC<CT>>(m, tpr, smem);
-        CT s = 0;
-#pragma unroll
-        for (int c = 0; c < NCHUNK; ++c)
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) {
-                CT d = x[c][j] - m;
-                CT e = exp_ct<T>(d);
-                s += e;
-                x[c][j] = KIND == NORM_SOFTMAX ? e : d;
-            }
-        s = row_all_reduce<SumC<CT>>(s, tpr, smem);
-        const CT k = KIND == NORM_SOFTMAX ? (CT)1 / s : log_ct<T>(s);
-#pragma unroll
-        for (int c = 0; c < NCHUNK; ++c)
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) x[c][j] = KIND == NORM_SOFTMAX ? x[c][j] * k : x[c][j] - k;
-    } else {
-        // Row statistics of f32 (and f64) rows are taken in f64: x - mean is then
-        // exact before it is rounded, so rows whose spread is small against
-        // their offset keep full f32 accuracy. Half types use f32.
-        using ST = typename StatType<T>::type;
-        ST* ssmem = reinterpret_cast<ST*>(smem_stat);
-        ST s = 0;
-#pragma unroll
-        for (int c = 0; c < NCHUNK; ++c)
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) s += (ST)x[c][j];
-        s = row_all_reduce<SumC<ST>>(s, tpr, ssmem);
-        const ST mean = s / (ST)a.cols;
-        ST q = 0;
+    // this thread's columns never change: keep gamma / beta in registers
+    Pack<T, VEC> gam[NCHUNK], bet[NCHUNK];
+    if constexpr (!kSoft) {
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
-            const bool in_row_c = ((int64_t)c * tpr + tx) < nv;
+            const int iv = c * tpr + tx;
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
-                const ST d = in_row_c ? (ST)x[c][j] - mean : (ST)0;
-                x[c][j] = (CT)d;
-                q += d * d;
+                gam[c].v[j] = Elem<T>::narrow((CT)1);
+                bet[c].v[j] = Elem<T>::narrow((CT)0);
             }
-        }
-        q = row_all_reduce<SumC<ST>>(q, tpr, ssmem);
-        const CT rstd = (CT)rsqrt_ct(q / (ST)a.cols + (ST)a.eps);
-#pragma unroll
-        for (int c = 0; c < NCHUNK; ++c) {
-            const int64_t iv = (int64_t)c * tpr + tx;
             if (iv < nv) {
                 if constexpr (VEC > 1) {
-                    if (a.gamma) {
-                        Pack<T, VEC> g = load_pack<T, VEC>((const T*)a.gamma + iv * VEC);
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) x[c][j] = x[c][j] * rstd * Elem<T>::widen(g.v[j]);
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) x[c][j] *= rstd;
-                    }
-                    if (a.beta) {
-                        Pack<T, VEC> b = load_pack<T, VEC>((const T*)a.beta + iv * VEC);
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) x[c][j] += Elem<T>::widen(b.v[j]);
-                    }
+                    if (a.gamma) gam[c] = load_pack<T, VEC>((const T*)a.gamma + (int64_t)iv * VEC);
+                    if (a.beta) bet[c] = load_pack<T, VEC>((const T*)a.beta + (int64_t)iv * VEC);
                 } else {
-                    CT y = x[c][0] * rstd;
-                    if (a.gamma) y *= Elem<T>::widen(((const T*)a.gamma)[iv]);
-                    if (a.beta) y += Elem<T>::widen(((const T*)a.beta)[iv]);
-                    x[c][0] = y;
+                    if (a.gamma) gam[c].v[0] = ((const T*)a.gamma)[iv];
+                    if (a.beta) bet[c].v[0] = ((const T*)a.beta)[iv];
                 }
             }
         }
     }
 
-    if (!valid) return;
+    const int64_t row_step = (int64_t)gridDim.x * a.rpb;
+    for (int64_t row0 = (int64_t)blockIdx.x * a.rpb; row0 < a.rows; row0 += row_step) {
+        const int64_t row = row0 + ty;
+        const bool valid = row < a.rows;
+        const T* in_row = (const T*)a.in + (valid ? offset_of(a.kept_in, row) : 0);
+        T* out_row = (T*)a.out + (valid ? row * a.cols : 0);
+
+        CT x[NCHUNK][VEC];
 #pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) {
-        const int64_t iv = (int64_t)c * tpr + tx;
-        if (iv < nv) {
-            if constexpr (VEC > 1) {
-                Pack<T, VEC> o;
+        for (int c = 0; c < NCHUNK; ++c) {
+            const int iv = c * tpr + tx;
+            if (valid && iv < nv) {
+                if constexpr (VEC > 1) {
+                    Pack<T, VEC> v = load_pack_stream<T, VEC>(in_row + (int64_t)iv * VEC);
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) o.v[j] = Elem<T>::narrow(x[c][j]);
-                store_pack<T, VEC>(out_row + iv * VEC, o);
+                    for (int j = 0; j < VEC; ++j) x[c][j] = Elem<T>::widen(v.v[j]);
+                } else {
+                    x[c][0] = Elem<T>::widen(in_row[(int64_t)iv * a.sa]);
+                }
             } else {
-                out_row[iv] = Elem<T>::narrow(x[c][0]);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) x[c][j] = fill;
+            }
+        }
+
+        if constexpr (kSoft) {
+            CT m = neg_inf<CT>();
+#pragma unroll
+            for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, x[c][j]);
+            m = row_all_reduce<MaxC<CT>>(m, tpr, ty, smem);
+            CT s = 0;
+#pragma unroll
+            for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    CT d = x[c][j] - m;
+                    CT e = exp_ct<T>(d);
+                    s += e;
+                    x[c][j] = KIND == NORM_SOFTMAX ? e : d;
+                }
+            s = row_all_reduce<SumC<CT>>(s, tpr, ty, smem);
+            const CT k = KIND == NORM_SOFTMAX ? (CT)1 / s : log_ct<T>(s);
+#pragma unroll
+            for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    x[c][j] = KIND == NORM_SOFTMAX ? x[c][j] * k : x[c][j] - k;
+        } else {
+            CT s = 0;
+#pragma unroll
+            for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) s += x[c][j];
+            // mean = sum / cols, as a reciprocal multiply plus one correction step
+            // (exact quotient for the cases that matter, e.g. constant rows)
+            const ST sum = row_all_reduce<SumC<ST>>((ST)s, tpr, ty, ssmem);
+            const ST m0 = sum * (ST)a.inv_cols;
+            const ST mean = fma_ct(fma_ct(-m0, (ST)a.cols, sum), (ST)a.inv_cols, m0);
+            const CT mean_hi = (CT)mean;
+            const CT mean_lo = (CT)(mean - (ST)mean_hi);  // 0 when ST is no wider than CT
+            CT q = 0;
+#pragma unroll
+            for (int c = 0; c < NCHUNK; ++c) {
+                const bool in_row_c = (c * tpr + tx) < nv;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const CT d = in_row_c ? (x[c][j] - mean_hi) - mean_lo : (CT)0;
+                    x[c][j] = d;
+                    q += d * d;
+                }
+            }
+            const ST var = row_all_reduce<SumC<ST>>((ST)q, tpr, ty, ssmem) * (ST)a.inv_cols;
+            const CT rstd = rsqrt_ct((CT)var + (CT)a.eps);
+#pragma unroll
+            for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    x[c][j] = x[c][j] * rstd * Elem<T>::widen(gam[c].v[j]) + Elem<T>::widen(bet[c].v[j]);
+        }
+
+        if (valid) {
+#pragma unroll
+            for (int c = 0; c < NCHUNK; ++c) {
+                const int iv = c * tpr + tx;
+                if (iv < nv) {
+                    if constexpr (VEC > 1) {
+                        Pack<T, VEC> o;
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) o.v[j] = Elem<T>::narrow(x[c][j]);
+                        store_pack_stream<T, VEC>(out_row + (int64_t)iv * VEC, o);
+                    } else {
+                        out_row[iv] = Elem<T>::narrow(x[c][0]);
+                    }
+                }
             }
         }
     }
@@ -314,43 +344,45 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
         using ST = typename StatType<T>::type;
         MomentStat<ST> st{(ST)0, (ST)0, (ST)0};
         if (valid) {
-            // Per thread: sums of (x - k) and (x - k)^2 around the first element k
-            // it sees (no division per element, no cancellation against a far
-            // origin), turned into (count, mean, M2) once at the end.
-            ST k = 0, s1 = 0, s2 = 0, n = 0;
+            // Per lane: sums of (x - k) and (x - k)^2 around the first element k it
+            // sees, in the compute type (no division per element, no cancellation
+            // against a far origin), turned into (count, mean, M2) once at the end.
+            CT k = 0, s1 = 0, s2 = 0;
+            int64_t n = 0;
             bool first = true;
             for (int64_t iv = tx; iv < nv; iv += tpr) {
                 CT x[VEC];
                 load(iv, x);
                 if (first) {
-                    k = (ST)x[0];
+                    k = x[0];
                     first = false;
                 }
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
-                    const ST d = (ST)x[j] - k;
+                    const CT d = x[j] - k;
                     s1 += d;
                     s2 += d * d;
                 }
-                n += (ST)VEC;
+                n += VEC;
             }
-            if (n > (ST)0) {
-                st.n = n;
-                st.mean = k + s1 / n;
-                st.m2 = s2 - s1 * s1 / n;
+            if (n > 0) {
+                st.n = (ST)n;
+                st.mean = (ST)k + (ST)s1 / st.n;
+                st.m2 = (ST)s2 - (ST)s1 * (ST)s1 / st.n;
                 if (st.m2 < (ST)0) st.m2 = 0;
             }
         }
         st = stat_all_reduce<MomentStatOp<ST>>(st, tpr, (MomentStat<ST>*)smem_raw);
         if (!valid) return;
-        const ST mean = st.mean;
-        const CT rstd = (CT)rsqrt_ct(st.m2 / (ST)a.cols + (ST)a.eps);
+        const CT mean_hi = (CT)st.mean;
+        const CT mean_lo = (CT)(st.mean - (ST)mean_hi);
+        const CT rstd = rsqrt_ct((CT)(st.m2 * (ST)a.inv_cols) + (CT)a.eps);
         for (int64_t iv = tx; iv < nv; iv += tpr) {
             CT x[VEC];
             load(iv, x);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
-                CT y = (CT)((ST)x[j] - mean) * rstd;
+                CT y = ((x[j] - mean_hi) - mean_lo) * rstd;
                 const int64_t col = iv * VEC + j;
                 if (a.gamma) y *= Elem<T>::widen(((const T*)a.gamma)[col]);
                 if (a.beta) y += Elem<T>::widen(((const T*)a.beta)[col]);

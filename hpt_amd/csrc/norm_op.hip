@@ -35,9 +35,13 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
     a.tpr = p.tpr;
     a.tpr_log2 = ilog2(p.tpr);
     a.rpb = p.rpb;
+    a.inv_cols = 1.0 / (double)p.cols;
     dim3 grid((unsigned)((p.rows + p.rpb - 1) / p.rpb));
     dim3 block((unsigned)(p.tpr * p.rpb));
     if (p.kind == NormKind::RowReg) {
+        // Layernorm workgroups walk the rows (gamma / beta stay in registers);
+        // softmax has nothing to reuse across rows and runs one row per group.
+        if (KIND == NORM_LAYERNORM && grid.x > (unsigned)p.max_blocks) grid.x = (unsigned)p.max_blocks;
         if (p.vec == FULL) launch_row_reg<T, FULL>(p, a, grid, block, st);
         else launch_row_reg<T, 1>(p, a, grid, block, st);
         return;

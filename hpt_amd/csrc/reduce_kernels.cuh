@@ -1,19 +1,26 @@
-// The two reduction kernels of libhpt_hip and their launcher.
+// The reduction kernels of libhpt_hip and their launcher.
 //
-//   row_reduce_kernel  lanes walk the reduced index space of one output
-//                      (a reduced dim owns the smallest stride): 128-bit loads
-//                      along the row, combine over the lanes of a wavefront by
-//                      cross-lane shuffles, over wavefronts through LDS.
-//   col_reduce_kernel  lanes walk neighbouring outputs (a kept dim owns the
-//                      smallest stride): every lane accumulates its own
-//                      outputs while thread rows stride over the reduced range;
-//                      the thread rows are combined through LDS.
+//   row kernels   lanes walk the reduced index space of one output (a reduced
+//                 dim owns the smallest stride): 128-bit streaming loads along
+//                 the row, combine over the lanes of a wavefront by cross-lane
+//                 shuffles, over wavefronts through LDS.
+//   col kernels   lanes walk neighbouring outputs (a kept dim owns the smallest
+//                 stride): every lane accumulates its own VEC outputs while it
+//                 strides over the reduced range; thread rows meet in LDS.
 //
-// When there are too few outputs to fill 256 CUs, several workgroups share one
-// output: each writes a partial accumulator, and the workgroup that arrives
-// last (a device-scope counter per output) folds the partials in a fixed order,
-// so results are bit-identical from run to run. The counter is reset by that
-// last workgroup, so the scratch needs no clearing between launches.
+// Each family has a lean form for the layouts that matter most (one reduced
+// dim, at most two kept dims, 32-bit extents: every benchmark configuration)
+// and a general form that walks up to 8 + 8 coalesced dims with 64-bit
+// arithmetic. The lean kernels exist because these launches last 15-50 us and
+// run thousands of short-lived workgroups: a long prologue of index arithmetic
+// costs a measurable share of the HBM bandwidth.
+//
+// When there are too few outputs to fill 256 CUs, several workgroups share an
+// output: each writes a partial accumulator and a second, tiny kernel folds the
+// partials in a fixed order (bit-identical from run to run). Two launches beat
+// the single-launch "last workgroup folds" scheme here: its device-scope fence
+// writes back the L2 and its counter is one contended address, and both
+// serialise (measured: 155 us against 19 us for a 100 MB full sum).
 //
 // These replace the eight kernel variants per op of the reference's device
 // path (hpt-cudakernels/src/reduce/reduce_template.cuh:8-198) and the CPU
@@ -25,13 +32,86 @@
 
 namespace hpt {
 
+template <class Op>
+__device__ __forceinline__ void write_out(void* out, int64_t o, typename Op::Acc acc, int init_out,
+                                          double count) {
+    typename Op::Out* p = (typename Op::Out*)out + o;
+    if (!init_out) acc = Op::comb(Op::from_out(*p), acc);
+    *p = Op::post(acc, count);
+}
+
+// ---- lean row kernel ---------------------------------------------------------
+// out[row] = reduce over i in [0, rin) of in[row * row_stride + i * sr].
+struct RowLeanArgs {
+    const void* in;
+    void* out;       // outputs, or partial accumulators when split > 1
+    int64_t row_stride;
+    double count;
+    int K;           // rows
+    int rin_v;       // row length in vectors
+    int sr;          // element stride along the row (1 when VEC > 1)
+    int ichunk;      // vectors per split
+    int tpr, tpr_log2, rpb, split, init_out;
+};
+
+template <class Op, int VEC>
+__global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
+    using T = typename Op::In;
+    using Acc = typename Op::Acc;
+    __shared__ Acc smem[16];
+    const int tpr = a.tpr;
+    const int tx = threadIdx.x & (tpr - 1);
+    const int ty = threadIdx.x >> a.tpr_log2;
+    const int row = blockIdx.x * a.rpb + ty;
+    const bool valid = row < a.K;
+    Acc acc = Op::identity();
+    if (valid) {
+        const T* p = (const T*)a.in + (int64_t)row * a.row_stride;
+        const int i0 = blockIdx.y * a.ichunk;
+        const int i1 = min(a.rin_v, i0 + a.ichunk);
+        int iv = i0 + tx;
+        if constexpr (VEC > 1) {
+            // batches of four loads in flight per lane before any is consumed
+            for (; iv + 3 * tpr < i1; iv += 4 * tpr) {
+                Pack<T, VEC> v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(p + (int64_t)(iv + u * tpr) * VEC);
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        acc = Op::comb(acc, Op::pre(v[u].v[j], (iv + u * tpr) * VEC + j));
+            }
+            for (; iv < i1; iv += tpr) {
+                Pack<T, VEC> v = load_pack_stream<T, VEC>(p + (int64_t)iv * VEC);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc = Op::comb(acc, Op::pre(v.v[j], iv * VEC + j));
+            }
+        } else {
+#pragma unroll 4
+            for (; iv < i1; iv += tpr) acc = Op::comb(acc, Op::pre(p[(int64_t)iv * a.sr], iv));
+        }
+    }
+    acc = group_reduce<Op>(acc, tpr < 64 ? tpr : 64);
+    if (tpr > 64) {
+        const int wpr = tpr >> 6;  // wavefronts per row
+        if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = acc;
+        __syncthreads();
+        if (tx == 0)
+            for (int w = 1; w < wpr; ++w) acc = Op::comb(acc, smem[ty * wpr + w]);
+    }
+    if (tx == 0 && valid) {
+        if (a.split == 1) write_out<Op>(a.out, row, acc, a.init_out, a.count);
+        else ((Acc*)a.out)[(int64_t)row * a.split + blockIdx.y] = acc;
+    }
+}
+
+// ---- general row kernel ---------------------------------------------------------
 struct RowArgs {
     const void* in;
-    void* out;
-    void* partial;
-    unsigned* counters;
-    Dims kept;   // output index -> input offset
-    Dims redo;   // outer reduced dims (all reduced dims but the innermost)
+    void* out;       // outputs, or partial accumulators when split > 1
+    Dims kept;       // output index -> input offset
+    Dims redo;       // outer reduced dims (all reduced dims but the innermost)
     int64_t K;       // outputs
     int64_t rout;    // product of redo sizes
     int64_t rin_v;   // innermost reduced length, in vectors
@@ -42,28 +122,17 @@ struct RowArgs {
     int tpr, tpr_log2, rpb, split_q, split_i, init_out;
 };
 
-struct ColArgs {
-    const void* in;
-    void* out;
-    void* partial;
-    unsigned* counters;
-    Dims kept_outer;  // kept dims except the innermost
-    Dims red;         // reduced dims
-    int64_t K;        // outputs
-    int64_t kin;      // innermost kept size
-    int64_t sk;       // its stride (1 when VEC > 1)
-    int64_t R;        // reduced elements per output
-    int64_t chunk;    // reduced indices per split
-    double count;
-    int split, init_out;
-};
-
-template <class Op>
-__device__ __forceinline__ void write_out(void* out, int64_t o, typename Op::Acc acc, int init_out,
-                                          double count) {
-    typename Op::Out* p = (typename Op::Out*)out + o;
-    if (!init_out) acc = Op::comb(Op::from_out(*p), acc);
-    *p = Op::post(acc, count);
+template <class Op, int VEC>
+__device__ __forceinline__ void row_step(typename Op::Acc& acc, const typename Op::In* p, int64_t iv,
+                                         int64_t sr) {
+    using T = typename Op::In;
+    if constexpr (VEC > 1) {
+        Pack<T, VEC> v = load_pack_stream<T, VEC>(p + iv * VEC);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc = Op::comb(acc, Op::pre(v.v[j], iv * VEC + j));
+    } else {
+        acc = Op::comb(acc, Op::pre(p[iv * sr], iv));
+    }
 }
 
 template <class Op, int VEC>
@@ -71,7 +140,6 @@ __global__ void __launch_bounds__(1024) row_reduce_kernel(const RowArgs a) {
     using T = typename Op::In;
     using Acc = typename Op::Acc;
     __shared__ Acc smem[16];
-    __shared__ int s_last;
 
     const int tpr = a.tpr;
     const int tx = threadIdx.x & (tpr - 1);
@@ -93,16 +161,7 @@ __global__ void __launch_bounds__(1024) row_reduce_kernel(const RowArgs a) {
             for (int64_t q = q0; q < q1; ++q) {
                 const T* p = base + offset_of(a.redo, q);
 #pragma unroll 4
-                for (int64_t iv = i0 + tx; iv < i1; iv += tpr) {
-                    if constexpr (VEC > 1) {
-                        Pack<T, VEC> v = load_pack<T, VEC>(p + iv * VEC);
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j)
-                            acc = Op::comb(acc, Op::pre(v.v[j], iv * VEC + j));
-                    } else {
-                        acc = Op::comb(acc, Op::pre(p[iv * a.sr], iv));
-                    }
-                }
+                for (int64_t iv = i0 + tx; iv < i1; iv += tpr) row_step<Op, VEC>(acc, p, iv, a.sr);
             }
         } else if (ni > 0) {
             // short inner runs: spread the lanes over (outer, inner) pairs
@@ -117,57 +176,135 @@ __global__ void __launch_bounds__(1024) row_reduce_kernel(const RowArgs a) {
                     dq = t / ni;
                     di = t - dq * ni;
                 }
-                const T* p = base + offset_of(a.redo, q0 + dq);
-                const int64_t iv = i0 + di;
-                if constexpr (VEC > 1) {
-                    Pack<T, VEC> v = load_pack<T, VEC>(p + iv * VEC);
-#pragma unroll
-                    for (int j = 0; j < VEC; ++j) acc = Op::comb(acc, Op::pre(v.v[j], iv * VEC + j));
-                } else {
-                    acc = Op::comb(acc, Op::pre(p[iv * a.sr], iv));
-                }
+                row_step<Op, VEC>(acc, base + offset_of(a.redo, q0 + dq), i0 + di, a.sr);
             }
         }
     }
 
-    if (tpr <= 64) acc = group_reduce<Op>(acc, tpr);
-    else acc = block_reduce<Op>(acc, smem);
-
-    const int split = a.split_q * a.split_i;
-    if (split == 1) {
-        if (tx == 0 && valid) write_out<Op>(a.out, row, acc, a.init_out, a.count);
-        return;
+    acc = group_reduce<Op>(acc, tpr < 64 ? tpr : 64);
+    if (tpr > 64) {
+        const int wpr = tpr >> 6;
+        if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = acc;
+        __syncthreads();
+        if (tx == 0)
+            for (int w = 1; w < wpr; ++w) acc = Op::comb(acc, smem[ty * wpr + w]);
     }
-
-    // several workgroups per output: one output per workgroup here (rpb == 1)
-    Acc* part = (Acc*)a.partial + row * split;
-    // Only the thread that wrote the partial releases it: a device-scope fence
-    // writes back the L2 of this XCD, so it must not run once per wavefront.
-    if (threadIdx.x == 0) {
-        part[blockIdx.y] = acc;
-        __threadfence();
-        unsigned prev = atomicAdd(&a.counters[row], 1u);
-        s_last = (prev == (unsigned)(split - 1));
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    acc = Op::identity();
-    for (int s = threadIdx.x; s < split; s += blockDim.x) acc = Op::comb(acc, part[s]);
-    acc = block_reduce<Op>(acc, smem);
-    if (threadIdx.x == 0) {
-        write_out<Op>(a.out, row, acc, a.init_out, a.count);
-        a.counters[row] = 0;
+    if (tx == 0 && valid) {
+        const int split = a.split_q * a.split_i;
+        if (split == 1) write_out<Op>(a.out, row, acc, a.init_out, a.count);
+        else ((Acc*)a.out)[row * split + blockIdx.y] = acc;
     }
 }
+
+// ---- column kernels ---------------------------------------------------------------
+// Fold the `by` thread rows of a workgroup: row 0 collects, in row order.
+template <class Op, int VEC>
+__device__ __forceinline__ void fold_thread_rows(typename Op::Acc (&acc)[VEC], typename Op::Acc* smem) {
+    const int bx = blockDim.x, by = blockDim.y;
+    const int tx = threadIdx.x, ty = threadIdx.y;
+    if (by == 1) return;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) smem[((size_t)ty * bx + tx) * VEC + j] = acc[j];
+    __syncthreads();
+    if (ty == 0) {
+        for (int y = 1; y < by; ++y) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], smem[((size_t)y * bx + tx) * VEC + j]);
+        }
+    }
+}
+
+// Lean form: outputs are (outer, inner) with inner the lane dim; one reduced dim.
+// out[outer * kin + inner] = reduce over r of in[outer * so + r * rs + inner * sk].
+struct ColLeanArgs {
+    const void* in;
+    void* out;       // outputs, or partials [split][K] when split > 1
+    int64_t so;      // stride of the outer kept dim
+    int64_t rs;      // stride of the reduced dim
+    int64_t K;       // outputs
+    double count;
+    int kin_v;       // inner kept length in vectors
+    int sk;          // inner kept stride in elements (1 when VEC > 1)
+    int R;           // reduced length
+    int chunk;       // reduced indices per split
+    int split, init_out;
+};
+
+template <class Op, int VEC>
+__global__ void __launch_bounds__(1024) col_lean_kernel(const ColLeanArgs a) {
+    using T = typename Op::In;
+    using Acc = typename Op::Acc;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int tx = threadIdx.x, ty = threadIdx.y, by = blockDim.y;
+    const int cv = blockIdx.x * blockDim.x + tx;  // vector column in the inner dim
+    const int outer = blockIdx.y;
+    const bool valid = cv < a.kin_v;
+    Acc acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = Op::identity();
+    if (valid) {
+        const T* base = (const T*)a.in + (int64_t)outer * a.so + (int64_t)cv * VEC * a.sk;
+        const int r0 = blockIdx.z * a.chunk;
+        const int r1 = min(a.R, r0 + a.chunk);
+        int r = r0 + ty;
+        // batches of eight loads in flight per lane before any is consumed: with one
+        // wavefront per 64 columns this is what keeps the memory pipeline full
+        for (; r + 7 * by < r1; r += 8 * by) {
+            Pack<T, VEC> v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const T* p = base + (int64_t)(r + u * by) * a.rs;
+                if constexpr (VEC > 1) v[u] = load_pack_stream<T, VEC>(p);
+                else v[u].v[0] = *p;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], Op::pre(v[u].v[j], r + u * by));
+        }
+        for (; r < r1; r += by) {
+            const T* p = base + (int64_t)r * a.rs;
+            if constexpr (VEC > 1) {
+                Pack<T, VEC> v = load_pack_stream<T, VEC>(p);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], Op::pre(v.v[j], r));
+            } else {
+                acc[0] = Op::comb(acc[0], Op::pre(*p, r));
+            }
+        }
+    }
+    fold_thread_rows<Op, VEC>(acc, (Acc*)smem_raw);
+    if (ty == 0 && valid) {
+        const int64_t o0 = ((int64_t)outer * a.kin_v + cv) * VEC;
+        if (a.split == 1) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) write_out<Op>(a.out, o0 + j, acc[j], a.init_out, a.count);
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) ((Acc*)a.out)[(int64_t)blockIdx.z * a.K + o0 + j] = acc[j];
+        }
+    }
+}
+
+struct ColArgs {
+    const void* in;
+    void* out;        // outputs, or partials [split][K] when split > 1
+    Dims kept_outer;  // kept dims except the innermost
+    Dims red;         // reduced dims
+    int64_t K;        // outputs
+    int64_t kin;      // innermost kept size
+    int64_t sk;       // its stride (1 when VEC > 1)
+    int64_t R;        // reduced elements per output
+    int64_t chunk;    // reduced indices per split
+    double count;
+    int split, init_out;
+};
 
 template <class Op, int VEC>
 __global__ void __launch_bounds__(1024) col_reduce_kernel(const ColArgs a) {
     using T = typename Op::In;
     using Acc = typename Op::Acc;
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    Acc* smem = (Acc*)smem_raw;
-    __shared__ int s_last;
 
     const int bx = blockDim.x, by = blockDim.y;
     const int tx = threadIdx.x, ty = threadIdx.y;
@@ -190,87 +327,53 @@ __global__ void __launch_bounds__(1024) col_reduce_kernel(const ColArgs a) {
         const T* base = (const T*)a.in + offset_of(a.kept_outer, outer) + inner * a.sk;
         const int64_t r0 = (int64_t)blockIdx.y * a.chunk;
         const int64_t r1 = min(a.R, r0 + a.chunk);
-        if (a.red.n <= 1) {
-            const int64_t rs = a.red.n ? a.red.stride[0] : 0;
-#pragma unroll 4
-            for (int64_t r = r0 + ty; r < r1; r += by) {
-                const T* p = base + r * rs;
-                if constexpr (VEC > 1) {
-                    Pack<T, VEC> v = load_pack<T, VEC>(p);
-#pragma unroll
-                    for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], Op::pre(v.v[j], r));
-                } else {
-                    acc[0] = Op::comb(acc[0], Op::pre(*p, r));
-                }
-            }
-        } else {
 #pragma unroll 2
-            for (int64_t r = r0 + ty; r < r1; r += by) {
-                const T* p = base + offset_of(a.red, r);
-                if constexpr (VEC > 1) {
-                    Pack<T, VEC> v = load_pack<T, VEC>(p);
+        for (int64_t r = r0 + ty; r < r1; r += by) {
+            const T* p = base + offset_of(a.red, r);
+            if constexpr (VEC > 1) {
+                Pack<T, VEC> v = load_pack_stream<T, VEC>(p);
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], Op::pre(v.v[j], r));
-                } else {
-                    acc[0] = Op::comb(acc[0], Op::pre(*p, r));
-                }
+                for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], Op::pre(v.v[j], r));
+            } else {
+                acc[0] = Op::comb(acc[0], Op::pre(*p, r));
             }
         }
     }
-
-    // fold the thread rows: row 0 collects, in row order
-    auto fold_rows = [&]() {
-        if (by == 1) return;
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) smem[((size_t)ty * bx + tx) * VEC + j] = acc[j];
-        __syncthreads();
-        if (ty == 0) {
-            for (int y = 1; y < by; ++y) {
-#pragma unroll
-                for (int j = 0; j < VEC; ++j)
-                    acc[j] = Op::comb(acc[j], smem[((size_t)y * bx + tx) * VEC + j]);
-            }
-        }
-    };
-    fold_rows();
-
-    if (a.split == 1) {
-        if (ty == 0 && valid) {
+    fold_thread_rows<Op, VEC>(acc, (Acc*)smem_raw);
+    if (ty == 0 && valid) {
+        if (a.split == 1) {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) write_out<Op>(a.out, o0 + j, acc[j], a.init_out, a.count);
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) ((Acc*)a.out)[(int64_t)blockIdx.y * a.K + o0 + j] = acc[j];
         }
-        return;
     }
+}
 
-    Acc* part = (Acc*)a.partial;
-    if (ty == 0 && valid) {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) part[(int64_t)blockIdx.y * a.K + o0 + j] = acc[j];
+// ---- second stage: fold the partials of the outputs that were split ---------------
+// Partial s of output o sits at part[o * so + s * ss]. BLOCK_PER_OUTPUT: a
+// workgroup folds one output (many partials, few outputs); otherwise a thread
+// folds one output (few partials, many outputs; lanes are neighbours in memory).
+template <class Op, bool BLOCK_PER_OUTPUT>
+__global__ void __launch_bounds__(256) finish_kernel(const void* part_, void* out, int64_t K, int split,
+                                                     int64_t so, int64_t ss, int init_out, double count) {
+    using Acc = typename Op::Acc;
+    const Acc* part = (const Acc*)part_;
+    if constexpr (BLOCK_PER_OUTPUT) {
+        __shared__ Acc smem[16];
+        const int64_t o = blockIdx.x;
+        Acc acc = Op::identity();
+        for (int s = threadIdx.x; s < split; s += blockDim.x) acc = Op::comb(acc, part[o * so + s * ss]);
+        acc = block_reduce<Op>(acc, smem);
+        if (threadIdx.x == 0) write_out<Op>(out, o, acc, init_out, count);
+    } else {
+        const int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (o >= K) return;
+        Acc acc = Op::identity();
+        for (int s = 0; s < split; ++s) acc = Op::comb(acc, part[o * so + s * ss]);
+        write_out<Op>(out, o, acc, init_out, count);
     }
-    if (ty == 0) __threadfence();  // the writers release their partials
-    __syncthreads();
-    if (tx == 0 && ty == 0) {
-        unsigned prev = atomicAdd(&a.counters[blockIdx.x], 1u);
-        s_last = (prev == (unsigned)(a.split - 1));
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) acc[j] = Op::identity();
-    if (valid) {
-        for (int s = ty; s < a.split; s += by) {
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], part[(int64_t)s * a.K + o0 + j]);
-        }
-    }
-    fold_rows();
-    if (ty == 0 && valid) {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) write_out<Op>(a.out, o0 + j, acc[j], a.init_out, a.count);
-    }
-    if (tx == 0 && ty == 0) a.counters[blockIdx.x] = 0;
 }
 
 // Fill `n` outputs with the op's identity (a reduced dim of size 0).
@@ -290,6 +393,7 @@ template <class Op>
 void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const ReduceScratch& sc,
                      hipStream_t st, int init_out) {
     using T = typename Op::In;
+    using Acc = typename Op::Acc;
     constexpr int FULL = 16 / sizeof(T);
     const double count = (double)p.R;
     if (p.kind == ReduceKind::Empty) return;
@@ -298,57 +402,103 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
         identity_fill_kernel<Op><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(out, p.K, init_out, count);
         return;
     }
+    const bool vec = p.vec == FULL && FULL > 1;
+    void* stage1_out = p.split > 1 ? sc.partial : out;
     if (p.kind == ReduceKind::Row) {
-        RowArgs a{};
-        a.in = in;
-        a.out = out;
-        a.partial = sc.partial;
-        a.counters = sc.counters;
-        a.kept = p.kept;
-        a.redo = p.red;
-        a.redo.n = p.red.n - 1;
-        a.K = p.K;
-        const int64_t rin = p.red.size[p.red.n - 1];
-        a.rout = p.R / rin;
-        a.rin_v = rin / p.vec;
-        a.sr = p.red.stride[p.red.n - 1];
-        a.qchunk = (a.rout + p.split_q - 1) / p.split_q;
-        a.ichunk = (a.rin_v + p.split_i - 1) / p.split_i;
-        a.count = count;
-        a.tpr = p.tpr;
-        a.tpr_log2 = ilog2(p.tpr);
-        a.rpb = p.rpb;
-        a.split_q = p.split_q;
-        a.split_i = p.split_i;
-        a.init_out = init_out;
         dim3 grid((unsigned)((p.K + p.rpb - 1) / p.rpb), (unsigned)p.split);
         dim3 block((unsigned)(p.tpr * p.rpb));
-        if (p.vec == FULL && FULL > 1) row_reduce_kernel<Op, FULL><<<grid, block, 0, st>>>(a);
-        else row_reduce_kernel<Op, 1><<<grid, block, 0, st>>>(a);
+        const int64_t rin = p.red.size[p.red.n - 1];
+        if (p.lean) {
+            RowLeanArgs a{};
+            a.in = in;
+            a.out = stage1_out;
+            a.row_stride = p.kept.n ? p.kept.stride[0] : 0;
+            a.count = count;
+            a.K = (int)p.K;
+            a.rin_v = (int)(rin / p.vec);
+            a.sr = (int)p.red.stride[0];
+            a.ichunk = (a.rin_v + p.split - 1) / p.split;
+            a.tpr = p.tpr;
+            a.tpr_log2 = ilog2(p.tpr);
+            a.rpb = p.rpb;
+            a.split = p.split;
+            a.init_out = init_out;
+            if (vec) row_lean_kernel<Op, FULL><<<grid, block, 0, st>>>(a);
+            else row_lean_kernel<Op, 1><<<grid, block, 0, st>>>(a);
+        } else {
+            RowArgs a{};
+            a.in = in;
+            a.out = stage1_out;
+            a.kept = p.kept;
+            a.redo = p.red;
+            a.redo.n = p.red.n - 1;
+            a.K = p.K;
+            a.rout = p.R / rin;
+            a.rin_v = rin / p.vec;
+            a.sr = p.red.stride[p.red.n - 1];
+            a.qchunk = (a.rout + p.split_q - 1) / p.split_q;
+            a.ichunk = (a.rin_v + p.split_i - 1) / p.split_i;
+            a.count = count;
+            a.tpr = p.tpr;
+            a.tpr_log2 = ilog2(p.tpr);
+            a.rpb = p.rpb;
+            a.split_q = p.split_q;
+            a.split_i = p.split_i;
+            a.init_out = init_out;
+            if (vec) row_reduce_kernel<Op, FULL><<<grid, block, 0, st>>>(a);
+            else row_reduce_kernel<Op, 1><<<grid, block, 0, st>>>(a);
+        }
+        if (p.split > 1)
+            finish_kernel<Op, true><<<dim3((unsigned)p.K), dim3(256), 0, st>>>(sc.partial, out, p.K, p.split,
+                                                                             p.split, 1, init_out, count);
         return;
     }
-    ColArgs a{};
-    a.in = in;
-    a.out = out;
-    a.partial = sc.partial;
-    a.counters = sc.counters;
-    a.kept_outer = p.kept;
-    a.kept_outer.n = p.kept.n > 0 ? p.kept.n - 1 : 0;
-    a.red = p.red;
-    a.K = p.K;
-    a.kin = p.kept.n ? p.kept.size[p.kept.n - 1] : 1;
-    a.sk = p.kept.n ? p.kept.stride[p.kept.n - 1] : 0;
-    a.R = p.R;
-    a.chunk = p.chunk;
-    a.count = count;
-    a.split = p.split;
-    a.init_out = init_out;
+    // Col
     const int64_t kv = p.K / p.vec;
-    dim3 grid((unsigned)((kv + p.bx - 1) / p.bx), (unsigned)p.split);
     dim3 block((unsigned)p.bx, (unsigned)p.by);
-    size_t smem = p.by > 1 ? (size_t)p.bx * p.by * p.vec * sizeof(typename Op::Acc) : 0;
-    if (p.vec == FULL && FULL > 1) col_reduce_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
-    else col_reduce_kernel<Op, 1><<<grid, block, smem, st>>>(a);
+    size_t smem = p.by > 1 ? (size_t)p.bx * p.by * p.vec * sizeof(Acc) : 0;
+    if (p.lean) {
+        ColLeanArgs a{};
+        const int nk = p.kept.n;
+        const int64_t kin = nk ? p.kept.size[nk - 1] : 1;
+        a.in = in;
+        a.out = stage1_out;
+        a.so = nk > 1 ? p.kept.stride[0] : 0;
+        a.rs = p.red.n ? p.red.stride[0] : 0;
+        a.K = p.K;
+        a.count = count;
+        a.kin_v = (int)(kin / p.vec);
+        a.sk = nk ? (int)p.kept.stride[nk - 1] : 1;
+        a.R = (int)p.R;
+        a.chunk = (int)p.chunk;
+        a.split = p.split;
+        a.init_out = init_out;
+        const int64_t outer = nk > 1 ? p.kept.size[0] : 1;
+        dim3 grid((unsigned)((a.kin_v + p.bx - 1) / p.bx), (unsigned)outer, (unsigned)p.split);
+        if (vec) col_lean_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
+        else col_lean_kernel<Op, 1><<<grid, block, smem, st>>>(a);
+    } else {
+        ColArgs a{};
+        a.in = in;
+        a.out = stage1_out;
+        a.kept_outer = p.kept;
+        a.kept_outer.n = p.kept.n > 0 ? p.kept.n - 1 : 0;
+        a.red = p.red;
+        a.K = p.K;
+        a.kin = p.kept.n ? p.kept.size[p.kept.n - 1] : 1;
+        a.sk = p.kept.n ? p.kept.stride[p.kept.n - 1] : 0;
+        a.R = p.R;
+        a.chunk = p.chunk;
+        a.count = count;
+        a.split = p.split;
+        a.init_out = init_out;
+        dim3 grid((unsigned)((kv + p.bx - 1) / p.bx), (unsigned)p.split);
+        if (vec) col_reduce_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
+        else col_reduce_kernel<Op, 1><<<grid, block, smem, st>>>(a);
+    }
+    if (p.split > 1)
+        finish_kernel<Op, false><<<dim3((unsigned)((p.K + 255) / 256)), dim3(256), 0, st>>>(
+            sc.partial, out, p.K, p.split, 1, p.K, init_out, count);
 }
 
 // Instantiate launch_reduce_t for every dtype of one op family.
