@@ -202,9 +202,30 @@ template <class A> __device__ __forceinline__ A shfl_xor_any(A v, int mask) {
     return out.a;
 }
 
+// Move every 32-bit word of v along a DPP lane pattern (a VALU modifier, a few
+// cycles) instead of through the LDS crossbar that __shfl uses.
+template <int CTRL, class A> __device__ __forceinline__ A dpp_move(A v) {
+    static_assert(sizeof(A) % 4 == 0, "DPP moves 32-bit words");
+    constexpr int W = sizeof(A) / 4;
+    union { A a; int w[W]; } in, out;
+    in.a = v;
+#pragma unroll
+    for (int i = 0; i < W; ++i) out.w[i] = __builtin_amdgcn_update_dpp(0, in.w[i], CTRL, 0xF, 0xF, true);
+    return out.a;
+}
+
 // All-reduce over aligned groups of `width` consecutive lanes (power of two, <= 64).
+// Inside a row of 16 lanes the butterfly runs on DPP patterns: swap within pairs
+// (quad_perm [1,0,3,2]), swap pairs (quad_perm [2,3,0,1]), mirror within 8
+// (row_half_mirror), mirror within 16 (row_mirror); rows are then combined with
+// two cross-lane shuffles. Every lane of a group ends with the same value.
 template <class Op, class A> __device__ __forceinline__ A group_reduce(A v, int width) {
-    for (int m = width >> 1; m > 0; m >>= 1) v = Op::comb(v, shfl_xor_any(v, m));
+    if (width >= 2) v = Op::comb(v, dpp_move<0xB1>(v));
+    if (width >= 4) v = Op::comb(v, dpp_move<0x4E>(v));
+    if (width >= 8) v = Op::comb(v, dpp_move<0x141>(v));
+    if (width >= 16) v = Op::comb(v, dpp_move<0x140>(v));
+    if (width >= 32) v = Op::comb(v, shfl_xor_any(v, 16));
+    if (width >= 64) v = Op::comb(v, shfl_xor_any(v, 32));
     return v;
 }
 

@@ -159,8 +159,8 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
         if (blocks < kBlocksToFill / 4) {
             // Too few outputs to fill the chip: several workgroups of 256 threads
             // per output, each with a long contiguous share (>= 16 loads per
-            // thread); about 1024 workgroups in all is the measured sweet spot.
-            int64_t want = (1024 + p.K - 1) / p.K;
+            // thread); about 512 workgroups in all is the measured sweet spot.
+            int64_t want = (512 + p.K - 1) / p.K;
             int64_t can = nv / (256 * 16);
             int64_t split = std::min<int64_t>(std::min(want, can), 4096);
             if (split > 1) {

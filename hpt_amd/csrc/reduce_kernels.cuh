@@ -80,16 +80,16 @@ __global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
                 for (int u = 0; u < 4; ++u)
 #pragma unroll
                     for (int j = 0; j < VEC; ++j)
-                        acc = Op::comb(acc, Op::pre(v[u].v[j], (iv + u * tpr) * VEC + j));
+                        fold_in<Op>(acc, v[u].v[j], (iv + u * tpr) * VEC + j);
             }
             for (; iv < i1; iv += tpr) {
                 Pack<T, VEC> v = load_pack_stream<T, VEC>(p + (int64_t)iv * VEC);
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) acc = Op::comb(acc, Op::pre(v.v[j], iv * VEC + j));
+                for (int j = 0; j < VEC; ++j) fold_in<Op>(acc, v.v[j], iv * VEC + j);
             }
         } else {
 #pragma unroll 4
-            for (; iv < i1; iv += tpr) acc = Op::comb(acc, Op::pre(p[(int64_t)iv * a.sr], iv));
+            for (; iv < i1; iv += tpr) fold_in<Op>(acc, p[(int64_t)iv * a.sr], iv);
         }
     }
     acc = group_reduce<Op>(acc, tpr < 64 ? tpr : 64);
@@ -129,9 +129,9 @@ __device__ __forceinline__ void row_step(typename Op::Acc& acc, const typename O
     if constexpr (VEC > 1) {
         Pack<T, VEC> v = load_pack_stream<T, VEC>(p + iv * VEC);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) acc = Op::comb(acc, Op::pre(v.v[j], iv * VEC + j));
+        for (int j = 0; j < VEC; ++j) fold_in<Op>(acc, v.v[j], iv * VEC + j);
     } else {
-        acc = Op::comb(acc, Op::pre(p[iv * sr], iv));
+        fold_in<Op>(acc, p[iv * sr], iv);
     }
 }
 
@@ -260,16 +260,16 @@ __global__ void __launch_bounds__(1024) col_lean_kernel(const ColLeanArgs a) {
 #pragma unroll
             for (int u = 0; u < 8; ++u)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], Op::pre(v[u].v[j], r + u * by));
+                for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v[u].v[j], r + u * by);
         }
         for (; r < r1; r += by) {
             const T* p = base + (int64_t)r * a.rs;
             if constexpr (VEC > 1) {
                 Pack<T, VEC> v = load_pack_stream<T, VEC>(p);
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], Op::pre(v.v[j], r));
+                for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v.v[j], r);
             } else {
-                acc[0] = Op::comb(acc[0], Op::pre(*p, r));
+                fold_in<Op>(acc[0], *p, r);
             }
         }
     }
@@ -333,9 +333,9 @@ __global__ void __launch_bounds__(1024) col_reduce_kernel(const ColArgs a) {
             if constexpr (VEC > 1) {
                 Pack<T, VEC> v = load_pack_stream<T, VEC>(p);
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], Op::pre(v.v[j], r));
+                for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v.v[j], r);
             } else {
-                acc[0] = Op::comb(acc[0], Op::pre(*p, r));
+                fold_in<Op>(acc[0], *p, r);
             }
         }
     }

@@ -221,6 +221,28 @@ template <bool IS_MAX, class T> struct ArgOp {
     }
     __device__ static __forceinline__ Out post(Acc a, double) { return (int64_t)a.idx; }
     __device__ static __forceinline__ Acc from_out(Out) { return identity(); }
+    // Fold element x at index r into acc when r only grows within the lane: the
+    // strict compare alone keeps the first extremum, exactly the CPU scan.
+    __device__ static __forceinline__ void accumulate(Acc& acc, T x, int64_t r) {
+        const C v = Elem<T>::cmp(x);
+        const bool better = IS_MAX ? (v > acc.val) : (v < acc.val);
+        if (better) {
+            acc.val = v;
+            acc.idx = (decltype(acc.idx))r;
+        }
+    }
 };
+
+// acc = comb(acc, pre(x, r)), or the op's own cheaper in-order form when it has one.
+template <class Op, class = void> struct HasAccumulate { static constexpr bool value = false; };
+template <class Op>
+struct HasAccumulate<Op, decltype(Op::accumulate(*(typename Op::Acc*)nullptr, typename Op::In{}, (int64_t)0))> {
+    static constexpr bool value = true;
+};
+template <class Op>
+__device__ __forceinline__ void fold_in(typename Op::Acc& acc, typename Op::In x, int64_t r) {
+    if constexpr (HasAccumulate<Op>::value) Op::accumulate(acc, x, r);
+    else acc = Op::comb(acc, Op::pre(x, r));
+}
 
 }  // namespace hpt
