@@ -364,6 +364,20 @@ static NormCall prepare_norm(const hpt_view* in, const void* out_data, int64_t a
     return c;
 }
 
+// Launch a normalisation; plans that need scratch (partial row statistics) get
+// the per-stream buffer, held under its lock from lookup to launch.
+static void launch_norm(int dev, hipStream_t st, NormLaunchFn fn, NormCall& c, const char* what) {
+    if (c.plan.scratch_bytes) {
+        std::lock_guard<std::mutex> g(g_scratch_mu);
+        c.args.scratch = scratch_for(dev, st, c.plan.scratch_bytes, 0).partial;
+        fn(c.plan, c.args, st);
+        check_launch(what);
+    } else {
+        fn(c.plan, c.args, st);
+        check_launch(what);
+    }
+}
+
 }  // namespace hpt
 
 using namespace hpt;
@@ -564,8 +578,7 @@ int32_t hpt_hip_softmax(int32_t dev, void* stream, int32_t log, const hpt_view* 
         NormLaunchFn fn = norm_launcher_for(log ? NORM_LOGSOFTMAX : NORM_SOFTMAX, in->dtype);
         if (!fn) fail(HPT_ERR_DTYPE, "softmax: unsupported dtype %s", dtype_name(in->dtype));
         use_device(dev);
-        fn(c.plan, c.args, (hipStream_t)stream);
-        check_launch("softmax");
+        launch_norm(dev, (hipStream_t)stream, fn, c, "softmax");
     });
 }
 
@@ -597,13 +610,16 @@ int32_t hpt_hip_layernorm(int32_t dev, void* stream, const hpt_view* in, int32_t
         // vector loads of gamma/beta need 16-byte alignment too
         if (c.plan.vec > 1 && (((uintptr_t)c.args.gamma | (uintptr_t)c.args.beta) % 16) != 0) {
             c.plan.vec = 1;
-            if (c.plan.kind == NormKind::RowReg) c.plan.kind = NormKind::Generic;
+            if (c.plan.kind == NormKind::RowReg || c.plan.kind == NormKind::Transposed) {
+                c.plan.kind = NormKind::Generic;
+                c.plan.scratch_bytes = 0;
+                c.plan.sstride = 1;
+            }
         }
         NormLaunchFn fn = norm_launcher_for(NORM_LAYERNORM, in->dtype);
         if (!fn) fail(HPT_ERR_DTYPE, "layernorm: unsupported dtype %s", dtype_name(in->dtype));
         use_device(dev);
-        fn(c.plan, c.args, (hipStream_t)stream);
-        check_launch("layernorm");
+        launch_norm(dev, (hipStream_t)stream, fn, c, "layernorm");
     });
 }
 

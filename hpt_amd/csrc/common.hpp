@@ -95,6 +95,7 @@ struct ReducePlan {
     int split_q = 1; // Row: how `split` divides the outer reduced dims ...
     int split_i = 1; // ... and the innermost reduced dim (split = split_q * split_i)
     int64_t chunk = 0;  // Col: reduced indices per split
+    int sstride = 1;    // lean kernels: 2 = elements along the lane dim sit at every second position
     bool lean = false;  // the layout fits the lean kernels (one reduced dim, <= 2 kept dims, 32-bit extents)
 };
 
@@ -126,8 +127,11 @@ struct NormPlan {
     int tpr = 1;      // threads per row (RowReg / RowStream / Generic)
     int rpb = 1;      // rows per block
     int nchunk = 1;   // RowReg: vectors held per thread
-    int max_blocks = 4096;  // RowReg layernorm: workgroups launched at most (they walk the rows)
+    int max_blocks = 1024;  // RowReg layernorm: workgroups launched at most (they walk the rows)
     int64_t inner = 1;  // Col: size of the contiguous inner dim the lanes walk
+    int sstride = 1;    // RowReg: 2 = the row's elements sit at every second position of full vectors
+    int tsplit = 1;     // Transposed: workgroups sharing the axis in the statistics pass
+    size_t scratch_bytes = 0;  // Transposed: partial statistics (rows * tsplit * 24 bytes at most)
 };
 
 // axis >= 0: softmax-style single axis; n_norm_dims > 0: trailing dims (layernorm).

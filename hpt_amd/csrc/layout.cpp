@@ -146,7 +146,13 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
             p.vec = legal_vec(data, elem_size, rin, p.kept, p.red, 0, 1);
         p.lean = p.red.n == 1 && p.kept.n <= 1 && p.K <= kI32 && rin <= kI32 &&
                  iabs(p.red.stride[0]) <= kI32;
-        int64_t nv = p.R / p.vec;  // vector loads per output
+        if (p.lean && p.red.stride[0] == 2 && elem_size <= 8 &&
+            legal_vec(data, elem_size, rin * 2, p.kept, p.red, 0, 1) > 1) {
+            // every second element along the row: full vectors, even positions kept
+            p.vec = (int)(16 / elem_size);
+            p.sstride = 2;
+        }
+        int64_t nv = p.R / (p.vec / p.sstride);  // vector loads per output
         // About 8 vector loads per lane; groups of one or two wavefronts per row
         // stream best (each wavefront walks its own long run of the row), and
         // only very long rows get a whole workgroup.
@@ -169,7 +175,7 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
                 int64_t rout = p.R / rin;
                 int64_t sq = std::min(split, rout);
                 int64_t si = std::max<int64_t>(1, split / sq);
-                int64_t can_i = std::max<int64_t>(1, (rin / p.vec) / p.tpr);
+                int64_t can_i = std::max<int64_t>(1, (rin / (p.vec / p.sstride)) / p.tpr);
                 si = std::min(si, can_i);
                 p.split_q = (int)sq;
                 p.split_i = (int)si;
@@ -187,7 +193,13 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
         const int64_t outer = nk > 1 ? p.kept.size[0] : 1;
         p.lean = p.red.n <= 1 && nk <= 2 && outer <= 65535 && kin <= kI32 && p.R <= kI32 &&
                  (nk == 0 || iabs(p.kept.stride[nk - 1]) <= kI32);
-        int64_t kv = (p.lean ? kin : p.K) / p.vec;  // vector columns the lanes spread over
+        if (p.lean && nk && p.kept.stride[nk - 1] == 2 && elem_size <= 8 &&
+            legal_vec(data, elem_size, kin * 2, p.kept, p.red, 1, 0) > 1) {
+            // neighbouring outputs sit at every second position: full vectors, even positions kept
+            p.vec = (int)(16 / elem_size);
+            p.sstride = 2;
+        }
+        int64_t kv = (p.lean ? kin : p.K) / (p.vec / p.sstride);  // vector columns the lanes spread over
         p.bx = (int)std::min<int64_t>(64, pow2_ceil(kv));
         int64_t xblocks = (kv + p.bx - 1) / p.bx * (p.lean ? outer : 1);
         // One wavefront per 64 vector columns streams best when there are enough
@@ -195,20 +207,30 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
         // with fewer, thread rows and then workgroups split the reduced range.
         const int base_by = 64 / p.bx;  // a workgroup is at least one wavefront
         const int64_t kWavesWanted = 768;
-        int by = base_by;
-        while (xblocks * (by / base_by) < kWavesWanted && by * p.bx < 1024 && p.R / (by * 2) >= 8) by *= 2;
-        // the thread rows meet in LDS: keep bx*by*vec accumulators within 64 KiB
-        while (by > 1 && (size_t)p.bx * by * p.vec * acc_size > (64u << 10)) by /= 2;
-        p.by = std::max(1, by);
+        const int uv = p.vec / p.sstride;
+        p.by = base_by;
         p.split = 1;
-        int64_t waves = xblocks * std::max(1, p.by / base_by);
-        int64_t per_thread = p.R / p.by;
-        if (waves < kWavesWanted && per_thread >= 64) {
-            int64_t want = (kWavesWanted + waves - 1) / waves;
-            int64_t can = per_thread / 32;
-            // bound the partial buffer: K * split accumulators <= 64 MiB
-            int64_t cap = std::max<int64_t>(1, (int64_t)((64ll << 20) / acc_size) / p.K);
-            p.split = (int)std::max<int64_t>(1, std::min(std::min(want, can), std::min<int64_t>(cap, 1024)));
+        // r-partitions wanted so that about 768 wavefronts run, each with >= 16 loads
+        const int64_t need = (kWavesWanted + xblocks - 1) / xblocks;
+        const int64_t can = std::max<int64_t>(1, p.R / 16);
+        const int64_t rp = std::min(need, can);
+        if (rp > 1) {
+            const int64_t bytes = p.K * p.R * (int64_t)elem_size;
+            if (bytes >= (8ll << 20)) {
+                // Large input: partition over WORKGROUPS first, so that the partitions land
+                // on different CUs (48 workgroups of 1024 threads leave 208 CUs idle), and
+                // fold the partials in a second launch.
+                int64_t cap = std::max<int64_t>(1, (int64_t)((64ll << 20) / acc_size) / p.K);
+                int64_t split = std::min<int64_t>(std::min<int64_t>(rp, 64), cap);
+                int64_t by = pow2_floor(std::max<int64_t>(1, rp / split));
+                p.split = (int)split;
+                p.by = (int)std::min<int64_t>(by, 4) * base_by;
+            } else {
+                // Small input: one launch, thread rows meet in LDS
+                int64_t by = std::min<int64_t>(pow2_ceil(rp), 1024 / p.bx / base_by) * base_by;
+                while (by > base_by && (size_t)p.bx * by * uv * acc_size > (64u << 10)) by /= 2;
+                p.by = (int)by;
+            }
         }
         p.chunk = (p.R + p.split - 1) / p.split;
     }
@@ -234,13 +256,14 @@ std::string describe(const ReducePlan& p) {
         case ReduceKind::Empty: return "empty";
         case ReduceKind::Identity: return "identity";
         case ReduceKind::Row:
-            snprintf(buf, sizeof buf, "row%s vec=%d tpr=%d rpb=%d rows=%lld cols=%lld split=%d(%dx%d) ",
-                     p.lean ? "" : "-general", p.vec, p.tpr, p.rpb, (long long)p.K, (long long)p.R,
-                     p.split, p.split_q, p.split_i);
+            snprintf(buf, sizeof buf, "row%s%s vec=%d tpr=%d rpb=%d rows=%lld cols=%lld split=%d(%dx%d) ",
+                     p.lean ? "" : "-general", p.sstride == 2 ? "-step2" : "", p.vec, p.tpr, p.rpb,
+                     (long long)p.K, (long long)p.R, p.split, p.split_q, p.split_i);
             break;
         case ReduceKind::Col:
-            snprintf(buf, sizeof buf, "col%s vec=%d bx=%d by=%d outs=%lld red=%lld split=%d ",
-                     p.lean ? "" : "-general", p.vec, p.bx, p.by, (long long)p.K, (long long)p.R, p.split);
+            snprintf(buf, sizeof buf, "col%s%s vec=%d bx=%d by=%d outs=%lld red=%lld split=%d ",
+                     p.lean ? "" : "-general", p.sstride == 2 ? "-step2" : "", p.vec, p.bx, p.by,
+                     (long long)p.K, (long long)p.R, p.split);
             break;
     }
     s = buf;
@@ -328,10 +351,27 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
 
     if (p.norm_in.n == 1 && p.out_axis_stride == 1) {
         // rows are contiguous in the output
-        bool transposed = sa != 1 && p.kept_in.n >= 1 && p.kept_in.stride[p.kept_in.n - 1] == 1 &&
-                          p.kept_in.size[p.kept_in.n - 1] >= 64 && p.cols >= 64 && sa > 0;
+        // input contiguous along the rows, output along the axis (a transposed view):
+        // statistics pass + register-tile transpose, when 128-bit access is legal both ways
+        const int nk = p.kept_in.n;
+        const int v = max_vec;
+        bool transposed = sa > 1 && nk >= 1 && nk <= 2 && p.kept_in.stride[nk - 1] == 1 && v > 1 &&
+                          p.kept_in.size[nk - 1] % v == 0 && p.cols % v == 0 && sa % v == 0 &&
+                          (nk == 1 || (p.kept_in.stride[0] % v == 0 && p.kept_in.size[0] <= 65535)) &&
+                          ((uintptr_t)in_data % 16) == 0 && ((uintptr_t)out_data % 16) == 0 &&
+                          p.kept_in.size[nk - 1] <= 0x7fffffff && p.cols <= 0x7fffffff &&
+                          p.kept_in.size[nk - 1] >= 8 * v && p.cols >= 8 * v;
         if (transposed) {
             p.kind = NormKind::Transposed;
+            p.vec = v;
+            // statistics pass: a wavefront covers 64*v rows; enough column splits for
+            // about 2048 wavefronts, each keeping at least 32 columns
+            const int64_t R = p.kept_in.size[nk - 1];
+            const int64_t batch = nk > 1 ? p.kept_in.size[0] : 1;
+            const int64_t groups = (R + 64 * v - 1) / (64 * v) * batch;
+            int64_t S = std::max<int64_t>(1, std::min<int64_t>((512 + groups - 1) / groups, p.cols / 128));
+            p.tsplit = (int)std::min<int64_t>(S, 64);
+            p.scratch_bytes = (size_t)p.rows * p.tsplit * 4 * 16 + (size_t)p.rows * 3 * 8;
             return p;
         }
         if (sa >= 1 && sa <= 4) {
@@ -342,9 +382,19 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 int vi = legal_vec(in_data, elem_size, p.cols, p.kept_in, none, 0, 0);
                 int vo = legal_vec(out_data, elem_size, p.cols, p.kept_out, none, 0, 0);
                 v = std::min(std::min(vi, vo), max_vec);
+            } else if (sa == 2 && max_vec >= 2) {
+                // every second element: load full vectors, keep the even positions
+                Dims none;
+                const int uv = max_vec / 2;
+                int vi = legal_vec(in_data, elem_size, p.cols * 2, p.kept_in, none, 0, 0);
+                bool out_ok = ((uintptr_t)out_data % (uv * elem_size)) == 0 && p.cols % uv == 0;
+                if (vi == max_vec && out_ok) {
+                    v = max_vec;
+                    p.sstride = 2;
+                }
             }
             p.vec = v;
-            int64_t nv = p.cols / v;
+            int64_t nv = p.cols / (v / p.sstride);
             if (nv <= 8192) {
                 p.kind = NormKind::RowReg;
                 p.tpr = (int)std::min<int64_t>(1024, pow2_ceil((nv + 3) / 4));
@@ -357,6 +407,10 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 p.kind = NormKind::RowStream;
                 p.tpr = 1024;
                 p.rpb = 1;
+                if (p.sstride == 2) {  // the streaming kernel gathers stride-2 rows element by element
+                    p.vec = 1;
+                    p.sstride = 1;
+                }
             }
             return p;
         }
@@ -378,8 +432,8 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
 std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "col", "transposed", "generic"};
     char buf[256];
-    snprintf(buf, sizeof buf, "%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+    snprintf(buf, sizeof buf, "%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     describe_dims(s, "rows_in", p.kept_in);

@@ -23,6 +23,7 @@ struct NormArgs {
     int64_t out_axis_stride;  // output stride along the row
     double eps;
     double inv_cols;  // 1 / cols
+    void* scratch;    // library-owned scratch (partial row statistics of the transposed form)
     int tpr, tpr_log2, rpb;
 };
 

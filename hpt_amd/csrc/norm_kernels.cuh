@@ -91,8 +91,14 @@ __device__ __forceinline__ A row_all_reduce(A v, int tpr, int ty, A* smem) {
 // grid.x workgroups walk the rows in steps of gridDim.x * rpb, so that gamma and
 // beta are fetched once per thread (they index by column, and a thread keeps its
 // columns) instead of once per row, and the launch prologue is paid once.
-template <int KIND, class T, int VEC, int NCHUNK>
+// SS = 2 reads a row whose elements sit at every second position (a [:, ::2] view):
+// full 128-bit vectors are loaded and the odd positions dropped, which moves the
+// same cache lines as a scalar gather with a fraction of the instructions. (A
+// 16-byte aligned vector that holds one valid element never leaves that element's
+// page, so the unused half of the last vector is safe to touch.)
+template <int KIND, class T, int VEC, int NCHUNK, int SS = 1>
 __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
+    constexpr int UV = VEC / SS;  // useful elements per vector
     using CT = typename Elem<T>::Wide;
     using ST = typename StatType<T>::type;
     __shared__ __align__(8) unsigned char smem_stat[16 * sizeof(double)];
@@ -101,25 +107,25 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     const int tpr = a.tpr;
     const int tx = threadIdx.x & (tpr - 1);
     const int ty = threadIdx.x >> a.tpr_log2;
-    const int nv = (int)(a.cols / VEC);
+    const int nv = (int)(a.cols / UV);
     constexpr bool kSoft = KIND != NORM_LAYERNORM;
     const CT fill = kSoft ? neg_inf<CT>() : (CT)0;
 
     // this thread's columns never change: keep gamma / beta in registers
-    Pack<T, VEC> gam[NCHUNK], bet[NCHUNK];
+    Pack<T, UV> gam[NCHUNK], bet[NCHUNK];
     if constexpr (!kSoft) {
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int iv = c * tpr + tx;
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) {
+            for (int j = 0; j < UV; ++j) {
                 gam[c].v[j] = Elem<T>::narrow((CT)1);
                 bet[c].v[j] = Elem<T>::narrow((CT)0);
             }
             if (iv < nv) {
                 if constexpr (VEC > 1) {
-                    if (a.gamma) gam[c] = load_pack<T, VEC>((const T*)a.gamma + (int64_t)iv * VEC);
-                    if (a.beta) bet[c] = load_pack<T, VEC>((const T*)a.beta + (int64_t)iv * VEC);
+                    if (a.gamma) gam[c] = load_pack<T, UV>((const T*)a.gamma + (int64_t)iv * UV);
+                    if (a.beta) bet[c] = load_pack<T, UV>((const T*)a.beta + (int64_t)iv * UV);
                 } else {
                     if (a.gamma) gam[c].v[0] = ((const T*)a.gamma)[iv];
                     if (a.beta) bet[c].v[0] = ((const T*)a.beta)[iv];
@@ -135,7 +141,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
         const T* in_row = (const T*)a.in + (valid ? offset_of(a.kept_in, row) : 0);
         T* out_row = (T*)a.out + (valid ? row * a.cols : 0);
 
-        CT x[NCHUNK][VEC];
+        CT x[NCHUNK][UV];
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int iv = c * tpr + tx;
@@ -143,13 +149,13 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                 if constexpr (VEC > 1) {
                     Pack<T, VEC> v = load_pack_stream<T, VEC>(in_row + (int64_t)iv * VEC);
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) x[c][j] = Elem<T>::widen(v.v[j]);
+                    for (int j = 0; j < UV; ++j) x[c][j] = Elem<T>::widen(v.v[j * SS]);
                 } else {
                     x[c][0] = Elem<T>::widen(in_row[(int64_t)iv * a.sa]);
                 }
             } else {
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) x[c][j] = fill;
+                for (int j = 0; j < UV; ++j) x[c][j] = fill;
             }
         }
 
@@ -158,13 +164,13 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, x[c][j]);
+                for (int j = 0; j < UV; ++j) m = MaxC<CT>::comb(m, x[c][j]);
             m = row_all_reduce<MaxC<CT>>(m, tpr, ty, smem);
             CT s = 0;
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) {
+                for (int j = 0; j < UV; ++j) {
                     CT d = x[c][j] - m;
                     CT e = exp_ct<T>(d);
                     s += e;
@@ -175,14 +181,14 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j)
+                for (int j = 0; j < UV; ++j)
                     x[c][j] = KIND == NORM_SOFTMAX ? x[c][j] * k : x[c][j] - k;
         } else {
             CT s = 0;
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) s += x[c][j];
+                for (int j = 0; j < UV; ++j) s += x[c][j];
             // mean = sum / cols, as a reciprocal multiply plus one correction step
             // (exact quotient for the cases that matter, e.g. constant rows)
             const ST sum = row_all_reduce<SumC<ST>>((ST)s, tpr, ty, ssmem);
@@ -195,7 +201,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
             for (int c = 0; c < NCHUNK; ++c) {
                 const bool in_row_c = (c * tpr + tx) < nv;
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) {
+                for (int j = 0; j < UV; ++j) {
                     const CT d = in_row_c ? (x[c][j] - mean_hi) - mean_lo : (CT)0;
                     x[c][j] = d;
                     q += d * d;
@@ -206,7 +212,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j)
+                for (int j = 0; j < UV; ++j)
                     x[c][j] = x[c][j] * rstd * Elem<T>::widen(gam[c].v[j]) + Elem<T>::widen(bet[c].v[j]);
         }
 
@@ -216,10 +222,10 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                 const int iv = c * tpr + tx;
                 if (iv < nv) {
                     if constexpr (VEC > 1) {
-                        Pack<T, VEC> o;
+                        Pack<T, UV> o;
 #pragma unroll
-                        for (int j = 0; j < VEC; ++j) o.v[j] = Elem<T>::narrow(x[c][j]);
-                        store_pack_stream<T, VEC>(out_row + (int64_t)iv * VEC, o);
+                        for (int j = 0; j < UV; ++j) o.v[j] = Elem<T>::narrow(x[c][j]);
+                        store_pack_stream<T, UV>(out_row + (int64_t)iv * UV, o);
                     } else {
                         out_row[iv] = Elem<T>::narrow(x[c][0]);
                     }

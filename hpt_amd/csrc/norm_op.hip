@@ -1,6 +1,6 @@
 // One normalisation kind (softmax, log_softmax or layernorm) for the four
 // float dtypes. Compiled once per kind with -DHPT_NORM_KIND=<0|1|2>.
-#include "norm_kernels.cuh"
+#include "transpose_norm.cuh"
 
 #ifndef HPT_NORM_KIND
 #error "compile with -DHPT_NORM_KIND=<kind>"
@@ -18,13 +18,13 @@ inline int ilog2(int v) {
     return l;
 }
 
-template <class T, int VEC>
+template <class T, int VEC, int SS = 1>
 void launch_row_reg(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block, hipStream_t st) {
     switch (p.nchunk) {
-        case 1: row_reg_kernel<KIND, T, VEC, 1><<<grid, block, 0, st>>>(a); break;
-        case 2: row_reg_kernel<KIND, T, VEC, 2><<<grid, block, 0, st>>>(a); break;
-        case 4: row_reg_kernel<KIND, T, VEC, 4><<<grid, block, 0, st>>>(a); break;
-        case 8: row_reg_kernel<KIND, T, VEC, 8><<<grid, block, 0, st>>>(a); break;
+        case 1: row_reg_kernel<KIND, T, VEC, 1, SS><<<grid, block, 0, st>>>(a); break;
+        case 2: row_reg_kernel<KIND, T, VEC, 2, SS><<<grid, block, 0, st>>>(a); break;
+        case 4: row_reg_kernel<KIND, T, VEC, 4, SS><<<grid, block, 0, st>>>(a); break;
+        case 8: row_reg_kernel<KIND, T, VEC, 8, SS><<<grid, block, 0, st>>>(a); break;
         default: fail(HPT_ERR_KERNEL, "row_reg: unsupported chunk count %d", p.nchunk);
     }
 }
@@ -38,11 +38,40 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
     a.inv_cols = 1.0 / (double)p.cols;
     dim3 grid((unsigned)((p.rows + p.rpb - 1) / p.rpb));
     dim3 block((unsigned)(p.tpr * p.rpb));
+    if (p.kind == NormKind::Transposed) {
+        constexpr int TILE = 8 * FULL;
+        TransposedArgs t{};
+        t.in = a.in;
+        t.out = a.out;
+        t.gamma = a.gamma;
+        t.beta = a.beta;
+        const int nk = p.kept_in.n;
+        const unsigned batch = nk > 1 ? (unsigned)p.kept_in.size[0] : 1u;
+        t.R = (int)p.kept_in.size[nk - 1];
+        t.cols = (int)p.cols;
+        t.S = p.tsplit;
+        // scratch: [batch][4 S][R] partial statistics (16 bytes each at most), then [batch][3][R] numbers
+        t.stats = a.scratch;
+        t.params = (char*)a.scratch + (size_t)batch * t.S * 4 * t.R * 16;
+        t.sa = a.sa;
+        t.bi = nk > 1 ? p.kept_in.stride[0] : 0;
+        t.eps = a.eps;
+        t.inv_cols = a.inv_cols;
+        t.cols_per_split = (t.cols + t.S - 1) / t.S;
+        const int tiles = (t.cols + TILE - 1) / TILE;
+        const unsigned rt = (unsigned)((t.R + TILE - 1) / TILE);
+        const unsigned rg = (unsigned)((t.R + 64 * FULL - 1) / (64 * FULL));
+        transposed_stats_kernel<KIND, T><<<dim3(rg, (unsigned)t.S, batch), dim3(256), 0, st>>>(t);
+        transposed_finalize_kernel<KIND, T><<<dim3((unsigned)((t.R + 15) / 16), 1, batch), dim3(16, 16), 0, st>>>(t);
+        transposed_apply_kernel<KIND, T><<<dim3(rt, (unsigned)((tiles + 3) / 4), batch), dim3(256), 0, st>>>(t);
+        return;
+    }
     if (p.kind == NormKind::RowReg) {
         // Layernorm workgroups walk the rows (gamma / beta stay in registers);
         // softmax has nothing to reuse across rows and runs one row per group.
         if (KIND == NORM_LAYERNORM && grid.x > (unsigned)p.max_blocks) grid.x = (unsigned)p.max_blocks;
-        if (p.vec == FULL) launch_row_reg<T, FULL>(p, a, grid, block, st);
+        if (p.vec == FULL && p.sstride == 2 && FULL > 1) launch_row_reg<T, FULL, 2>(p, a, grid, block, st);
+        else if (p.vec == FULL) launch_row_reg<T, FULL>(p, a, grid, block, st);
         else launch_row_reg<T, 1>(p, a, grid, block, st);
         return;
     }

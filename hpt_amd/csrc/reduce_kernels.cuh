@@ -54,10 +54,13 @@ struct RowLeanArgs {
     int tpr, tpr_log2, rpb, split, init_out;
 };
 
-template <class Op, int VEC>
+// SS = 2: the row's elements sit at every second position; full vectors are
+// loaded and the odd positions dropped (see row_reg_kernel).
+template <class Op, int VEC, int SS = 1>
 __global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
     using T = typename Op::In;
     using Acc = typename Op::Acc;
+    constexpr int UV = VEC / SS;
     __shared__ Acc smem[16];
     const int tpr = a.tpr;
     const int tx = threadIdx.x & (tpr - 1);
@@ -79,13 +82,13 @@ __global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
 #pragma unroll
                 for (int u = 0; u < 4; ++u)
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j)
-                        fold_in<Op>(acc, v[u].v[j], (iv + u * tpr) * VEC + j);
+                    for (int j = 0; j < UV; ++j)
+                        fold_in<Op>(acc, v[u].v[j * SS], (iv + u * tpr) * UV + j);
             }
             for (; iv < i1; iv += tpr) {
                 Pack<T, VEC> v = load_pack_stream<T, VEC>(p + (int64_t)iv * VEC);
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) fold_in<Op>(acc, v.v[j], iv * VEC + j);
+                for (int j = 0; j < UV; ++j) fold_in<Op>(acc, v.v[j * SS], iv * UV + j);
             }
         } else {
 #pragma unroll 4
@@ -230,20 +233,21 @@ struct ColLeanArgs {
     int split, init_out;
 };
 
-template <class Op, int VEC>
+template <class Op, int VEC, int SS = 1>
 __global__ void __launch_bounds__(1024) col_lean_kernel(const ColLeanArgs a) {
     using T = typename Op::In;
     using Acc = typename Op::Acc;
+    constexpr int UV = VEC / SS;  // outputs per lane (SS = 2: every second position of a vector)
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int tx = threadIdx.x, ty = threadIdx.y, by = blockDim.y;
     const int cv = blockIdx.x * blockDim.x + tx;  // vector column in the inner dim
     const int outer = blockIdx.y;
     const bool valid = cv < a.kin_v;
-    Acc acc[VEC];
+    Acc acc[UV];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) acc[j] = Op::identity();
+    for (int j = 0; j < UV; ++j) acc[j] = Op::identity();
     if (valid) {
-        const T* base = (const T*)a.in + (int64_t)outer * a.so + (int64_t)cv * VEC * a.sk;
+        const T* base = (const T*)a.in + (int64_t)outer * a.so + (int64_t)cv * (VEC > 1 ? VEC : a.sk);
         const int r0 = blockIdx.z * a.chunk;
         const int r1 = min(a.R, r0 + a.chunk);
         int r = r0 + ty;
@@ -260,28 +264,28 @@ __global__ void __launch_bounds__(1024) col_lean_kernel(const ColLeanArgs a) {
 #pragma unroll
             for (int u = 0; u < 8; ++u)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v[u].v[j], r + u * by);
+                for (int j = 0; j < UV; ++j) fold_in<Op>(acc[j], v[u].v[j * SS], r + u * by);
         }
         for (; r < r1; r += by) {
             const T* p = base + (int64_t)r * a.rs;
             if constexpr (VEC > 1) {
                 Pack<T, VEC> v = load_pack_stream<T, VEC>(p);
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v.v[j], r);
+                for (int j = 0; j < UV; ++j) fold_in<Op>(acc[j], v.v[j * SS], r);
             } else {
                 fold_in<Op>(acc[0], *p, r);
             }
         }
     }
-    fold_thread_rows<Op, VEC>(acc, (Acc*)smem_raw);
+    fold_thread_rows<Op, UV>(acc, (Acc*)smem_raw);
     if (ty == 0 && valid) {
-        const int64_t o0 = ((int64_t)outer * a.kin_v + cv) * VEC;
+        const int64_t o0 = ((int64_t)outer * a.kin_v + cv) * UV;
         if (a.split == 1) {
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) write_out<Op>(a.out, o0 + j, acc[j], a.init_out, a.count);
+            for (int j = 0; j < UV; ++j) write_out<Op>(a.out, o0 + j, acc[j], a.init_out, a.count);
         } else {
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) ((Acc*)a.out)[(int64_t)blockIdx.z * a.K + o0 + j] = acc[j];
+            for (int j = 0; j < UV; ++j) ((Acc*)a.out)[(int64_t)blockIdx.z * a.K + o0 + j] = acc[j];
         }
     }
 }
@@ -415,7 +419,7 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.row_stride = p.kept.n ? p.kept.stride[0] : 0;
             a.count = count;
             a.K = (int)p.K;
-            a.rin_v = (int)(rin / p.vec);
+            a.rin_v = (int)(rin / (p.vec / p.sstride));
             a.sr = (int)p.red.stride[0];
             a.ichunk = (a.rin_v + p.split - 1) / p.split;
             a.tpr = p.tpr;
@@ -423,7 +427,8 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.rpb = p.rpb;
             a.split = p.split;
             a.init_out = init_out;
-            if (vec) row_lean_kernel<Op, FULL><<<grid, block, 0, st>>>(a);
+            if (vec && p.sstride == 2) row_lean_kernel<Op, FULL, 2><<<grid, block, 0, st>>>(a);
+            else if (vec) row_lean_kernel<Op, FULL><<<grid, block, 0, st>>>(a);
             else row_lean_kernel<Op, 1><<<grid, block, 0, st>>>(a);
         } else {
             RowArgs a{};
@@ -456,7 +461,7 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
     // Col
     const int64_t kv = p.K / p.vec;
     dim3 block((unsigned)p.bx, (unsigned)p.by);
-    size_t smem = p.by > 1 ? (size_t)p.bx * p.by * p.vec * sizeof(Acc) : 0;
+    size_t smem = p.by > 1 ? (size_t)p.bx * p.by * (p.vec / p.sstride) * sizeof(Acc) : 0;
     if (p.lean) {
         ColLeanArgs a{};
         const int nk = p.kept.n;
@@ -467,7 +472,7 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
         a.rs = p.red.n ? p.red.stride[0] : 0;
         a.K = p.K;
         a.count = count;
-        a.kin_v = (int)(kin / p.vec);
+        a.kin_v = (int)(kin / (p.vec / p.sstride));
         a.sk = nk ? (int)p.kept.stride[nk - 1] : 1;
         a.R = (int)p.R;
         a.chunk = (int)p.chunk;
@@ -475,7 +480,8 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
         a.init_out = init_out;
         const int64_t outer = nk > 1 ? p.kept.size[0] : 1;
         dim3 grid((unsigned)((a.kin_v + p.bx - 1) / p.bx), (unsigned)outer, (unsigned)p.split);
-        if (vec) col_lean_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
+        if (vec && p.sstride == 2) col_lean_kernel<Op, FULL, 2><<<grid, block, smem, st>>>(a);
+        else if (vec) col_lean_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
         else col_lean_kernel<Op, 1><<<grid, block, smem, st>>>(a);
     } else {
         ColArgs a{};

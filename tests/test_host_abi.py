@@ -92,10 +92,11 @@ def test_plans_for_the_benchmark_configurations(hpt):
     c4 = hpt.Tensor.from_numpy(np.zeros((64, 2048), np.uint16), hpt.bf16)
     assert hpt.normalize_plan(c4, 1).startswith("rowreg rows=64 cols=2048 vec=8 tpr=64 rpb=4 nchunk=4")
     c5 = hpt.Tensor.from_numpy(np.zeros((64, 128), np.float16))
-    assert hpt.normalize_plan(c5.permute([1, 0]), 1).startswith("transposed rows=128 cols=64")
+    assert hpt.normalize_plan(c5.permute([1, 0]), 1).startswith("transposed rows=128 cols=64 vec=8")
     assert hpt.reduce_plan(c5.permute([1, 0]), hpt.SUM, [0]).startswith("row vec=8")
-    assert "norm_in=[64:2]" in hpt.normalize_plan(c5[:, ::2], 1)
-    assert hpt.reduce_plan(c5[:, ::2], hpt.SUM, [0]).startswith("col vec=1")
+    assert hpt.normalize_plan(c5[:, ::2], 1).startswith("rowreg-step2") and "norm_in=[64:2]" in hpt.normalize_plan(c5[:, ::2], 1)
+    assert hpt.reduce_plan(c5[:, ::2], hpt.SUM, [0]).startswith("col-step2 vec=8")
+    assert hpt.reduce_plan(c5[:, 1::2], hpt.SUM, [0]).startswith("col vec=1")   # odd start: vectors would be misaligned
     # misaligned base pointer or odd row length: scalar loads
     assert hpt.reduce_plan(f32(7, 1023), hpt.SUM, [1]).startswith("row vec=1")
     assert hpt.reduce_plan(f32(8, 1024)[:, 1:], hpt.SUM, [1]).startswith("row vec=1")
