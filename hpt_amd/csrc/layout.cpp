@@ -371,7 +371,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             const int64_t groups = (R + 64 * v - 1) / (64 * v) * batch;
             int64_t S = std::max<int64_t>(1, std::min<int64_t>((512 + groups - 1) / groups, p.cols / 128));
             p.tsplit = (int)std::min<int64_t>(S, 64);
-            p.scratch_bytes = (size_t)p.rows * p.tsplit * 4 * 16 + (size_t)p.rows * 3 * 8;
+            p.scratch_bytes = (size_t)p.rows * p.tsplit * 16 + (size_t)p.rows * 3 * 8;
             return p;
         }
         if (sa >= 1 && sa <= 4) {

@@ -50,9 +50,9 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         t.R = (int)p.kept_in.size[nk - 1];
         t.cols = (int)p.cols;
         t.S = p.tsplit;
-        // scratch: [batch][4 S][R] partial statistics (16 bytes each at most), then [batch][3][R] numbers
+        // scratch: [batch][S][R] partial statistics (16 bytes each at most), then [batch][3][R] numbers
         t.stats = a.scratch;
-        t.params = (char*)a.scratch + (size_t)batch * t.S * 4 * t.R * 16;
+        t.params = (char*)a.scratch + (size_t)batch * t.S * t.R * 16;
         t.sa = a.sa;
         t.bi = nk > 1 ? p.kept_in.stride[0] : 0;
         t.eps = a.eps;

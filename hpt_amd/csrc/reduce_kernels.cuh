@@ -248,25 +248,28 @@ __global__ void __launch_bounds__(1024) col_lean_kernel(const ColLeanArgs a) {
     for (int j = 0; j < UV; ++j) acc[j] = Op::identity();
     if (valid) {
         const T* base = (const T*)a.in + (int64_t)outer * a.so + (int64_t)cv * (VEC > 1 ? VEC : a.sk);
-        const int r0 = blockIdx.z * a.chunk;
-        const int r1 = min(a.R, r0 + a.chunk);
-        int r = r0 + ty;
+        // The reduced range is dealt out round-robin: thread row ty of workgroup z takes
+        // r = z * by + ty, then steps by (by * splits). Wavefronts that run at the same
+        // time therefore read neighbouring rows, which keeps a power-of-two row pitch
+        // from sending them all to the same memory channels.
+        const int step = by * a.split;
+        int r = blockIdx.z * by + ty;
         // batches of eight loads in flight per lane before any is consumed: with one
         // wavefront per 64 columns this is what keeps the memory pipeline full
-        for (; r + 7 * by < r1; r += 8 * by) {
+        for (; r + 7 * step < a.R; r += 8 * step) {
             Pack<T, VEC> v[8];
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
-                const T* p = base + (int64_t)(r + u * by) * a.rs;
+                const T* p = base + (int64_t)(r + u * step) * a.rs;
                 if constexpr (VEC > 1) v[u] = load_pack_stream<T, VEC>(p);
                 else v[u].v[0] = *p;
             }
 #pragma unroll
             for (int u = 0; u < 8; ++u)
 #pragma unroll
-                for (int j = 0; j < UV; ++j) fold_in<Op>(acc[j], v[u].v[j * SS], r + u * by);
+                for (int j = 0; j < UV; ++j) fold_in<Op>(acc[j], v[u].v[j * SS], r + u * step);
         }
-        for (; r < r1; r += by) {
+        for (; r < a.R; r += step) {
             const T* p = base + (int64_t)r * a.rs;
             if constexpr (VEC > 1) {
                 Pack<T, VEC> v = load_pack_stream<T, VEC>(p);
@@ -356,28 +359,45 @@ __global__ void __launch_bounds__(1024) col_reduce_kernel(const ColArgs a) {
 }
 
 // ---- second stage: fold the partials of the outputs that were split ---------------
-// Partial s of output o sits at part[o * so + s * ss]. BLOCK_PER_OUTPUT: a
-// workgroup folds one output (many partials, few outputs); otherwise a thread
-// folds one output (few partials, many outputs; lanes are neighbours in memory).
-template <class Op, bool BLOCK_PER_OUTPUT>
-__global__ void __launch_bounds__(256) finish_kernel(const void* part_, void* out, int64_t K, int split,
-                                                     int64_t so, int64_t ss, int init_out, double count) {
+// finish_rows_kernel: few outputs with many partials each (row splits; partial s of
+// output o at part[o * split + s]): a workgroup folds one output.
+template <class Op>
+__global__ void __launch_bounds__(256) finish_rows_kernel(const void* part_, void* out, int split, int init_out,
+                                                          double count) {
     using Acc = typename Op::Acc;
     const Acc* part = (const Acc*)part_;
-    if constexpr (BLOCK_PER_OUTPUT) {
-        __shared__ Acc smem[16];
-        const int64_t o = blockIdx.x;
-        Acc acc = Op::identity();
-        for (int s = threadIdx.x; s < split; s += blockDim.x) acc = Op::comb(acc, part[o * so + s * ss]);
-        acc = block_reduce<Op>(acc, smem);
-        if (threadIdx.x == 0) write_out<Op>(out, o, acc, init_out, count);
-    } else {
-        const int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-        if (o >= K) return;
-        Acc acc = Op::identity();
-        for (int s = 0; s < split; ++s) acc = Op::comb(acc, part[o * so + s * ss]);
-        write_out<Op>(out, o, acc, init_out, count);
+    __shared__ Acc smem[16];
+    const int64_t o = blockIdx.x;
+    Acc acc = Op::identity();
+    for (int s = threadIdx.x; s < split; s += blockDim.x) acc = Op::comb(acc, part[o * split + s]);
+    acc = block_reduce<Op>(acc, smem);
+    if (threadIdx.x == 0) write_out<Op>(out, o, acc, init_out, count);
+}
+
+// finish_cols_kernel: many outputs (column splits; partial s of output o at
+// part[s * K + o]): 64 neighbouring outputs per workgroup, the partials of each dealt
+// over blockDim.y thread rows so that no thread walks a long chain of dependent
+// loads, then folded through LDS.
+template <class Op>
+__global__ void __launch_bounds__(1024) finish_cols_kernel(const void* part_, void* out, int64_t K, int split,
+                                                           int init_out, double count) {
+    using Acc = typename Op::Acc;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    Acc* sm = (Acc*)smem_raw;
+    const Acc* part = (const Acc*)part_;
+    const int tx = threadIdx.x, ty = threadIdx.y, by = blockDim.y;
+    const int64_t o = (int64_t)blockIdx.x * 64 + tx;
+    const bool valid = o < K;
+    Acc acc = Op::identity();
+    if (valid)
+        for (int s = ty; s < split; s += by) acc = Op::comb(acc, part[(int64_t)s * K + o]);
+    if (by > 1) {
+        sm[ty * 64 + tx] = acc;
+        __syncthreads();
+        if (ty == 0)
+            for (int y = 1; y < by; ++y) acc = Op::comb(acc, sm[y * 64 + tx]);
     }
+    if (ty == 0 && valid) write_out<Op>(out, o, acc, init_out, count);
 }
 
 // Fill `n` outputs with the op's identity (a reduced dim of size 0).
@@ -454,8 +474,8 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             else row_reduce_kernel<Op, 1><<<grid, block, 0, st>>>(a);
         }
         if (p.split > 1)
-            finish_kernel<Op, true><<<dim3((unsigned)p.K), dim3(256), 0, st>>>(sc.partial, out, p.K, p.split,
-                                                                             p.split, 1, init_out, count);
+            finish_rows_kernel<Op><<<dim3((unsigned)p.K), dim3(256), 0, st>>>(sc.partial, out, p.split, init_out,
+                                                                              count);
         return;
     }
     // Col
@@ -502,9 +522,13 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
         if (vec) col_reduce_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
         else col_reduce_kernel<Op, 1><<<grid, block, smem, st>>>(a);
     }
-    if (p.split > 1)
-        finish_kernel<Op, false><<<dim3((unsigned)((p.K + 255) / 256)), dim3(256), 0, st>>>(
-            sc.partial, out, p.K, p.split, 1, p.K, init_out, count);
+    if (p.split > 1) {
+        int fy = 1;  // thread rows sharing an output's partials: about two partials per thread
+        while (fy < 16 && fy * 2 < p.split) fy <<= 1;
+        finish_cols_kernel<Op><<<dim3((unsigned)((p.K + 63) / 64)), dim3(64, (unsigned)fy),
+                                 fy > 1 ? (size_t)fy * 64 * sizeof(Acc) : 0, st>>>(sc.partial, out, p.K, p.split,
+                                                                                    init_out, count);
+    }
 }
 
 // Instantiate launch_reduce_t for every dtype of one op family.

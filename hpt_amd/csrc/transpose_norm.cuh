@@ -56,8 +56,9 @@ template <int KIND, class T> struct RowPartial {
 
 // Pass 1: partial row statistics. Lanes run along the rows (a wavefront reads 1 KiB
 // of consecutive rows per column), so every lane owns its VEC rows outright: no
-// cross-lane merge, no LDS. Every wavefront takes its own column range and writes
-// one partial per row: partial p of row r goes to stats[b][p][r], p = split * 4 + wave.
+// cross-lane merge. Every wavefront takes its own columns; the four wavefronts of a
+// workgroup meet in LDS and write one partial per row: partial y of row r goes to
+// stats[b][y][r], y = blockIdx.y.
 template <int KIND, class T>
 __global__ void __launch_bounds__(256) transposed_stats_kernel(const TransposedArgs a) {
     using CT = typename Elem<T>::Wide;
@@ -68,12 +69,15 @@ __global__ void __launch_bounds__(256) transposed_stats_kernel(const TransposedA
     const int lane = threadIdx.x & 63;
     // the wavefront index is uniform: say so, and the column arithmetic stays scalar
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int r0 = (blockIdx.x * 64 + lane) * VEC;
-    if (r0 >= a.R) return;
-    // this wavefront's column range inside the workgroup's split
-    const int cpw = (a.cols_per_split + NW - 1) / NW;
-    const int cb = blockIdx.y * a.cols_per_split + w * cpw;
-    const int ce = min(min(a.cols, (int)(blockIdx.y + 1) * a.cols_per_split), cb + cpw);
+    // lanes past the last row keep going (they meet the others at the barrier below) on row 0
+    const bool valid = (blockIdx.x * 64 + lane) * VEC < a.R;
+    const int r0 = valid ? (blockIdx.x * 64 + lane) * VEC : 0;
+    // Columns are dealt out round-robin over all P = 4 S wavefronts that share these
+    // rows: wavefront p takes columns p, p + P, ... Wavefronts running at the same time
+    // then read neighbouring columns, which keeps a power-of-two column pitch from
+    // sending them all to the same memory channels.
+    const int P = a.S * NW;
+    const int pid = blockIdx.y * NW + w;
     const T* base = (const T*)a.in + (int64_t)blockIdx.z * a.bi + r0;
 
     // per row: softmax (m, s); layernorm s = sum (x - k), s2 = sum (x - k)^2, k = x[row][0]
@@ -119,36 +123,58 @@ __global__ void __launch_bounds__(256) transposed_stats_kernel(const TransposedA
             }
         }
     };
-    const T* p = base + (int64_t)cb * a.sa;
-    int c = cb;
-    for (; c + 8 <= ce; c += 8) {  // eight columns in flight per lane
+    const int64_t stepb = (int64_t)P * a.sa;
+    const T* p = base + (int64_t)pid * a.sa;
+    int c = pid;
+    for (; c + 7 * P < a.cols; c += 8 * P) {  // eight columns in flight per lane
         Pack<T, VEC> v[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = load_pack<T, VEC>(p + (int64_t)i * a.sa);
-        p += 8 * a.sa;
+        for (int i = 0; i < 8; ++i) v[i] = load_pack<T, VEC>(p + i * stepb);
+        p += 8 * stepb;
         // keep the scheduler from sinking loads into the arithmetic: all eight stay in flight
         __builtin_amdgcn_sched_barrier(0);
         fold(v, std::integral_constant<int, 8>{});
     }
-    for (; c < ce; ++c) {
+    for (; c < a.cols; c += P) {
         Pack<T, VEC> v = load_pack<T, VEC>(p);
-        p += a.sa;
+        p += stepb;
         fold(&v, std::integral_constant<int, 1>{});
     }
 
-    const int P = a.S * NW;
-    Part* dst = (Part*)a.stats + ((int64_t)blockIdx.z * P + blockIdx.y * NW + w) * a.R + r0;
+    // The four wavefronts hold partials of the same rows: fold them through LDS so
+    // that one partial per row and workgroup goes to memory.
+    __shared__ Part sm[NW - 1][VEC][64];
+    Part t[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; ++k) {
-        Part t;
         if constexpr (KIND == NORM_LAYERNORM) {
-            t.s1 = s[k];
-            t.s2 = s2[k];
+            t[k].s1 = s[k];
+            t[k].s2 = s2[k];
         } else {
-            t.m = m[k];
-            t.s = s[k];
+            t[k].m = m[k];
+            t[k].s = s[k];
         }
-        dst[k] = t;
+    }
+    if (w > 0) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) sm[w - 1][k][lane] = t[k];
+    }
+    __syncthreads();
+    if (w > 0 || !valid) return;
+    Part* dst = (Part*)a.stats + ((int64_t)blockIdx.z * a.S + blockIdx.y) * a.R + r0;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+#pragma unroll
+        for (int o = 0; o < NW - 1; ++o) {
+            const Part u = sm[o][k][lane];
+            if constexpr (KIND == NORM_LAYERNORM) {
+                t[k].s1 += u.s1;
+                t[k].s2 += u.s2;
+            } else {
+                t[k] = SoftStatOp<T, CT>::comb(t[k], u);
+            }
+        }
+        dst[k] = t[k];
     }
 }
 
@@ -161,11 +187,11 @@ __global__ void __launch_bounds__(256) transposed_finalize_kernel(const Transpos
     using CT = typename Elem<T>::Wide;
     using ST = typename StatType<T>::type;
     using Part = typename RowPartial<KIND, T>::type;
-    constexpr int NW = 4, LY = 16;
+    constexpr int LY = 16;
     __shared__ ST sm0[LY][16], sm1[LY][16];
     const int r = blockIdx.x * 16 + threadIdx.x;
     const bool ok = r < a.R;
-    const int P = a.S * NW;
+    const int P = a.S;
     ST acc0, acc1;  // layernorm: sums of s1, s2; softmax: running max, rescaled sum
     if constexpr (KIND == NORM_LAYERNORM) { acc0 = 0; acc1 = 0; }
     else { acc0 = (ST)neg_inf<CT>(); acc1 = 0; }
