@@ -33,6 +33,11 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+# HBM bytes one headline launch moves, from two hardware-counter runs of this script
+# (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, with --copy-calibration), each counter scaled
+# by what it reads for the plain 134217728-byte copy in the same run: fetch 131406.7 KiB +
+# write 131091.1 KiB. A measured constant, not something this script can read live.
+HEADLINE_TRAFFIC_BYTES = 268797803
 
 
 # ---- HIP events on the launch stream (the null stream: the library is called with stream=NULL) ----
@@ -356,7 +361,7 @@ def main():
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1),
         "rows_per_s": round(8192 * args.steps / wall, 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": HEADLINE_TRAFFIC_BYTES,
                      "kernel": "hpt::row_reg_kernel<2, float, 4, 4, 1>", "kernel_us": round(kernel_us, 2)},
         "cpu_baseline": cpu,
         "ops": ops,
