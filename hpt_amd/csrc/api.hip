@@ -610,7 +610,8 @@ int32_t hpt_hip_layernorm(int32_t dev, void* stream, const hpt_view* in, int32_t
         // vector loads of gamma/beta need 16-byte alignment too
         if (c.plan.vec > 1 && (((uintptr_t)c.args.gamma | (uintptr_t)c.args.beta) % 16) != 0) {
             c.plan.vec = 1;
-            if (c.plan.kind == NormKind::RowReg || c.plan.kind == NormKind::Transposed) {
+            if (c.plan.kind == NormKind::RowReg || c.plan.kind == NormKind::Transposed ||
+                c.plan.kind == NormKind::TransposedTile) {
                 c.plan.kind = NormKind::Generic;
                 c.plan.scratch_bytes = 0;
                 c.plan.sstride = 1;

@@ -112,7 +112,8 @@ enum class NormKind {
     RowReg,     // a row sits in the registers of `tpr` threads; one HBM read, one write
     RowStream,  // rows too long for registers: statistics pass, then a second read
     Col,        // the normalised axis is strided in input and output alike; lanes walk the inner dim
-    Transposed, // input contiguous along the rows, output along the axis: statistics + LDS tile transpose
+    Transposed, // input contiguous along the rows, output along the axis: statistics, then a register-tile transpose
+    TransposedTile,  // same layout, a block of rows fits one compute unit's registers: one read, one write
     Generic     // anything else: one block per row, per-element offset arithmetic
 };
 
@@ -124,8 +125,8 @@ struct NormPlan {
     Dims norm_in;        // input (size, stride) of the normalised dims, logical order, coalesced
     int64_t out_axis_stride = 1;  // output stride between consecutive elements of a row
     int vec = 1;
-    int tpr = 1;      // threads per row (RowReg / RowStream / Generic)
-    int rpb = 1;      // rows per block
+    int tpr = 1;      // threads per row (RowReg / RowStream / Generic); TransposedTile: lanes along the rows (rgN)
+    int rpb = 1;      // rows per block; TransposedTile: wavefronts per workgroup
     int nchunk = 1;   // RowReg: vectors held per thread
     int max_blocks = 1024;  // RowReg layernorm: workgroups launched at most (they walk the rows)
     int64_t inner = 1;  // Col: size of the contiguous inner dim the lanes walk

@@ -362,8 +362,28 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                           p.kept_in.size[nk - 1] <= 0x7fffffff && p.cols <= 0x7fffffff &&
                           p.kept_in.size[nk - 1] >= 8 * v && p.cols >= 8 * v;
         if (transposed) {
-            p.kind = NormKind::Transposed;
             p.vec = v;
+            {
+                // Single pass when 16 vectors per thread hold (16 * rgN bytes of rows) x (all
+                // columns): rgN lanes along the rows, 1024 / rgN thread columns of 16 columns
+                // each. Prefer long row segments, but keep at least ~one workgroup per
+                // compute unit; below 64-byte segments the three-pass form is used.
+                const int64_t R = p.kept_in.size[nk - 1];
+                const int64_t batch = nk > 1 ? p.kept_in.size[0] : 1;
+                const int64_t cgroups = (p.cols + 15) / 16;
+                int rgN = 16;
+                while (rgN >= 4 && cgroups * rgN > 1024) rgN >>= 1;
+                while (rgN > 8 && (R + rgN * v - 1) / (rgN * v) * batch < 256) rgN >>= 1;
+                const int64_t blocks = rgN >= 4 ? (R + rgN * v - 1) / (rgN * v) * batch : 0;
+                if (rgN >= 4 && blocks >= 128 && !getenv("HPT_NO_TILE")) {
+                    p.kind = NormKind::TransposedTile;
+                    p.tpr = rgN;
+                    const int64_t cols_per_wave = 16 * (64 / rgN);
+                    p.rpb = (int)((p.cols + cols_per_wave - 1) / cols_per_wave);
+                    return p;
+                }
+            }
+            p.kind = NormKind::Transposed;
             // statistics pass: a wavefront covers 64*v rows; enough column splits for
             // about 2048 wavefronts, each keeping at least 32 columns
             const int64_t R = p.kept_in.size[nk - 1];
@@ -371,6 +391,9 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             const int64_t groups = (R + 64 * v - 1) / (64 * v) * batch;
             int64_t S = std::max<int64_t>(1, std::min<int64_t>((512 + groups - 1) / groups, p.cols / 128));
             p.tsplit = (int)std::min<int64_t>(S, 64);
+            p.tpr = 4;  // wavefronts per workgroup of the statistics pass
+            if (const char* e = getenv("HPT_TSPLIT")) p.tsplit = atoi(e);
+            if (const char* e = getenv("HPT_TNW")) p.tpr = atoi(e);
             p.scratch_bytes = (size_t)p.rows * p.tsplit * 16 + (size_t)p.rows * 3 * 8;
             return p;
         }
@@ -430,7 +453,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
 }
 
 std::string describe(const NormPlan& p) {
-    static const char* names[] = {"empty", "rowreg", "rowstream", "col", "transposed", "generic"};
+    static const char* names[] = {"empty", "rowreg", "rowstream", "col", "transposed", "transposed-tile", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
              names[(int)p.kind], p.sstride == 2 ? "-step2" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,

@@ -38,6 +38,26 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
     a.inv_cols = 1.0 / (double)p.cols;
     dim3 grid((unsigned)((p.rows + p.rpb - 1) / p.rpb));
     dim3 block((unsigned)(p.tpr * p.rpb));
+    if (p.kind == NormKind::TransposedTile) {
+        TileArgs t{};
+        t.in = a.in;
+        t.out = a.out;
+        t.gamma = a.gamma;
+        t.beta = a.beta;
+        const int nk = p.kept_in.n;
+        const unsigned batch = nk > 1 ? (unsigned)p.kept_in.size[0] : 1u;
+        t.R = (int)p.kept_in.size[nk - 1];
+        t.cols = (int)p.cols;
+        t.sa = a.sa;
+        t.bi = nk > 1 ? p.kept_in.stride[0] : 0;
+        t.eps = a.eps;
+        t.inv_cols = a.inv_cols;
+        t.rg_log2 = ilog2(p.tpr);
+        t.pair = p.tpr == 4;
+        const unsigned blocks = (unsigned)((t.R + p.tpr * FULL - 1) / (p.tpr * FULL));
+        transposed_tile_kernel<KIND, T><<<dim3(blocks, batch), dim3(64u * (unsigned)p.rpb), 0, st>>>(t);
+        return;
+    }
     if (p.kind == NormKind::Transposed) {
         constexpr int TILE = 8 * FULL;
         TransposedArgs t{};
@@ -61,7 +81,10 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         const int tiles = (t.cols + TILE - 1) / TILE;
         const unsigned rt = (unsigned)((t.R + TILE - 1) / TILE);
         const unsigned rg = (unsigned)((t.R + 64 * FULL - 1) / (64 * FULL));
-        transposed_stats_kernel<KIND, T><<<dim3(rg, (unsigned)t.S, batch), dim3(256), 0, st>>>(t);
+        using Part = typename RowPartial<KIND, T>::type;
+        const unsigned nw = (unsigned)p.tpr;  // wavefronts per workgroup of the statistics pass
+        transposed_stats_kernel<KIND, T>
+            <<<dim3(rg, (unsigned)t.S, batch), dim3(64 * nw), (size_t)nw * FULL * 64 * sizeof(Part), st>>>(t);
         transposed_finalize_kernel<KIND, T><<<dim3((unsigned)((t.R + 15) / 16), 1, batch), dim3(16, 16), 0, st>>>(t);
         transposed_apply_kernel<KIND, T><<<dim3(rt, (unsigned)((tiles + 3) / 4), batch), dim3(256), 0, st>>>(t);
         return;

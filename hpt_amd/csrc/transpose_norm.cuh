@@ -56,15 +56,16 @@ template <int KIND, class T> struct RowPartial {
 
 // Pass 1: partial row statistics. Lanes run along the rows (a wavefront reads 1 KiB
 // of consecutive rows per column), so every lane owns its VEC rows outright: no
-// cross-lane merge. Every wavefront takes its own columns; the four wavefronts of a
+// cross-lane merge. Every wavefront takes its own columns; the wavefronts of a
 // workgroup meet in LDS and write one partial per row: partial y of row r goes to
 // stats[b][y][r], y = blockIdx.y.
 template <int KIND, class T>
-__global__ void __launch_bounds__(256) transposed_stats_kernel(const TransposedArgs a) {
+__global__ void __launch_bounds__(1024) transposed_stats_kernel(const TransposedArgs a) {
     using CT = typename Elem<T>::Wide;
     using Part = typename RowPartial<KIND, T>::type;
     constexpr int VEC = 16 / sizeof(T);
-    constexpr int NW = 4;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int NW = blockDim.x >> 6;  // wavefronts per workgroup (1...16)
 
     const int lane = threadIdx.x & 63;
     // the wavefront index is uniform: say so, and the column arithmetic stays scalar
@@ -141,40 +142,37 @@ __global__ void __launch_bounds__(256) transposed_stats_kernel(const TransposedA
         fold(&v, std::integral_constant<int, 1>{});
     }
 
-    // The four wavefronts hold partials of the same rows: fold them through LDS so
+    // The wavefronts of a workgroup hold partials of the same rows: they meet in LDS
+    // (sm[wavefront][k][lane]) and wavefront w folds row k = w, w + NW, ... of every lane, so
     // that one partial per row and workgroup goes to memory.
-    __shared__ Part sm[NW - 1][VEC][64];
-    Part t[VEC];
+    Part* sm = (Part*)smem_raw;
 #pragma unroll
     for (int k = 0; k < VEC; ++k) {
+        Part t;
         if constexpr (KIND == NORM_LAYERNORM) {
-            t[k].s1 = s[k];
-            t[k].s2 = s2[k];
+            t.s1 = s[k];
+            t.s2 = s2[k];
         } else {
-            t[k].m = m[k];
-            t[k].s = s[k];
+            t.m = m[k];
+            t.s = s[k];
         }
-    }
-    if (w > 0) {
-#pragma unroll
-        for (int k = 0; k < VEC; ++k) sm[w - 1][k][lane] = t[k];
+        sm[(w * VEC + k) * 64 + lane] = t;
     }
     __syncthreads();
-    if (w > 0 || !valid) return;
+    if (!valid) return;
     Part* dst = (Part*)a.stats + ((int64_t)blockIdx.z * a.S + blockIdx.y) * a.R + r0;
-#pragma unroll
-    for (int k = 0; k < VEC; ++k) {
-#pragma unroll
-        for (int o = 0; o < NW - 1; ++o) {
-            const Part u = sm[o][k][lane];
+    for (int k = w; k < VEC; k += NW) {
+        Part t = sm[k * 64 + lane];
+        for (int o = 1; o < NW; ++o) {
+            const Part u = sm[(o * VEC + k) * 64 + lane];
             if constexpr (KIND == NORM_LAYERNORM) {
-                t[k].s1 += u.s1;
-                t[k].s2 += u.s2;
+                t.s1 += u.s1;
+                t.s2 += u.s2;
             } else {
-                t[k] = SoftStatOp<T, CT>::comb(t[k], u);
+                t = SoftStatOp<T, CT>::comb(t, u);
             }
         }
-        dst[k] = t[k];
+        dst[k] = t;
     }
 }
 
@@ -295,6 +293,319 @@ __global__ void __launch_bounds__(256) transposed_apply_kernel(const TransposedA
             o.v[i] = Elem<T>::narrow(y);
         }
         store_pack_stream<T, VEC>(out + (int64_t)k * a.cols, o);
+    }
+}
+
+// ---- single pass: the whole row block lives in registers -------------------------
+// When (16 * rgN bytes of consecutive rows) x (all columns) fits the register file of
+// one compute unit (16 vectors per thread, up to 1024 threads), a workgroup loads its
+// row block ONCE, takes the row statistics from registers (the reference's two-pass
+// forms, no shifted sums needed), and stores the transposed result: one HBM read and
+// one HBM write per element instead of two reads and one write.
+//
+// Lane (rg, cgl) of wavefront w: rg = lane % rgN picks VEC consecutive rows (one
+// 128-bit vector along the rows); it holds 16 columns as H = 16 / VEC groups of VEC
+// consecutive columns, group h starting at column w * 16 * CGW + h * VEC * CGW + cgl * VEC
+// (CGW = 64 / rgN). A load instruction therefore reads 16 * rgN contiguous bytes per
+// column; a store instruction writes, per row, VEC * CGW consecutive columns.
+//
+// With rgN = 4 a 128-byte line of the input is shared by two workgroups. Workgroups
+// are handed to the eight XCDs (each with its own L2) round-robin, so the row blocks
+// are renumbered to put both halves of a line on workgroups i and i + 8: same XCD,
+// dispatched together, and the second one hits in L2.
+struct TileArgs {
+    const void* in;
+    void* out;
+    const void* gamma;
+    const void* beta;
+    int64_t sa;  // input stride along the normalised axis
+    int64_t bi;  // input stride of the batch dim
+    double eps, inv_cols;
+    int R;       // rows per batch (contiguous in the input)
+    int cols;
+    int rg_log2; // log2(rgN), rgN = 4, 8 or 16
+    int pair;    // 1: renumber row blocks so that line-sharing pairs meet on one XCD
+};
+
+// All-reduce of VEC row values over every thread that holds a piece of the same rows:
+// shuffles over the lanes of a wavefront that share rg, then LDS across wavefronts.
+template <class Op, class A, int VEC>
+__device__ __forceinline__ void tile_all_reduce(A (&v)[VEC], int rgN, int rg, int cgl, int w, int nw, A* part,
+                                                A* res) {
+    for (int m = rgN; m < 64; m <<= 1) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) v[k] = Op::comb(v[k], shfl_xor_any(v[k], m));
+    }
+    if (nw == 1) return;
+    const int rows = rgN * VEC;
+    __syncthreads();  // the slots may still be read from the previous use
+    if (cgl == 0) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) part[w * rows + rg * VEC + k] = v[k];
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < rows) {
+        A r = part[threadIdx.x];
+        for (int o = 1; o < nw; ++o) r = Op::comb(r, part[o * rows + threadIdx.x]);
+        res[threadIdx.x] = r;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) v[k] = res[rg * VEC + k];
+}
+
+// Make the compiler forget what it knows about the tile's registers. Between two
+// sweeps over a tile of 2-byte elements it would otherwise keep the widened (f32)
+// copies of the first sweep alive for the second: twice the registers of the tile
+// itself, i.e. spills to scratch memory. Widening again costs one conversion.
+template <class T, int VEC> __device__ __forceinline__ void forget_values(Pack<T, VEC> (&v)[16]) {
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&v[j])));
+    }
+}
+
+template <int KIND, class T>
+__global__ void __launch_bounds__(1024) transposed_tile_kernel(const TileArgs a) {
+    using CT = typename Elem<T>::Wide;
+    using ST = typename StatType<T>::type;
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr int H = 16 / VEC;
+    constexpr bool kSoft = KIND != NORM_LAYERNORM;
+    constexpr bool kKeepExp = kSoft && sizeof(T) == sizeof(CT);  // exp(x - max) fits back into the tile
+    __shared__ __align__(8) unsigned char smem_raw[(16 * 128 + 128) * sizeof(double)];
+    ST* part = reinterpret_cast<ST*>(smem_raw);
+    ST* res = part + 16 * 128;
+
+    const int rgN = 1 << a.rg_log2;
+    const int cgw = 64 >> a.rg_log2;
+    const int lane = threadIdx.x & 63;
+    const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int rg = lane & (rgN - 1), cgl = lane >> a.rg_log2;
+
+    int b = blockIdx.x;
+    if (a.pair && b < (int)(gridDim.x & ~15u)) {
+        const int x = b & 7, q = b >> 3;
+        b = ((x + 8 * (q >> 1)) << 1) | (q & 1);
+    }
+    const int r0 = (b * rgN + rg) * VEC;
+    const bool row_ok = r0 < a.R;
+    const int gw = VEC * cgw;                       // columns a wavefront covers per group
+    const int c_first = w * 16 * cgw + cgl * VEC;   // first column of group 0
+    bool col_ok[H];
+#pragma unroll
+    for (int h = 0; h < H; ++h) col_ok[h] = c_first + h * gw < a.cols;
+
+    // Every thread loads 16 vectors, unconditionally: a thread whose rows or columns lie
+    // outside the tensor reads row block 0 / column 0 instead (always there), and is
+    // left out where it would count: its column groups are skipped when the per-thread
+    // statistics are folded, and nothing of it is stored. No branch sits between the
+    // loads, so all 16 are in flight at once and the first sweep below consumes them in
+    // the order they return.
+    Pack<T, VEC> v[16];
+    {
+        const T* base = (const T*)a.in + (int64_t)blockIdx.y * a.bi + (row_ok ? r0 : 0);
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            const T* p = base + (col_ok[h] ? (int64_t)(c_first + h * gw) * a.sa : (int64_t)0);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) v[h * VEC + i] = load_pack<T, VEC>(p + i * a.sa);
+        }
+    }
+    // gamma / beta of this thread's columns, fetched before anything is stored: a load
+    // issued between the stores would have to wait for every store before it. (f64
+    // holds too many registers for that and loads them group by group.)
+    constexpr bool kHoistAffine = !kSoft && sizeof(T) <= 4;
+    Pack<T, VEC> gam[kHoistAffine ? H : 1], bet[kHoistAffine ? H : 1];
+    // (an absent gamma / beta still loads, from the start of the input, and the value is
+    // then replaced: a load under a branch would make the compiler wait for it, and for
+    // every load issued before it, at the end of the branch)
+    auto load_affine = [&](int h, Pack<T, VEC>& gp, Pack<T, VEC>& bp) {
+        const int c = col_ok[h] ? c_first + h * gw : 0;
+        const T* gsrc = a.gamma ? (const T*)a.gamma + c : (const T*)a.in;
+        const T* bsrc = a.beta ? (const T*)a.beta + c : (const T*)a.in;
+        gp = load_pack<T, VEC>(gsrc);
+        bp = load_pack<T, VEC>(bsrc);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            gp.v[i] = a.gamma ? gp.v[i] : Elem<T>::narrow((CT)1);
+            bp.v[i] = a.beta ? bp.v[i] : Elem<T>::narrow((CT)0);
+        }
+    };
+    if constexpr (kHoistAffine) {
+#pragma unroll
+        for (int h = 0; h < H; ++h) load_affine(h, gam[h], bet[h]);
+    }
+
+    // per row k: p0, p1 (and p2) are what the output pass needs
+    CT p0[VEC], p1[VEC], p2[VEC];
+    if constexpr (kSoft) {
+        CT m[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) m[k] = neg_inf<CT>();
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            CT mh[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) mh[k] = neg_inf<CT>();
+#pragma unroll
+            for (int i = 0; i < VEC; ++i)
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) mh[k] = MaxC<CT>::comb(mh[k], Elem<T>::widen(v[h * VEC + i].v[k]));
+            if (col_ok[h]) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) m[k] = MaxC<CT>::comb(m[k], mh[k]);
+            }
+        }
+        forget_values(v);
+        tile_all_reduce<MaxC<CT>, CT, VEC>(m, rgN, rg, cgl, w, nw, (CT*)part, (CT*)res);
+        CT s[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) s[k] = 0;
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            CT sh[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) sh[k] = 0;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i)
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    const CT e = exp_ct<T>(Elem<T>::widen(v[h * VEC + i].v[k]) - m[k]);
+                    sh[k] += e;
+                    if constexpr (kKeepExp && KIND == NORM_SOFTMAX) v[h * VEC + i].v[k] = Elem<T>::narrow(e);
+                }
+            if (col_ok[h]) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) s[k] += sh[k];
+            }
+        }
+        forget_values(v);
+        tile_all_reduce<SumC<CT>, CT, VEC>(s, rgN, rg, cgl, w, nw, (CT*)part, (CT*)res);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            p0[k] = m[k];
+            p1[k] = KIND == NORM_SOFTMAX ? (CT)1 / s[k] : log_ct<T>(s[k]);
+            p2[k] = 0;
+        }
+    } else {
+        ST sum[VEC];
+        {
+            CT t[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) t[k] = 0;
+#pragma unroll
+            for (int h = 0; h < H; ++h) {
+                CT th[VEC];
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) th[k] = 0;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i)
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) th[k] += Elem<T>::widen(v[h * VEC + i].v[k]);
+                if (col_ok[h]) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) t[k] += th[k];
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) sum[k] = (ST)t[k];
+        }
+        forget_values(v);
+        tile_all_reduce<SumC<ST>, ST, VEC>(sum, rgN, rg, cgl, w, nw, part, res);
+        ST q[VEC];
+        {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                // mean = sum / cols: reciprocal multiply plus one correction step
+                const ST m0 = sum[k] * (ST)a.inv_cols;
+                const ST mean = fma_ct(fma_ct(-m0, (ST)a.cols, sum[k]), (ST)a.inv_cols, m0);
+                p0[k] = (CT)mean;
+                if constexpr (sizeof(ST) > sizeof(CT)) p1[k] = (CT)(mean - (ST)p0[k]);
+                else p1[k] = 0;
+            }
+            CT t[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) t[k] = 0;
+#pragma unroll
+            for (int h = 0; h < H; ++h) {
+                CT th[VEC];
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) th[k] = 0;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i)
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) {
+                        CT d = Elem<T>::widen(v[h * VEC + i].v[k]) - p0[k];
+                        if constexpr (sizeof(ST) > sizeof(CT)) d -= p1[k];
+                        th[k] += d * d;
+                    }
+                if (col_ok[h]) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) t[k] += th[k];
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) q[k] = (ST)t[k];
+        }
+        forget_values(v);
+        tile_all_reduce<SumC<ST>, ST, VEC>(q, rgN, rg, cgl, w, nw, part, res);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) p2[k] = rsqrt_ct((CT)(q[k] * (ST)a.inv_cols) + (CT)a.eps);
+    }
+
+    if (!row_ok) return;
+    if constexpr (kHoistAffine) {
+        // gamma / beta must have arrived before the first store is issued: loads and
+        // stores share one counter, so waiting for them later would also wait for
+        // every store issued in between
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&gam[h])));
+            asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&bet[h])));
+        }
+    }
+    T* out = (T*)a.out + ((int64_t)blockIdx.y * a.R + r0) * a.cols + c_first;
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+        if (!col_ok[h]) continue;
+        CT g[VEC], bt[VEC];
+        if constexpr (!kSoft) {
+            Pack<T, VEC> gp, bp;
+            if constexpr (kHoistAffine) {
+                gp = gam[h];
+                bp = bet[h];
+            } else {
+                load_affine(h, gp, bp);
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                g[i] = Elem<T>::widen(gp.v[i]);
+                bt[i] = Elem<T>::widen(bp.v[i]);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            Pack<T, VEC> o;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                const CT x = Elem<T>::widen(v[h * VEC + i].v[k]);
+                CT y;
+                if constexpr (KIND == NORM_LAYERNORM) {
+                    y = x - p0[k];
+                    if constexpr (sizeof(ST) > sizeof(CT)) y -= p1[k];
+                    y = y * p2[k] * g[i] + bt[i];
+                } else if constexpr (KIND == NORM_SOFTMAX) {
+                    y = (kKeepExp ? x : exp_ct<T>(x - p0[k])) * p1[k];
+                } else {
+                    y = (x - p0[k]) - p1[k];
+                }
+                o.v[i] = Elem<T>::narrow(y);
+            }
+            store_pack_stream<T, VEC>(out + (int64_t)k * a.cols + h * gw, o);
+            // one output vector at a time: interleaving several only adds live registers
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
 }
 

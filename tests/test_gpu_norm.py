@@ -167,3 +167,78 @@ def test_layernorm_half_types(hpt, orc, dev, name):
             else:
                 want = tof(orc.layernorm(a, 1, g, b, 1e-5, acc=orc.ACC_F32, dtype=odt))
             assert_close(got, want, HALF_RTOL, half_atol(want, bits), f"layernorm {name} {shape} {lname}")
+
+
+# ---- transposed views whose row blocks fit the register file: the single-pass kernel ----------
+# (base shape [cols, rows] viewed as [rows, cols]; the expected plan prefix pins the kernel)
+TILE_CASES = [
+    # name, numpy dtype / "bf16", base shape, perm, expected plan prefix
+    ("f32 rg8 one wavefront", np.float32, [40, 8192], [1, 0], "transposed-tile rows=8192 cols=40 vec=4 tpr=8 rpb=1 "),
+    ("f32 rg4 paired blocks", np.float32, [4096, 2048], [1, 0], "transposed-tile rows=2048 cols=4096 vec=4 tpr=4 rpb=16 "),
+    ("f16 ragged rows and cols", np.float16, [264, 16392], [1, 0], "transposed-tile rows=16392 cols=264 vec=8 tpr=8 rpb=3 "),
+    ("bf16 rg8", "bf16", [1000, 16384], [1, 0], "transposed-tile rows=16384 cols=1000 vec=8 tpr=8 rpb=8 "),
+    ("f64 rg4", np.float64, [3000, 1024], [1, 0], "transposed-tile rows=1024 cols=3000 vec=2 tpr=4 rpb=12 "),
+    ("f32 batched", np.float32, [3, 520, 2048], [0, 2, 1], "transposed-tile rows=6144 cols=520 vec=4 tpr=8 rpb=5 "),
+    ("f32 too many columns: three passes", np.float32, [4100, 2048], [1, 0], "transposed rows=2048 cols=4100 "),
+]
+
+
+@pytest.mark.parametrize("case", TILE_CASES, ids=[c[0] for c in TILE_CASES])
+def test_transposed_tile_softmax_layernorm(hpt, orc, dev, case):
+    name, npdt, shape, perm, plan = case
+    rng = np.random.default_rng(206)
+    x = (rng.standard_normal(shape) * 2 + rng.uniform(-3, 3, shape[:-1] + [1])).astype(np.float32)
+    if npdt == "bf16":
+        cv, dt, odt, bits, tof, acc = hpt.f32_to_bf16_bits, hpt.bf16, orc.BF16, 8, hpt.bf16_bits_to_f32, orc.ACC_F32
+    elif npdt == np.float16:
+        cv, dt, odt, bits, tof, acc = (lambda v: v.astype(np.float16)), None, None, 11, (lambda v: v.astype(np.float32)), orc.ACC_F32
+    else:
+        cv, dt, odt, bits, tof, acc = (lambda v: v.astype(npdt)), None, None, 0, (lambda v: v), orc.ACC_F64
+    base = cv(x)
+    t, a = upload(hpt, base, (("permute", tuple(perm)),), dtype=dt, dev=dev)
+    axis = a.ndim - 1
+    assert hpt.normalize_plan(t, axis).startswith(plan), hpt.normalize_plan(t, axis)
+    n = a.shape[-1]
+    g, b = cv(rng.normal(1, 0.1, n).astype(np.float32)), cv(rng.normal(0, 0.1, n).astype(np.float32))
+    tg, tb = hpt.Tensor.from_numpy(g, dt).to_hip(dev), hpt.Tensor.from_numpy(b, dt).to_hip(dev)
+
+    def check(got, want, what):
+        got, want = tof(got), tof(want)
+        if bits:
+            atol = half_atol(want, bits)
+            if npdt == np.float16:
+                atol = max(atol, 6e-8)
+            assert_close(got, want, HALF_RTOL, atol, f"{what} {name}")
+        else:
+            assert_close(got, want, F32_RTOL, 2e-6, f"{what} {name}")
+
+    check(t.softmax(axis).numpy(), orc.softmax(a, axis, acc=acc, dtype=odt), "softmax")
+    check(t.log_softmax(axis).numpy(), orc.softmax(a, axis, log=True, acc=acc, dtype=odt), "log_softmax")
+    check(t.layernorm([n], tg, tb, 1e-5).numpy(), orc.layernorm(a, 1, g, b, 1e-5, acc=acc, dtype=odt), "layernorm")
+    check(t.layernorm([n], None, None, 1e-5).numpy(), orc.layernorm(a, 1, None, None, 1e-5, acc=acc, dtype=odt),
+          "layernorm without gamma/beta")
+
+
+def test_transposed_tile_masked_and_constant_rows(hpt, dev):
+    """Closed forms through the single-pass kernel: a row with one finite entry -> one-hot; an all -inf
+    row -> NaN; constant rows -> beta exactly."""
+    base = np.full((96, 4096), -np.inf, np.float32)   # viewed as [4096 rows, 96 cols]
+    base[5, 0] = 2.0
+    base[:, 1] = np.arange(96)
+    base[95, 2] = -1.0
+    t = hpt.Tensor.from_numpy(base).to_hip(dev).permute([1, 0])
+    assert hpt.normalize_plan(t, 1).startswith("transposed-tile")
+    s = t.softmax(1).numpy()
+    assert s[0, 5] == 1.0 and s[0].sum() == 1.0
+    assert s[2, 95] == 1.0 and s[2].sum() == 1.0
+    assert np.all(np.isnan(s[3]))
+    e = np.exp(np.arange(96, dtype=np.float64) - 95)
+    assert_close(s[1], e / e.sum(), F32_RTOL, F32_ATOL, "dense row")
+    # (multiples of 1/4: the sum of a row is exact in f32, so the mean is too)
+    c = np.repeat((np.round(np.linspace(-4, 4, 4096) * 4) / 4).astype(np.float32)[None, :], 200, 0)   # [200 cols, 4096 rows]
+    g = np.linspace(0.5, 2, 200).astype(np.float32)
+    b = np.linspace(-1, 1, 200).astype(np.float32)
+    tc = hpt.Tensor.from_numpy(c).to_hip(dev).permute([1, 0])
+    assert hpt.normalize_plan(tc, 1).startswith("transposed-tile")
+    out = tc.layernorm([200], hpt.Tensor.from_numpy(g).to_hip(dev), hpt.Tensor.from_numpy(b).to_hip(dev), 1e-5).numpy()
+    assert np.array_equal(out, np.broadcast_to(b, out.shape))
