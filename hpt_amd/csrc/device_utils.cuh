@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -35,16 +36,11 @@ template <> struct DType<HPT_F64> { using type = double; };
 __device__ __forceinline__ float bf16_to_float(bf16_t h) {
     return __uint_as_float((uint32_t)h.bits << 16);
 }
-// round-to-nearest-even, NaN stays a quiet NaN
+// round-to-nearest-even, NaN stays a quiet NaN: gfx950 converts in hardware
+// (v_cvt_pk_bf16_f32, two values per instruction when neighbours are converted together)
 __device__ __forceinline__ bf16_t float_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
     bf16_t r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-        r.bits = (uint16_t)((u >> 16) | 0x0040u);
-    } else {
-        u += 0x7fffu + ((u >> 16) & 1u);
-        r.bits = (uint16_t)(u >> 16);
-    }
+    r.bits = __builtin_bit_cast(uint16_t, (__bf16)f);
     return r;
 }
 
@@ -162,6 +158,25 @@ __device__ __forceinline__ void store_pack_stream(T* p, const Pack<T, N>& v) {
     } else
 #endif
         store_pack<T, N>(p, v);
+}
+
+// ---- f16 data used straight from its packed registers ---------------------------
+// v_fma_mix_f32 reads a half out of either side of a 32-bit register and widens it
+// inside the multiply-add: (float)x * b + c costs one instruction instead of a
+// conversion plus the arithmetic, with the same single rounding. The compiler picks it
+// for fma(widened half, b, c) as long as it cannot fold the multiplication away, so
+// where b is 1 the caller passes a 1.0 the compiler cannot see through (opaque_one).
+__device__ __forceinline__ float opaque_one() {
+    float one = 1.0f;
+    asm volatile("" : "+v"(one));
+    return one;
+}
+
+// widen(x) * b + c for any element type; one instruction for f16.
+template <class T>
+__device__ __forceinline__ typename Elem<T>::Wide widen_fma(T x, typename Elem<T>::Wide b, typename Elem<T>::Wide c) {
+    if constexpr (std::is_same<T, f16_t>::value) return __builtin_fmaf((float)x, b, c);
+    else return Elem<T>::widen(x) * b + c;
 }
 
 // ---- index arithmetic -----------------------------------------------------

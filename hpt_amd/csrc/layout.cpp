@@ -375,7 +375,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 while (rgN >= 4 && cgroups * rgN > 1024) rgN >>= 1;
                 while (rgN > 8 && (R + rgN * v - 1) / (rgN * v) * batch < 256) rgN >>= 1;
                 const int64_t blocks = rgN >= 4 ? (R + rgN * v - 1) / (rgN * v) * batch : 0;
-                if (rgN >= 4 && blocks >= 128 && !getenv("HPT_NO_TILE")) {
+                if (rgN >= 4 && blocks >= 128) {
                     p.kind = NormKind::TransposedTile;
                     p.tpr = rgN;
                     const int64_t cols_per_wave = 16 * (64 / rgN);
@@ -392,8 +392,6 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             int64_t S = std::max<int64_t>(1, std::min<int64_t>((512 + groups - 1) / groups, p.cols / 128));
             p.tsplit = (int)std::min<int64_t>(S, 64);
             p.tpr = 4;  // wavefronts per workgroup of the statistics pass
-            if (const char* e = getenv("HPT_TSPLIT")) p.tsplit = atoi(e);
-            if (const char* e = getenv("HPT_TNW")) p.tpr = atoi(e);
             p.scratch_bytes = (size_t)p.rows * p.tsplit * 16 + (size_t)p.rows * 3 * 8;
             return p;
         }

@@ -134,30 +134,41 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
         }
     }
 
+    // Where registers allow (2-byte elements, few values per thread), the loads of the
+    // NEXT row this workgroup will take are issued before the current row's statistics
+    // and stores, so that the memory pipeline never drains between rows. With 4-byte
+    // elements the extra live registers cost more than the overlap gains (measured).
+    constexpr bool kPrefetch = sizeof(T) == 2 && NCHUNK * UV <= (kSoft ? 32 : 16);
     const int64_t row_step = (int64_t)gridDim.x * a.rpb;
+    Pack<T, VEC> raw[NCHUNK];
+    auto issue_loads = [&](int64_t row0) {
+        const int64_t row = row0 + ty;
+        if (row >= a.rows) return;
+        const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            const int iv = c * tpr + tx;
+            if (iv < nv) {
+                if constexpr (VEC > 1) raw[c] = load_pack_stream<T, VEC>(in_row + (int64_t)iv * VEC);
+                else raw[c].v[0] = in_row[(int64_t)iv * a.sa];
+            }
+        }
+    };
+    if constexpr (kPrefetch) issue_loads((int64_t)blockIdx.x * a.rpb);
     for (int64_t row0 = (int64_t)blockIdx.x * a.rpb; row0 < a.rows; row0 += row_step) {
+        if constexpr (!kPrefetch) issue_loads(row0);
         const int64_t row = row0 + ty;
         const bool valid = row < a.rows;
-        const T* in_row = (const T*)a.in + (valid ? offset_of(a.kept_in, row) : 0);
         T* out_row = (T*)a.out + (valid ? row * a.cols : 0);
 
         CT x[NCHUNK][UV];
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int iv = c * tpr + tx;
-            if (valid && iv < nv) {
-                if constexpr (VEC > 1) {
-                    Pack<T, VEC> v = load_pack_stream<T, VEC>(in_row + (int64_t)iv * VEC);
 #pragma unroll
-                    for (int j = 0; j < UV; ++j) x[c][j] = Elem<T>::widen(v.v[j * SS]);
-                } else {
-                    x[c][0] = Elem<T>::widen(in_row[(int64_t)iv * a.sa]);
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < UV; ++j) x[c][j] = fill;
-            }
+            for (int j = 0; j < UV; ++j) x[c][j] = (valid && iv < nv) ? Elem<T>::widen(raw[c].v[j * SS]) : fill;
         }
+        if constexpr (kPrefetch) issue_loads(row0 + row_step);
 
         if constexpr (kSoft) {
             CT m = neg_inf<CT>();

@@ -53,7 +53,7 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         t.eps = a.eps;
         t.inv_cols = a.inv_cols;
         t.rg_log2 = ilog2(p.tpr);
-        t.pair = p.tpr == 4;
+        t.share_log2 = p.tpr >= 8 ? 0 : (p.tpr == 4 ? 1 : 2);
         const unsigned blocks = (unsigned)((t.R + p.tpr * FULL - 1) / (p.tpr * FULL));
         transposed_tile_kernel<KIND, T><<<dim3(blocks, batch), dim3(64u * (unsigned)p.rpb), 0, st>>>(t);
         return;

@@ -309,10 +309,10 @@ __global__ void __launch_bounds__(256) transposed_apply_kernel(const TransposedA
 // (CGW = 64 / rgN). A load instruction therefore reads 16 * rgN contiguous bytes per
 // column; a store instruction writes, per row, VEC * CGW consecutive columns.
 //
-// With rgN = 4 a 128-byte line of the input is shared by two workgroups. Workgroups
-// are handed to the eight XCDs (each with its own L2) round-robin, so the row blocks
-// are renumbered to put both halves of a line on workgroups i and i + 8: same XCD,
-// dispatched together, and the second one hits in L2.
+// With rgN = 4 (2) a 128-byte line of the input is shared by two (four) workgroups.
+// Workgroups are handed to the eight XCDs (each with its own L2) round-robin, so the
+// row blocks are renumbered to put the parts of a line on workgroups i, i + 8, (i + 16,
+// i + 24): same XCD, dispatched together, and all but the first hit in L2.
 struct TileArgs {
     const void* in;
     void* out;
@@ -323,8 +323,8 @@ struct TileArgs {
     double eps, inv_cols;
     int R;       // rows per batch (contiguous in the input)
     int cols;
-    int rg_log2; // log2(rgN), rgN = 4, 8 or 16
-    int pair;    // 1: renumber row blocks so that line-sharing pairs meet on one XCD
+    int rg_log2; // log2(rgN), rgN = 2, 4, 8 or 16
+    int share_log2;  // log2 of the workgroups that share a 128-byte line of the input (0, 1 or 2)
 };
 
 // All-reduce of VEC row values over every thread that holds a piece of the same rows:
@@ -352,6 +352,25 @@ __device__ __forceinline__ void tile_all_reduce(A (&v)[VEC], int rgN, int rg, in
     __syncthreads();
 #pragma unroll
     for (int k = 0; k < VEC; ++k) v[k] = res[rg * VEC + k];
+}
+
+// The four pairs of halves of a Pack<f16_t, 8>.
+typedef f16_t half2_t __attribute__((ext_vector_type(2)));
+struct alignas(16) HalfPairs {
+    half2_t p[4];
+};
+
+// exp(x - m) of a tile element. f16: exp2(x * log2(e) - m * log2(e)) with the
+// scaling folded into the one multiply-add that also widens x (`nml` = -m * log2(e));
+// a row of -inf only still yields NaN (-inf + inf). Other types: as everywhere else.
+template <class T>
+__device__ __forceinline__ typename Elem<T>::Wide tile_exp(T x, typename Elem<T>::Wide m, typename Elem<T>::Wide nml) {
+    using CT = typename Elem<T>::Wide;
+    if constexpr (std::is_same<T, f16_t>::value) {
+        return __builtin_amdgcn_exp2f(widen_fma(x, (CT)1.4426950408889634, nml));
+    } else {
+        return exp_ct<T>(Elem<T>::widen(x) - m);
+    }
 }
 
 // Make the compiler forget what it knows about the tile's registers. Between two
@@ -384,9 +403,9 @@ __global__ void __launch_bounds__(1024) transposed_tile_kernel(const TileArgs a)
     const int rg = lane & (rgN - 1), cgl = lane >> a.rg_log2;
 
     int b = blockIdx.x;
-    if (a.pair && b < (int)(gridDim.x & ~15u)) {
+    if (a.share_log2 && b < (int)(gridDim.x & ~((8u << a.share_log2) - 1))) {
         const int x = b & 7, q = b >> 3;
-        b = ((x + 8 * (q >> 1)) << 1) | (q & 1);
+        b = ((x + 8 * (q >> a.share_log2)) << a.share_log2) | (q & ((1 << a.share_log2) - 1));
     }
     const int r0 = (b * rgN + rg) * VEC;
     const bool row_ok = r0 < a.R;
@@ -395,6 +414,8 @@ __global__ void __launch_bounds__(1024) transposed_tile_kernel(const TileArgs a)
     bool col_ok[H];
 #pragma unroll
     for (int h = 0; h < H; ++h) col_ok[h] = c_first + h * gw < a.cols;
+
+    const CT one = std::is_same<T, f16_t>::value ? (CT)opaque_one() : (CT)1;  // see widen_fma
 
     // Every thread loads 16 vectors, unconditionally: a thread whose rows or columns lie
     // outside the tensor reads row block 0 / column 0 instead (always there), and is
@@ -426,11 +447,16 @@ __global__ void __launch_bounds__(1024) transposed_tile_kernel(const TileArgs a)
         const T* bsrc = a.beta ? (const T*)a.beta + c : (const T*)a.in;
         gp = load_pack<T, VEC>(gsrc);
         bp = load_pack<T, VEC>(bsrc);
+        Pack<T, VEC> ones, zeros;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
-            gp.v[i] = a.gamma ? gp.v[i] : Elem<T>::narrow((CT)1);
-            bp.v[i] = a.beta ? bp.v[i] : Elem<T>::narrow((CT)0);
+            ones.v[i] = Elem<T>::narrow((CT)1);
+            zeros.v[i] = Elem<T>::narrow((CT)0);
         }
+        // chosen per 32-bit word, not per element
+        const u32x4 gw4 = __builtin_bit_cast(u32x4, gp), bw4 = __builtin_bit_cast(u32x4, bp);
+        gp = __builtin_bit_cast(Pack<T, VEC>, a.gamma ? gw4 : __builtin_bit_cast(u32x4, ones));
+        bp = __builtin_bit_cast(Pack<T, VEC>, a.beta ? bw4 : __builtin_bit_cast(u32x4, zeros));
     };
     if constexpr (kHoistAffine) {
 #pragma unroll
@@ -443,25 +469,52 @@ __global__ void __launch_bounds__(1024) transposed_tile_kernel(const TileArgs a)
         CT m[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) m[k] = neg_inf<CT>();
+        if constexpr (std::is_same<T, f16_t>::value) {
+            // a maximum is exact in any precision: take it on the packed halves, two rows
+            // per instruction, and widen the VEC results once
+            HalfPairs mp;
 #pragma unroll
-        for (int h = 0; h < H; ++h) {
-            CT mh[VEC];
+            for (int q = 0; q < 4; ++q) mp.p[q] = half2_t{(f16_t)-__builtin_huge_valf(), (f16_t)-__builtin_huge_valf()};
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) mh[k] = neg_inf<CT>();
+            for (int h = 0; h < H; ++h) {
+                HalfPairs mh = __builtin_bit_cast(HalfPairs, v[h * VEC]);
 #pragma unroll
-            for (int i = 0; i < VEC; ++i)
+                for (int i = 1; i < VEC; ++i) {
+                    const HalfPairs x = __builtin_bit_cast(HalfPairs, v[h * VEC + i]);
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) mh[k] = MaxC<CT>::comb(mh[k], Elem<T>::widen(v[h * VEC + i].v[k]));
-            if (col_ok[h]) {
+                    for (int q = 0; q < 4; ++q) mh.p[q] = __builtin_elementwise_max(mh.p[q], x.p[q]);
+                }
+                if (col_ok[h]) {
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) m[k] = MaxC<CT>::comb(m[k], mh[k]);
+                    for (int q = 0; q < 4; ++q) mp.p[q] = __builtin_elementwise_max(mp.p[q], mh.p[q]);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) m[k] = (CT)mp.p[k >> 1][k & 1];
+        } else {
+#pragma unroll
+            for (int h = 0; h < H; ++h) {
+                CT mh[VEC];
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) mh[k] = neg_inf<CT>();
+#pragma unroll
+                for (int i = 0; i < VEC; ++i)
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) mh[k] = MaxC<CT>::comb(mh[k], Elem<T>::widen(v[h * VEC + i].v[k]));
+                if (col_ok[h]) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) m[k] = MaxC<CT>::comb(m[k], mh[k]);
+                }
             }
         }
         forget_values(v);
         tile_all_reduce<MaxC<CT>, CT, VEC>(m, rgN, rg, cgl, w, nw, (CT*)part, (CT*)res);
-        CT s[VEC];
+        CT s[VEC], nml[VEC];
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) s[k] = 0;
+        for (int k = 0; k < VEC; ++k) {
+            s[k] = 0;
+            nml[k] = -m[k] * (CT)1.4426950408889634;  // -max * log2(e), see tile_exp
+        }
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             CT sh[VEC];
@@ -471,7 +524,7 @@ __global__ void __launch_bounds__(1024) transposed_tile_kernel(const TileArgs a)
             for (int i = 0; i < VEC; ++i)
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) {
-                    const CT e = exp_ct<T>(Elem<T>::widen(v[h * VEC + i].v[k]) - m[k]);
+                    const CT e = tile_exp<T>(v[h * VEC + i].v[k], m[k], nml[k]);
                     sh[k] += e;
                     if constexpr (kKeepExp && KIND == NORM_SOFTMAX) v[h * VEC + i].v[k] = Elem<T>::narrow(e);
                 }
@@ -486,7 +539,7 @@ __global__ void __launch_bounds__(1024) transposed_tile_kernel(const TileArgs a)
         for (int k = 0; k < VEC; ++k) {
             p0[k] = m[k];
             p1[k] = KIND == NORM_SOFTMAX ? (CT)1 / s[k] : log_ct<T>(s[k]);
-            p2[k] = 0;
+            p2[k] = nml[k];
         }
     } else {
         ST sum[VEC];
@@ -502,7 +555,7 @@ __global__ void __launch_bounds__(1024) transposed_tile_kernel(const TileArgs a)
 #pragma unroll
                 for (int i = 0; i < VEC; ++i)
 #pragma unroll
-                    for (int k = 0; k < VEC; ++k) th[k] += Elem<T>::widen(v[h * VEC + i].v[k]);
+                    for (int k = 0; k < VEC; ++k) th[k] = widen_fma(v[h * VEC + i].v[k], one, th[k]);
                 if (col_ok[h]) {
 #pragma unroll
                     for (int k = 0; k < VEC; ++k) t[k] += th[k];
@@ -536,7 +589,7 @@ __global__ void __launch_bounds__(1024) transposed_tile_kernel(const TileArgs a)
                 for (int i = 0; i < VEC; ++i)
 #pragma unroll
                     for (int k = 0; k < VEC; ++k) {
-                        CT d = Elem<T>::widen(v[h * VEC + i].v[k]) - p0[k];
+                        CT d = widen_fma(v[h * VEC + i].v[k], one, -p0[k]);
                         if constexpr (sizeof(ST) > sizeof(CT)) d -= p1[k];
                         th[k] += d * d;
                     }
@@ -589,16 +642,18 @@ __global__ void __launch_bounds__(1024) transposed_tile_kernel(const TileArgs a)
             Pack<T, VEC> o;
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
-                const CT x = Elem<T>::widen(v[h * VEC + i].v[k]);
+                // x - p0 (max or mean) first, in one step
+                const CT d = widen_fma(v[h * VEC + i].v[k], one, -p0[k]);
                 CT y;
                 if constexpr (KIND == NORM_LAYERNORM) {
-                    y = x - p0[k];
+                    y = d;
                     if constexpr (sizeof(ST) > sizeof(CT)) y -= p1[k];
                     y = y * p2[k] * g[i] + bt[i];
                 } else if constexpr (KIND == NORM_SOFTMAX) {
-                    y = (kKeepExp ? x : exp_ct<T>(x - p0[k])) * p1[k];
+                    if constexpr (kKeepExp) y = Elem<T>::widen(v[h * VEC + i].v[k]) * p1[k];
+                    else y = tile_exp<T>(v[h * VEC + i].v[k], p0[k], p2[k]) * p1[k];
                 } else {
-                    y = (x - p0[k]) - p1[k];
+                    y = d - p1[k];
                 }
                 o.v[i] = Elem<T>::narrow(y);
             }
