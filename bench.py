@@ -245,13 +245,48 @@ def cases_c5(P):
     return cases
 
 
+def cases_c6(P):
+    """The steps either side of the path at the headline / C5 shapes: contiguous() of the C5 views, the
+    affine steps of layernorm as separate in-place passes, full()."""
+    import hpt_amd as hpt
+    l, check, ffi = P.l, P.ffi.check, P.ffi
+    rng = np.random.default_rng(6)
+    c5 = (rng.standard_normal((4096, 8192), dtype=np.float32) * 2).astype(np.float16)
+    c5s = [hpt.Tensor.from_numpy(np.roll(c5, k, 0)).to_hip(0) for k in range(6)]
+    n5 = c5.nbytes
+    cases = []
+
+    def copy_case(name, cfg, views, algo):
+        outs = [hpt.Tensor.empty(v.shape, v.dtype, 0) for v in views]
+        vi, vo = [P.view(v) for v in views], [P.view(o) for o in outs]
+        n = len(views)
+        run = lambda i: check(l.hpt_hip_contiguous(0, None, vi[i % n], vo[i % n]))
+        cases.append(Case(name, cfg, "f16", views[0].shape[0], algo, run, n))
+
+    copy_case("contiguous", "C5a f16 [4096,8192].permute(1,0)", [t.permute([1, 0]) for t in c5s], 2 * n5)
+    copy_case("contiguous", "C5b f16 [4096,8192][:, ::2]", [t[:, ::2] for t in c5s], n5)
+    copy_case("contiguous", "f16 [4096,8192][:, 1024:5120] (row segments)", [t[:, 1024:5120] for t in c5s], n5)
+    x = rng.standard_normal((8192, 4096), dtype=np.float32)
+    g = rng.normal(1, 0.1, 4096).astype(np.float32)
+    xs = [hpt.Tensor.from_numpy(np.roll(x, k, 0)).to_hip(0) for k in range(4)]
+    tg = hpt.Tensor.from_numpy(g).to_hip(0).expand([8192, 4096])
+    vx, vg = [P.view(t) for t in xs], P.view(tg)
+    run = lambda i: check(l.hpt_hip_binary(0, None, hpt.BIN_MUL, vx[i % 4], vg, vx[i % 4]))
+    cases.append(Case("mul_(gamma) in place", "C2 f32 [8192,4096] * [4096]", "f32", 8192, 2 * x.nbytes + g.nbytes, run, 4))
+    one = np.array([1.5], np.float32)
+    P.keep.append(one)
+    run = lambda i: check(l.hpt_hip_fill(0, None, vx[i % 4], one.ctypes.data))
+    cases.append(Case("full", "C2 f32 [8192,4096]", "f32", 8192, x.nbytes, run, 4))
+    return cases
+
+
 def build_cases(which: str, configs=None):
     """Synthetic inputs of the benchmark configurations, uploaded once; outputs preallocated.
     The headline (C2 layernorm) is always first; `configs` limits the others (e.g. {"c3"})."""
     P = Prepared()
     cases, head = cases_c2(P, which == "headline")
     if which != "headline":
-        for name, fn in (("c1", cases_c1), ("c3", cases_c3), ("c4", cases_c4), ("c5", cases_c5)):
+        for name, fn in (("c1", cases_c1), ("c3", cases_c3), ("c4", cases_c4), ("c5", cases_c5), ("c6", cases_c6)):
             if configs is None or name in configs:
                 cases += fn(P)
     return cases, P, head
@@ -296,7 +331,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--ops", choices=["all", "headline"], default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--configs", default="", help="comma list of c1,c3,c4,c5 to measure besides the headline")
+    ap.add_argument("--configs", default="", help="comma list of c1,c3,c4,c5,c6 to measure besides the headline (c6 = the steps either side: contiguous / in-place affine / full)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region, run one plain device-to-device copy of the headline input "
                          "(134217728 bytes read + as many written): the known-size dispatch that hardware "

@@ -36,7 +36,8 @@ N_NORM_KINDS = 3
 
 def units():
     """(object name, source, extra flags)"""
-    u = [("layout.o", CSRC / "layout.cpp", ["-x", "hip"]), ("api.o", CSRC / "api.hip", [])]
+    u = [("layout.o", CSRC / "layout.cpp", ["-x", "hip"]), ("api.o", CSRC / "api.hip", []),
+         ("elementwise.o", CSRC / "elementwise.hip", [])]
     for e in range(N_REDUCE_ENTRIES):
         u.append((f"reduce_op_{e}.o", CSRC / "reduce_op.hip", [f"-DHPT_REDUCE_ENTRY={e}"]))
     for k in range(N_NORM_KINDS):

@@ -10,6 +10,7 @@
 #include <vector>
 
 #include "common.hpp"
+#include "elementwise_entry.hpp"
 #include "norm_entry.hpp"
 #include "reduce_entry.hpp"
 
@@ -621,6 +622,95 @@ int32_t hpt_hip_layernorm(int32_t dev, void* stream, const hpt_view* in, int32_t
         if (!fn) fail(HPT_ERR_DTYPE, "layernorm: unsupported dtype %s", dtype_name(in->dtype));
         use_device(dev);
         launch_norm(dev, (hipStream_t)stream, fn, c, "layernorm");
+    });
+}
+
+// ---- the steps either side of the path ------------------------------------------------
+
+static void check_same_shape(const hpt_view* a, const hpt_view* b, const char* what) {
+    bool same = a->ndim == b->ndim;
+    for (int i = 0; same && i < a->ndim; ++i) same = a->shape[i] == b->shape[i];
+    if (!same) fail(HPT_ERR_SHAPE, "%s: shapes differ", what);
+}
+
+static EwPlan prepare_copy(const hpt_view* in, const hpt_view* out) {
+    check_view(in, "contiguous input", true);
+    check_out(out, in->dtype, view_size(in), "contiguous output");
+    check_same_shape(in, out, "contiguous");
+    const void* datas[1] = {in->data};
+    const int64_t* strides[1] = {in->strides};
+    return plan_elementwise(out->data, in->shape, in->ndim, 1, datas, strides, dtype_size(in->dtype), true);
+}
+
+int32_t hpt_hip_contiguous(int32_t dev, void* stream, const hpt_view* in, hpt_view* out) {
+    return guarded([&] {
+        const EwPlan p = prepare_copy(in, out);
+        if (p.kind == EwKind::Empty) return;
+        use_device(dev);
+        launch_strided_copy(in->dtype, p, out->data, in->data, (hipStream_t)stream);
+        check_launch("contiguous");
+    });
+}
+
+int32_t hpt_hip_contiguous_plan(const hpt_view* in, const hpt_view* out, char* buf, size_t buflen) {
+    return guarded([&] {
+        if (!buf || !buflen) fail(HPT_ERR_PARAM, "contiguous_plan: no buffer");
+        snprintf(buf, buflen, "%s", describe(prepare_copy(in, out)).c_str());
+    });
+}
+
+int32_t hpt_hip_fill(int32_t dev, void* stream, hpt_view* out, const void* value) {
+    return guarded([&] {
+        check_view(out, "fill output", true);
+        if (!view_contiguous(out)) fail(HPT_ERR_SHAPE, "fill output: output tensor must be contiguous");
+        if (!value) fail(HPT_ERR_PARAM, "fill: value pointer is null");
+        const int64_t n = view_size(out);
+        if (n == 0) return;
+        use_device(dev);
+        launch_fill(out->dtype, out->data, n, value, (hipStream_t)stream);
+        check_launch("fill");
+    });
+}
+
+int32_t hpt_hip_binary(int32_t dev, void* stream, int32_t op, const hpt_view* lhs, const hpt_view* rhs,
+                       hpt_view* out) {
+    return guarded([&] {
+        check_view(lhs, "binary lhs", true);
+        check_view(rhs, "binary rhs", true);
+        if (lhs->dtype != rhs->dtype)
+            fail(HPT_ERR_DTYPE, "binary: operands must share one dtype, got %s and %s", dtype_name(lhs->dtype),
+                 dtype_name(rhs->dtype));
+        check_out(out, lhs->dtype, view_size(lhs), "binary output");
+        check_same_shape(lhs, out, "binary lhs / out");
+        check_same_shape(rhs, out, "binary rhs / out");
+        // The output may be one of the operands (in place) but must not overlap one otherwise:
+        // every element is read before it is written only when the two walk the same addresses.
+        const size_t es = dtype_size(out->dtype);
+        const char* ob = (const char*)out->data;
+        const char* oe = ob + view_size(out) * es;
+        const hpt_view* ops[2] = {lhs, rhs};
+        for (const hpt_view* v : ops) {
+            // extent of the operand in memory
+            int64_t lo = 0, hi = 0;
+            for (int i = 0; i < v->ndim; ++i) {
+                const int64_t span = (v->shape[i] - 1) * v->strides[i];
+                if (span < 0) lo += span;
+                else hi += span;
+            }
+            const char* vb = (const char*)v->data + lo * (int64_t)es;
+            const char* ve = (const char*)v->data + (hi + 1) * (int64_t)es;
+            const bool overlap = view_size(out) > 0 && vb < oe && ob < ve;
+            const bool same = v->data == out->data && view_contiguous(v);
+            if (overlap && !same)
+                fail(HPT_ERR_PARAM, "binary: out overlaps an operand without being that operand");
+        }
+        const void* datas[2] = {lhs->data, rhs->data};
+        const int64_t* strides[2] = {lhs->strides, rhs->strides};
+        const EwPlan p = plan_elementwise(out->data, out->shape, out->ndim, 2, datas, strides, es, false);
+        if (p.kind == EwKind::Empty) return;
+        use_device(dev);
+        launch_binary(op, out->dtype, p, out->data, lhs->data, rhs->data, (hipStream_t)stream);
+        check_launch("binary");
     });
 }
 

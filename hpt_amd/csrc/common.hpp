@@ -142,4 +142,32 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
 
 std::string describe(const NormPlan& p);
 
+// ---- elementwise: strided copy (contiguous()), fill, binary ops with broadcasting ----
+
+enum class EwKind {
+    Empty,
+    Inner,      // lanes walk the innermost coalesced dim (vectors where every operand allows them)
+    Transpose   // copy only: some other dim is the contiguous one in the input: register-tile transpose
+};
+
+// The output is contiguous over `size[0..n)`; `stride[k][i]` is operand k's stride (in
+// elements, 0 = broadcast) along dim i. Dims are coalesced across all operands at once.
+struct EwPlan {
+    EwKind kind = EwKind::Empty;
+    int n = 0;     // coalesced dims
+    int nin = 0;   // input operands (1 or 2)
+    int64_t size[kMaxDims] = {};
+    int64_t stride[2][kMaxDims] = {};
+    int64_t total = 0;
+    int vec = 1;   // output elements per thread along the innermost dim
+    int sstride = 1;  // 2: (copy) the innermost input stride is 2: full vectors in, every second element kept
+    // Transpose: dim `tdim` has input stride 1; the innermost dim is strided in the input
+    int tdim = -1;
+};
+
+EwPlan plan_elementwise(const void* out_data, const int64_t* shape, int ndim, int nin, const void* const* in_data,
+                        const int64_t* const* in_strides, size_t elem_size, bool allow_transpose);
+
+std::string describe(const EwPlan& p);
+
 }  // namespace hpt

@@ -1,0 +1,343 @@
+// The steps either side of the reduction / normalisation path, on device:
+//   strided copy   `contiguous()` of any view (hpt-cudakernels/src/strided_copy.cu:6-14,
+//                  hpt/src/backends/cuda/tensor_internal/normal_out_unary.rs:286-310)
+//   fill           `set_val` (hpt-cudakernels/src/set_val.cu:4-12)
+//   add/sub/mul/div with broadcasting, also in place: the `add_` / `mul_` that layernorm's
+//                  single-affine branches use (hpt/src/backends/cpu/tensor_internal/
+//                  normalization.rs:187-192; trait hpt-traits/src/ops/binary.rs:9-152)
+// All are HBM-bound: the work is in keeping both sides of the copy on whole cache lines.
+#include <cstring>
+
+#include "device_utils.cuh"
+#include "elementwise_entry.hpp"
+
+namespace hpt {
+
+namespace {
+
+struct EwArgs {
+    void* out;
+    const void* in[2];
+    int64_t stride[2][kMaxDims];
+    int size[kMaxDims];
+    int n;
+    int64_t total_v;  // vectors (of VEC output elements) in all
+    int inner_v;      // vectors along the innermost dim
+};
+
+// ---- operators ---------------------------------------------------------------------
+// Integers wrap (hpt-types/src/scalars/impls.rs:31-48); bool add is OR and mul is AND;
+// f16 / bf16 widen to f32, operate, round once (what the `half` crate does per operation).
+template <int OP, class T> struct BinOp {
+    __device__ static __forceinline__ T apply(T x, T y) {
+        if constexpr (Elem<T>::is_bool) {
+            const bool a = x.v != 0, b = y.v != 0;
+            return bool8{(uint8_t)(OP == EW_ADD ? (a || b) : (a && b))};
+        } else {
+            using W = typename Elem<T>::Wide;
+            const W a = Elem<T>::widen(x), b = Elem<T>::widen(y);
+            W r;
+            if constexpr (OP == EW_ADD) r = a + b;
+            else if constexpr (OP == EW_SUB) r = a - b;
+            else if constexpr (OP == EW_MUL) r = a * b;
+            else r = a / b;
+            return Elem<T>::narrow(r);
+        }
+    }
+};
+
+// ---- lanes along the innermost dim ---------------------------------------------------
+// Thread t of a workgroup takes vectors t, t + 256, t + 512, t + 768 of the workgroup's
+// 1024: four loads per operand are in flight before the first result is stored.
+// SS = 2 (copy only): the innermost dim has input stride 2 (a [:, ::2] view): two full
+// vectors are loaded per output vector and the odd positions dropped, which moves the same
+// cache lines as a gather of single elements with a fraction of the instructions. (A
+// 16-byte aligned vector that holds one valid element never leaves that element's page, so
+// the unused last element of the last vector is safe to touch.)
+template <int OP, class T, int VEC, int NIN, int SS = 1>
+__global__ void __launch_bounds__(256) ew_inner_kernel(const EwArgs a) {
+    constexpr int UNR = 4;
+    Pack<T, VEC> x[UNR], y[UNR];
+    int64_t vi[UNR];
+    const int last = a.n - 1;
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+        const int64_t v = ((int64_t)blockIdx.x * UNR + u) * 256 + threadIdx.x;
+        vi[u] = v;
+        if (v >= a.total_v) continue;
+        // innermost position and the operands' offsets of the outer position
+        int64_t off[2] = {0, 0};
+        int64_t iv;
+        if (((uint64_t)a.total_v >> 31) == 0) {
+            uint32_t r = (uint32_t)v;
+            uint32_t q = r / (uint32_t)a.inner_v;
+            iv = r - q * (uint32_t)a.inner_v;
+            for (int i = last - 1; i >= 0; --i) {
+                const uint32_t s = (uint32_t)a.size[i];
+                const uint32_t q2 = q / s;
+                const uint32_t idx = q - q2 * s;
+                q = q2;
+#pragma unroll
+                for (int k = 0; k < NIN; ++k) off[k] += (int64_t)idx * a.stride[k][i];
+            }
+        } else {
+            int64_t q = v / a.inner_v;
+            iv = v - q * a.inner_v;
+            for (int i = last - 1; i >= 0; --i) {
+                const int64_t q2 = q / a.size[i];
+                const int64_t idx = q - q2 * a.size[i];
+                q = q2;
+#pragma unroll
+                for (int k = 0; k < NIN; ++k) off[k] += idx * a.stride[k][i];
+            }
+        }
+        auto fetch = [&](int k, Pack<T, VEC>& dst) {
+            const T* p = (const T*)a.in[k] + off[k];
+            const int64_t s = a.stride[k][last];
+            if constexpr (SS == 2) {
+                const Pack<T, VEC> lo = load_pack_stream<T, VEC>(p + iv * (2 * VEC));
+                const Pack<T, VEC> hi = load_pack_stream<T, VEC>(p + iv * (2 * VEC) + VEC);
+#pragma unroll
+                for (int j = 0; j < VEC / 2; ++j) {
+                    dst.v[j] = lo.v[2 * j];
+                    dst.v[VEC / 2 + j] = hi.v[2 * j];
+                }
+            } else if constexpr (VEC > 1) {
+                if (s == 1) {
+                    dst = load_pack_stream<T, VEC>(p + iv * VEC);
+                } else {  // broadcast along the innermost dim
+                    const T e = *p;
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) dst.v[j] = e;
+                }
+            } else {
+                dst.v[0] = p[iv * s];
+            }
+        };
+        fetch(0, x[u]);
+        if constexpr (NIN == 2) fetch(1, y[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+        if (vi[u] >= a.total_v) continue;
+        Pack<T, VEC> r;
+        if constexpr (NIN == 2) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) r.v[j] = BinOp<OP, T>::apply(x[u].v[j], y[u].v[j]);
+        } else {
+            r = x[u];
+        }
+        T* o = (T*)a.out + vi[u] * VEC;
+        if constexpr (VEC > 1) store_pack_stream<T, VEC>(o, r);
+        else *o = r.v[0];
+    }
+}
+
+// ---- copy of a view whose contiguous dim is not the innermost one ------------------------
+// Dim B (size nB) is contiguous in the input, dim A (the innermost of the output, size nA)
+// has input stride sA. A wavefront moves an (8 VEC along B) x (8 VEC along A) tile: lane
+// (rg, cl) loads VEC vectors of VEC consecutive B positions (one per A position) and stores
+// VEC vectors of VEC consecutive A positions. Both sides move whole 128-byte lines; the
+// transpose itself is a renaming of registers. The other dims ride on blockIdx.z.
+struct TransposeArgs {
+    const void* in;
+    void* out;
+    int64_t sA;         // input stride of A (elements)
+    int64_t oB;         // output stride of B
+    int nA, nB;
+    int nother;
+    int osize[kMaxDims];
+    int64_t oin[kMaxDims], oout[kMaxDims];  // strides of the other dims in input / output
+};
+
+template <class U>
+__global__ void __launch_bounds__(256) ew_transpose_kernel(const TransposeArgs a) {
+    constexpr int VEC = 16 / sizeof(U);
+    constexpr int TB = 8 * VEC, TA = 8 * VEC;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int rg = lane & 7, cl = lane >> 3;
+    // neighbouring workgroups take neighbouring B tiles: their reads are adjacent in memory
+    const int b0 = blockIdx.x * TB + rg * VEC;
+    const int a0 = (blockIdx.y * 4 + w) * TA + cl * VEC;
+    if (b0 >= a.nB || a0 >= a.nA) return;
+    int64_t ioff = 0, ooff = 0;
+    {
+        uint32_t q = blockIdx.z;
+        for (int i = a.nother - 1; i >= 0; --i) {
+            const uint32_t s = (uint32_t)a.osize[i];
+            const uint32_t q2 = q / s;
+            const uint32_t idx = q - q2 * s;
+            q = q2;
+            ioff += (int64_t)idx * a.oin[i];
+            ooff += (int64_t)idx * a.oout[i];
+        }
+    }
+    const U* in = (const U*)a.in + ioff + b0;
+    Pack<U, VEC> v[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = load_pack_stream<U, VEC>(in + (int64_t)(a0 + i) * a.sA);
+    U* out = (U*)a.out + ooff + (int64_t)b0 * a.oB + a0;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        Pack<U, VEC> o;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) o.v[i] = v[i].v[k];
+        store_pack_stream<U, VEC>(out + (int64_t)k * a.oB, o);
+    }
+}
+
+// ---- fill -----------------------------------------------------------------------------
+// `pattern` holds the element replicated over 16 bytes.
+__global__ void __launch_bounds__(256) fill_vec_kernel(u32x4* out, u32x4 pattern, int64_t nvec) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < nvec) __builtin_nontemporal_store(pattern, out + i);
+}
+template <class U> __global__ void __launch_bounds__(256) fill_scalar_kernel(U* out, U value, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = value;
+}
+
+EwArgs make_args(const EwPlan& p, void* out, const void* in0, const void* in1) {
+    EwArgs a{};
+    a.out = out;
+    a.in[0] = in0;
+    a.in[1] = in1;
+    a.n = p.n;
+    for (int i = 0; i < p.n; ++i) {
+        a.size[i] = (int)p.size[i];
+        for (int k = 0; k < p.nin; ++k) a.stride[k][i] = p.stride[k][i];
+    }
+    a.inner_v = (int)(p.size[p.n - 1] / p.vec);
+    a.total_v = p.total / p.vec;
+    return a;
+}
+
+template <int OP, class T, int NIN>
+void launch_inner(const EwPlan& p, void* out, const void* in0, const void* in1, hipStream_t st) {
+    constexpr int FULL = 16 / sizeof(T);
+    const EwArgs a = make_args(p, out, in0, in1);
+    const int64_t blocks = (a.total_v + 1023) / 1024;
+    if (blocks > 0x7fffffff) fail(HPT_ERR_SHAPE, "elementwise: tensor too large for one launch");
+    if constexpr (NIN == 1 && FULL > 1) {
+        if (p.vec == FULL && p.sstride == 2) {
+            ew_inner_kernel<OP, T, FULL, NIN, 2><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a);
+            return;
+        }
+    }
+    if (p.vec == FULL && FULL > 1) ew_inner_kernel<OP, T, FULL, NIN><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a);
+    else ew_inner_kernel<OP, T, 1, NIN><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a);
+}
+
+template <class U> void launch_transpose(const EwPlan& p, void* out, const void* in, hipStream_t st) {
+    constexpr int VEC = 16 / sizeof(U);
+    TransposeArgs t{};
+    const int last = p.n - 1;
+    t.in = in;
+    t.out = out;
+    t.nA = (int)p.size[last];
+    t.sA = p.stride[0][last];
+    t.nB = (int)p.size[p.tdim];
+    int64_t ostride[kMaxDims];
+    int64_t acc = 1;
+    for (int i = last; i >= 0; --i) {
+        ostride[i] = acc;
+        acc *= p.size[i];
+    }
+    t.oB = ostride[p.tdim];
+    int64_t others = 1;
+    for (int i = 0; i < p.n; ++i) {
+        if (i == p.tdim || i == last) continue;
+        t.osize[t.nother] = (int)p.size[i];
+        t.oin[t.nother] = p.stride[0][i];
+        t.oout[t.nother] = ostride[i];
+        ++t.nother;
+        others *= p.size[i];
+    }
+    constexpr int TILE = 8 * VEC;
+    dim3 grid((unsigned)((t.nB + TILE - 1) / TILE), (unsigned)((t.nA + 4 * TILE - 1) / (4 * TILE)), (unsigned)others);
+    if (grid.y > 65535) fail(HPT_ERR_SHAPE, "strided copy: innermost dim too long for the transposing kernel");
+    ew_transpose_kernel<U><<<grid, dim3(256), 0, st>>>(t);
+}
+
+template <class U> void launch_copy_sized(const EwPlan& p, void* out, const void* in, hipStream_t st) {
+    if (p.kind == EwKind::Transpose) launch_transpose<U>(p, out, in, st);
+    else launch_inner<EW_COPY, U, 1>(p, out, in, nullptr, st);
+}
+
+template <int OP> void launch_binary_op(int dtype, const EwPlan& p, void* out, const void* a, const void* b, hipStream_t st) {
+    switch (dtype) {
+#define HPT_CASE(DT)                                                                 \
+    case DT:                                                                         \
+        launch_inner<OP, typename DType<DT>::type, 2>(p, out, a, b, st);             \
+        return;
+        HPT_CASE(HPT_I8) HPT_CASE(HPT_I16) HPT_CASE(HPT_I32) HPT_CASE(HPT_I64) HPT_CASE(HPT_U8) HPT_CASE(HPT_U16)
+        HPT_CASE(HPT_U32) HPT_CASE(HPT_U64) HPT_CASE(HPT_F16) HPT_CASE(HPT_BF16) HPT_CASE(HPT_F32) HPT_CASE(HPT_F64)
+#undef HPT_CASE
+        case HPT_BOOL:
+            if constexpr (OP == EW_ADD || OP == EW_MUL) {
+                launch_inner<OP, bool8, 2>(p, out, a, b, st);
+                return;
+            }
+            break;
+        default: break;
+    }
+    fail(HPT_ERR_DTYPE, "binary: unsupported dtype %s for this operator", dtype_name(dtype));
+}
+
+}  // namespace
+
+void launch_strided_copy(int dtype, const EwPlan& p, void* out, const void* in, hipStream_t st) {
+    if (p.kind == EwKind::Empty) return;
+    switch (dtype_size(dtype)) {
+        case 1: launch_copy_sized<uint8_t>(p, out, in, st); break;
+        case 2: launch_copy_sized<uint16_t>(p, out, in, st); break;
+        case 4: launch_copy_sized<uint32_t>(p, out, in, st); break;
+        case 8: launch_copy_sized<uint64_t>(p, out, in, st); break;
+        default: fail(HPT_ERR_DTYPE, "strided copy: invalid dtype %d", dtype);
+    }
+}
+
+void launch_binary(int op, int dtype, const EwPlan& p, void* out, const void* a, const void* b, hipStream_t st) {
+    if (p.kind == EwKind::Empty) return;
+    const bool is_float = dtype == HPT_F16 || dtype == HPT_BF16 || dtype == HPT_F32 || dtype == HPT_F64;
+    switch (op) {
+        case EW_ADD: launch_binary_op<EW_ADD>(dtype, p, out, a, b, st); break;
+        case EW_SUB: launch_binary_op<EW_SUB>(dtype, p, out, a, b, st); break;
+        case EW_MUL: launch_binary_op<EW_MUL>(dtype, p, out, a, b, st); break;
+        case EW_DIV:
+            // integer division promotes to a float type in Hpt (a different output dtype): not provided
+            if (!is_float) fail(HPT_ERR_DTYPE, "binary: div is provided for float dtypes only, got %s", dtype_name(dtype));
+            launch_binary_op<EW_DIV>(dtype, p, out, a, b, st);
+            break;
+        default: fail(HPT_ERR_PARAM, "binary: unknown operator %d", op);
+    }
+}
+
+void launch_fill(int dtype, void* out, int64_t n, const void* value, hipStream_t st) {
+    if (n == 0) return;
+    const size_t es = dtype_size(dtype);
+    unsigned char pat[16];
+    for (size_t i = 0; i < 16; ++i) pat[i] = ((const unsigned char*)value)[i % es];
+    unsigned char* p = (unsigned char*)out;
+    int64_t done = 0;
+    if (((uintptr_t)p % 16) == 0 && n * (int64_t)es >= 16) {
+        const int64_t nvec = n * (int64_t)es / 16;
+        u32x4 pattern;
+        memcpy(&pattern, pat, 16);
+        fill_vec_kernel<<<dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0, st>>>((u32x4*)p, pattern, nvec);
+        done = nvec * 16 / (int64_t)es;
+    }
+    const int64_t rest = n - done;
+    if (rest > 0) {
+        const unsigned blocks = (unsigned)((rest + 255) / 256);
+        unsigned char* q = p + done * es;
+        switch (es) {
+            case 1: { uint8_t v; memcpy(&v, value, 1); fill_scalar_kernel<uint8_t><<<blocks, 256, 0, st>>>((uint8_t*)q, v, rest); break; }
+            case 2: { uint16_t v; memcpy(&v, value, 2); fill_scalar_kernel<uint16_t><<<blocks, 256, 0, st>>>((uint16_t*)q, v, rest); break; }
+            case 4: { uint32_t v; memcpy(&v, value, 4); fill_scalar_kernel<uint32_t><<<blocks, 256, 0, st>>>((uint32_t*)q, v, rest); break; }
+            default: { uint64_t v; memcpy(&v, value, 8); fill_scalar_kernel<uint64_t><<<blocks, 256, 0, st>>>((uint64_t*)q, v, rest); break; }
+        }
+    }
+}
+
+}  // namespace hpt

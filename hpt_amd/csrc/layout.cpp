@@ -463,4 +463,119 @@ std::string describe(const NormPlan& p) {
     return s;
 }
 
+// ---- elementwise ------------------------------------------------------------------
+
+EwPlan plan_elementwise(const void* out_data, const int64_t* shape, int ndim, int nin, const void* const* in_data,
+                        const int64_t* const* in_strides, size_t elem_size, bool allow_transpose) {
+    EwPlan p;
+    p.nin = nin;
+    p.total = 1;
+    for (int i = 0; i < ndim; ++i) p.total *= shape[i];
+    if (p.total == 0) return p;
+    // coalesce: drop size-1 dims; merge dim i into i+1 when every operand (and the
+    // contiguous output, which always can) steps over dim i+1 exactly once per step of i
+    for (int i = 0; i < ndim; ++i) {
+        if (shape[i] == 1) continue;
+        bool merge = p.n > 0;
+        if (merge) {
+            for (int k = 0; k < nin; ++k)
+                if (p.stride[k][p.n - 1] != in_strides[k][i] * shape[i]) merge = false;
+        }
+        if (merge) {
+            p.size[p.n - 1] *= shape[i];
+            for (int k = 0; k < nin; ++k) p.stride[k][p.n - 1] = in_strides[k][i];
+        } else {
+            if (p.n == kMaxDims)
+                fail(HPT_ERR_SHAPE, "elementwise: the view does not coalesce to %d dims or fewer", kMaxDims);
+            p.size[p.n] = shape[i];
+            for (int k = 0; k < nin; ++k) p.stride[k][p.n] = in_strides[k][i];
+            ++p.n;
+        }
+    }
+    if (p.n == 0) {  // a single element
+        p.n = 1;
+        p.size[0] = 1;
+        for (int k = 0; k < nin; ++k) p.stride[k][0] = 1;
+    }
+    for (int i = 0; i < p.n; ++i)
+        if (p.size[i] > 0x7fffffff) fail(HPT_ERR_SHAPE, "elementwise: a coalesced dim exceeds 2^31 - 1 elements");
+    p.kind = EwKind::Inner;
+    const int full = (int)(16 / elem_size);
+    const int last = p.n - 1;
+    auto aligned = [&](const void* ptr) { return ((uintptr_t)ptr % 16) == 0; };
+    // vectors along the innermost dim: every operand is either contiguous there (stride 1,
+    // with 16-byte aligned base and outer strides) or broadcast there (stride 0)
+    bool vec_ok = full > 1 && p.size[last] % full == 0 && aligned(out_data);
+    for (int k = 0; k < nin && vec_ok; ++k) {
+        const int64_t s = p.stride[k][last];
+        if (s == 1) {
+            if (!aligned(in_data[k])) vec_ok = false;
+            for (int i = 0; i < last; ++i)
+                if (p.stride[k][i] % full != 0) vec_ok = false;
+        } else if (s != 0) {
+            vec_ok = false;
+        }
+    }
+    if (vec_ok) {
+        p.vec = full;
+        return p;
+    }
+    // copy of a view whose innermost stride is 2: full vectors in, the even positions kept
+    if (nin == 1 && full > 1 && p.stride[0][last] == 2 && p.size[last] % full == 0 && aligned(out_data) &&
+        aligned(in_data[0])) {
+        bool ok = true;
+        for (int i = 0; i < last; ++i)
+            if (p.stride[0][i] % full != 0) ok = false;
+        if (ok) {
+            p.vec = full;
+            p.sstride = 2;
+            return p;
+        }
+    }
+    // copy of a view whose contiguous dim is not the innermost one: transpose in registers
+    if (allow_transpose && nin == 1 && full > 1 && p.stride[0][last] != 1 && p.stride[0][last] != 0) {
+        int t = -1;
+        for (int i = 0; i < last; ++i)
+            if (p.stride[0][i] == 1) t = i;
+        if (t >= 0 && p.n <= 6) {
+            bool ok = aligned(out_data) && aligned(in_data[0]) && p.size[last] % full == 0 && p.size[t] % full == 0 &&
+                      p.size[last] >= 2 * full && p.size[t] >= 2 * full;
+            for (int i = 0; i < p.n; ++i)
+                if (i != t && p.stride[0][i] % full != 0) ok = false;
+            // the remaining dims ride on blockIdx.z
+            int64_t others = 1;
+            for (int i = 0; i < p.n; ++i)
+                if (i != t && i != last) others *= p.size[i];
+            if (ok && others <= 65535) {
+                p.kind = EwKind::Transpose;
+                p.vec = full;
+                p.tdim = t;
+            }
+        }
+    }
+    return p;
+}
+
+std::string describe(const EwPlan& p) {
+    static const char* names[] = {"empty", "inner", "transpose"};
+    char buf[128];
+    snprintf(buf, sizeof buf, "%s%s vec=%d total=%lld dims=[", names[(int)p.kind], p.sstride == 2 ? "-step2" : "", p.vec,
+             (long long)p.total);
+    std::string s = buf;
+    for (int i = 0; i < p.n; ++i) {
+        snprintf(buf, sizeof buf, "%s%lld:", i ? "," : "", (long long)p.size[i]);
+        s += buf;
+        for (int k = 0; k < p.nin; ++k) {
+            snprintf(buf, sizeof buf, "%s%lld", k ? "/" : "", (long long)p.stride[k][i]);
+            s += buf;
+        }
+    }
+    s += "]";
+    if (p.kind == EwKind::Transpose) {
+        snprintf(buf, sizeof buf, " tdim=%d", p.tdim);
+        s += buf;
+    }
+    return s;
+}
+
 }  // namespace hpt

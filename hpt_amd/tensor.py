@@ -57,6 +57,7 @@ _BY_NP = {d.np_dtype: d for d in DTYPES if d is not bf16}
 
 # hpt_reduce_op
 SUM, PROD, MAX, MIN, MEAN, NANSUM, NANPROD, REDUCEL1, REDUCEL2, REDUCEL3, SUM_SQUARE, LOGSUMEXP, ALL, ANY = range(14)
+BIN_ADD, BIN_SUB, BIN_MUL, BIN_DIV = range(4)  # hpt_binary_op
 
 
 def f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
@@ -180,10 +181,17 @@ class Tensor:
         return out
 
     def to_cpu(self) -> "Tensor":
-        """to_cpu (hpt/src/backends/cuda/tensor_impls.rs:142-169): contiguous copy back to the host."""
+        """to_cpu (hpt/src/backends/cuda/tensor_impls.rs:142-169): a view is first made contiguous ON
+        THE DEVICE (:154-160), then copied back with one synchronous transfer."""
         if self.backend != "hip":
             raise ParamError(_ffi.ERR_PARAM, "to_cpu expects a hip tensor")
-        return Tensor.from_numpy(self.numpy(), self.dtype)
+        src = self if (self.is_contiguous() and self.parent is None) else self.contiguous()
+        arr = np.empty(self.shape, self.dtype.np_dtype)
+        if arr.nbytes:
+            check(_ffi.lib().hpt_hip_stream_synchronize(self.device, None))
+            check(_ffi.lib().hpt_hip_memcpy_d2h_sync(self.device, C.c_void_p(arr.ctypes.data),
+                                                     C.c_void_p(src.ptr), arr.nbytes))
+        return Tensor.from_numpy(arr, self.dtype)
 
     def numpy(self) -> np.ndarray:
         """Contiguous numpy copy of this (possibly strided) tensor; bf16 comes back as uint16 bits."""
@@ -443,6 +451,106 @@ class Tensor:
         del keep
         return res
 
+    # ---- the steps either side of the path ------------------------------------------
+    def contiguous(self, stream=None) -> "Tensor":
+        """Contiguous::contiguous (hpt/src/backends/cuda/tensor_internal/normal_out_unary.rs:286-310):
+        a new contiguous tensor with this view's elements."""
+        self._require_hip("contiguous")
+        res = Tensor.empty(self.shape, self.dtype, self.device)
+        vin, k1 = self._c_view()
+        vout, k2 = res._c_view()
+        check(_ffi.lib().hpt_hip_contiguous(self.device, stream, C.byref(vin), C.byref(vout)))
+        del k1, k2
+        return res
+
+    @classmethod
+    def full(cls, value, shape, dtype: DType, device: int = 0, stream=None) -> "Tensor":
+        """TensorCreator::full on the device (set_val, hpt-cudakernels/src/set_val.cu:4-12). For bf16 `value`
+        is a float (rounded to nearest even)."""
+        res = cls.empty(shape, dtype, device)
+        if dtype.name == "bf16":
+            host = f32_to_bf16_bits(np.array([value], np.float32))
+        else:
+            host = np.array([value]).astype(dtype.np_dtype)
+        v, k = res._c_view()
+        check(_ffi.lib().hpt_hip_fill(device, stream, C.byref(v), C.c_void_p(host.ctypes.data)))
+        del k
+        return res
+
+    @classmethod
+    def zeros(cls, shape, dtype: DType, device: int = 0) -> "Tensor":
+        return cls.full(0, shape, dtype, device)
+
+    @classmethod
+    def ones(cls, shape, dtype: DType, device: int = 0) -> "Tensor":
+        return cls.full(1, shape, dtype, device)
+
+    def expand(self, shape) -> "Tensor":
+        """ShapeManipulate::expand (hpt-common/src/layout/layout_utils.rs:107-): broadcast size-1 dims (and
+        missing leading dims) to `shape` with stride 0."""
+        shape = [int(x) for x in shape]
+        if len(shape) < self.ndim:
+            raise ShapeError(_ffi.ERR_SHAPE, f"expand: cannot expand {self.shape} to {shape}")
+        pad = len(shape) - self.ndim
+        strides = [0] * len(shape)
+        for i, d in enumerate(shape):
+            if i < pad:
+                continue
+            old = self.shape[i - pad]
+            if old == d:
+                strides[i] = self.strides[i - pad]
+            elif old != 1:
+                raise ShapeError(_ffi.ERR_SHAPE, f"expand: cannot broadcast {self.shape} to {shape}")
+        return self._view(self.ptr, shape, strides)
+
+    def _binary(self, op: int, rhs: "Tensor", out: Optional["Tensor"] = None, stream=None) -> "Tensor":
+        self._require_hip("binary op")
+        rhs._require_hip("binary op rhs")
+        # predict_broadcast_shape (hpt-common/src/shape/shape_utils.rs): numpy's rule
+        nd = max(self.ndim, rhs.ndim)
+        sa = [1] * (nd - self.ndim) + list(self.shape)
+        sb = [1] * (nd - rhs.ndim) + list(rhs.shape)
+        shape = []
+        for x, y in zip(sa, sb):
+            if x != y and x != 1 and y != 1:
+                raise ShapeError(_ffi.ERR_SHAPE, f"broadcast failed: lhs shape {self.shape}, rhs shape {rhs.shape}")
+            shape.append(max(x, y) if min(x, y) != 0 else 0)
+        a, b = self.expand(shape), rhs.expand(shape)
+        res = out if out is not None else Tensor.empty(shape, self.dtype, self.device)
+        va, k1 = a._c_view()
+        vb, k2 = b._c_view()
+        vo, k3 = res._c_view()
+        check(_ffi.lib().hpt_hip_binary(self.device, stream, op, C.byref(va), C.byref(vb), C.byref(vo)))
+        del k1, k2, k3
+        return res
+
+    def add(self, rhs: "Tensor", **kw) -> "Tensor":
+        return self._binary(BIN_ADD, rhs, **kw)
+
+    def sub(self, rhs: "Tensor", **kw) -> "Tensor":
+        return self._binary(BIN_SUB, rhs, **kw)
+
+    def mul(self, rhs: "Tensor", **kw) -> "Tensor":
+        return self._binary(BIN_MUL, rhs, **kw)
+
+    def div(self, rhs: "Tensor", **kw) -> "Tensor":
+        return self._binary(BIN_DIV, rhs, **kw)
+
+    def add_(self, rhs: "Tensor", out: "Tensor", **kw) -> "Tensor":
+        """NormalBinOps::add_ (hpt-traits/src/ops/binary.rs:34): the result goes to `out` (which may be self)."""
+        return self._binary(BIN_ADD, rhs, out=out, **kw)
+
+    def sub_(self, rhs: "Tensor", out: "Tensor", **kw) -> "Tensor":
+        return self._binary(BIN_SUB, rhs, out=out, **kw)
+
+    def mul_(self, rhs: "Tensor", out: "Tensor", **kw) -> "Tensor":
+        return self._binary(BIN_MUL, rhs, out=out, **kw)
+
+    def div_(self, rhs: "Tensor", out: "Tensor", **kw) -> "Tensor":
+        return self._binary(BIN_DIV, rhs, out=out, **kw)
+
+    __add__, __sub__, __mul__, __truediv__ = add, sub, mul, div
+
     def __repr__(self):
         return f"Tensor<{self.dtype.name}, {self.backend}, {self.device}>(shape={self.shape}, strides={self.strides})"
 
@@ -454,6 +562,16 @@ def reduce_plan(t: Tensor, op: int, axes) -> str:
     buf = C.create_string_buffer(512)
     check(_ffi.lib().hpt_hip_reduce_plan(op, C.byref(v), _ffi.i64_array(axes), len(axes), buf, 512))
     del k
+    return buf.value.decode()
+
+
+def contiguous_plan(t: Tensor) -> str:
+    """The kernel `t.contiguous()` would use (no device needed; the output is assumed 16-byte aligned)."""
+    v, k = t._c_view()
+    out, k2 = make_view(4096, t.shape, _contiguous_strides(t.shape), t.dtype.code)
+    buf = C.create_string_buffer(512)
+    check(_ffi.lib().hpt_hip_contiguous_plan(C.byref(v), C.byref(out), buf, 512))
+    del k, k2
     return buf.value.decode()
 
 

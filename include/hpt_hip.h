@@ -209,6 +209,39 @@ int32_t hpt_hip_softmax(int32_t dev, void* stream, int32_t log, const hpt_view* 
 int32_t hpt_hip_layernorm(int32_t dev, void* stream, const hpt_view* in, int32_t n_norm_dims,
                           const hpt_view* gamma, const hpt_view* beta, double eps, hpt_view* out);
 
+/* ---- the steps either side of the path ------------------------------------
+ * What the callers of reductions and normalisations do to their operands just
+ * before and after, kept on the device. */
+
+/* Contiguous::contiguous (hpt-traits/src/ops/unary.rs:882; device
+ * hpt/src/backends/cuda/tensor_internal/normal_out_unary.rs:286-310 launching
+ * hpt-cudakernels/src/strided_copy.cu:6-14): copy any strided view into the
+ * contiguous `out` of the same shape and dtype. This is also the first step of
+ * `to_cpu` on a view (hpt/src/backends/cuda/tensor_impls.rs:154-160). */
+int32_t hpt_hip_contiguous(int32_t dev, void* stream, const hpt_view* in, hpt_view* out);
+/* Describes the kernel hpt_hip_contiguous would pick (tests, tuning). */
+int32_t hpt_hip_contiguous_plan(const hpt_view* in, const hpt_view* out, char* buf, size_t buflen);
+
+/* set_val (hpt-cudakernels/src/set_val.cu:4-12; used by `full` / `zeros` / `ones`,
+ * hpt/src/backends/cuda/tensor_internal/normal_creation.rs): every element of the
+ * contiguous `out` becomes `*value`, one element of out's dtype in HOST memory. */
+int32_t hpt_hip_fill(int32_t dev, void* stream, hpt_view* out, const void* value);
+
+typedef enum hpt_binary_op { HPT_BIN_ADD = 0, HPT_BIN_SUB = 1, HPT_BIN_MUL = 2, HPT_BIN_DIV = 3 } hpt_binary_op;
+
+/* NormalBinOps::add_ / sub_ / mul_ / div_ (hpt-traits/src/ops/binary.rs:34,52,70,149;
+ * device hpt/src/backends/cuda/utils/binary/binary_normal.rs:29-) for operands of ONE
+ * dtype: out = lhs (op) rhs. `lhs` and `rhs` are strided views of out's shape; a
+ * broadcast dim is passed with stride 0, as Hpt's `expand` produces it
+ * (hpt-common/src/layout/layout_utils.rs `broadcast`). `out` is contiguous and may be
+ * the very tensor `lhs` or `rhs` views (same data, shape and strides): the in-place
+ * `add_` / `mul_` that layernorm's single-affine branches call
+ * (hpt/src/backends/cpu/tensor_internal/normalization.rs:187-192). Integers wrap; bool
+ * add is OR and mul is AND (sub / div undefined); div is for float dtypes (Hpt's
+ * integer division changes the dtype). f16 / bf16 compute in f32 and round once. */
+int32_t hpt_hip_binary(int32_t dev, void* stream, int32_t op, const hpt_view* lhs, const hpt_view* rhs,
+                       hpt_view* out);
+
 #ifdef __cplusplus
 }
 #endif

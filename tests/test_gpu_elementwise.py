@@ -1,0 +1,203 @@
+"""GPU parity of the steps either side of the path, through the C ABI: contiguous() of any view
+(hpt/src/backends/cuda/tensor_internal/normal_out_unary.rs:286-310), full (set_val), and add / sub / mul /
+div with broadcasting and in place (hpt-traits/src/ops/binary.rs:34-152). Every result is bit-exact against
+oracle/elementwise.py."""
+import numpy as np
+import pytest
+
+from oracle import elementwise as ew
+from util import apply_view_np, apply_view_t, layouts_for
+
+pytestmark = pytest.mark.gpu
+
+NP_DTYPES = [np.bool_, np.int8, np.int16, np.int32, np.int64, np.uint8, np.uint16, np.uint32, np.uint64,
+             np.float16, np.float32, np.float64]
+
+
+def rand(rng, shape, npdt):
+    if npdt == np.bool_:
+        return rng.integers(0, 2, shape).astype(np.bool_)
+    if np.dtype(npdt).kind in "iu":
+        info = np.iinfo(npdt)
+        return rng.integers(info.min, info.max, shape, dtype=npdt, endpoint=True)
+    return (rng.standard_normal(shape) * 4).astype(npdt)
+
+
+def same_bits(got, want, msg):
+    assert got.shape == want.shape and got.dtype == want.dtype, msg
+    assert np.array_equal(got.view(np.uint8) if got.size else got, want.view(np.uint8) if want.size else want), msg
+
+
+# ---- contiguous ------------------------------------------------------------------------------------
+
+COPY_CASES = [
+    # name, base shape, view ops, expected plan prefix
+    ("2-D transpose, ragged tiles", [200, 136], (("permute", (1, 0)),), "transpose"),
+    ("3-D rotate", [24, 40, 72], (("permute", (2, 0, 1)),), "transpose"),
+    ("batched transpose", [3, 80, 48], (("permute", (0, 2, 1)),), "transpose"),
+    ("4-D middle swap keeps inner rows", [4, 6, 10, 64], (("permute", (0, 2, 1, 3)),), "inner"),
+    ("row slice", [50, 128], (("slice", ((3, 41, 1), (0, 128, 1))),), "inner"),
+    ("column slice (unaligned rows)", [50, 128], (("slice", ((0, 50, 1), (5, 77, 1))),), "inner"),
+    ("step 2 columns", [50, 128], (("slice", ((0, 50, 1), (0, 128, 2))),), "inner-step2"),
+    ("step 2 columns, odd start", [50, 128], (("slice", ((0, 50, 1), (1, 128, 2))),), "inner vec=1"),
+    ("step 2 rows and columns", [50, 128], (("slice", ((1, 50, 2), (0, 128, 2))),), "inner-step2"),
+    ("negative steps", [9, 31], (("slice", ((8, None, -1), (30, None, -3))),), "inner"),
+    ("transpose too small for tiles", [5, 7], (("permute", (1, 0)),), "inner"),
+    ("5-D permute", [3, 4, 5, 6, 8], (("permute", (4, 2, 0, 3, 1)),), ""),
+    ("one element", [1, 1], (), "inner"),
+]
+
+
+@pytest.mark.parametrize("case", COPY_CASES, ids=[c[0] for c in COPY_CASES])
+def test_contiguous_all_dtypes(hpt, dev, case):
+    name, shape, ops, plan = case
+    rng = np.random.default_rng(300)
+    for npdt in NP_DTYPES:
+        base = rand(rng, shape, npdt)
+        t = apply_view_t(hpt.Tensor.from_numpy(base).to_hip(dev), ops)
+        a = apply_view_np(base, ops)
+        if np.dtype(npdt).itemsize == 4 and plan:
+            assert hpt.contiguous_plan(t).startswith(plan), hpt.contiguous_plan(t)
+        c = t.contiguous()
+        assert c.is_contiguous() and c.shape == list(a.shape)
+        same_bits(c.numpy(), ew.contiguous(a), f"contiguous {name} {np.dtype(npdt).name}")
+        # to_cpu of a view goes through the same device copy (tensor_impls.rs:154-160)
+        same_bits(t.to_cpu().numpy(), ew.contiguous(a), f"to_cpu {name} {np.dtype(npdt).name}")
+
+
+def test_contiguous_bf16_random_layouts_and_empty(hpt, dev):
+    rng = np.random.default_rng(301)
+    for shape in ([33, 129], [4, 18, 40], [2, 3, 4, 5]):
+        base = rng.integers(0, 65536, shape).astype(np.uint16)
+        for lname, ops in layouts_for(shape, rng):
+            t = apply_view_t(hpt.Tensor.from_numpy(base, hpt.bf16).to_hip(dev), ops)
+            same_bits(t.contiguous().numpy(), ew.contiguous(apply_view_np(base, ops)), f"bf16 {shape} {lname}")
+    e = hpt.Tensor.from_numpy(np.zeros((4, 0, 3), np.float32)).to_hip(dev).permute([2, 1, 0]).contiguous()
+    assert e.shape == [3, 0, 4] and e.numpy().size == 0
+
+
+def test_contiguous_large_transpose_and_errors(hpt, dev):
+    """f16 [4096, 2048] transposed: 16 MiB through the register-tile kernel; f64 [1024, 1536]."""
+    rng = np.random.default_rng(302)
+    for npdt, shape in ((np.float16, [4096, 2048]), (np.float64, [1024, 1536]), (np.int8, [2048, 4096])):
+        base = rand(rng, shape, npdt)
+        t = hpt.Tensor.from_numpy(base).to_hip(dev).permute([1, 0])
+        assert hpt.contiguous_plan(t).startswith("transpose")
+        same_bits(t.contiguous().numpy(), ew.contiguous(base.T), f"large transpose {np.dtype(npdt).name}")
+    from hpt_amd import _ffi
+    import ctypes as C
+    a = hpt.Tensor.from_numpy(np.zeros((4, 6), np.float32)).to_hip(dev)
+    bad = hpt.Tensor.empty([6, 5], hpt.f32, dev)
+    va, k1 = a.permute([1, 0])._c_view()
+    vb, k2 = bad._c_view()
+    with pytest.raises(hpt.ShapeError):
+        _ffi.check(hpt.lib().hpt_hip_contiguous(dev, None, C.byref(va), C.byref(vb)))
+    wrong = hpt.Tensor.empty([6, 4], hpt.i32, dev)
+    vw, k3 = wrong._c_view()
+    with pytest.raises(hpt.DTypeError):
+        _ffi.check(hpt.lib().hpt_hip_contiguous(dev, None, C.byref(va), C.byref(vw)))
+
+
+# ---- fill -------------------------------------------------------------------------------------------
+
+def test_full_all_dtypes_and_unaligned_views(hpt, dev):
+    vals = {np.bool_: True, np.int8: -7, np.int16: -1234, np.int32: -123456789, np.int64: -(1 << 40) - 3,
+            np.uint8: 200, np.uint16: 54321, np.uint32: 4000000000, np.uint64: (1 << 63) + 5,
+            np.float16: 1.5, np.float32: -2.25, np.float64: 3.141592653589793}
+    for npdt, v in vals.items():
+        t = hpt.Tensor.from_numpy(np.zeros(1, npdt))   # only to look the dtype up
+        for shape in ([1], [5], [1000], [3, 7, 11], [0]):
+            f = hpt.Tensor.full(v, shape, t.dtype, dev)
+            same_bits(f.numpy(), ew.full(v, shape, npdt), f"full {np.dtype(npdt).name} {shape}")
+    b = hpt.Tensor.full(1.0 / 3.0, [9], hpt.bf16, dev).numpy()
+    assert np.all(b == ew.f32_to_bf16_bits(np.array([1.0 / 3.0], np.float32))[0])
+    assert np.all(hpt.Tensor.zeros([4, 4], hpt.f32, dev).numpy() == 0)
+    assert np.all(hpt.Tensor.ones([4, 4], hpt.i64, dev).numpy() == 1)
+    # fill a contiguous tail that starts off a 16-byte boundary: the rest of the block must stay untouched
+    from hpt_amd import _ffi
+    import ctypes as C
+    base = hpt.Tensor.from_numpy(np.arange(100, dtype=np.int16)).to_hip(dev)
+    tail = base[3:90]
+    val = np.array([-5], np.int16)
+    v, k = tail._c_view()
+    _ffi.check(hpt.lib().hpt_hip_fill(dev, None, C.byref(v), C.c_void_p(val.ctypes.data)))
+    want = np.arange(100, dtype=np.int16)
+    want[3:90] = -5
+    same_bits(base.numpy(), want, "fill of an unaligned tail")
+
+
+# ---- binary -----------------------------------------------------------------------------------------
+
+OPS = (("add", ew.ADD), ("sub", ew.SUB), ("mul", ew.MUL), ("div", ew.DIV))
+
+
+@pytest.mark.parametrize("npdt", NP_DTYPES, ids=[np.dtype(d).name for d in NP_DTYPES])
+def test_binary_broadcast_patterns(hpt, dev, npdt):
+    rng = np.random.default_rng(310)
+    shapes = [([37, 64], [37, 64]),      # same shape: flat vectors
+              ([37, 64], [64]),          # bias over rows (layernorm's add_ / mul_)
+              ([37, 64], [37, 1]),       # per-row scalar: broadcast along the inner dim
+              ([5, 1, 24], [1, 7, 24]),  # both sides broadcast
+              ([6, 10], [1]),            # scalar tensor
+              ([3, 5], [3, 5])]          # tiny, not vectorisable
+    for sa, sb in shapes:
+        a, b = rand(rng, sa, npdt), rand(rng, sb, npdt)
+        if np.dtype(npdt).kind == "f":
+            b = np.where(np.abs(b) < 0.25, npdt(1.0), b)   # keep quotients tame
+        ta, tb = hpt.Tensor.from_numpy(a).to_hip(dev), hpt.Tensor.from_numpy(b).to_hip(dev)
+        for name, op in OPS:
+            ok = not (npdt == np.bool_ and op in (ew.SUB, ew.DIV)) and not (op == ew.DIV and np.dtype(npdt).kind != "f")
+            if not ok:
+                with pytest.raises(hpt.DTypeError):
+                    getattr(ta, name)(tb)
+                continue
+            got = getattr(ta, name)(tb).numpy()
+            same_bits(got, ew.binary(op, a, b), f"{name} {np.dtype(npdt).name} {sa} {sb}")
+
+
+def test_binary_strided_operands_inplace_and_bf16(hpt, dev):
+    rng = np.random.default_rng(311)
+    base = rand(rng, [48, 80], np.float32)
+    other = rand(rng, [80, 48], np.float32)
+    ta, tb = hpt.Tensor.from_numpy(base).to_hip(dev), hpt.Tensor.from_numpy(other).to_hip(dev)
+    same_bits(ta.add(tb.permute([1, 0])).numpy(), ew.binary(ew.ADD, base, other.T), "add of a transposed operand")
+    same_bits(ta[:, ::2].mul(tb.permute([1, 0])[:, 1::2]).numpy(), ew.binary(ew.MUL, base[:, ::2], other.T[:, 1::2]),
+              "mul of stepped views")
+    # in place: res.add_(beta, res) / res.mul_(gamma, res), as normalization.rs:187-192
+    res = hpt.Tensor.from_numpy(base).to_hip(dev)
+    gamma = rand(rng, [80], np.float32)
+    tg = hpt.Tensor.from_numpy(gamma).to_hip(dev)
+    out = res.mul_(tg, res)
+    assert out is res
+    same_bits(res.numpy(), ew.binary(ew.MUL, base, gamma), "mul_ in place")
+    res.add_(tg, res)
+    same_bits(res.numpy(), ew.binary(ew.ADD, ew.binary(ew.MUL, base, gamma), gamma), "add_ in place")
+    # out overlapping an operand without being it is refused
+    with pytest.raises(hpt.ParamError):
+        ta[1:].add_(ta[1:], ta[:-1])
+    # bf16
+    xa = ew.f32_to_bf16_bits(rand(rng, [33, 40], np.float32))
+    xb = ew.f32_to_bf16_bits(rand(rng, [40], np.float32))
+    t1, t2 = hpt.Tensor.from_numpy(xa, hpt.bf16).to_hip(dev), hpt.Tensor.from_numpy(xb, hpt.bf16).to_hip(dev)
+    for name, op in OPS[:3]:
+        same_bits(getattr(t1, name)(t2).numpy(), ew.binary(op, xa, xb, bf16=True), f"bf16 {name}")
+    # dtype mismatch and shape mismatch
+    with pytest.raises(hpt.DTypeError):
+        ta.add(hpt.Tensor.from_numpy(np.zeros([48, 80], np.float64)).to_hip(dev))
+    with pytest.raises(hpt.ShapeError):
+        ta.add(hpt.Tensor.from_numpy(np.zeros([48, 81], np.float32)).to_hip(dev))
+
+
+def test_layernorm_equals_normalise_then_affine_steps(hpt, orc, dev):
+    """The reference applies gamma / beta as separate mul_ / add_ passes after normalising
+    (normalization.rs:187-192); the fused kernel must agree with those steps done on the device."""
+    rng = np.random.default_rng(312)
+    x = rng.standard_normal((64, 256)).astype(np.float32)
+    g = rng.normal(1, 0.1, 256).astype(np.float32)
+    b = rng.normal(0, 0.1, 256).astype(np.float32)
+    tx, tg, tb = (hpt.Tensor.from_numpy(v).to_hip(dev) for v in (x, g, b))
+    fused = tx.layernorm([256], tg, tb, 1e-5).numpy()
+    steps = tx.layernorm([256], None, None, 1e-5)
+    steps.mul_(tg, steps)
+    steps.add_(tb, steps)
+    np.testing.assert_allclose(steps.numpy(), fused, rtol=2e-6, atol=2e-7)
