@@ -245,6 +245,32 @@ def cases_c5(P):
     return cases
 
 
+def cases_c7(P):
+    """The fused forms at the C4 / C2 shapes: the causal mask as a parameter (the masked half of the logits is
+    never read), and layernorm(x + residual)."""
+    import hpt_amd as hpt
+    l, check = P.l, P.ffi.check
+    rng = np.random.default_rng(7)
+    c4 = hpt.f32_to_bf16_bits(rng.standard_normal((32, 2048, 2048), dtype=np.float32) * 3)
+    ins = [hpt.Tensor.from_numpy(c4, hpt.bf16).to_hip(0), hpt.Tensor.from_numpy(np.roll(c4, 1, 0), hpt.bf16).to_hip(0)]
+    outs = [hpt.Tensor.empty(t.shape, t.dtype, 0) for t in ins]
+    vi, vo = [P.view(t) for t in ins], [P.view(t) for t in outs]
+    run = lambda i: check(l.hpt_hip_softmax_causal(0, None, 0, vi[i % 2], 0.125, 0, vo[i % 2]))
+    kept = 32 * 2048 * 2049 // 2     # logits below or on the diagonal
+    cases = [Case("softmax_causal(scale)", "C4 bf16 [32,2048,2048] causal mask as a parameter", "bf16", 65536,
+                  kept * 2 + c4.nbytes, run, 2)]
+    x, g, b = gen_c2()
+    xs = [hpt.Tensor.from_numpy(np.roll(x, k, axis=0)).to_hip(0) for k in range(3)]
+    rs = [hpt.Tensor.from_numpy(np.roll(x, k + 5, axis=0)).to_hip(0) for k in range(3)]
+    tg, tb = hpt.Tensor.from_numpy(g).to_hip(0), hpt.Tensor.from_numpy(b).to_hip(0)
+    os_ = [hpt.Tensor.empty(t.shape, t.dtype, 0) for t in xs]
+    vx, vr, vo2, vg, vb = [P.view(t) for t in xs], [P.view(t) for t in rs], [P.view(t) for t in os_], P.view(tg), P.view(tb)
+    run2 = lambda i: check(l.hpt_hip_add_layernorm(0, None, vx[i % 3], vr[i % 3], 1, vg, vb, 1e-5, vo2[i % 3]))
+    cases.append(Case("add_layernorm", "C2 f32 [8192,4096] + residual, gamma,beta", "f32", 8192,
+                      3 * x.nbytes + g.nbytes + b.nbytes, run2, 3))
+    return cases
+
+
 def cases_c6(P):
     """The steps either side of the path at the headline / C5 shapes: contiguous() of the C5 views, the
     affine steps of layernorm as separate in-place passes, full()."""
@@ -286,7 +312,8 @@ def build_cases(which: str, configs=None):
     P = Prepared()
     cases, head = cases_c2(P, which == "headline")
     if which != "headline":
-        for name, fn in (("c1", cases_c1), ("c3", cases_c3), ("c4", cases_c4), ("c5", cases_c5), ("c6", cases_c6)):
+        for name, fn in (("c1", cases_c1), ("c3", cases_c3), ("c4", cases_c4), ("c5", cases_c5), ("c6", cases_c6),
+                         ("c7", cases_c7)):
             if configs is None or name in configs:
                 cases += fn(P)
     return cases, P, head

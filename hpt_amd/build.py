@@ -31,7 +31,7 @@ FLAGS = [
 ]
 
 N_REDUCE_ENTRIES = 16  # 14 reduce ops + argmin + argmax
-N_NORM_KINDS = 3
+N_NORM_KINDS = 6  # softmax, log_softmax, layernorm, add+layernorm, causal softmax / log_softmax
 
 
 def units():

@@ -226,6 +226,9 @@ NormLaunchFn norm_launcher_for(int kind, int dtype) {
         case NORM_SOFTMAX: return norm_launcher<NORM_SOFTMAX>(dtype);
         case NORM_LOGSOFTMAX: return norm_launcher<NORM_LOGSOFTMAX>(dtype);
         case NORM_LAYERNORM: return norm_launcher<NORM_LAYERNORM>(dtype);
+        case NORM_ADD_LAYERNORM: return norm_launcher<NORM_ADD_LAYERNORM>(dtype);
+        case NORM_SOFTMAX_CAUSAL: return norm_launcher<NORM_SOFTMAX_CAUSAL>(dtype);
+        case NORM_LOGSOFTMAX_CAUSAL: return norm_launcher<NORM_LOGSOFTMAX_CAUSAL>(dtype);
         default: return nullptr;
     }
 }
@@ -583,45 +586,86 @@ int32_t hpt_hip_softmax(int32_t dev, void* stream, int32_t log, const hpt_view* 
     });
 }
 
+// layernorm, optionally of (in + residual)
+static void run_layernorm(int dev, void* stream, const hpt_view* in, const hpt_view* residual, int n_norm_dims,
+                          const hpt_view* gamma, const hpt_view* beta, double eps, hpt_view* out) {
+    check_view(in, "layernorm input", true);
+    if (n_norm_dims <= 0) fail(HPT_ERR_SHAPE, "layernorm: normalized_shape must not be empty");
+    check_out(out, in->dtype, view_size(in), "layernorm output");
+    NormCall c = prepare_norm(in, out->data, 0, n_norm_dims);
+    const hpt_view* gb[2] = {gamma, beta};
+    const char* names[2] = {"layernorm gamma", "layernorm beta"};
+    for (int k = 0; k < 2; ++k) {
+        if (!gb[k]) continue;
+        check_view(gb[k], names[k], true);
+        if (gb[k]->dtype != in->dtype)
+            fail(HPT_ERR_DTYPE, "%s: dtype is %s, expected %s", names[k], dtype_name(gb[k]->dtype),
+                 dtype_name(in->dtype));
+        if (!view_contiguous(gb[k])) fail(HPT_ERR_SHAPE, "%s: must be contiguous", names[k]);
+        // shape must equal the normalised dims (leading 1s aside)
+        if (view_size(gb[k]) != c.plan.cols && c.plan.kind != NormKind::Empty)
+            fail(HPT_ERR_SHAPE, "%s: Size mismatch: expected %lld, got %lld", names[k],
+                 (long long)c.plan.cols, (long long)view_size(gb[k]));
+    }
+    if (residual) {
+        check_view(residual, "layernorm residual", true);
+        if (residual->dtype != in->dtype)
+            fail(HPT_ERR_DTYPE, "layernorm residual: dtype is %s, expected %s", dtype_name(residual->dtype),
+                 dtype_name(in->dtype));
+        if (!view_contiguous(residual)) fail(HPT_ERR_SHAPE, "layernorm residual: must be contiguous");
+        bool same = residual->ndim == in->ndim;
+        for (int i = 0; same && i < in->ndim; ++i) same = residual->shape[i] == in->shape[i];
+        if (!same) fail(HPT_ERR_SHAPE, "layernorm residual: shape differs from the input's");
+    }
+    if (c.plan.kind == NormKind::Empty) return;
+    c.args.gamma = gamma ? gamma->data : nullptr;
+    c.args.beta = beta ? beta->data : nullptr;
+    c.args.residual = residual ? residual->data : nullptr;
+    c.args.eps = eps;
+    // the fused form runs on the row kernels only
+    if (residual && (c.plan.kind == NormKind::Transposed || c.plan.kind == NormKind::TransposedTile))
+        demote_to_generic(c.plan);
+    // vector loads of gamma / beta / residual need 16-byte alignment too
+    if (c.plan.vec > 1 &&
+        (((uintptr_t)c.args.gamma | (uintptr_t)c.args.beta | (uintptr_t)c.args.residual) % 16) != 0)
+        demote_to_generic(c.plan);
+    NormLaunchFn fn = norm_launcher_for(residual ? NORM_ADD_LAYERNORM : NORM_LAYERNORM, in->dtype);
+    if (!fn) fail(HPT_ERR_DTYPE, "layernorm: unsupported dtype %s", dtype_name(in->dtype));
+    use_device(dev);
+    launch_norm(dev, (hipStream_t)stream, fn, c, "layernorm");
+}
+
 int32_t hpt_hip_layernorm(int32_t dev, void* stream, const hpt_view* in, int32_t n_norm_dims,
                           const hpt_view* gamma, const hpt_view* beta, double eps, hpt_view* out) {
+    return guarded([&] { run_layernorm(dev, stream, in, nullptr, n_norm_dims, gamma, beta, eps, out); });
+}
+
+int32_t hpt_hip_add_layernorm(int32_t dev, void* stream, const hpt_view* in, const hpt_view* residual,
+                              int32_t n_norm_dims, const hpt_view* gamma, const hpt_view* beta, double eps,
+                              hpt_view* out) {
     return guarded([&] {
-        check_view(in, "layernorm input", true);
-        if (n_norm_dims <= 0) fail(HPT_ERR_SHAPE, "layernorm: normalized_shape must not be empty");
-        check_out(out, in->dtype, view_size(in), "layernorm output");
-        NormCall c = prepare_norm(in, out->data, 0, n_norm_dims);
-        const hpt_view* gb[2] = {gamma, beta};
-        const char* names[2] = {"layernorm gamma", "layernorm beta"};
-        for (int k = 0; k < 2; ++k) {
-            if (!gb[k]) continue;
-            check_view(gb[k], names[k], true);
-            if (gb[k]->dtype != in->dtype)
-                fail(HPT_ERR_DTYPE, "%s: dtype is %s, expected %s", names[k], dtype_name(gb[k]->dtype),
-                     dtype_name(in->dtype));
-            if (!view_contiguous(gb[k])) fail(HPT_ERR_SHAPE, "%s: must be contiguous", names[k]);
-            // shape must equal the normalised dims (leading 1s aside)
-            if (view_size(gb[k]) != c.plan.cols && c.plan.kind != NormKind::Empty)
-                fail(HPT_ERR_SHAPE, "%s: Size mismatch: expected %lld, got %lld", names[k],
-                     (long long)c.plan.cols, (long long)view_size(gb[k]));
-        }
+        if (!residual) fail(HPT_ERR_PARAM, "add_layernorm: residual is null");
+        run_layernorm(dev, stream, in, residual, n_norm_dims, gamma, beta, eps, out);
+    });
+}
+
+int32_t hpt_hip_softmax_causal(int32_t dev, void* stream, int32_t log, const hpt_view* in, double scale,
+                               int64_t causal_offset, hpt_view* out) {
+    return guarded([&] {
+        check_view(in, "softmax_causal input", true);
+        check_out(out, in->dtype, view_size(in), "softmax_causal output");
+        if (in->ndim < 2) fail(HPT_ERR_SHAPE, "softmax_causal: needs at least 2 dims (queries x keys)");
+        NormCall c = prepare_norm(in, out->data, in->ndim - 1, 0);
         if (c.plan.kind == NormKind::Empty) return;
-        c.args.gamma = gamma ? gamma->data : nullptr;
-        c.args.beta = beta ? beta->data : nullptr;
-        c.args.eps = eps;
-        // vector loads of gamma/beta need 16-byte alignment too
-        if (c.plan.vec > 1 && (((uintptr_t)c.args.gamma | (uintptr_t)c.args.beta) % 16) != 0) {
-            c.plan.vec = 1;
-            if (c.plan.kind == NormKind::RowReg || c.plan.kind == NormKind::Transposed ||
-                c.plan.kind == NormKind::TransposedTile) {
-                c.plan.kind = NormKind::Generic;
-                c.plan.scratch_bytes = 0;
-                c.plan.sstride = 1;
-            }
-        }
-        NormLaunchFn fn = norm_launcher_for(NORM_LAYERNORM, in->dtype);
-        if (!fn) fail(HPT_ERR_DTYPE, "layernorm: unsupported dtype %s", dtype_name(in->dtype));
+        if (c.plan.kind == NormKind::Transposed || c.plan.kind == NormKind::TransposedTile)
+            demote_to_generic(c.plan);
+        c.args.scale = scale;
+        c.args.q_rows = in->shape[in->ndim - 2];
+        c.args.causal_offset = causal_offset;
+        NormLaunchFn fn = norm_launcher_for(log ? NORM_LOGSOFTMAX_CAUSAL : NORM_SOFTMAX_CAUSAL, in->dtype);
+        if (!fn) fail(HPT_ERR_DTYPE, "softmax_causal: unsupported dtype %s", dtype_name(in->dtype));
         use_device(dev);
-        launch_norm(dev, (hipStream_t)stream, fn, c, "layernorm");
+        launch_norm(dev, (hipStream_t)stream, fn, c, "softmax_causal");
     });
 }
 

@@ -142,6 +142,10 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
 
 std::string describe(const NormPlan& p);
 
+// Turn a plan into the generic row form (one group of lanes per row, per-element offsets):
+// what the caller falls back to when an operand rules the specialised kernels out.
+void demote_to_generic(NormPlan& p);
+
 // ---- elementwise: strided copy (contiguous()), fill, binary ops with broadcasting ----
 
 enum class EwKind {

@@ -450,6 +450,17 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
     return p;
 }
 
+void demote_to_generic(NormPlan& p) {
+    p.kind = NormKind::Generic;
+    p.vec = 1;
+    p.sstride = 1;
+    p.nchunk = 1;
+    p.scratch_bytes = 0;
+    p.tpr = (int)std::min<int64_t>(1024, pow2_ceil((p.cols + 3) / 4));
+    if (p.tpr > 64 && p.tpr < 256) p.tpr = 256;
+    p.rpb = std::max(1, 256 / p.tpr);
+}
+
 std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "col", "transposed", "transposed-tile", "generic"};
     char buf[256];

@@ -1,5 +1,5 @@
 // Launch table of the normalisation kernels: one object file per kind
-// (softmax, log_softmax, layernorm), one launcher per float dtype.
+// (softmax, log_softmax, layernorm and their fused forms), one launcher per float dtype.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -8,7 +8,18 @@
 
 namespace hpt {
 
-enum { NORM_SOFTMAX = 0, NORM_LOGSOFTMAX = 1, NORM_LAYERNORM = 2 };
+enum {
+    NORM_SOFTMAX = 0,
+    NORM_LOGSOFTMAX = 1,
+    NORM_LAYERNORM = 2,
+    NORM_ADD_LAYERNORM = 3,       // layernorm(in + residual)
+    NORM_SOFTMAX_CAUSAL = 4,      // softmax(scale * in) with the causal mask as a parameter
+    NORM_LOGSOFTMAX_CAUSAL = 5,
+    NORM_KIND_COUNT = 6
+};
+constexpr bool norm_is_layer(int k) { return k == NORM_LAYERNORM || k == NORM_ADD_LAYERNORM; }
+constexpr bool norm_is_log(int k) { return k == NORM_LOGSOFTMAX || k == NORM_LOGSOFTMAX_CAUSAL; }
+constexpr bool norm_is_causal(int k) { return k == NORM_SOFTMAX_CAUSAL || k == NORM_LOGSOFTMAX_CAUSAL; }
 
 struct NormArgs {
     const void* in;
@@ -24,6 +35,10 @@ struct NormArgs {
     double eps;
     double inv_cols;  // 1 / cols
     void* scratch;    // library-owned scratch (partial row statistics of the transposed form)
+    const void* residual;  // NORM_ADD_LAYERNORM: contiguous tensor of out's shape, added to `in` first
+    double scale;          // causal kinds: the input is multiplied by this (and rounded to its dtype) first
+    int64_t q_rows;        // causal kinds: rows per attention matrix (size of the dim before the axis)
+    int64_t causal_offset; // causal kinds: row q keeps columns 0 .. q + causal_offset
     int tpr, tpr_log2, rpb;
 };
 

@@ -108,7 +108,10 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     const int tx = threadIdx.x & (tpr - 1);
     const int ty = threadIdx.x >> a.tpr_log2;
     const int nv = (int)(a.cols / UV);
-    constexpr bool kSoft = KIND != NORM_LAYERNORM;
+    constexpr bool kSoft = !norm_is_layer(KIND);
+    constexpr bool kLog = norm_is_log(KIND);
+    constexpr bool kCausal = norm_is_causal(KIND);
+    constexpr bool kRes = KIND == NORM_ADD_LAYERNORM;
     const CT fill = kSoft ? neg_inf<CT>() : (CT)0;
 
     // this thread's columns never change: keep gamma / beta in registers
@@ -138,19 +141,41 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     // NEXT row this workgroup will take are issued before the current row's statistics
     // and stores, so that the memory pipeline never drains between rows. With 4-byte
     // elements the extra live registers cost more than the overlap gains (measured).
-    constexpr bool kPrefetch = sizeof(T) == 2 && NCHUNK * UV <= (kSoft ? 32 : 16);
+    constexpr bool kPrefetch = sizeof(T) == 2 && NCHUNK * UV <= (kSoft ? 32 : 16) && !kRes;
     const int64_t row_step = (int64_t)gridDim.x * a.rpb;
     Pack<T, VEC> raw[NCHUNK];
+    Pack<T, UV> raw_res[kRes ? NCHUNK : 1];
+    // causal kinds: row q of each (q_rows x cols) matrix keeps columns 0 .. q + causal_offset;
+    // the rest is never read and counts as -inf
+    // the scalar operand of the unfused mul_ has the tensor's dtype
+    const CT scale_t = kCausal ? Elem<T>::widen(Elem<T>::narrow((CT)a.scale)) : (CT)1;
+    auto row_limit = [&](int64_t row) -> int64_t {
+        if constexpr (kCausal) {
+            // (rows and q_rows fit 32 bits whenever this kernel runs: a row fits registers)
+            const int64_t q = ((uint64_t)(row | a.q_rows) >> 32) == 0 ? (int64_t)((uint32_t)row % (uint32_t)a.q_rows)
+                                                                      : row % a.q_rows;
+            const int64_t lim = q + a.causal_offset + 1;
+            return lim < 0 ? 0 : (lim < a.cols ? lim : a.cols);
+        } else {
+            return a.cols;
+        }
+    };
     auto issue_loads = [&](int64_t row0) {
         const int64_t row = row0 + ty;
         if (row >= a.rows) return;
         const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
+        const int nv_row = kCausal ? (int)((row_limit(row) + UV - 1) / UV) : nv;
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int iv = c * tpr + tx;
-            if (iv < nv) {
+            if (iv < nv_row) {
                 if constexpr (VEC > 1) raw[c] = load_pack_stream<T, VEC>(in_row + (int64_t)iv * VEC);
                 else raw[c].v[0] = in_row[(int64_t)iv * a.sa];
+                if constexpr (kRes) {
+                    const T* res_row = (const T*)a.residual + row * a.cols;
+                    if constexpr (VEC > 1) raw_res[c] = load_pack_stream<T, UV>(res_row + (int64_t)iv * UV);
+                    else raw_res[c].v[0] = res_row[iv];
+                }
             }
         }
     };
@@ -160,13 +185,22 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
         const int64_t row = row0 + ty;
         const bool valid = row < a.rows;
         T* out_row = (T*)a.out + (valid ? row * a.cols : 0);
+        const int limit = valid ? (int)row_limit(row) : 0;  // cols <= 8192 vectors here
 
         CT x[NCHUNK][UV];
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int iv = c * tpr + tx;
 #pragma unroll
-            for (int j = 0; j < UV; ++j) x[c][j] = (valid && iv < nv) ? Elem<T>::widen(raw[c].v[j * SS]) : fill;
+            for (int j = 0; j < UV; ++j) {
+                const bool have = valid && iv < nv && (!kCausal || iv * UV + j < limit);
+                CT e = have ? Elem<T>::widen(raw[c].v[j * SS]) : fill;
+                // the fused forms round the intermediate (in + residual, scale * in) to the tensor's
+                // dtype, as the separate add / mul_ of the unfused sequence would have stored it
+                if constexpr (kRes) e = have ? Elem<T>::widen(Elem<T>::narrow(e + Elem<T>::widen(raw_res[c].v[j]))) : fill;
+                if constexpr (kCausal) e = have ? Elem<T>::widen(Elem<T>::narrow(e * scale_t)) : fill;
+                x[c][j] = e;
+            }
         }
         if constexpr (kPrefetch) issue_loads(row0 + row_step);
 
@@ -185,15 +219,15 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                     CT d = x[c][j] - m;
                     CT e = exp_ct<T>(d);
                     s += e;
-                    x[c][j] = KIND == NORM_SOFTMAX ? e : d;
+                    x[c][j] = kLog ? d : e;
                 }
             s = row_all_reduce<SumC<CT>>(s, tpr, ty, smem);
-            const CT k = KIND == NORM_SOFTMAX ? (CT)1 / s : log_ct<T>(s);
+            const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
                 for (int j = 0; j < UV; ++j)
-                    x[c][j] = KIND == NORM_SOFTMAX ? x[c][j] * k : x[c][j] - k;
+                    x[c][j] = kLog ? x[c][j] - k : x[c][j] * k;
         } else {
             CT s = 0;
 #pragma unroll
@@ -303,15 +337,41 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
     const T* in_row = (const T*)a.in + (valid ? offset_of(a.kept_in, row) : 0);
     T* out_row = (T*)a.out + (valid ? offset_of(a.kept_out, row) : 0);
     const bool one_dim = a.norm_in.n <= 1;
+    constexpr bool kLog = norm_is_log(KIND);
+    constexpr bool kCausal = norm_is_causal(KIND);
+    constexpr bool kRes = KIND == NORM_ADD_LAYERNORM;
+    // causal kinds: this row keeps columns 0 .. limit - 1; the rest is never read and counts as -inf
+    int64_t limit = a.cols;
+    if constexpr (kCausal) {
+        limit = valid ? row % a.q_rows + a.causal_offset + 1 : 0;
+        limit = limit < 0 ? 0 : (limit < a.cols ? limit : a.cols);
+    }
+    const int64_t nv_lim = kCausal ? (limit + VEC - 1) / VEC : nv;
+    // the scalar operand of the unfused mul_ has the tensor's dtype
+    const CT scale_t = kCausal ? Elem<T>::widen(Elem<T>::narrow((CT)a.scale)) : (CT)1;
+    const T* res_row = kRes ? (const T*)a.residual + (valid ? row * a.cols : 0) : nullptr;
 
+    // The fused forms round the intermediate (in + residual, scale * in) to the tensor's dtype, as
+    // the separate add / mul_ of the unfused sequence would have stored it.
     auto load = [&](int64_t iv, CT* x) {
         if constexpr (VEC > 1) {
             Pack<T, VEC> v = load_pack<T, VEC>(in_row + iv * VEC);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) x[j] = Elem<T>::widen(v.v[j]);
+            if constexpr (kRes) {
+                Pack<T, VEC> r = load_pack<T, VEC>(res_row + iv * VEC);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) x[j] = Elem<T>::widen(Elem<T>::narrow(x[j] + Elem<T>::widen(r.v[j])));
+            }
         } else {
             const int64_t off = one_dim ? iv * a.sa : offset_of(a.norm_in, iv);
             x[0] = Elem<T>::widen(in_row[off]);
+            if constexpr (kRes) x[0] = Elem<T>::widen(Elem<T>::narrow(x[0] + Elem<T>::widen(res_row[iv])));
+        }
+        if constexpr (kCausal) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                x[j] = iv * VEC + j < limit ? Elem<T>::widen(Elem<T>::narrow(x[j] * scale_t)) : neg_inf<CT>();
         }
     };
     auto store = [&](int64_t iv, const CT* y) {
@@ -325,10 +385,10 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
         }
     };
 
-    if constexpr (KIND != NORM_LAYERNORM) {
+    if constexpr (!norm_is_layer(KIND)) {
         SoftStat<CT> st{neg_inf<CT>(), (CT)0};
         if (valid) {
-            for (int64_t iv = tx; iv < nv; iv += tpr) {
+            for (int64_t iv = tx; iv < nv_lim; iv += tpr) {
                 CT x[VEC];
                 load(iv, x);
                 CT cm = x[0];
@@ -346,14 +406,19 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
         }
         st = stat_all_reduce<SoftStatOp<T, CT>>(st, tpr, (SoftStat<CT>*)smem_raw);
         if (!valid) return;
-        const CT k = KIND == NORM_SOFTMAX ? (CT)1 / st.s : log_ct<T>(st.s);
+        const CT k = kLog ? log_ct<T>(st.s) : (CT)1 / st.s;
         for (int64_t iv = tx; iv < nv; iv += tpr) {
             CT x[VEC];
-            load(iv, x);
+            if (iv < nv_lim) {
+                load(iv, x);
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) x[j] = neg_inf<CT>();
+            }
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
                 CT d = x[j] - st.m;
-                x[j] = KIND == NORM_SOFTMAX ? exp_ct<T>(d) * k : d - k;
+                x[j] = kLog ? d - k : exp_ct<T>(d) * k;
             }
             store(iv, x);
         }

@@ -1,5 +1,5 @@
 // One normalisation kind (softmax, log_softmax or layernorm) for the four
-// float dtypes. Compiled once per kind with -DHPT_NORM_KIND=<0|1|2>.
+// float dtypes. Compiled once per kind with -DHPT_NORM_KIND=<0...5>.
 #include "transpose_norm.cuh"
 
 #ifndef HPT_NORM_KIND
@@ -29,15 +29,9 @@ void launch_row_reg(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block,
     }
 }
 
-template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) {
+// The transposed forms (kinds 0..2 only).
+template <class T> void launch_transposed(const NormPlan& p, const NormArgs& a, hipStream_t st) {
     constexpr int FULL = 16 / sizeof(T);
-    if (p.kind == NormKind::Empty) return;
-    a.tpr = p.tpr;
-    a.tpr_log2 = ilog2(p.tpr);
-    a.rpb = p.rpb;
-    a.inv_cols = 1.0 / (double)p.cols;
-    dim3 grid((unsigned)((p.rows + p.rpb - 1) / p.rpb));
-    dim3 block((unsigned)(p.tpr * p.rpb));
     if (p.kind == NormKind::TransposedTile) {
         TileArgs t{};
         t.in = a.in;
@@ -89,10 +83,27 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         transposed_apply_kernel<KIND, T><<<dim3(rt, (unsigned)((tiles + 3) / 4), batch), dim3(256), 0, st>>>(t);
         return;
     }
+}
+
+template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) {
+    constexpr int FULL = 16 / sizeof(T);
+    if (p.kind == NormKind::Empty) return;
+    a.tpr = p.tpr;
+    a.tpr_log2 = ilog2(p.tpr);
+    a.rpb = p.rpb;
+    a.inv_cols = 1.0 / (double)p.cols;
+    dim3 grid((unsigned)((p.rows + p.rpb - 1) / p.rpb));
+    dim3 block((unsigned)(p.tpr * p.rpb));
+    if (p.kind == NormKind::TransposedTile || p.kind == NormKind::Transposed) {
+        // the fused kinds run on the row kernels only (the caller demotes transposed plans)
+        if constexpr (KIND > NORM_LAYERNORM) fail(HPT_ERR_KERNEL, "fused normalisation: no transposed kernel for this kind");
+        else launch_transposed<T>(p, a, st);
+        return;
+    }
     if (p.kind == NormKind::RowReg) {
         // Layernorm workgroups walk the rows (gamma / beta stay in registers);
         // softmax has nothing to reuse across rows and runs one row per group.
-        if (KIND == NORM_LAYERNORM && grid.x > (unsigned)p.max_blocks) grid.x = (unsigned)p.max_blocks;
+        if (norm_is_layer(KIND) && grid.x > (unsigned)p.max_blocks) grid.x = (unsigned)p.max_blocks;
         if (p.vec == FULL && p.sstride == 2 && FULL > 1) launch_row_reg<T, FULL, 2>(p, a, grid, block, st);
         else if (p.vec == FULL) launch_row_reg<T, FULL>(p, a, grid, block, st);
         else launch_row_reg<T, 1>(p, a, grid, block, st);

@@ -424,7 +424,7 @@ class Tensor:
         return self._softmax(True, axis, **kw)
 
     def layernorm(self, normalized_shape, gamma: Optional["Tensor"] = None, beta: Optional["Tensor"] = None,
-                  eps: float = 1e-5, stream=None) -> "Tensor":
+                  eps: float = 1e-5, stream=None, residual: Optional["Tensor"] = None) -> "Tensor":
         self._require_hip("layernorm")
         ns = [int(s) for s in (normalized_shape if isinstance(normalized_shape, Iterable) else [normalized_shape])]
         if len(ns) > self.ndim or (ns and self.shape[self.ndim - len(ns):] != ns) or not ns:
@@ -445,11 +445,38 @@ class Tensor:
             beta._require_hip("layernorm beta")
             bv, k = beta._c_view()
             keep.append(k)
-        check(_ffi.lib().hpt_hip_layernorm(self.device, stream, C.byref(vin), len(ns),
-                                           C.byref(gv) if gv is not None else None,
-                                           C.byref(bv) if bv is not None else None, float(eps), C.byref(vout)))
+        gp = C.byref(gv) if gv is not None else None
+        bp = C.byref(bv) if bv is not None else None
+        if residual is not None:
+            residual._require_hip("layernorm residual")
+            rv, k = residual._c_view()
+            keep.append(k)
+            check(_ffi.lib().hpt_hip_add_layernorm(self.device, stream, C.byref(vin), C.byref(rv), len(ns), gp, bp,
+                                                   float(eps), C.byref(vout)))
+        else:
+            check(_ffi.lib().hpt_hip_layernorm(self.device, stream, C.byref(vin), len(ns), gp, bp, float(eps),
+                                               C.byref(vout)))
         del keep
         return res
+
+    # ---- fused forms of what the callers do around softmax / layernorm -----------------
+    def softmax_causal(self, scale: float = 1.0, causal_offset: int = 0, log: bool = False, stream=None) -> "Tensor":
+        """softmax(-1) of scale * self with keys above query + causal_offset masked out: the sequence
+        `scores.mul_(scaling)`, fill -inf where key > query, `softmax(-1)` of
+        hpt-examples/examples/transformer/main.rs:233-246 in one pass; the masked part is never read."""
+        self._require_hip("softmax_causal")
+        res = Tensor.empty(self.shape, self.dtype, self.device)
+        vin, k1 = self._c_view()
+        vout, k2 = res._c_view()
+        check(_ffi.lib().hpt_hip_softmax_causal(self.device, stream, int(log), C.byref(vin), float(scale),
+                                                int(causal_offset), C.byref(vout)))
+        del k1, k2
+        return res
+
+    def add_layernorm(self, residual: "Tensor", normalized_shape, gamma: Optional["Tensor"] = None,
+                      beta: Optional["Tensor"] = None, eps: float = 1e-5, stream=None) -> "Tensor":
+        """layernorm(self + residual) (hpt-examples/examples/transformer/main.rs:87-91) in one pass."""
+        return self.layernorm(normalized_shape, gamma, beta, eps, stream=stream, residual=residual)
 
     # ---- the steps either side of the path ------------------------------------------
     def contiguous(self, stream=None) -> "Tensor":

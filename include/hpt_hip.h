@@ -209,6 +209,30 @@ int32_t hpt_hip_softmax(int32_t dev, void* stream, int32_t log, const hpt_view* 
 int32_t hpt_hip_layernorm(int32_t dev, void* stream, const hpt_view* in, int32_t n_norm_dims,
                           const hpt_view* gamma, const hpt_view* beta, double eps, hpt_view* out);
 
+/* ---- fused forms of what the callers do around softmax / layernorm ---------
+ * No trait of the reference has these signatures; they fuse the exact sequences its
+ * transformer example runs (hpt-examples/examples/transformer/main.rs) and give the
+ * results those sequences give. */
+
+/* scores.mul_(scaling) -> fill -inf where key > query -> softmax(-1)
+ * (hpt-examples/examples/transformer/main.rs:233-246, with the mask of :79 `tri`): the
+ * causal mask is a PARAMETER, not data: row q of every (Q x K) matrix (Q = in.shape[ndim-2],
+ * K = the last dim) keeps keys 0 .. q + causal_offset; the masked part of the input is never
+ * read (its outputs are 0, or -inf for log). `scale` is rounded to in's dtype (the scalar
+ * operand of `mul_` has it) and scale * x is rounded to in's dtype before the softmax, as
+ * the separate `mul_` would have stored it. A row with no key left is NaN, like
+ * softmax of a row of -inf. `in` any strided view of a float dtype with ndim >= 2, `out`
+ * contiguous. */
+int32_t hpt_hip_softmax_causal(int32_t dev, void* stream, int32_t log, const hpt_view* in, double scale,
+                               int64_t causal_offset, hpt_view* out);
+
+/* layernorm(x + residual) (hpt-examples/examples/transformer/main.rs:87-91): the sum is
+ * rounded to the tensors' dtype, as the separate `+` would have stored it, then
+ * normalised as hpt_hip_layernorm does. `residual`: contiguous, in's shape and dtype. */
+int32_t hpt_hip_add_layernorm(int32_t dev, void* stream, const hpt_view* in, const hpt_view* residual,
+                              int32_t n_norm_dims, const hpt_view* gamma, const hpt_view* beta, double eps,
+                              hpt_view* out);
+
 /* ---- the steps either side of the path ------------------------------------
  * What the callers of reductions and normalisations do to their operands just
  * before and after, kept on the device. */
