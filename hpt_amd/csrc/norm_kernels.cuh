@@ -282,17 +282,18 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
 
 // ---- streaming rows: online statistics, then a second sweep ------------------
 
-// running (max, sum of exp(x - max))
-template <class CT> struct SoftStat {
-    CT m, s;
+// running (max, sum of exp(x - max)); the sum may be carried in a wider type ST
+template <class CT, class ST = CT> struct SoftStat {
+    CT m;
+    ST s;
 };
-template <class T, class CT> struct SoftStatOp {
-    __device__ static __forceinline__ SoftStat<CT> comb(SoftStat<CT> a, SoftStat<CT> b) {
-        SoftStat<CT> r;
+template <class T, class CT, class ST = CT> struct SoftStatOp {
+    __device__ static __forceinline__ SoftStat<CT, ST> comb(SoftStat<CT, ST> a, SoftStat<CT, ST> b) {
+        SoftStat<CT, ST> r;
         r.m = MaxC<CT>::comb(a.m, b.m);
         // a side that has seen nothing (m = -inf, s = 0) must not produce inf - inf
-        CT sa = a.s == (CT)0 ? (CT)0 : a.s * exp_ct<T>(a.m - r.m);
-        CT sb = b.s == (CT)0 ? (CT)0 : b.s * exp_ct<T>(b.m - r.m);
+        ST sa = a.s == (ST)0 ? (ST)0 : a.s * (ST)exp_ct<T>(a.m - r.m);
+        ST sb = b.s == (ST)0 ? (ST)0 : b.s * (ST)exp_ct<T>(b.m - r.m);
         r.s = sa + sb;
         return r;
     }
@@ -386,7 +387,11 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
     };
 
     if constexpr (!norm_is_layer(KIND)) {
-        SoftStat<CT> st{neg_inf<CT>(), (CT)0};
+        // A lane may sum a whole row by itself here (tpr = 1: thousands of terms one after the
+        // other), so f32 rows carry the sum of exponentials in f64: sequential f32 addition would
+        // lose about sqrt(n) ulps, which shows in log_softmax values near zero.
+        using ST = typename StatType<T>::type;
+        SoftStat<CT, ST> st{neg_inf<CT>(), (ST)0};
         if (valid) {
             for (int64_t iv = tx; iv < nv_lim; iv += tpr) {
                 CT x[VEC];
@@ -395,18 +400,20 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
 #pragma unroll
                 for (int j = 1; j < VEC; ++j) cm = MaxC<CT>::comb(cm, x[j]);
                 if (cm > st.m) {
-                    st.s = st.s == (CT)0 ? (CT)0 : st.s * exp_ct<T>(st.m - cm);
+                    st.s = st.s == (ST)0 ? (ST)0 : st.s * (ST)exp_ct<T>(st.m - cm);
                     st.m = cm;
                 }
                 if (st.m > neg_inf<CT>()) {
+                    CT part = 0;  // the few elements of one vector add up in the compute type
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) st.s += exp_ct<T>(x[j] - st.m);
+                    for (int j = 0; j < VEC; ++j) part += exp_ct<T>(x[j] - st.m);
+                    st.s += (ST)part;
                 }
             }
         }
-        st = stat_all_reduce<SoftStatOp<T, CT>>(st, tpr, (SoftStat<CT>*)smem_raw);
+        st = stat_all_reduce<SoftStatOp<T, CT, ST>>(st, tpr, (SoftStat<CT, ST>*)smem_raw);
         if (!valid) return;
-        const CT k = kLog ? log_ct<T>(st.s) : (CT)1 / st.s;
+        const CT k = kLog ? log_ct<T>((CT)st.s) : (CT)((ST)1 / st.s);
         for (int64_t iv = tx; iv < nv; iv += tpr) {
             CT x[VEC];
             if (iv < nv_lim) {

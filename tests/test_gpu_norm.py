@@ -242,3 +242,17 @@ def test_transposed_tile_masked_and_constant_rows(hpt, dev):
     assert hpt.normalize_plan(tc, 1).startswith("transposed-tile")
     out = tc.layernorm([200], hpt.Tensor.from_numpy(g).to_hip(dev), hpt.Tensor.from_numpy(b).to_hip(dev), 1e-5).numpy()
     assert np.array_equal(out, np.broadcast_to(b, out.shape))
+
+
+def test_log_softmax_long_columns_keep_the_absolute_tolerance(hpt, orc, dev):
+    """Column softmax where one lane sums a whole column (1012 terms one after the other): the entry at the
+    column's maximum is -ln(sum) ~ -0.004, so the sum must be right to better than 1e-6 relative for the
+    absolute tolerance to hold; the running sum is carried in f64."""
+    rng = np.random.default_rng(207)
+    base = (rng.standard_normal((1012, 1266)) * 3).astype(np.float32)
+    t, a = upload(hpt, base, dev=dev)
+    assert hpt.normalize_plan(t, 0).startswith("col")
+    got = t.log_softmax(0).numpy()
+    want = orc.softmax(a, 0, log=True, acc=orc.ACC_F64)
+    assert_close(got, want, F32_RTOL, F32_ATOL, "log_softmax over 1012-term columns")
+    assert_close(t.softmax(0).numpy(), orc.softmax(a, 0, acc=orc.ACC_F64), F32_RTOL, F32_ATOL, "softmax columns")
