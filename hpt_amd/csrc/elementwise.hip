@@ -15,6 +15,13 @@ namespace hpt {
 
 namespace {
 
+#ifndef EW_UNR2
+#define EW_UNR2 2
+#endif
+// vectors per thread: a copy keeps four loads in flight per thread; with two operands two
+// vectors each are better (more workgroups resident, the same bytes in flight)
+template <int NIN> constexpr int ew_unroll() { return NIN == 2 ? EW_UNR2 : 4; }
+
 struct EwArgs {
     void* out;
     const void* in[2];
@@ -47,8 +54,8 @@ template <int OP, class T> struct BinOp {
 };
 
 // ---- lanes along the innermost dim ---------------------------------------------------
-// Thread t of a workgroup takes vectors t, t + 256, t + 512, t + 768 of the workgroup's
-// 1024: four loads per operand are in flight before the first result is stored.
+// Thread t of a workgroup takes vectors t, t + 256, ... of the workgroup's 256 * UNR: UNR loads
+// per operand are in flight before the first result is stored.
 // SS = 2 (copy only): the innermost dim has input stride 2 (a [:, ::2] view): two full
 // vectors are loaded per output vector and the odd positions dropped, which moves the same
 // cache lines as a gather of single elements with a fraction of the instructions. (A
@@ -56,7 +63,7 @@ template <int OP, class T> struct BinOp {
 // the unused last element of the last vector is safe to touch.)
 template <int OP, class T, int VEC, int NIN, int SS = 1>
 __global__ void __launch_bounds__(256) ew_inner_kernel(const EwArgs a) {
-    constexpr int UNR = 4;
+    constexpr int UNR = ew_unroll<NIN>();
     Pack<T, VEC> x[UNR], y[UNR];
     int64_t vi[UNR];
     const int last = a.n - 1;
@@ -216,7 +223,7 @@ template <int OP, class T, int NIN>
 void launch_inner(const EwPlan& p, void* out, const void* in0, const void* in1, hipStream_t st) {
     constexpr int FULL = 16 / sizeof(T);
     const EwArgs a = make_args(p, out, in0, in1);
-    const int64_t blocks = (a.total_v + 1023) / 1024;
+    const int64_t blocks = (a.total_v + 256 * ew_unroll<NIN>() - 1) / (256 * ew_unroll<NIN>());
     if (blocks > 0x7fffffff) fail(HPT_ERR_SHAPE, "elementwise: tensor too large for one launch");
     if constexpr (NIN == 1 && FULL > 1) {
         if (p.vec == FULL && p.sstride == 2) {
