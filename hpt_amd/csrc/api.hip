@@ -156,16 +156,14 @@ static DeviceAllocator& allocator_of(int dev) {
 struct StreamScratch {
     void* partial = nullptr;
     size_t partial_bytes = 0;
-    unsigned* counters = nullptr;
-    size_t n_counters = 0;
 };
 
 static std::mutex g_scratch_mu;  // held from lookup to launch
 static std::map<std::pair<int, hipStream_t>, StreamScratch> g_scratch;
 
 // Requires g_scratch_mu. Grows the scratch of (dev, stream); growing frees the
-// old buffers, which waits for the device to go idle first.
-static ReduceScratch scratch_for(int dev, hipStream_t st, size_t partial_bytes, size_t counters) {
+// old buffer, which waits for the device to go idle first.
+static ReduceScratch scratch_for(int dev, hipStream_t st, size_t partial_bytes) {
     StreamScratch& s = g_scratch[{dev, st}];
     if (partial_bytes > s.partial_bytes) {
         if (s.partial) hip_check(hipFree(s.partial), HPT_ERR_MEMORY, "hipFree(scratch)");
@@ -175,26 +173,13 @@ static ReduceScratch scratch_for(int dev, hipStream_t st, size_t partial_bytes, 
         hip_check(hipMalloc(&s.partial, want), HPT_ERR_MEMORY, "hipMalloc(scratch)");
         s.partial_bytes = want;
     }
-    if (counters > s.n_counters) {
-        if (s.counters) hip_check(hipFree(s.counters), HPT_ERR_MEMORY, "hipFree(counters)");
-        s.counters = nullptr;
-        s.n_counters = 0;
-        size_t want = std::max<size_t>(counters, 4096);
-        hip_check(hipMalloc((void**)&s.counters, want * sizeof(unsigned)), HPT_ERR_MEMORY,
-                  "hipMalloc(counters)");
-        hip_check(hipMemset(s.counters, 0, want * sizeof(unsigned)), HPT_ERR_MEMORY,
-                  "hipMemset(counters)");
-        s.n_counters = want;
-    }
     ReduceScratch r;
     r.partial = s.partial;
-    r.counters = s.counters;
     return r;
 }
 
-void scratch_need(const ReducePlan& p, size_t acc_size, size_t* partial_bytes, size_t* counters) {
-    *counters = 0;
-    *partial_bytes = p.split > 1 ? (size_t)p.K * p.split * acc_size : 0;
+size_t scratch_need(const ReducePlan& p, size_t acc_size) {
+    return p.split > 1 ? (size_t)p.K * p.split * acc_size : 0;
 }
 
 // ---- dispatch tables -----------------------------------------------------------
@@ -319,11 +304,10 @@ static void run_reduce(int dev, void* stream, int entry_id, const hpt_view* in, 
     use_device(dev);
     hipStream_t st = (hipStream_t)stream;
     ReduceLaunchFn fn = c.entry->launch[in->dtype];
-    size_t pbytes, ncount;
-    scratch_need(c.plan, c.entry->acc_size[in->dtype], &pbytes, &ncount);
+    const size_t pbytes = scratch_need(c.plan, c.entry->acc_size[in->dtype]);
     if (pbytes) {
         std::lock_guard<std::mutex> g(g_scratch_mu);
-        ReduceScratch sc = scratch_for(dev, st, pbytes, ncount);
+        ReduceScratch sc = scratch_for(dev, st, pbytes);
         fn(c.plan, in->data, out->data, sc, st, init_out);
         check_launch("reduce");
     } else {
@@ -373,7 +357,7 @@ static NormCall prepare_norm(const hpt_view* in, const void* out_data, int64_t a
 static void launch_norm(int dev, hipStream_t st, NormLaunchFn fn, NormCall& c, const char* what) {
     if (c.plan.scratch_bytes) {
         std::lock_guard<std::mutex> g(g_scratch_mu);
-        c.args.scratch = scratch_for(dev, st, c.plan.scratch_bytes, 0).partial;
+        c.args.scratch = scratch_for(dev, st, c.plan.scratch_bytes).partial;
         fn(c.plan, c.args, st);
         check_launch(what);
     } else {

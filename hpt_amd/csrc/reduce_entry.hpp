@@ -9,15 +9,14 @@
 
 namespace hpt {
 
-// Library-owned scratch of the multi-workgroup reductions: partial
-// accumulators and one arrival counter per output group (zero between launches).
+// Library-owned scratch of the reductions that are split over workgroups: the
+// partial accumulators the first stage writes and the second stage folds.
 struct ReduceScratch {
     void* partial = nullptr;
-    unsigned* counters = nullptr;
 };
 
-// Bytes of partial-accumulator scratch and number of counters a plan needs.
-void scratch_need(const ReducePlan& p, size_t acc_size, size_t* partial_bytes, size_t* counters);
+// Bytes of partial-accumulator scratch a plan needs (0: a single stage).
+size_t scratch_need(const ReducePlan& p, size_t acc_size);
 
 using ReduceLaunchFn = void (*)(const ReducePlan&, const void* in, void* out,
                                 const ReduceScratch&, hipStream_t, int init_out);

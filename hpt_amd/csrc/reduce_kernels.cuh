@@ -229,7 +229,6 @@ struct ColLeanArgs {
     int kin_v;       // inner kept length in vectors
     int sk;          // inner kept stride in elements (1 when VEC > 1)
     int R;           // reduced length
-    int chunk;       // reduced indices per split
     int split, init_out;
 };
 
@@ -495,7 +494,6 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
         a.kin_v = (int)(kin / (p.vec / p.sstride));
         a.sk = nk ? (int)p.kept.stride[nk - 1] : 1;
         a.R = (int)p.R;
-        a.chunk = (int)p.chunk;
         a.split = p.split;
         a.init_out = init_out;
         const int64_t outer = nk > 1 ? p.kept.size[0] : 1;
