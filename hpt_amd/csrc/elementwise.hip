@@ -26,10 +26,10 @@ struct EwArgs {
     void* out;
     const void* in[2];
     int64_t stride[2][kMaxDims];
-    int size[kMaxDims];
+    int64_t size[kMaxDims];
     int n;
     int64_t total_v;  // vectors (of VEC output elements) in all
-    int inner_v;      // vectors along the innermost dim
+    int64_t inner_v;  // vectors along the innermost dim
 };
 
 // ---- operators ---------------------------------------------------------------------
@@ -211,10 +211,10 @@ EwArgs make_args(const EwPlan& p, void* out, const void* in0, const void* in1) {
     a.in[1] = in1;
     a.n = p.n;
     for (int i = 0; i < p.n; ++i) {
-        a.size[i] = (int)p.size[i];
+        a.size[i] = p.size[i];
         for (int k = 0; k < p.nin; ++k) a.stride[k][i] = p.stride[k][i];
     }
-    a.inner_v = (int)(p.size[p.n - 1] / p.vec);
+    a.inner_v = p.size[p.n - 1] / p.vec;
     a.total_v = p.total / p.vec;
     return a;
 }

@@ -136,7 +136,9 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
     int64_t sr = p.red.n ? iabs(p.red.stride[p.red.n - 1]) : INT64_MAX;
     int64_t sk = p.kept.n ? iabs(p.kept.stride[p.kept.n - 1]) : INT64_MAX;
 
-    const int64_t kI32 = 0x7fffffff;
+    // the lean kernels index with 32-bit integers and form sums of two such values
+    // (chunk starts plus chunk lengths, positions plus batch steps): stay below 2^30
+    const int64_t kI32 = 1 << 30;
     if (p.red.n > 0 && (p.kept.n == 0 || sr <= sk)) {
         // ---- Row: lanes walk the reduced index space ---------------------
         p.kind = ReduceKind::Row;
@@ -508,8 +510,6 @@ EwPlan plan_elementwise(const void* out_data, const int64_t* shape, int ndim, in
         p.size[0] = 1;
         for (int k = 0; k < nin; ++k) p.stride[k][0] = 1;
     }
-    for (int i = 0; i < p.n; ++i)
-        if (p.size[i] > 0x7fffffff) fail(HPT_ERR_SHAPE, "elementwise: a coalesced dim exceeds 2^31 - 1 elements");
     p.kind = EwKind::Inner;
     const int full = (int)(16 / elem_size);
     const int last = p.n - 1;
@@ -550,7 +550,8 @@ EwPlan plan_elementwise(const void* out_data, const int64_t* shape, int ndim, in
             if (p.stride[0][i] == 1) t = i;
         if (t >= 0 && p.n <= 6) {
             bool ok = aligned(out_data) && aligned(in_data[0]) && p.size[last] % full == 0 && p.size[t] % full == 0 &&
-                      p.size[last] >= 2 * full && p.size[t] >= 2 * full;
+                      p.size[last] >= 2 * full && p.size[t] >= 2 * full && p.size[last] <= (1 << 30) &&
+                      p.size[t] <= (1 << 30);
             for (int i = 0; i < p.n; ++i)
                 if (i != t && p.stride[0][i] % full != 0) ok = false;
             // the remaining dims ride on blockIdx.z
