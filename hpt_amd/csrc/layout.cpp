@@ -361,7 +361,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                           p.kept_in.size[nk - 1] % v == 0 && p.cols % v == 0 && sa % v == 0 &&
                           (nk == 1 || (p.kept_in.stride[0] % v == 0 && p.kept_in.size[0] <= 65535)) &&
                           ((uintptr_t)in_data % 16) == 0 && ((uintptr_t)out_data % 16) == 0 &&
-                          p.kept_in.size[nk - 1] <= 0x7fffffff && p.cols <= 0x7fffffff &&
+                          p.kept_in.size[nk - 1] <= (1 << 30) && p.cols <= (1 << 30) &&  // 32-bit positions
                           p.kept_in.size[nk - 1] >= 8 * v && p.cols >= 8 * v;
         if (transposed) {
             p.vec = v;
