@@ -42,3 +42,33 @@ def test_two_dims_total_beyond_int32(hpt, dev):
     assert np.array_equal(tt.sum([0]).numpy(), a.sum(1, dtype=np.int8))
     c = tt[(1 << 30) - 5:].contiguous().numpy()                                  # offsets beyond 2^31 bytes
     assert np.array_equal(c, a.T[(1 << 30) - 5:])
+
+
+def test_normalisation_beyond_int32_elements(hpt, orc, dev):
+    """f16 [2^20, 2304] (2.4 G elements): row kernels with 64-bit row offsets; checked on the first and last
+    rows against the oracle and on every row through the sum-to-one property."""
+    from conftest import assert_close
+    rows, cols = 1 << 20, 2304
+    rng = np.random.default_rng(502)
+    block = (rng.standard_normal((1 << 12, cols)) * 2).astype(np.float16)
+    a = np.tile(block, (rows >> 12, 1))
+    a[-3:] += np.float16(1.5)          # make the last rows differ from the tiled pattern
+    t = hpt.Tensor.from_numpy(a).to_hip(dev)
+    s = t.softmax(1).numpy()
+    sel = np.r_[0:64, rows - 64:rows]
+    want = orc.softmax(np.ascontiguousarray(a[sel]), 1, acc=orc.ACC_F32).astype(np.float32)
+    assert_close(s[sel].astype(np.float32), want, 1e-2, 6e-8, "softmax rows at both ends")
+    sums = s.astype(np.float32).sum(1)
+    assert np.all(np.abs(sums - 1) < 2e-2)
+    del s
+    g = rng.normal(1, 0.1, cols).astype(np.float16)
+    ln = t.layernorm([cols], hpt.Tensor.from_numpy(g).to_hip(dev), None, 1e-5).numpy()
+    want = orc.layernorm(np.ascontiguousarray(a[sel]), 1, g, None, 1e-5, acc=orc.ACC_F32).astype(np.float32)
+    assert_close(ln[sel].astype(np.float32), want, 1e-2, 2e-3, "layernorm rows at both ends")
+    del ln
+    # columns: softmax over axis 0 of the transposed view's base layout ([cols, rows] rows contiguous)
+    b = np.ascontiguousarray(a[:, :8].T)          # [8, 2^20]
+    tb = hpt.Tensor.from_numpy(b).to_hip(dev)
+    got = tb.softmax(0).numpy().astype(np.float32)
+    want = orc.softmax(b, 0, acc=orc.ACC_F32).astype(np.float32)
+    assert_close(got, want, 1e-2, 6e-8, "column softmax")
