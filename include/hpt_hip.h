@@ -113,7 +113,9 @@ int32_t hpt_hip_device_count(int32_t* n);
 /* Allocator::allocate / allocate_zeroed (hpt-allocator/src/traits.rs:25-41). */
 int32_t hpt_hip_alloc(int32_t dev, size_t bytes, size_t align, int32_t zeroed, void** out);
 /* Allocator::deallocate (hpt-allocator/src/traits.rs:43-50): returns the block
- * to the cache. `p` must come from hpt_hip_alloc with the same (bytes, align). */
+ * to the cache. `p` must come from hpt_hip_alloc with the same (bytes, align).
+ * The block may be handed out again at once: free it only after the stream that
+ * last used it has finished with it. */
 int32_t hpt_hip_free(int32_t dev, void* p, size_t bytes, size_t align);
 /* resize_cuda_lru_cache (hpt/src/lib.rs:449-450). Evicted blocks are released. */
 int32_t hpt_hip_cache_resize(int32_t dev, size_t entries);
