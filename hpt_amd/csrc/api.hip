@@ -687,6 +687,31 @@ int32_t hpt_hip_contiguous_plan(const hpt_view* in, const hpt_view* out, char* b
     });
 }
 
+int32_t hpt_hip_cast(int32_t dev, void* stream, const hpt_view* in, hpt_view* out) {
+    return guarded([&] {
+        check_view(in, "cast input", true);
+        check_view(out, "cast output", true);
+        if (!view_contiguous(out)) fail(HPT_ERR_SHAPE, "cast output: output tensor must be contiguous");
+        check_same_shape(in, out, "cast");
+        if (in->dtype == out->dtype) {
+            const EwPlan p = prepare_copy(in, out);
+            if (p.kind == EwKind::Empty) return;
+            use_device(dev);
+            launch_strided_copy(in->dtype, p, out->data, in->data, (hipStream_t)stream);
+            check_launch("cast");
+            return;
+        }
+        const size_t es = std::max(dtype_size(in->dtype), dtype_size(out->dtype));
+        const void* datas[1] = {in->data};
+        const int64_t* strides[1] = {in->strides};
+        const EwPlan p = plan_elementwise(out->data, in->shape, in->ndim, 1, datas, strides, es, false);
+        if (p.kind == EwKind::Empty) return;
+        use_device(dev);
+        launch_cast(in->dtype, out->dtype, p, out->data, in->data, (hipStream_t)stream);
+        check_launch("cast");
+    });
+}
+
 int32_t hpt_hip_fill(int32_t dev, void* stream, hpt_view* out, const void* value) {
     return guarded([&] {
         check_view(out, "fill output", true);

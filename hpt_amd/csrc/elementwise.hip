@@ -53,6 +53,37 @@ template <int OP, class T> struct BinOp {
     }
 };
 
+// Innermost position (in vectors) of output vector `v` and the operands' element offsets of
+// its outer position.
+template <int NIN>
+__device__ __forceinline__ void ew_locate(const EwArgs& a, int64_t v, int64_t& iv, int64_t (&off)[2]) {
+    const int last = a.n - 1;
+    off[0] = off[1] = 0;
+    if (((uint64_t)a.total_v >> 31) == 0) {
+        uint32_t r = (uint32_t)v;
+        uint32_t q = r / (uint32_t)a.inner_v;
+        iv = r - q * (uint32_t)a.inner_v;
+        for (int i = last - 1; i >= 0; --i) {
+            const uint32_t s = (uint32_t)a.size[i];
+            const uint32_t q2 = q / s;
+            const uint32_t idx = q - q2 * s;
+            q = q2;
+#pragma unroll
+            for (int k = 0; k < NIN; ++k) off[k] += (int64_t)idx * a.stride[k][i];
+        }
+    } else {
+        int64_t q = v / a.inner_v;
+        iv = v - q * a.inner_v;
+        for (int i = last - 1; i >= 0; --i) {
+            const int64_t q2 = q / a.size[i];
+            const int64_t idx = q - q2 * a.size[i];
+            q = q2;
+#pragma unroll
+            for (int k = 0; k < NIN; ++k) off[k] += idx * a.stride[k][i];
+        }
+    }
+}
+
 // ---- lanes along the innermost dim ---------------------------------------------------
 // Thread t of a workgroup takes vectors t, t + 256, ... of the workgroup's 256 * UNR: UNR loads
 // per operand are in flight before the first result is stored.
@@ -72,32 +103,8 @@ __global__ void __launch_bounds__(256) ew_inner_kernel(const EwArgs a) {
         const int64_t v = ((int64_t)blockIdx.x * UNR + u) * 256 + threadIdx.x;
         vi[u] = v;
         if (v >= a.total_v) continue;
-        // innermost position and the operands' offsets of the outer position
-        int64_t off[2] = {0, 0};
-        int64_t iv;
-        if (((uint64_t)a.total_v >> 31) == 0) {
-            uint32_t r = (uint32_t)v;
-            uint32_t q = r / (uint32_t)a.inner_v;
-            iv = r - q * (uint32_t)a.inner_v;
-            for (int i = last - 1; i >= 0; --i) {
-                const uint32_t s = (uint32_t)a.size[i];
-                const uint32_t q2 = q / s;
-                const uint32_t idx = q - q2 * s;
-                q = q2;
-#pragma unroll
-                for (int k = 0; k < NIN; ++k) off[k] += (int64_t)idx * a.stride[k][i];
-            }
-        } else {
-            int64_t q = v / a.inner_v;
-            iv = v - q * a.inner_v;
-            for (int i = last - 1; i >= 0; --i) {
-                const int64_t q2 = q / a.size[i];
-                const int64_t idx = q - q2 * a.size[i];
-                q = q2;
-#pragma unroll
-                for (int k = 0; k < NIN; ++k) off[k] += idx * a.stride[k][i];
-            }
-        }
+        int64_t off[2], iv;
+        ew_locate<NIN>(a, v, iv, off);
         auto fetch = [&](int k, Pack<T, VEC>& dst) {
             const T* p = (const T*)a.in[k] + off[k];
             const int64_t s = a.stride[k][last];
@@ -190,6 +197,70 @@ __global__ void __launch_bounds__(256) ew_transpose_kernel(const TransposeArgs a
 #pragma unroll
         for (int i = 0; i < VEC; ++i) o.v[i] = v[i].v[k];
         store_pack_stream<U, VEC>(out + (int64_t)k * a.oB, o);
+    }
+}
+
+// ---- dtype casts ----------------------------------------------------------------------
+// Scalar<T>::cast as astype uses it (hpt/src/backends/cuda/tensor_impls.rs:129-140): integers go
+// to a float type through Rust's `as` (round to nearest even; f16 / bf16 through f32, as the
+// generated conversions do), floats to floats with ONE rounding. f64 -> f16 / bf16 has no
+// hardware instruction: the value is first rounded to f32 "to odd" (truncate, then set the
+// last bit if anything was lost), which makes the second, nearest-even rounding exact.
+__device__ __forceinline__ float double_to_float_round_to_odd(double d) {
+    float f = (float)d;
+    if ((double)f != d && d == d && fabsf(f) != __builtin_huge_valf()) {
+        uint32_t u = __float_as_uint(f);
+        if (fabs((double)f) > fabs(d)) u -= 1;  // step back towards zero
+        u |= 1u;
+        f = __uint_as_float(u);
+    }
+    return f;
+}
+
+template <class TI, class TO> __device__ __forceinline__ TO cast_elem(TI x) {
+    if constexpr (std::is_same<TI, TO>::value) {
+        return x;
+    } else if constexpr (Elem<TO>::is_float) {
+        using WO = typename Elem<TO>::Wide;
+        if constexpr (Elem<TI>::is_bool) {
+            return Elem<TO>::narrow((WO)(x.v != 0));
+        } else if constexpr (Elem<TI>::is_float) {
+            if constexpr (std::is_same<TI, double>::value && sizeof(TO) == 2)
+                return Elem<TO>::narrow(double_to_float_round_to_odd(x));
+            else
+                return Elem<TO>::narrow((WO)Elem<TI>::widen(x));
+        } else {
+            return Elem<TO>::narrow((WO)x);
+        }
+    } else {
+        static_assert(sizeof(TI) == 0, "cast to a non-float dtype is not provided");
+    }
+}
+
+template <class TI, class TO, int VEC>
+__global__ void __launch_bounds__(256) ew_cast_kernel(const EwArgs a) {
+    constexpr int UNR = 4;
+    Pack<TI, VEC> x[UNR];
+    int64_t vi[UNR];
+    const int last = a.n - 1;
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+        const int64_t v = ((int64_t)blockIdx.x * UNR + u) * 256 + threadIdx.x;
+        vi[u] = v;
+        if (v >= a.total_v) continue;
+        int64_t off[2], iv;
+        ew_locate<1>(a, v, iv, off);
+        const TI* p = (const TI*)a.in[0] + off[0];
+        if constexpr (VEC > 1) x[u] = load_pack<TI, VEC>(p + iv * VEC);
+        else x[u].v[0] = p[iv * a.stride[0][last]];
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+        if (vi[u] >= a.total_v) continue;
+        Pack<TO, VEC> r;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) r.v[j] = cast_elem<TI, TO>(x[u].v[j]);
+        store_pack<TO, VEC>((TO*)a.out + vi[u] * VEC, r);
     }
 }
 
@@ -345,6 +416,48 @@ void launch_fill(int dtype, void* out, int64_t n, const void* value, hipStream_t
             default: { uint64_t v; memcpy(&v, value, 8); fill_scalar_kernel<uint64_t><<<blocks, 256, 0, st>>>((uint64_t*)q, v, rest); break; }
         }
     }
+}
+
+namespace {
+
+template <class TI, class TO> void launch_cast_t(const EwPlan& p, void* out, const void* in, hipStream_t st) {
+    // vector width of the wider of the two types (the plan was made for it)
+    constexpr int FULL = 16 / (sizeof(TI) > sizeof(TO) ? sizeof(TI) : sizeof(TO));
+    const EwArgs a = make_args(p, out, in, nullptr);
+    const int64_t blocks = (a.total_v + 1023) / 1024;
+    if (blocks > 0x7fffffff) fail(HPT_ERR_SHAPE, "cast: tensor too large for one launch");
+    if (p.vec == FULL && FULL > 1) ew_cast_kernel<TI, TO, FULL><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a);
+    else ew_cast_kernel<TI, TO, 1><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a);
+}
+
+template <class TO> bool launch_cast_to(int in_dtype, const EwPlan& p, void* out, const void* in, hipStream_t st) {
+    switch (in_dtype) {
+#define HPT_CASE(DT)                                                      \
+    case DT:                                                              \
+        launch_cast_t<typename DType<DT>::type, TO>(p, out, in, st);      \
+        return true;
+        HPT_CASE(HPT_BOOL) HPT_CASE(HPT_I8) HPT_CASE(HPT_I16) HPT_CASE(HPT_I32) HPT_CASE(HPT_I64) HPT_CASE(HPT_U8)
+        HPT_CASE(HPT_U16) HPT_CASE(HPT_U32) HPT_CASE(HPT_U64) HPT_CASE(HPT_F16) HPT_CASE(HPT_BF16) HPT_CASE(HPT_F32)
+        HPT_CASE(HPT_F64)
+#undef HPT_CASE
+        default: return false;
+    }
+}
+
+}  // namespace
+
+void launch_cast(int in_dtype, int out_dtype, const EwPlan& p, void* out, const void* in, hipStream_t st) {
+    if (p.kind == EwKind::Empty) return;
+    bool ok = false;
+    switch (out_dtype) {
+        case HPT_F16: ok = launch_cast_to<f16_t>(in_dtype, p, out, in, st); break;
+        case HPT_BF16: ok = launch_cast_to<bf16_t>(in_dtype, p, out, in, st); break;
+        case HPT_F32: ok = launch_cast_to<float>(in_dtype, p, out, in, st); break;
+        case HPT_F64: ok = launch_cast_to<double>(in_dtype, p, out, in, st); break;
+        default: break;
+    }
+    if (!ok) fail(HPT_ERR_DTYPE, "cast: %s -> %s is not provided (the output must be a float dtype)", dtype_name(in_dtype),
+                  dtype_name(out_dtype));
 }
 
 }  // namespace hpt

@@ -410,6 +410,10 @@ class Tensor:
     # ---- NormalizationOps (hpt-traits/src/ops/normalization.rs:6-64) ------------
     def _softmax(self, log: bool, axis: int, stream=None) -> "Tensor":
         self._require_hip("softmax")
+        ft = self._float_binary_type()
+        if ft is not self.dtype:
+            # NormalizationOps::Output = Tensor<FloatBinaryType<T>>: a non-float input is cast first
+            return self.astype(ft, stream=stream)._softmax(log, axis, stream=stream)
         res = Tensor.empty(self.shape, self.dtype, self.device)
         vin, k1 = self._c_view()
         vout, k2 = res._c_view()
@@ -432,6 +436,10 @@ class Tensor:
             raise ShapeError(_ffi.ERR_SHAPE,
                              "normalized dims must match last dims of input tensor, "
                              f"shape: {self.shape}, normalized_shape: {ns}")
+        ft = self._float_binary_type()
+        if ft is not self.dtype:
+            return self.astype(ft, stream=stream).layernorm(normalized_shape, gamma, beta, eps, stream=stream,
+                                                            residual=residual)
         res = Tensor.empty(self.shape, self.dtype, self.device)
         vin, k1 = self._c_view()
         vout, k2 = res._c_view()
@@ -479,6 +487,22 @@ class Tensor:
         return self.layernorm(normalized_shape, gamma, beta, eps, stream=stream, residual=residual)
 
     # ---- the steps either side of the path ------------------------------------------
+    def astype(self, dtype: DType, stream=None) -> "Tensor":
+        """astype (hpt/src/backends/cuda/tensor_impls.rs:129-140) to a float dtype (or to the same dtype)."""
+        self._require_hip("astype")
+        res = Tensor.empty(self.shape, dtype, self.device)
+        vin, k1 = self._c_view()
+        vout, k2 = res._c_view()
+        check(_ffi.lib().hpt_hip_cast(self.device, stream, C.byref(vin), C.byref(vout)))
+        del k1, k2
+        return res
+
+    def _float_binary_type(self) -> DType:
+        """FloatBinaryType<T> (hpt-types/src/type_promote.rs): the output dtype of the float-valued entries."""
+        out = C.c_int32()
+        check(_ffi.lib().hpt_hip_reduce_out_dtype(MEAN, self.dtype.code, C.byref(out)))
+        return DTYPES[out.value]
+
     def contiguous(self, stream=None) -> "Tensor":
         """Contiguous::contiguous (hpt/src/backends/cuda/tensor_internal/normal_out_unary.rs:286-310):
         a new contiguous tensor with this view's elements."""

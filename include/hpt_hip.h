@@ -248,6 +248,14 @@ int32_t hpt_hip_contiguous(int32_t dev, void* stream, const hpt_view* in, hpt_vi
 /* Describes the kernel hpt_hip_contiguous would pick (tests, tuning). */
 int32_t hpt_hip_contiguous_plan(const hpt_view* in, const hpt_view* out, char* buf, size_t buflen);
 
+/* astype (hpt/src/backends/cuda/tensor_impls.rs:129-140; the cast every FloatReduce /
+ * NormalizationOps entry applies to a non-float input, whose output dtype is
+ * FloatBinaryType<T>: hpt-types/src/type_promote.rs): `in` any strided view, `out`
+ * contiguous, same shape, a FLOAT dtype (or in's own dtype: a plain strided copy).
+ * Integers convert as Rust's `as` does (nearest even; to f16 / bf16 through f32), floats
+ * with one rounding. */
+int32_t hpt_hip_cast(int32_t dev, void* stream, const hpt_view* in, hpt_view* out);
+
 /* set_val (hpt-cudakernels/src/set_val.cu:4-12; used by `full` / `zeros` / `ones`,
  * hpt/src/backends/cuda/tensor_internal/normal_creation.rs): every element of the
  * contiguous `out` becomes `*value`, one element of out's dtype in HOST memory. */

@@ -67,3 +67,56 @@ def binary(op: int, a: np.ndarray, b: np.ndarray, bf16: bool = False) -> np.ndar
                 raise TypeError("div: float dtypes only")
             return a / b
         return (a + b, a - b, a * b)[op].astype(dt)   # numpy integer arithmetic wraps
+
+
+def cast(a: np.ndarray, to, bf16_in: bool = False):
+    """Scalar<T>::cast as astype uses it (hpt/src/backends/cuda/tensor_impls.rs:129-140), to a float dtype.
+    `to`: a numpy float dtype, or the string "bf16" (result: uint16 bit patterns). Integers -> f16 / bf16 go
+    through f32 (the generated conversions do `self as f32` first); everything else is one rounding, which is
+    what numpy's astype does. Pinned by: exact rational arithmetic on tie cases (tests/test_oracle_elementwise.py)."""
+    src = bf16_bits_to_f32(a) if bf16_in else a
+    if to == "bf16":
+        with np.errstate(all="ignore"):
+            return f32_to_bf16_bits(src.astype(np.float32)) if src.dtype != np.float64 else _f64_to_bf16(src)
+    with np.errstate(all="ignore"):
+        return src.astype(to)
+
+
+def _f64_to_bf16(d: np.ndarray) -> np.ndarray:
+    """One rounding (nearest even) of f64 to bf16, on the bit patterns."""
+    u = np.ascontiguousarray(d, np.float64).view(np.uint64)
+    sign = ((u >> 63) & 1).astype(np.uint16) << 15
+    mag = u & np.uint64(0x7fffffffffffffff)
+    out = np.zeros(d.shape, np.uint16)
+    flat_mag, flat_out = mag.ravel(), out.ravel()
+    vals = np.abs(d).ravel()
+    for i, (m, v) in enumerate(zip(flat_mag, vals)):
+        if np.isnan(v):
+            flat_out[i] = 0x7fc0
+        elif np.isinf(v):
+            flat_out[i] = 0x7f80
+        else:
+            from fractions import Fraction
+            fr = Fraction(float(v))
+            if fr == 0:
+                flat_out[i] = 0
+                continue
+            e = 0
+            t = fr
+            while t >= 2:
+                t /= 2; e += 1
+            while t < 1:
+                t *= 2; e -= 1
+            e_eff = max(e, -126)
+            scale = Fraction(2) ** (e_eff - 7)
+            q = fr / scale
+            n = q.numerator // q.denominator
+            rem = q - n
+            if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and n % 2 == 1):
+                n += 1
+            r = n * scale
+            if r >= Fraction(2) ** 128:
+                flat_out[i] = 0x7f80
+            else:
+                flat_out[i] = f32_to_bf16_bits(np.array([float(r)], np.float32))[0]
+    return (out | sign.reshape(out.shape)).astype(np.uint16)

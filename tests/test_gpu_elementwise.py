@@ -201,3 +201,64 @@ def test_layernorm_equals_normalise_then_affine_steps(hpt, orc, dev):
     steps.mul_(tg, steps)
     steps.add_(tb, steps)
     np.testing.assert_allclose(steps.numpy(), fused, rtol=2e-6, atol=2e-7)
+
+
+# ---- casts ------------------------------------------------------------------------------------------
+
+def test_astype_to_float_dtypes_bit_exact(hpt, dev):
+    rng = np.random.default_rng(320)
+    targets = [(hpt.f16, np.float16), (hpt.f32, np.float32), (hpt.f64, np.float64), (hpt.bf16, "bf16")]
+    for npdt in NP_DTYPES:
+        for shape, ops in (([37, 64], ()), ([40, 24], (("permute", (1, 0)),)), ([5, 7, 3], (("slice", ((0, 5, 2), (1, 7, 1), (0, 3, 1))),))):
+            base = rand(rng, shape, npdt)
+            if np.dtype(npdt).kind == "f":
+                base = (base.astype(np.float64) * rng.choice([1e-6, 1.0, 300.0, 7e4], shape)).astype(npdt)
+            t = apply_view_t(hpt.Tensor.from_numpy(base).to_hip(dev), ops)
+            a = apply_view_np(base, ops)
+            for hdt, to in targets:
+                got = t.astype(hdt).numpy()
+                want = np.ascontiguousarray(ew.cast(a, to))
+                same_bits(got, want, f"astype {np.dtype(npdt).name} -> {hdt.name} {shape} {ops}")
+    # bf16 source
+    xb = ew.f32_to_bf16_bits((rng.standard_normal((33, 16)) * 100).astype(np.float32))
+    tb = hpt.Tensor.from_numpy(xb, hpt.bf16).to_hip(dev)
+    for hdt, to in targets:
+        same_bits(tb.astype(hdt).numpy(), np.ascontiguousarray(ew.cast(xb, to, bf16_in=True)), f"astype bf16 -> {hdt.name}")
+    # the f64 -> half tie cases that a detour through f32 gets wrong
+    d = np.array([1 + 2.0 ** -11 + 2.0 ** -40, 1 + 2.0 ** -11, 65519.999, 65520.0, 6e-8, -2.5e-8, np.nan, np.inf,
+                  1 + 2.0 ** -8 + 2.0 ** -40, 3.4e38])
+    td = hpt.Tensor.from_numpy(d).to_hip(dev)
+    got = td.astype(hpt.f16).numpy()
+    want = ew.cast(d, np.float16)
+    assert np.array_equal(got.view(np.uint16)[~np.isnan(want)], want.view(np.uint16)[~np.isnan(want)]) and np.isnan(got[6])
+    gb = td.astype(hpt.bf16).numpy()
+    wb = ew.cast(d, "bf16")
+    keep = ~np.isnan(d)
+    assert np.array_equal(gb[keep], wb[keep]) and np.isnan(ew.bf16_bits_to_f32(gb)[6])
+    with pytest.raises(hpt.DTypeError):
+        td.astype(hpt.i32)
+    same_bits(hpt.Tensor.from_numpy(np.arange(12, dtype=np.int32).reshape(3, 4)).to_hip(dev).permute([1, 0]).astype(hpt.i32).numpy(),
+              np.ascontiguousarray(np.arange(12, dtype=np.int32).reshape(3, 4).T), "astype to the same dtype is a copy")
+
+
+def test_integer_inputs_of_softmax_and_layernorm_promote(hpt, orc, dev):
+    """NormalizationOps::Output = Tensor<FloatBinaryType<T>>: i32 -> f32, i16 -> f16, i64 -> f64."""
+    from conftest import assert_close
+    rng = np.random.default_rng(321)
+    xi = rng.integers(-6, 7, (19, 200)).astype(np.int32)
+    t = hpt.Tensor.from_numpy(xi).to_hip(dev)
+    s = t.softmax(1)
+    assert s.dtype is hpt.f32
+    assert_close(s.numpy(), orc.softmax(xi.astype(np.float32), 1, acc=orc.ACC_F64), 1e-5, 1e-6, "softmax of i32")
+    ln = t.layernorm([200])
+    assert ln.dtype is hpt.f32
+    assert_close(ln.numpy(), orc.layernorm(xi.astype(np.float32), 1, None, None, 1e-5, acc=orc.ACC_F64), 1e-5, 2e-6, "layernorm of i32")
+    x16 = rng.integers(-5, 6, (7, 64)).astype(np.int16)
+    s16 = hpt.Tensor.from_numpy(x16).to_hip(dev).log_softmax(-1)
+    assert s16.dtype is hpt.f16
+    want = orc.softmax(x16.astype(np.float16), 1, log=True, acc=orc.ACC_F32).astype(np.float32)
+    assert_close(s16.numpy().astype(np.float32), want, 1e-2, 1e-3, "log_softmax of i16")
+    x64 = rng.integers(-5, 6, (3, 5, 9)).astype(np.int64)
+    s64 = hpt.Tensor.from_numpy(x64).to_hip(dev).permute([2, 0, 1]).softmax(0)
+    assert s64.dtype is hpt.f64
+    assert_close(s64.numpy(), orc.softmax(x64.astype(np.float64).transpose(2, 0, 1), 0, acc=orc.ACC_F64), 1e-12, 1e-14, "softmax of i64")

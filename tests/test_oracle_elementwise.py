@@ -118,3 +118,22 @@ def test_bool_and_broadcast():
     x = np.arange(6, dtype=np.float32).reshape(2, 3)
     assert ew.binary(ew.MUL, x, np.array([1, 10, 100], np.float32)).tolist() == [[0, 10, 200], [3, 40, 500]]
     assert ew.full(7, (2, 2), np.int16).tolist() == [[7, 7], [7, 7]]
+
+
+def test_cast_ties_and_ranges():
+    # f64 -> f16: values a hair above a tie must round up (a detour through f32 would round to even first)
+    d = np.array([1 + 2.0 ** -11 + 2.0 ** -40, 1 + 2.0 ** -11, 1 + 3 * 2.0 ** -11, 65519.999, 65520.0, 6e-8, -2.5e-8])
+    got = ew.cast(d, np.float16)
+    want = [1 + 2.0 ** -10, 1.0, 1 + 2.0 ** -9, 65504.0, np.inf, 2.0 ** -24, -0.0]
+    assert [float(v) for v in got] == want
+    for x, g in zip(d[:4], got[:4]):
+        assert Fraction(float(g)) == _round_to(Fraction(float(x)), 11, -14, 15)
+    # f64 -> bf16, one rounding
+    b = ew.cast(np.array([1 + 2.0 ** -8 + 2.0 ** -40, 1 + 2.0 ** -8, 3.0e38, 3.4e38]), "bf16")
+    assert ew.bf16_bits_to_f32(b).tolist()[:2] == [1 + 2.0 ** -7, 1.0]
+    assert np.isfinite(ew.bf16_bits_to_f32(b)[2]) and np.isinf(ew.bf16_bits_to_f32(b)[3])
+    # integers
+    assert ew.cast(np.array([32767, -32768, 2049, 2051], np.int16), np.float16).tolist() == [32768.0, -32768.0, 2048.0, 2052.0]
+    assert ew.cast(np.array([16777217, -16777219], np.int32), np.float32).tolist() == [16777216.0, -16777220.0]
+    assert ew.cast(np.array([(1 << 53) + 1, (1 << 64) - 1], np.uint64), np.float64).tolist() == [float(1 << 53), float(1 << 64)]
+    assert ew.cast(np.array([True, False]), np.float16).tolist() == [1.0, 0.0]
