@@ -213,7 +213,15 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
             m = row_all_reduce<MaxC<CT>>(m, tpr, ty, smem);
             CT s = 0;
 #pragma unroll
-            for (int c = 0; c < NCHUNK; ++c)
+            for (int c = 0; c < NCHUNK; ++c) {
+                // causal kinds: a chunk that lies wholly above the diagonal (the same for every lane
+                // of the row) is all -inf: its exponentials are 0 without computing them. A row with
+                // no key at all takes the ordinary way and comes out NaN, as -inf - -inf does.
+                if (kCausal && limit > 0 && c * tpr * UV >= limit) {
+#pragma unroll
+                    for (int j = 0; j < UV; ++j) x[c][j] = kLog ? neg_inf<CT>() : (CT)0;
+                    continue;
+                }
 #pragma unroll
                 for (int j = 0; j < UV; ++j) {
                     CT d = x[c][j] - m;
@@ -221,6 +229,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                     s += e;
                     x[c][j] = kLog ? d : e;
                 }
+            }
             s = row_all_reduce<SumC<CT>>(s, tpr, ty, smem);
             const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
 #pragma unroll
