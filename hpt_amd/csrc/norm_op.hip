@@ -80,7 +80,7 @@ template <class T> void launch_transposed(const NormPlan& p, const NormArgs& a, 
         transposed_stats_kernel<KIND, T>
             <<<dim3(rg, (unsigned)t.S, batch), dim3(64 * nw), (size_t)nw * FULL * 64 * sizeof(Part), st>>>(t);
         transposed_finalize_kernel<KIND, T><<<dim3((unsigned)((t.R + 15) / 16), 1, batch), dim3(16, 16), 0, st>>>(t);
-        transposed_apply_kernel<KIND, T><<<dim3(rt, (unsigned)((tiles + 3) / 4), batch), dim3(256), 0, st>>>(t);
+        transposed_apply_kernel<KIND, T><<<dim3((rt + 3) / 4, (unsigned)((tiles + 1) / 2), batch), dim3(256), 0, st>>>(t);
         return;
     }
 }

@@ -240,60 +240,70 @@ __global__ void __launch_bounds__(256) transposed_finalize_kernel(const Transpos
     }
 }
 
-// Pass 3: normalise and transpose, one (8*VEC rows) x (8*VEC cols) tile per wavefront.
+// Pass 3: normalise and transpose in (8*VEC rows) x (8*VEC cols) register tiles. The four
+// wavefronts of a workgroup take neighbouring row tiles (512 contiguous bytes of the input per
+// column) and each wavefront takes two neighbouring column tiles (256 contiguous bytes of
+// the output per row).
 template <int KIND, class T>
 __global__ void __launch_bounds__(256) transposed_apply_kernel(const TransposedArgs a) {
     using CT = typename Elem<T>::Wide;
     constexpr int VEC = 16 / sizeof(T);
-    constexpr int TR = 8 * VEC, TC = 8 * VEC;
+    constexpr int TR = 8 * VEC, TC = 8 * VEC, NC = 2;
 
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int rg = lane & 7, cl = lane >> 3;
-    // neighbouring workgroups take neighbouring row tiles: their 128-byte reads are
-    // adjacent in memory
-    const int r0 = blockIdx.x * TR + rg * VEC;
-    const int c0 = (blockIdx.y * 4 + w) * TC + cl * VEC;
-    if (r0 >= a.R || c0 >= a.cols) return;
+    const int r0 = (blockIdx.x * 4 + w) * TR + rg * VEC;
+    const int c_base = blockIdx.y * (NC * TC) + cl * VEC;
+    if (r0 >= a.R || c_base >= a.cols) return;
 
     const CT* pp = (const CT*)a.params + (int64_t)blockIdx.z * 3 * a.R + r0;
     const Pack<CT, VEC> p0 = *reinterpret_cast<const Pack<CT, VEC>*>(pp);
     const Pack<CT, VEC> p1 = *reinterpret_cast<const Pack<CT, VEC>*>(pp + a.R);
     Pack<CT, VEC> p2 = p0;
     if constexpr (KIND == NORM_LAYERNORM) p2 = *reinterpret_cast<const Pack<CT, VEC>*>(pp + 2 * (int64_t)a.R);
-    Pack<T, VEC> gam, bet;
-    if constexpr (KIND == NORM_LAYERNORM) {
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            gam.v[i] = Elem<T>::narrow((CT)1);
-            bet.v[i] = Elem<T>::narrow((CT)0);
-        }
-        if (a.gamma) gam = load_pack<T, VEC>((const T*)a.gamma + c0);
-        if (a.beta) bet = load_pack<T, VEC>((const T*)a.beta + c0);
-    }
 
     const T* base = (const T*)a.in + (int64_t)blockIdx.z * a.bi + r0;
-    Pack<T, VEC> v[VEC];
+    Pack<T, VEC> v[NC][VEC], gam[NC], bet[NC];
+    bool have[NC];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) v[i] = load_pack<T, VEC>(base + (int64_t)(c0 + i) * a.sa);
-
-    T* out = (T*)a.out + ((int64_t)blockIdx.z * a.R + r0) * a.cols + c0;
+    for (int s = 0; s < NC; ++s) {
+        const int c0 = c_base + s * TC;
+        have[s] = c0 < a.cols;
+        if (!have[s]) continue;
 #pragma unroll
-    for (int k = 0; k < VEC; ++k) {
-        Pack<T, VEC> o;
+        for (int i = 0; i < VEC; ++i) v[s][i] = load_pack<T, VEC>(base + (int64_t)(c0 + i) * a.sa);
+        if constexpr (KIND == NORM_LAYERNORM) {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            const CT x = Elem<T>::widen(v[i].v[k]);
-            CT y;
-            if constexpr (KIND == NORM_LAYERNORM)
-                y = ((x - p0.v[k]) - p1.v[k]) * p2.v[k] * Elem<T>::widen(gam.v[i]) + Elem<T>::widen(bet.v[i]);
-            else if constexpr (KIND == NORM_SOFTMAX)
-                y = exp_ct<T>(x - p0.v[k]) * p1.v[k];
-            else
-                y = (x - p0.v[k]) - p1.v[k];
-            o.v[i] = Elem<T>::narrow(y);
+            for (int i = 0; i < VEC; ++i) {
+                gam[s].v[i] = Elem<T>::narrow((CT)1);
+                bet[s].v[i] = Elem<T>::narrow((CT)0);
+            }
+            if (a.gamma) gam[s] = load_pack<T, VEC>((const T*)a.gamma + c0);
+            if (a.beta) bet[s] = load_pack<T, VEC>((const T*)a.beta + c0);
         }
-        store_pack_stream<T, VEC>(out + (int64_t)k * a.cols, o);
     }
+
+    T* out = (T*)a.out + ((int64_t)blockIdx.z * a.R + r0) * a.cols + c_base;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k)
+#pragma unroll
+        for (int s = 0; s < NC; ++s) {
+            if (!have[s]) continue;
+            Pack<T, VEC> o;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                const CT x = Elem<T>::widen(v[s][i].v[k]);
+                CT y;
+                if constexpr (KIND == NORM_LAYERNORM)
+                    y = ((x - p0.v[k]) - p1.v[k]) * p2.v[k] * Elem<T>::widen(gam[s].v[i]) + Elem<T>::widen(bet[s].v[i]);
+                else if constexpr (KIND == NORM_SOFTMAX)
+                    y = exp_ct<T>(x - p0.v[k]) * p1.v[k];
+                else
+                    y = (x - p0.v[k]) - p1.v[k];
+                o.v[i] = Elem<T>::narrow(y);
+            }
+            store_pack_stream<T, VEC>(out + (int64_t)k * a.cols + s * TC, o);
+        }
 }
 
 // ---- single pass: the whole row block lives in registers -------------------------
