@@ -85,7 +85,27 @@ def build(force: bool = False, jobs: int | None = None, verbose: bool = True) ->
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("link failed:\n" + r.stderr)
+    build_host_test(force)
     return LIB
+
+
+HOST_TEST_SRC = ROOT.parent / "tests" / "cpp" / "host_api_test.cpp"
+HOST_TEST_BIN = ROOT / "lib" / "host_api_test"
+
+
+def build_host_test(force: bool = False) -> Path:
+    """The C++ host side (include/hpt_hip.hpp) and its device test program, compiled with the host
+    compiler alone: the ABI is plain C, no HIP header is needed above it."""
+    deps = [HOST_TEST_SRC, INCLUDE / "hpt_hip.hpp", INCLUDE / "hpt_hip.h", LIB]
+    if not force and HOST_TEST_BIN.exists() and HOST_TEST_BIN.stat().st_mtime > max(d.stat().st_mtime for d in deps):
+        return HOST_TEST_BIN
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-Wall", f"-I{INCLUDE}", str(HOST_TEST_SRC),
+           "-o", str(HOST_TEST_BIN), f"-L{LIB.parent}", "-lhpt_hip", "-Wl,-rpath,$ORIGIN",
+           "-Wl,-rpath-link,/opt/rocm/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("host test build failed:\n" + r.stderr)
+    return HOST_TEST_BIN
 
 
 if __name__ == "__main__":

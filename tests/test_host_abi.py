@@ -161,3 +161,15 @@ def test_views_follow_the_reference_slice_rules(hpt, orc):
     assert p.shape == [5, 3, 4] and p.strides == [1, 20, 5] and not p.is_contiguous()
     assert np.array_equal(p[:, ::2].numpy(), a.transpose(2, 0, 1)[:, ::2])
     assert np.array_equal(t[::-1].numpy(), a[::-1])
+
+
+def test_cpp_host_header_compiles_standalone(tmp_path):
+    """include/hpt_hip.hpp needs only the C header and a C++17 host compiler."""
+    import subprocess
+    from pathlib import Path
+    inc = Path(__file__).resolve().parent.parent / "include"
+    src = tmp_path / "t.cpp"
+    src.write_text('#include "hpt_hip.hpp"\nint main() { hpt::Tensor<float>* t = nullptr; (void)t; return 0; }\n')
+    r = subprocess.run(["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", f"-I{inc}", str(src)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
