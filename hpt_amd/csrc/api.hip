@@ -641,7 +641,8 @@ int32_t hpt_hip_softmax_causal(int32_t dev, void* stream, int32_t log, const hpt
         if (in->ndim < 2) fail(HPT_ERR_SHAPE, "softmax_causal: needs at least 2 dims (queries x keys)");
         NormCall c = prepare_norm(in, out->data, in->ndim - 1, 0);
         if (c.plan.kind == NormKind::Empty) return;
-        if (c.plan.kind == NormKind::Transposed || c.plan.kind == NormKind::TransposedTile)
+        if (c.plan.kind == NormKind::Transposed || c.plan.kind == NormKind::TransposedTile ||
+            c.plan.kind == NormKind::ColSplit)
             demote_to_generic(c.plan);
         c.args.scale = scale;
         c.args.q_rows = in->shape[in->ndim - 2];

@@ -112,6 +112,7 @@ enum class NormKind {
     RowReg,     // a row sits in the registers of `tpr` threads; one HBM read, one write
     RowStream,  // rows too long for registers: statistics pass, then a second read
     Col,        // the normalised axis is strided in input and output alike; lanes walk the inner dim
+    ColSplit,   // same layout, vectorisable inner dim: statistics over workgroups, finalize, apply in place
     Transposed, // input contiguous along the rows, output along the axis: statistics, then a register-tile transpose
     TransposedTile,  // same layout, a block of rows fits one compute unit's registers: one read, one write
     Generic     // anything else: one block per row, per-element offset arithmetic

@@ -438,8 +438,29 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             return p;
         }
     }
-    if (p.norm_in.n == 1 && p.out_axis_stride > 1) {
-        // normalised axis is not the last one: lanes walk the trailing dims
+    if (p.norm_in.n == 1 && p.out_axis_stride > 1 && n_norm_dims <= 0) {
+        // Softmax over an axis that is not the last: the inner kept dim is contiguous in the output.
+        // When it is in the input too, three passes spread over the whole chip: partial statistics
+        // (lanes along the inner dim, the axis dealt over wavefronts and workgroups), finalize, apply.
+        const int nk = p.kept_in.n;
+        if (nk >= 1 && nk <= 2 && p.kept_in.stride[nk - 1] == 1 && p.kept_out.stride[nk - 1] == 1 &&
+            p.kept_in.size[nk - 1] == p.out_axis_stride && p.kept_in.size[nk - 1] <= (1 << 30) && p.cols <= (1 << 30) &&
+            (nk == 1 || p.kept_in.size[0] <= 65535)) {
+            const int64_t L = p.kept_in.size[nk - 1];
+            const int64_t batch = nk > 1 ? p.kept_in.size[0] : 1;
+            int v = max_vec;
+            const bool vec_ok = v > 1 && L % v == 0 && sa % v == 0 && (nk == 1 || p.kept_in.stride[0] % v == 0) &&
+                                ((uintptr_t)in_data % 16) == 0 && ((uintptr_t)out_data % 16) == 0;
+            if (!vec_ok) v = 1;
+            p.kind = NormKind::ColSplit;
+            p.vec = v;
+            const int64_t groups = (L + 64 * v - 1) / (64 * v) * batch;
+            int64_t S = std::max<int64_t>(1, std::min<int64_t>((512 + groups - 1) / groups, p.cols / 32));
+            p.tsplit = (int)std::min<int64_t>(S, 64);
+            p.tpr = 4;  // wavefronts per workgroup of the statistics pass
+            p.scratch_bytes = (size_t)p.rows * p.tsplit * 16 + (size_t)p.rows * 3 * 8;
+            return p;
+        }
         p.kind = NormKind::Col;
         p.inner = p.out_axis_stride;
         if (p.rows >= 1024) {
@@ -464,7 +485,7 @@ void demote_to_generic(NormPlan& p) {
 }
 
 std::string describe(const NormPlan& p) {
-    static const char* names[] = {"empty", "rowreg", "rowstream", "col", "transposed", "transposed-tile", "generic"};
+    static const char* names[] = {"empty", "rowreg", "rowstream", "col", "col-split", "transposed", "transposed-tile", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
              names[(int)p.kind], p.sstride == 2 ? "-step2" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,

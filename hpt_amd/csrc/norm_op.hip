@@ -1,5 +1,7 @@
 // One normalisation kind (softmax, log_softmax or layernorm) for the four
 // float dtypes. Compiled once per kind with -DHPT_NORM_KIND=<0...5>.
+#include <algorithm>
+
 #include "transpose_norm.cuh"
 
 #ifndef HPT_NORM_KIND
@@ -27,6 +29,36 @@ void launch_row_reg(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block,
         case 8: row_reg_kernel<KIND, T, VEC, 8, SS><<<grid, block, 0, st>>>(a); break;
         default: fail(HPT_ERR_KERNEL, "row_reg: unsupported chunk count %d", p.nchunk);
     }
+}
+
+// Softmax / log_softmax over an axis that is strided in the output too: three passes.
+template <class T, int VEC> void launch_col_split(const NormPlan& p, const NormArgs& a, hipStream_t st) {
+    TransposedArgs t{};
+    t.in = a.in;
+    t.out = a.out;
+    const int nk = p.kept_in.n;
+    const unsigned batch = nk > 1 ? (unsigned)p.kept_in.size[0] : 1u;
+    t.R = (int)p.kept_in.size[nk - 1];
+    t.cols = (int)p.cols;
+    t.S = p.tsplit;
+    t.stats = a.scratch;
+    t.params = (char*)a.scratch + (size_t)batch * t.S * t.R * 16;
+    t.sa = a.sa;
+    t.bi = nk > 1 ? p.kept_in.stride[0] : 0;
+    t.inv_cols = a.inv_cols;
+    using Part = typename RowPartial<KIND, T>::type;
+    const unsigned nw = (unsigned)p.tpr;
+    const unsigned rg = (unsigned)((t.R + 64 * VEC - 1) / (64 * VEC));
+    transposed_stats_kernel<KIND, T, VEC>
+        <<<dim3(rg, (unsigned)t.S, batch), dim3(64 * nw), (size_t)nw * VEC * 64 * sizeof(Part), st>>>(t);
+    transposed_finalize_kernel<KIND, T><<<dim3((unsigned)((t.R + 15) / 16), 1, batch), dim3(16, 16), 0, st>>>(t);
+    // apply: enough axis chunks for ~2048 workgroups, at least 16 positions each
+    int64_t want = (2048 + (int64_t)rg * batch - 1) / ((int64_t)rg * batch);
+    int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(want, (t.cols + 15) / 16));
+    chunks = std::min<int64_t>(chunks, 65535);
+    const int chunk = (int)((t.cols + chunks - 1) / chunks);
+    chunks = (t.cols + chunk - 1) / chunk;
+    col_apply_kernel<KIND, T, VEC><<<dim3(rg, (unsigned)chunks, batch), dim3(256), 0, st>>>(t, chunk);
 }
 
 // The transposed forms (kinds 0..2 only).
@@ -94,6 +126,15 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
     a.inv_cols = 1.0 / (double)p.cols;
     dim3 grid((unsigned)((p.rows + p.rpb - 1) / p.rpb));
     dim3 block((unsigned)(p.tpr * p.rpb));
+    if (p.kind == NormKind::ColSplit) {
+        if constexpr (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX) {
+            if (p.vec == FULL && FULL > 1) launch_col_split<T, FULL>(p, a, st);
+            else launch_col_split<T, 1>(p, a, st);
+        } else {
+            fail(HPT_ERR_KERNEL, "col-split is a softmax plan");
+        }
+        return;
+    }
     if (p.kind == NormKind::TransposedTile || p.kind == NormKind::Transposed) {
         // the fused kinds run on the row kernels only (the caller demotes transposed plans)
         if constexpr (KIND > NORM_LAYERNORM) fail(HPT_ERR_KERNEL, "fused normalisation: no transposed kernel for this kind");

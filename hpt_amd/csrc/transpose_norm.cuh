@@ -59,11 +59,10 @@ template <int KIND, class T> struct RowPartial {
 // cross-lane merge. Every wavefront takes its own columns; the wavefronts of a
 // workgroup meet in LDS and write one partial per row: partial y of row r goes to
 // stats[b][y][r], y = blockIdx.y.
-template <int KIND, class T>
+template <int KIND, class T, int VEC = 16 / sizeof(T)>
 __global__ void __launch_bounds__(1024) transposed_stats_kernel(const TransposedArgs a) {
     using CT = typename Elem<T>::Wide;
     using Part = typename RowPartial<KIND, T>::type;
-    constexpr int VEC = 16 / sizeof(T);
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int NW = blockDim.x >> 6;  // wavefronts per workgroup (1...16)
 
@@ -304,6 +303,45 @@ __global__ void __launch_bounds__(256) transposed_apply_kernel(const TransposedA
             }
             store_pack_stream<T, VEC>(out + (int64_t)k * a.cols + s * TC, o);
         }
+}
+
+// ---- the normalised axis is strided in input AND output (softmax over a middle dim) ----------
+// Same statistics and finalize passes (the rows are the contiguous inner kept dim, the
+// "columns" the axis); the last pass keeps the layout: lanes along the inner dim, each thread
+// holds the VEC per-row numbers in registers and walks a slice of the axis with batches of
+// loads in flight. out is contiguous: [batch][cols][R].
+template <int KIND, class T, int VEC>
+__global__ void __launch_bounds__(256) col_apply_kernel(const TransposedArgs a, int chunk) {
+    using CT = typename Elem<T>::Wide;
+    constexpr bool kLog = KIND == NORM_LOGSOFTMAX;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int r0 = (blockIdx.x * 64 + tx) * VEC;
+    if (r0 >= a.R) return;
+    const CT* pp = (const CT*)a.params + (int64_t)blockIdx.z * 3 * a.R + r0;
+    const Pack<CT, VEC> p0 = *reinterpret_cast<const Pack<CT, VEC>*>(pp);
+    const Pack<CT, VEC> p1 = *reinterpret_cast<const Pack<CT, VEC>*>(pp + a.R);
+    const T* in = (const T*)a.in + (int64_t)blockIdx.z * a.bi + r0;
+    T* out = (T*)a.out + (int64_t)blockIdx.z * a.cols * a.R + r0;
+    const int c_end = min(a.cols, (int)(blockIdx.y + 1) * chunk);
+    auto apply = [&](const Pack<T, VEC>& v, int c) {
+        Pack<T, VEC> o;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            const CT d = Elem<T>::widen(v.v[k]) - p0.v[k];
+            o.v[k] = Elem<T>::narrow(kLog ? d - p1.v[k] : exp_ct<T>(d) * p1.v[k]);
+        }
+        if constexpr (VEC > 1) store_pack_stream<T, VEC>(out + (int64_t)c * a.R, o);
+        else out[(int64_t)c * a.R] = o.v[0];
+    };
+    int c = blockIdx.y * chunk + ty;
+    for (; c + 12 < c_end; c += 16) {  // four positions in flight per thread (thread rows are 4 apart)
+        Pack<T, VEC> v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = load_pack<T, VEC>(in + (int64_t)(c + 4 * u) * a.sa);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) apply(v[u], c + 4 * u);
+    }
+    for (; c < c_end; c += 4) apply(load_pack<T, VEC>(in + (int64_t)c * a.sa), c);
 }
 
 // ---- single pass: the whole row block lives in registers -------------------------
