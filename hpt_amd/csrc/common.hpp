@@ -111,6 +111,7 @@ enum class NormKind {
     Empty,
     RowReg,     // a row sits in the registers of `tpr` threads; one HBM read, one write
     RowStream,  // rows too long for registers: statistics pass, then a second read
+    RowSplit,   // few, very long rows: several workgroups per row (statistics, finalize, apply)
     Col,        // the normalised axis is strided in input and output alike; lanes walk the inner dim
     ColSplit,   // same layout, vectorisable inner dim: statistics over workgroups, finalize, apply in place
     Transposed, // input contiguous along the rows, output along the axis: statistics, then a register-tile transpose

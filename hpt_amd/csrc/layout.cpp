@@ -418,6 +418,19 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             }
             p.vec = v;
             int64_t nv = p.cols / (v / p.sstride);
+            // Few, very long contiguous rows: share each row among workgroups. (One workgroup per
+            // row would leave a chip of 256 compute units mostly idle.)
+            if (sa == 1 && p.rows <= 128 && p.cols >= 16384 && p.cols % v == 0) {
+                const int64_t nvec = p.cols / v;
+                int64_t S = std::min<int64_t>(512, std::max<int64_t>(1, 1024 / p.rows));
+                S = std::min<int64_t>(S, std::max<int64_t>(1, nvec / 1024));  // at least 4 vectors per thread
+                if (S >= 2) {
+                    p.kind = NormKind::RowSplit;
+                    p.tsplit = (int)S;
+                    p.scratch_bytes = (size_t)p.rows * S * 16 + (size_t)p.rows * 3 * 8;
+                    return p;
+                }
+            }
             if (nv <= 8192) {
                 p.kind = NormKind::RowReg;
                 p.tpr = (int)std::min<int64_t>(1024, pow2_ceil((nv + 3) / 4));
@@ -485,7 +498,7 @@ void demote_to_generic(NormPlan& p) {
 }
 
 std::string describe(const NormPlan& p) {
-    static const char* names[] = {"empty", "rowreg", "rowstream", "col", "col-split", "transposed", "transposed-tile", "generic"};
+    static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
              names[(int)p.kind], p.sstride == 2 ? "-step2" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,

@@ -491,4 +491,180 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
     }
 }
 
+// ---- few, very long rows: a row is shared by many workgroups ------------------------------
+// One workgroup per row leaves most of the chip idle when there are fewer rows than compute
+// units (a batch of 32 rows of 131072 logits). Here S workgroups take a slice of the row each:
+//   row_split_stats_kernel     partial statistics of a slice: softmax (max, sum of exp(x - max)),
+//                              layernorm sums of (x - k), (x - k)^2 with k the row's first element
+//   row_split_finalize_kernel  folds the S partials of a row into (max, 1/sum or ln sum) or
+//                              (mean_hi, mean_lo, rstd)
+//   row_split_apply_kernel     re-reads the slice and writes the result
+// Input rows are contiguous along the axis (any row offsets), the output is contiguous.
+struct RowSplitArgs {
+    const void* in;
+    void* out;
+    const void* gamma;
+    const void* beta;
+    const void* residual;  // NORM_ADD_LAYERNORM
+    void* part;            // [rows][S] partials (16 bytes each at most)
+    void* params;          // [rows][3] numbers for the last pass
+    Dims kept_in;
+    int64_t rows, cols;
+    int64_t chunk_v;       // vectors per slice
+    double eps, inv_cols;
+    int S;
+};
+
+template <class ST> struct SumPair {
+    ST a, b;
+};
+template <class ST> struct SumPairOp {
+    __device__ static __forceinline__ SumPair<ST> comb(SumPair<ST> x, SumPair<ST> y) { return SumPair<ST>{x.a + y.a, x.b + y.b}; }
+};
+
+// element `j` of vector `iv` of a row, with the residual added where the kind says so
+template <int KIND, class T, int VEC>
+__device__ __forceinline__ void row_split_load(const RowSplitArgs& a, const T* in_row, int64_t row, int64_t iv,
+                                               typename Elem<T>::Wide (&x)[VEC]) {
+    using CT = typename Elem<T>::Wide;
+    const Pack<T, VEC> v = load_pack<T, VEC>(in_row + iv * VEC);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) x[j] = Elem<T>::widen(v.v[j]);
+    if constexpr (KIND == NORM_ADD_LAYERNORM) {
+        const Pack<T, VEC> r = load_pack<T, VEC>((const T*)a.residual + row * a.cols + iv * VEC);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) x[j] = Elem<T>::widen(Elem<T>::narrow(x[j] + Elem<T>::widen(r.v[j])));
+    }
+    (void)sizeof(CT);
+}
+
+template <int KIND, class T, int VEC>
+__global__ void __launch_bounds__(256) row_split_stats_kernel(const RowSplitArgs a) {
+    using CT = typename Elem<T>::Wide;
+    using ST = typename StatType<T>::type;
+    __shared__ __align__(16) unsigned char smem_raw[16 * 2 * sizeof(double)];
+    const int64_t row = blockIdx.y;
+    const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
+    const int64_t nv = a.cols / VEC;
+    const int64_t v0 = (int64_t)blockIdx.x * a.chunk_v, v1 = min(nv, v0 + a.chunk_v);
+    if constexpr (!norm_is_layer(KIND)) {
+        SoftStat<CT, ST> st{neg_inf<CT>(), (ST)0};
+        for (int64_t iv = v0 + threadIdx.x; iv < v1; iv += 256) {
+            CT x[VEC];
+            row_split_load<KIND, T, VEC>(a, in_row, row, iv, x);
+            CT cm = x[0];
+#pragma unroll
+            for (int j = 1; j < VEC; ++j) cm = MaxC<CT>::comb(cm, x[j]);
+            if (cm > st.m) {
+                st.s = st.s == (ST)0 ? (ST)0 : st.s * (ST)exp_ct<T>(st.m - cm);
+                st.m = cm;
+            }
+            if (st.m > neg_inf<CT>()) {
+                CT part = 0;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) part += exp_ct<T>(x[j] - st.m);
+                st.s += (ST)part;
+            }
+        }
+        st = block_reduce<SoftStatOp<T, CT, ST>>(st, (SoftStat<CT, ST>*)smem_raw);
+        if (threadIdx.x == 0) ((SoftStat<CT, ST>*)a.part)[row * a.S + blockIdx.x] = st;
+    } else {
+        // the shift k is the row's first element (after the residual, if any): the same for every slice
+        CT k;
+        {
+            CT x0[VEC];
+            row_split_load<KIND, T, VEC>(a, in_row, row, 0, x0);
+            k = x0[0];
+        }
+        CT s1 = 0, s2 = 0;
+        for (int64_t iv = v0 + threadIdx.x; iv < v1; iv += 256) {
+            CT x[VEC];
+            row_split_load<KIND, T, VEC>(a, in_row, row, iv, x);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const CT d = x[j] - k;
+                s1 += d;
+                s2 += d * d;
+            }
+        }
+        SumPair<ST> sp{(ST)s1, (ST)s2};
+        sp = block_reduce<SumPairOp<ST>>(sp, (SumPair<ST>*)smem_raw);
+        if (threadIdx.x == 0) ((SumPair<ST>*)a.part)[row * a.S + blockIdx.x] = sp;
+    }
+}
+
+// one wavefront per row folds its S partials
+template <int KIND, class T, int VEC>
+__global__ void __launch_bounds__(64) row_split_finalize_kernel(const RowSplitArgs a) {
+    using CT = typename Elem<T>::Wide;
+    using ST = typename StatType<T>::type;
+    const int64_t row = blockIdx.x;
+    const int lane = threadIdx.x;
+    CT* p = (CT*)a.params + row * 3;
+    if constexpr (!norm_is_layer(KIND)) {
+        SoftStat<CT, ST> st{neg_inf<CT>(), (ST)0};
+        for (int i = lane; i < a.S; i += 64) st = SoftStatOp<T, CT, ST>::comb(st, ((const SoftStat<CT, ST>*)a.part)[row * a.S + i]);
+        st = group_reduce<SoftStatOp<T, CT, ST>>(st, 64);
+        if (lane == 0) {
+            p[0] = st.m;
+            p[1] = norm_is_log(KIND) ? log_ct<T>((CT)st.s) : (CT)((ST)1 / st.s);
+            p[2] = 0;
+        }
+    } else {
+        SumPair<ST> sp{(ST)0, (ST)0};
+        for (int i = lane; i < a.S; i += 64) sp = SumPairOp<ST>::comb(sp, ((const SumPair<ST>*)a.part)[row * a.S + i]);
+        sp = group_reduce<SumPairOp<ST>>(sp, 64);
+        if (lane == 0) {
+            const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
+            CT x0[VEC];
+            row_split_load<KIND, T, VEC>(a, in_row, row, 0, x0);
+            const ST mean = (ST)x0[0] + sp.a * (ST)a.inv_cols;
+            ST m2 = sp.b - sp.a * sp.a * (ST)a.inv_cols;
+            if (m2 < (ST)0) m2 = 0;
+            const CT hi = (CT)mean;
+            p[0] = hi;
+            p[1] = (CT)(mean - (ST)hi);
+            p[2] = rsqrt_ct((CT)(m2 * (ST)a.inv_cols) + (CT)a.eps);
+        }
+    }
+}
+
+template <int KIND, class T, int VEC>
+__global__ void __launch_bounds__(256) row_split_apply_kernel(const RowSplitArgs a) {
+    using CT = typename Elem<T>::Wide;
+    const int64_t row = blockIdx.y;
+    const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
+    T* out_row = (T*)a.out + row * a.cols;
+    const CT* p = (const CT*)a.params + row * 3;
+    const CT p0 = p[0], p1 = p[1], p2 = p[2];
+    const int64_t nv = a.cols / VEC;
+    const int64_t v0 = (int64_t)blockIdx.x * a.chunk_v, v1 = min(nv, v0 + a.chunk_v);
+    for (int64_t iv = v0 + threadIdx.x; iv < v1; iv += 256) {
+        CT x[VEC];
+        row_split_load<KIND, T, VEC>(a, in_row, row, iv, x);
+        Pack<T, VEC> o;
+        if constexpr (norm_is_layer(KIND)) {
+            Pack<T, VEC> g, b;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                g.v[j] = Elem<T>::narrow((CT)1);
+                b.v[j] = Elem<T>::narrow((CT)0);
+            }
+            if (a.gamma) g = load_pack<T, VEC>((const T*)a.gamma + iv * VEC);
+            if (a.beta) b = load_pack<T, VEC>((const T*)a.beta + iv * VEC);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                o.v[j] = Elem<T>::narrow(((x[j] - p0) - p1) * p2 * Elem<T>::widen(g.v[j]) + Elem<T>::widen(b.v[j]));
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const CT d = x[j] - p0;
+                o.v[j] = Elem<T>::narrow(norm_is_log(KIND) ? d - p1 : exp_ct<T>(d) * p1);
+            }
+        }
+        if constexpr (VEC > 1) store_pack_stream<T, VEC>(out_row + iv * VEC, o);
+        else out_row[iv] = o.v[0];
+    }
+}
+
 }  // namespace hpt

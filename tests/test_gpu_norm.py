@@ -256,3 +256,52 @@ def test_log_softmax_long_columns_keep_the_absolute_tolerance(hpt, orc, dev):
     want = orc.softmax(a, 0, log=True, acc=orc.ACC_F64)
     assert_close(got, want, F32_RTOL, F32_ATOL, "log_softmax over 1012-term columns")
     assert_close(t.softmax(0).numpy(), orc.softmax(a, 0, acc=orc.ACC_F64), F32_RTOL, F32_ATOL, "softmax columns")
+
+
+ROW_SPLIT_CASES = [
+    ("a decode batch of logits", np.float32, [32, 131072], ()),
+    ("one row", np.float32, [1, 65544], ()),
+    ("odd length: one element per access", np.float32, [7, 20001], ()),
+    ("rows of a wider buffer", np.float32, [12, 40000], (("slice", ((1, 11, 1), (64, 32832, 1))),)),
+    ("f64", np.float64, [5, 33000], ()),
+    ("f16", np.float16, [16, 65536], ()),
+    ("bf16", "bf16", [9, 49152], ()),
+]
+
+
+@pytest.mark.parametrize("case", ROW_SPLIT_CASES, ids=[c[0] for c in ROW_SPLIT_CASES])
+def test_few_long_rows_are_shared_by_workgroups(hpt, orc, dev, case):
+    name, npdt, shape, ops = case
+    rng = np.random.default_rng(208)
+    x = (rng.standard_normal(shape) * 3 + rng.uniform(-4, 4, shape[:1] + [1])).astype(np.float32)
+    if npdt == "bf16":
+        cv, dt, odt, bits, tof, acc = hpt.f32_to_bf16_bits, hpt.bf16, orc.BF16, 8, hpt.bf16_bits_to_f32, orc.ACC_F32
+    elif npdt == np.float16:
+        cv, dt, odt, bits, tof, acc = (lambda v: v.astype(np.float16)), None, None, 11, (lambda v: v.astype(np.float32)), orc.ACC_F32
+    else:
+        cv, dt, odt, bits, tof, acc = (lambda v: v.astype(npdt)), None, None, 0, (lambda v: v), orc.ACC_F64
+    base = cv(x)
+    t, a = upload(hpt, base, ops, dtype=dt, dev=dev)
+    assert hpt.normalize_plan(t, 1).startswith("rowsplit"), hpt.normalize_plan(t, 1)
+    n = a.shape[-1]
+    g, b = cv(rng.normal(1, 0.1, n).astype(np.float32)), cv(rng.normal(0, 0.1, n).astype(np.float32))
+    r = cv(rng.standard_normal(a.shape).astype(np.float32))
+    tg, tb, tr = (hpt.Tensor.from_numpy(v, dt).to_hip(dev) for v in (g, b, r))
+
+    def check(got, want, what, atol32=F32_ATOL):
+        got, want = tof(got), tof(want)
+        if bits:
+            assert_close(got, want, HALF_RTOL, max(half_atol(want[np.isfinite(want)], bits), 6e-8), f"{what} {name}")
+        else:
+            assert_close(got, want, F32_RTOL, atol32, f"{what} {name}")
+
+    ac = np.ascontiguousarray(a)
+    check(t.softmax(1).numpy(), orc.softmax(ac, 1, acc=acc, dtype=odt), "softmax")
+    check(t.log_softmax(-1).numpy(), orc.softmax(ac, 1, log=True, acc=acc, dtype=odt), "log_softmax", 2e-6)
+    check(t.layernorm([n], tg, tb, 1e-5).numpy(), orc.layernorm(ac, 1, g, b, 1e-5, acc=acc, dtype=odt), "layernorm", 4e-6)
+    check(t.layernorm([n], None, None, 1e-5).numpy(), orc.layernorm(ac, 1, None, None, 1e-5, acc=acc, dtype=odt),
+          "layernorm without gamma / beta", 4e-6)
+    if not bits:
+        from oracle import elementwise as ew
+        summed = ew.binary(ew.ADD, ac, r)
+        check(t.add_layernorm(tr, [n], tg, tb, 1e-5).numpy(), orc.layernorm(summed, 1, g, b, 1e-5, acc=acc), "add_layernorm", 4e-6)
