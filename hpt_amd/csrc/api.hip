@@ -609,8 +609,11 @@ static void run_layernorm(int dev, void* stream, const hpt_view* in, const hpt_v
     // the fused form runs on the row kernels only
     if (residual && (c.plan.kind == NormKind::Transposed || c.plan.kind == NormKind::TransposedTile))
         demote_to_generic(c.plan);
-    // vector loads of gamma / beta / residual need 16-byte alignment too
-    if (c.plan.vec > 1 &&
+    // shifted rows: the residual's rows must be misaligned like the output's
+    if (c.plan.shift && residual && (((uintptr_t)residual->data ^ (uintptr_t)out->data) & 15) != 0) demote_to_generic(c.plan);
+    // vector loads of gamma / beta / residual need 16-byte alignment too (the shifted streaming
+    // kernel reads gamma / beta element by element and the residual with the rows' own shift)
+    if (c.plan.vec > 1 && !c.plan.shift &&
         (((uintptr_t)c.args.gamma | (uintptr_t)c.args.beta | (uintptr_t)c.args.residual) % 16) != 0)
         demote_to_generic(c.plan);
     NormLaunchFn fn = norm_launcher_for(residual ? NORM_ADD_LAYERNORM : NORM_LAYERNORM, in->dtype);

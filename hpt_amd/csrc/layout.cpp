@@ -417,6 +417,22 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 }
             }
             p.vec = v;
+            // Rows that start off 16-byte boundaries (odd row lengths): the streaming kernel can still
+            // move aligned vectors and mask the two ends of a row, provided input and output rows are
+            // misaligned by the same amount: equal bases and row pitches modulo 16 bytes.
+            if (sa == 1 && v == 1 && max_vec > 1 && p.cols >= 1024 && p.rows > 128) {
+                bool same = (((uintptr_t)in_data ^ (uintptr_t)out_data) & 15) == 0 && ((uintptr_t)in_data % elem_size) == 0;
+                for (int i = 0; i < p.kept_in.n; ++i)
+                    if (((p.kept_in.stride[i] - p.kept_out.stride[i]) * (int64_t)elem_size) % 16 != 0) same = false;
+                if (same) {
+                    p.kind = NormKind::RowStream;
+                    p.vec = max_vec;
+                    p.shift = 1;
+                    p.tpr = p.cols >= 4096 * max_vec ? 1024 : 256;
+                    p.rpb = 1;
+                    return p;
+                }
+            }
             int64_t nv = p.cols / (v / p.sstride);
             // Few, very long contiguous rows: share each row among workgroups. (One workgroup per
             // row would leave a chip of 256 compute units mostly idle.)
@@ -431,9 +447,16 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     return p;
                 }
             }
-            if (nv <= 8192) {
+            // A row fits the registers of a workgroup up to 8 vectors per thread; layernorm also keeps
+            // gamma and beta there (the eight-vector form spills), so it stops at four and streams
+            // longer rows (two sweeps; gamma / beta as vectors).
+            const int64_t reg_limit = (n_norm_dims > 0 && v > 1) ? 4096 : 8192;
+            if (nv <= reg_limit) {
                 p.kind = NormKind::RowReg;
-                p.tpr = (int)std::min<int64_t>(1024, pow2_ceil((nv + 3) / 4));
+                // about four 128-bit vectors per thread; rows that only allow single elements
+                // take eight per thread (fewer, busier threads: a 257-element row stays in one
+                // wavefront instead of four that meet in LDS)
+                p.tpr = (int)std::min<int64_t>(1024, v > 1 ? pow2_ceil((nv + 3) / 4) : pow2_ceil((nv + 7) / 8));
                 if (p.tpr > 64 && p.tpr < 256) p.tpr = 256;
                 int64_t nc = (nv + p.tpr - 1) / p.tpr;
                 p.nchunk = std::max(1, pow2_ceil(nc));
@@ -489,6 +512,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
 void demote_to_generic(NormPlan& p) {
     p.kind = NormKind::Generic;
     p.vec = 1;
+    p.shift = 0;
     p.sstride = 1;
     p.nchunk = 1;
     p.scratch_bytes = 0;
@@ -501,7 +525,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.shift ? "-shift" : ""), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     describe_dims(s, "rows_in", p.kept_in);

@@ -334,8 +334,15 @@ template <class Op, class S> __device__ __forceinline__ S stat_all_reduce(S v, i
     return block_reduce<Op>(v, smem);
 }
 
-template <int KIND, class T, int VEC>
+// SHIFT (VEC > 1 only): rows contiguous along the axis whose START is only element-aligned (odd
+// row lengths: 50257-wide logits). Vectors are taken at 16-byte aligned addresses all the same:
+// vector iv of a row covers its elements iv * VEC - m ... + VEC - 1, m = the row's misalignment,
+// and positions outside 0 .. cols - 1 are masked. (An aligned vector that holds one valid
+// element lies in that element's page, so the over-read at both ends is safe.) Input, output
+// and residual rows share m: the caller checks that their bases and row pitches agree mod 16 bytes.
+template <int KIND, class T, int VEC, bool SHIFT = false>
 __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
+    static_assert(!SHIFT || VEC > 1, "SHIFT is a vector mode");
     using CT = typename Elem<T>::Wide;
     __shared__ __align__(16) unsigned char smem_raw[16 * 3 * sizeof(double)];
     const int tpr = a.tpr;
@@ -343,9 +350,16 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
     const int ty = threadIdx.x >> a.tpr_log2;
     const int64_t row = (int64_t)blockIdx.x * a.rpb + ty;
     const bool valid = row < a.rows;
-    const int64_t nv = a.cols / VEC;
     const T* in_row = (const T*)a.in + (valid ? offset_of(a.kept_in, row) : 0);
     T* out_row = (T*)a.out + (valid ? offset_of(a.kept_out, row) : 0);
+    const int m = SHIFT ? (int)(((uintptr_t)in_row / sizeof(T)) % VEC) : 0;
+    const int64_t nv = SHIFT ? (a.cols + m + VEC - 1) / VEC : a.cols / VEC;
+    // is element j of vector iv inside the row?
+    auto inside = [&](int64_t iv, int j) {
+        if constexpr (!SHIFT) return true;
+        const int64_t e = iv * VEC + j - m;
+        return e >= 0 && e < a.cols;
+    };
     const bool one_dim = a.norm_in.n <= 1;
     constexpr bool kLog = norm_is_log(KIND);
     constexpr bool kCausal = norm_is_causal(KIND);
@@ -356,7 +370,7 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
         limit = valid ? row % a.q_rows + a.causal_offset + 1 : 0;
         limit = limit < 0 ? 0 : (limit < a.cols ? limit : a.cols);
     }
-    const int64_t nv_lim = kCausal ? (limit + VEC - 1) / VEC : nv;
+    const int64_t nv_lim = kCausal ? (limit + m + VEC - 1) / VEC : nv;
     // the scalar operand of the unfused mul_ has the tensor's dtype
     const CT scale_t = kCausal ? Elem<T>::widen(Elem<T>::narrow((CT)a.scale)) : (CT)1;
     const T* res_row = kRes ? (const T*)a.residual + (valid ? row * a.cols : 0) : nullptr;
@@ -365,11 +379,11 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
     // the separate add / mul_ of the unfused sequence would have stored it.
     auto load = [&](int64_t iv, CT* x) {
         if constexpr (VEC > 1) {
-            Pack<T, VEC> v = load_pack<T, VEC>(in_row + iv * VEC);
+            Pack<T, VEC> v = load_pack<T, VEC>(in_row - m + iv * VEC);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) x[j] = Elem<T>::widen(v.v[j]);
             if constexpr (kRes) {
-                Pack<T, VEC> r = load_pack<T, VEC>(res_row + iv * VEC);
+                Pack<T, VEC> r = load_pack<T, VEC>(res_row - m + iv * VEC);
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) x[j] = Elem<T>::widen(Elem<T>::narrow(x[j] + Elem<T>::widen(r.v[j])));
             }
@@ -381,7 +395,7 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
         if constexpr (kCausal) {
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
-                x[j] = iv * VEC + j < limit ? Elem<T>::widen(Elem<T>::narrow(x[j] * scale_t)) : neg_inf<CT>();
+                x[j] = iv * VEC + j - m < limit ? Elem<T>::widen(Elem<T>::narrow(x[j] * scale_t)) : neg_inf<CT>();
         }
     };
     auto store = [&](int64_t iv, const CT* y) {
@@ -389,7 +403,18 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
             Pack<T, VEC> o;
 #pragma unroll
             for (int j = 0; j < VEC; ++j) o.v[j] = Elem<T>::narrow(y[j]);
-            store_pack<T, VEC>(out_row + iv * VEC, o);
+            if constexpr (SHIFT) {
+                const int64_t e0 = iv * VEC - m;
+                if (e0 >= 0 && e0 + VEC <= a.cols) {
+                    store_pack<T, VEC>(out_row + e0, o);
+                } else {  // the partial vectors at both ends of the row
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        if (e0 + j >= 0 && e0 + j < a.cols) out_row[e0 + j] = o.v[j];
+                }
+            } else {
+                store_pack<T, VEC>(out_row + iv * VEC, o);
+            }
         } else {
             out_row[iv * a.out_axis_stride] = Elem<T>::narrow(y[0]);
         }
@@ -405,6 +430,11 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
             for (int64_t iv = tx; iv < nv_lim; iv += tpr) {
                 CT x[VEC];
                 load(iv, x);
+                if constexpr (SHIFT) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        if (!inside(iv, j)) x[j] = neg_inf<CT>();
+                }
                 CT cm = x[0];
 #pragma unroll
                 for (int j = 1; j < VEC; ++j) cm = MaxC<CT>::comb(cm, x[j]);
@@ -452,16 +482,24 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
                 CT x[VEC];
                 load(iv, x);
                 if (first) {
-                    k = x[0];
+                    k = x[0];  // the first element of the row this lane sees
+                    if constexpr (SHIFT) {
+                        if (iv == 0) {
+#pragma unroll
+                            for (int j = 1; j < VEC; ++j)
+                                if (j == m) k = x[j];
+                        }
+                    }
                     first = false;
                 }
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
-                    const CT d = x[j] - k;
+                    const bool in_row_j = inside(iv, j);
+                    const CT d = in_row_j ? x[j] - k : (CT)0;
                     s1 += d;
                     s2 += d * d;
+                    n += in_row_j;
                 }
-                n += VEC;
             }
             if (n > 0) {
                 st.n = (ST)n;
@@ -478,13 +516,30 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
         for (int64_t iv = tx; iv < nv; iv += tpr) {
             CT x[VEC];
             load(iv, x);
+            if constexpr (VEC > 1 && !SHIFT) {
+                // aligned rows: gamma / beta come as vectors too (the caller checked their alignment)
+                Pack<T, VEC> g, b;
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) {
-                CT y = ((x[j] - mean_hi) - mean_lo) * rstd;
-                const int64_t col = iv * VEC + j;
-                if (a.gamma) y *= Elem<T>::widen(((const T*)a.gamma)[col]);
-                if (a.beta) y += Elem<T>::widen(((const T*)a.beta)[col]);
-                x[j] = y;
+                for (int j = 0; j < VEC; ++j) {
+                    g.v[j] = Elem<T>::narrow((CT)1);
+                    b.v[j] = Elem<T>::narrow((CT)0);
+                }
+                if (a.gamma) g = load_pack<T, VEC>((const T*)a.gamma + iv * VEC);
+                if (a.beta) b = load_pack<T, VEC>((const T*)a.beta + iv * VEC);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    x[j] = ((x[j] - mean_hi) - mean_lo) * rstd * Elem<T>::widen(g.v[j]) + Elem<T>::widen(b.v[j]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    CT y = ((x[j] - mean_hi) - mean_lo) * rstd;
+                    const int64_t col = iv * VEC + j - m;
+                    if (inside(iv, j)) {
+                        if (a.gamma) y *= Elem<T>::widen(((const T*)a.gamma)[col]);
+                        if (a.beta) y += Elem<T>::widen(((const T*)a.beta)[col]);
+                    }
+                    x[j] = y;
+                }
             }
             store(iv, x);
         }

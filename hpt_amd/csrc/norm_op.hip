@@ -183,6 +183,12 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         else launch_row_reg<T, 1>(p, a, grid, block, st);
         return;
     }
+    if constexpr (FULL > 1) {
+        if (p.vec == FULL && p.shift) {
+            row_stream_kernel<KIND, T, FULL, true><<<grid, block, 0, st>>>(a);
+            return;
+        }
+    }
     if (p.vec == FULL) row_stream_kernel<KIND, T, FULL><<<grid, block, 0, st>>>(a);
     else row_stream_kernel<KIND, T, 1><<<grid, block, 0, st>>>(a);
 }
