@@ -223,10 +223,20 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
                 // on different CUs (48 workgroups of 1024 threads leave 208 CUs idle), and
                 // fold the partials in a second launch.
                 int64_t cap = std::max<int64_t>(1, (int64_t)((64ll << 20) / acc_size) / p.K);
-                int64_t split = std::min<int64_t>(std::min<int64_t>(rp, 64), cap);
-                int64_t by = pow2_floor(std::max<int64_t>(1, rp / split));
-                p.split = (int)split;
-                p.by = (int)std::min<int64_t>(by, 4) * base_by;
+                if (need > 64) {
+                    // Very few column blocks (a narrow inner dim: [N, 3], [N, 33]): aim for ~2048
+                    // wavefronts, sixteen per workgroup, up to 256 workgroups per column block.
+                    const int64_t slices = std::min((2048 + xblocks - 1) / xblocks, can);
+                    int64_t by_waves = std::min<int64_t>(16, pow2_floor(slices));
+                    while (by_waves > 1 && (size_t)64 * by_waves * uv * acc_size > (64u << 10)) by_waves /= 2;
+                    p.split = (int)std::min<int64_t>(std::min<int64_t>((slices + by_waves - 1) / by_waves, 256), cap);
+                    p.by = (int)by_waves * base_by;
+                } else {
+                    int64_t split = std::min<int64_t>(std::min<int64_t>(rp, 64), cap);
+                    int64_t by = pow2_floor(std::max<int64_t>(1, rp / split));
+                    p.split = (int)split;
+                    p.by = (int)std::min<int64_t>(by, 4) * base_by;
+                }
             } else {
                 // Small input: one launch, thread rows meet in LDS
                 int64_t by = std::min<int64_t>(pow2_ceil(rp), 1024 / p.bx / base_by) * base_by;
