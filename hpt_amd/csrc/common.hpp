@@ -97,6 +97,10 @@ struct ReducePlan {
     int64_t chunk = 0;  // Col: reduced indices per split
     int sstride = 1;    // lean kernels: 2 = elements along the lane dim sit at every second position
     bool lean = false;  // the layout fits the lean kernels (one reduced dim, <= 2 kept dims, 32-bit extents)
+    int flat_t = 0;     // Col, > 0: contiguous [R, kin] slab walked as a flat array by this many threads
+    int flat_xb = 0;    // > 0: a period of the flat walk is wider than a workgroup and spans this many of them;
+                        // `split` then counts the partials per output (slices x row phases)
+    int flat_phases = 1;  // rows per period in that case
 };
 
 // Build the plan for reducing `axes` (already normalised) of a view.

@@ -200,20 +200,39 @@ __global__ void __launch_bounds__(1024) row_reduce_kernel(const RowArgs a) {
 }
 
 // ---- column kernels ---------------------------------------------------------------
-// Fold the `by` thread rows of a workgroup: row 0 collects, in row order.
+// Fold the `by` thread rows of a workgroup into row 0.
 template <class Op, int VEC>
 __device__ __forceinline__ void fold_thread_rows(typename Op::Acc (&acc)[VEC], typename Op::Acc* smem) {
     const int bx = blockDim.x, by = blockDim.y;
     const int tx = threadIdx.x, ty = threadIdx.y;
     if (by == 1) return;
+    if (by <= 4) {
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) smem[((size_t)ty * bx + tx) * VEC + j] = acc[j];
-    __syncthreads();
-    if (ty == 0) {
-        for (int y = 1; y < by; ++y) {
+        for (int j = 0; j < VEC; ++j) smem[((size_t)ty * bx + tx) * VEC + j] = acc[j];
+        __syncthreads();
+        if (ty == 0) {
+            for (int y = 1; y < by; ++y) {
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], smem[((size_t)y * bx + tx) * VEC + j]);
+                for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], smem[((size_t)y * bx + tx) * VEC + j]);
+            }
         }
+        return;
+    }
+    // Many thread rows (a narrow inner dim): halve them step by step; rows [s, 2s) hand their
+    // values to rows [0, s) through LDS. The pairing is fixed, so the result is deterministic.
+    int top = 1;
+    while (top < by) top <<= 1;
+    for (int s = top >> 1; s >= 1; s >>= 1) {
+        if (ty >= s && ty < 2 * s) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) smem[((size_t)(ty - s) * bx + tx) * VEC + j] = acc[j];
+        }
+        __syncthreads();
+        if (ty < s && ty + s < by) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[j] = Op::comb(acc[j], smem[((size_t)ty * bx + tx) * VEC + j]);
+        }
+        __syncthreads();
     }
 }
 
@@ -290,6 +309,149 @@ __global__ void __launch_bounds__(1024) col_lean_kernel(const ColLeanArgs a) {
             for (int j = 0; j < UV; ++j) ((Acc*)a.out)[(int64_t)blockIdx.z * a.K + o0 + j] = acc[j];
         }
     }
+}
+
+// A contiguous [R, kin] slab per outer index whose rows are not whole vectors, walked as a flat
+// array: thread t owns elements [t * VEC, t * VEC + VEC) of every period of L = threads * VEC
+// elements. L is a multiple of kin, so slot (t, j) always sees column (t * VEC + j) % kin and
+// row (t * VEC + j) / kin + period * (L / kin). All loads are aligned 128-bit vectors whatever kin is.
+struct ColFlatArgs {
+    const void* in;
+    void* out;      // outputs, or partials [split][K] when split > 1
+    int64_t so;     // stride of the outer kept dim
+    int64_t total;  // elements per outer index: R * kin
+    int64_t K;      // outputs: outer * kin
+    double count;
+    int kin;        // inner kept length (columns)
+    int threads;    // threads that take part (a multiple of kin / gcd(kin, VEC))
+    int split, init_out;
+};
+
+template <class Op, int VEC>
+__global__ void __launch_bounds__(1024) col_flat_kernel(const ColFlatArgs a) {
+    using T = typename Op::In;
+    using Acc = typename Op::Acc;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    Acc* smem = (Acc*)smem_raw;
+    const int t = threadIdx.x;
+    const int outer = blockIdx.y;
+    const int L = a.threads * VEC;
+    const int rows_per_period = L / a.kin;
+    const int p0 = t * VEC;
+    Acc acc[VEC];
+    int row[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        acc[j] = Op::identity();
+        row[j] = (p0 + j) / a.kin;
+    }
+    if (t < a.threads) {
+        const T* base = (const T*)a.in + (int64_t)outer * a.so;
+        const int64_t whole = a.total / L;  // periods that lie wholly inside the slab
+        const int split = a.split;
+        int64_t it = blockIdx.z;  // periods are dealt round-robin over the workgroups of a slab
+        for (; it + 3 * split < whole; it += 4 * split) {
+            Pack<T, VEC> v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(base + (it + u * split) * L + p0);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    fold_in<Op>(acc[j], v[u].v[j], row[j] + (int)(it + u * split) * rows_per_period);
+        }
+        for (; it < whole; it += split) {
+            Pack<T, VEC> v = load_pack_stream<T, VEC>(base + it * L + p0);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v.v[j], row[j] + (int)it * rows_per_period);
+        }
+        if (it == whole) {  // the last, partial period: element by element
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const int64_t pos = whole * L + p0 + j;
+                if (pos < a.total) fold_in<Op>(acc[j], base[pos], row[j] + (int)whole * rows_per_period);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) smem[p0 + j] = acc[j];
+    }
+    __syncthreads();
+    // Slot p holds column p % kin: fold the L / kin slot rows pairwise, upper half into lower half.
+    int top = 1;
+    while (top < rows_per_period) top <<= 1;
+    for (int s = top >> 1; s >= 1; s >>= 1) {
+        const int n = s * a.kin;
+        for (int i = t; i < n; i += blockDim.x)
+            if (i + n < L) smem[i] = Op::comb(smem[i], smem[i + n]);
+        __syncthreads();
+    }
+    for (int c = t; c < a.kin; c += blockDim.x) {
+        const int64_t o = (int64_t)outer * a.kin + c;
+        if (a.split == 1) write_out<Op>(a.out, o, smem[c], a.init_out, a.count);
+        else ((Acc*)a.out)[(int64_t)blockIdx.z * a.K + o] = smem[c];
+    }
+}
+
+// The same flat walk for rows wider than a workgroup can cover: the period (phases rows, the
+// shortest run after which row starts repeat their alignment) is spread over gridDim.x workgroups.
+// Each vector slot is then a single (row phase, column) pair; the partials are [slice][phase][K].
+struct ColFlatWideArgs {
+    const void* in;
+    void* partial;
+    int64_t so;      // stride of the outer kept dim
+    int64_t total;   // elements per outer index: R * kin
+    int64_t K;       // outputs: outer * kin
+    int kin;         // inner kept length (columns)
+    int vecs;        // vectors per period: kin * phases / VEC
+    int phases;      // rows per period
+    int slices;      // workgroups along the reduced range
+};
+
+template <class Op, int VEC>
+__global__ void __launch_bounds__(1024) col_flat_wide_kernel(const ColFlatWideArgs a) {
+    using T = typename Op::In;
+    using Acc = typename Op::Acc;
+    const int q = blockIdx.x * blockDim.x + threadIdx.x;  // vector within the period
+    if (q >= a.vecs) return;
+    const int outer = blockIdx.y;
+    const int64_t L = (int64_t)a.vecs * VEC;
+    const int p0 = q * VEC;
+    Acc acc[VEC];
+    int row[VEC], col[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        acc[j] = Op::identity();
+        row[j] = (p0 + j) / a.kin;
+        col[j] = (p0 + j) - row[j] * a.kin;
+    }
+    const T* base = (const T*)a.in + (int64_t)outer * a.so;
+    const int64_t whole = a.total / L;
+    const int slices = a.slices;
+    int64_t it = blockIdx.z;
+    for (; it + 3 * slices < whole; it += 4 * slices) {
+        Pack<T, VEC> v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(base + (it + u * slices) * L + p0);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v[u].v[j], row[j] + (int)(it + u * slices) * a.phases);
+    }
+    for (; it < whole; it += slices) {
+        Pack<T, VEC> v = load_pack_stream<T, VEC>(base + it * L + p0);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v.v[j], row[j] + (int)it * a.phases);
+    }
+    if (it == whole) {  // the last, partial period
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            const int64_t pos = whole * L + p0 + j;
+            if (pos < a.total) fold_in<Op>(acc[j], base[pos], row[j] + (int)whole * a.phases);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+        ((Acc*)a.partial)[((int64_t)blockIdx.z * a.phases + row[j]) * a.K + (int64_t)outer * a.kin + col[j]] = acc[j];
 }
 
 struct ColArgs {
@@ -478,47 +640,86 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
         return;
     }
     // Col
-    const int64_t kv = p.K / p.vec;
-    dim3 block((unsigned)p.bx, (unsigned)p.by);
-    size_t smem = p.by > 1 ? (size_t)p.bx * p.by * (p.vec / p.sstride) * sizeof(Acc) : 0;
-    if (p.lean) {
-        ColLeanArgs a{};
-        const int nk = p.kept.n;
-        const int64_t kin = nk ? p.kept.size[nk - 1] : 1;
-        a.in = in;
-        a.out = stage1_out;
-        a.so = nk > 1 ? p.kept.stride[0] : 0;
-        a.rs = p.red.n ? p.red.stride[0] : 0;
-        a.K = p.K;
-        a.count = count;
-        a.kin_v = (int)(kin / (p.vec / p.sstride));
-        a.sk = nk ? (int)p.kept.stride[nk - 1] : 1;
-        a.R = (int)p.R;
-        a.split = p.split;
-        a.init_out = init_out;
-        const int64_t outer = nk > 1 ? p.kept.size[0] : 1;
-        dim3 grid((unsigned)((a.kin_v + p.bx - 1) / p.bx), (unsigned)outer, (unsigned)p.split);
-        if (vec && p.sstride == 2) col_lean_kernel<Op, FULL, 2><<<grid, block, smem, st>>>(a);
-        else if (vec) col_lean_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
-        else col_lean_kernel<Op, 1><<<grid, block, smem, st>>>(a);
+    if (p.flat_xb > 0) {
+        if constexpr (FULL > 1) {
+            const int nk = p.kept.n;
+            const int64_t kin = p.kept.size[nk - 1];
+            const int64_t outer = nk > 1 ? p.kept.size[0] : 1;
+            ColFlatWideArgs a{};
+            a.in = in;
+            a.partial = sc.partial;
+            a.so = nk > 1 ? p.kept.stride[0] : 0;
+            a.total = kin * p.R;
+            a.K = p.K;
+            a.kin = (int)kin;
+            a.vecs = (int)(kin * p.flat_phases / FULL);
+            a.phases = p.flat_phases;
+            a.slices = p.split / p.flat_phases;
+            col_flat_wide_kernel<Op, FULL><<<dim3((unsigned)p.flat_xb, (unsigned)outer, (unsigned)a.slices),
+                                             dim3((unsigned)p.flat_t), 0, st>>>(a);
+        }
+    } else if (p.flat_t > 0) {
+        if constexpr (FULL > 1) {
+            const int nk = p.kept.n;
+            const int64_t kin = p.kept.size[nk - 1];
+            const int64_t outer = nk > 1 ? p.kept.size[0] : 1;
+            ColFlatArgs a{};
+            a.in = in;
+            a.out = stage1_out;
+            a.so = nk > 1 ? p.kept.stride[0] : 0;
+            a.total = kin * p.R;
+            a.K = p.K;
+            a.count = count;
+            a.kin = (int)kin;
+            a.threads = p.flat_t;
+            a.split = p.split;
+            a.init_out = init_out;
+            col_flat_kernel<Op, FULL><<<dim3(1, (unsigned)outer, (unsigned)p.split), dim3((unsigned)p.bx),
+                                        (size_t)p.flat_t * FULL * sizeof(Acc), st>>>(a);
+        }
     } else {
-        ColArgs a{};
-        a.in = in;
-        a.out = stage1_out;
-        a.kept_outer = p.kept;
-        a.kept_outer.n = p.kept.n > 0 ? p.kept.n - 1 : 0;
-        a.red = p.red;
-        a.K = p.K;
-        a.kin = p.kept.n ? p.kept.size[p.kept.n - 1] : 1;
-        a.sk = p.kept.n ? p.kept.stride[p.kept.n - 1] : 0;
-        a.R = p.R;
-        a.chunk = p.chunk;
-        a.count = count;
-        a.split = p.split;
-        a.init_out = init_out;
-        dim3 grid((unsigned)((kv + p.bx - 1) / p.bx), (unsigned)p.split);
-        if (vec) col_reduce_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
-        else col_reduce_kernel<Op, 1><<<grid, block, smem, st>>>(a);
+        const int64_t kv = p.K / p.vec;
+        dim3 block((unsigned)p.bx, (unsigned)p.by);
+        size_t smem = p.by > 1 ? (size_t)p.bx * p.by * (p.vec / p.sstride) * sizeof(Acc) : 0;
+        if (p.lean) {
+            ColLeanArgs a{};
+            const int nk = p.kept.n;
+            const int64_t kin = nk ? p.kept.size[nk - 1] : 1;
+            a.in = in;
+            a.out = stage1_out;
+            a.so = nk > 1 ? p.kept.stride[0] : 0;
+            a.rs = p.red.n ? p.red.stride[0] : 0;
+            a.K = p.K;
+            a.count = count;
+            a.kin_v = (int)(kin / (p.vec / p.sstride));
+            a.sk = nk ? (int)p.kept.stride[nk - 1] : 1;
+            a.R = (int)p.R;
+            a.split = p.split;
+            a.init_out = init_out;
+            const int64_t outer = nk > 1 ? p.kept.size[0] : 1;
+            dim3 grid((unsigned)((a.kin_v + p.bx - 1) / p.bx), (unsigned)outer, (unsigned)p.split);
+            if (vec && p.sstride == 2) col_lean_kernel<Op, FULL, 2><<<grid, block, smem, st>>>(a);
+            else if (vec) col_lean_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
+            else col_lean_kernel<Op, 1><<<grid, block, smem, st>>>(a);
+        } else {
+            ColArgs a{};
+            a.in = in;
+            a.out = stage1_out;
+            a.kept_outer = p.kept;
+            a.kept_outer.n = p.kept.n > 0 ? p.kept.n - 1 : 0;
+            a.red = p.red;
+            a.K = p.K;
+            a.kin = p.kept.n ? p.kept.size[p.kept.n - 1] : 1;
+            a.sk = p.kept.n ? p.kept.stride[p.kept.n - 1] : 0;
+            a.R = p.R;
+            a.chunk = p.chunk;
+            a.count = count;
+            a.split = p.split;
+            a.init_out = init_out;
+            dim3 grid((unsigned)((kv + p.bx - 1) / p.bx), (unsigned)p.split);
+            if (vec) col_reduce_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
+            else col_reduce_kernel<Op, 1><<<grid, block, smem, st>>>(a);
+        }
     }
     if (p.split > 1) {
         int fy = 1;  // thread rows sharing an output's partials: about two partials per thread

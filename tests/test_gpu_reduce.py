@@ -201,6 +201,44 @@ def test_multi_stage_and_large_shapes(hpt, orc, dev):
         assert np.array_equal(t.sum(axes).numpy().view(np.uint32), t.sum(axes).numpy().view(np.uint32))
 
 
+def test_narrow_inner_dim_flat_walk(hpt, orc, dev):
+    """Contiguous [N, k] slabs with k not a whole number of 128-bit vectors (3, 33, 257 columns),
+    reduced over N: the slab is walked as a flat array of aligned vectors. Sizes leave a partial
+    last period; one case has an outer kept dim; ties and all-equal columns check the index rule."""
+    rng = np.random.default_rng(116)
+    assert "col-flat " in hpt.reduce_plan(hpt.Tensor.empty([700001, 3], hpt.f32, dev), hpt.SUM, [0])
+    assert "col-flat-wide" in hpt.reduce_plan(hpt.Tensor.empty([2051, 4097], hpt.f32, dev), hpt.SUM, [0])
+    for shape, axis, npdt in (((700001, 3), 0, np.float32), ((70003, 33), 0, np.float32), ((4, 500000, 5), 1, np.float32),
+                              ((140001, 33), 0, np.float16), ((20001, 257), 0, np.float16), ((1100003, 1, 3), 0, np.float64),
+                              ((2100001, 3), 0, np.int32), ((3000001, 3), 0, np.uint8), ((600011, 7), 0, np.int16),
+                              # rows wider than a workgroup: the period spans several workgroups ("flat-wide")
+                              ((2051, 4097), 0, np.float32), ((1031, 5003), 0, np.float16), ((2, 1028, 2051), 1, np.float32),
+                              ((1101, 8191), 0, np.uint8), ((1501, 2051), 0, np.int32), ((301, 4099), 0, np.float64)):
+        if np.issubdtype(npdt, np.floating):
+            base = rng.standard_normal(shape).astype(npdt)
+        else:
+            base = rng.integers(0, 100, shape).astype(npdt)   # many ties
+        t, a = upload(hpt, base, dev=dev)
+        tag = f"{np.dtype(npdt).name} {shape} axis={axis}"
+        gi, wi = t.argmax(axis).numpy(), orc.argreduce(True, a, axis)
+        assert np.array_equal(gi, wi), tag
+        assert np.array_equal(t.argmin(axis).numpy(), orc.argreduce(False, a, axis)), tag
+        assert np.array_equal(t.max([axis]).numpy(), a.max(axis)), tag
+        if npdt == np.float16:
+            want = orc.reduce(orc.SUM, a, [axis], acc=orc.ACC_F32)
+            assert_close(t.sum([axis]).numpy().astype(np.float32), want.astype(np.float32), HALF_RTOL, half_atol(want.astype(np.float32), 11), tag)
+        elif np.issubdtype(npdt, np.floating):
+            want = orc.reduce(orc.SUM, a, [axis], acc=orc.ACC_F64)
+            assert_close(t.sum([axis]).numpy(), want, F32_RTOL, F32_ATOL if npdt == np.float32 else 1e-9, tag)
+            assert_close(t.mean([axis]).numpy(), a.astype(np.float64).mean(axis), F32_RTOL, F32_ATOL, tag)
+        else:
+            assert np.array_equal(t.sum([axis]).numpy(), orc.reduce(orc.SUM, a, [axis])), tag
+    # a constant slab: every index ties, the lowest wins on every path
+    c = hpt.Tensor.full(2.5, [900001, 3], hpt.f32, dev)
+    assert c.argmax(0).numpy().tolist() == [0, 0, 0] and c.argmin(0).numpy().tolist() == [0, 0, 0]
+    assert c.sum([0]).numpy().tolist() == [900001 * 2.5] * 3
+
+
 def test_sum_inplace_out_and_accumulate(hpt, orc, dev):
     """sum_ with init_out: true overwrites, false adds to what `out` holds (reduce.rs:84-92)."""
     rng = np.random.default_rng(107)
