@@ -121,6 +121,15 @@ template <class T, int N>
 __device__ __forceinline__ void store_pack(T* p, const Pack<T, N>& v) {
     *reinterpret_cast<Pack<T, N>*>(p) = v;
 }
+// N consecutive elements from an address that is only element-aligned: one wide load all the
+// same (global memory takes unaligned vector accesses), at the cost of touching two lines now and
+// then. For small operands that sit in cache: gamma / beta of a row that starts off a boundary.
+template <class T, int N>
+__device__ __forceinline__ Pack<T, N> load_pack_unaligned(const T* p) {
+    Pack<T, N> v;
+    __builtin_memcpy(&v, p, sizeof(T) * N);
+    return v;
+}
 
 // Streaming (non-temporal) forms for data that is touched exactly once: the
 // access is marked so that it does not displace reusable lines from the caches.

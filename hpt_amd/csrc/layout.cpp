@@ -475,14 +475,20 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 }
             }
             p.vec = v;
-            // Rows that start off 16-byte boundaries (odd row lengths): the streaming kernel can still
-            // move aligned vectors and mask the two ends of a row, provided input and output rows are
+            // Rows that start off 16-byte boundaries (odd row lengths): the row kernels can still move
+            // aligned vectors and mask the two ends of a row, provided input and output rows are
             // misaligned by the same amount: equal bases and row pitches modulo 16 bytes.
-            if (sa == 1 && v == 1 && max_vec > 1 && p.cols >= 1024 && p.rows > 128) {
+            // (few, very long rows are shared among workgroups below, element by element). Measured: the
+            // register kernel gains from this between about 16 and 2048 vectors per row (f32 [130561, 257]
+            // softmax 3.5 -> 4.9 TB/s, [8190, 4097] 3.1 -> 4.1); shorter rows are mostly row ends and stay
+            // element-wise, longer ones stream (two sweeps) at the same speed.
+            if (sa == 1 && v == 1 && max_vec > 1 && p.cols >= 16 * max_vec && !(p.rows <= 128 && p.cols >= 16384)) {
                 bool same = (((uintptr_t)in_data ^ (uintptr_t)out_data) & 15) == 0 && ((uintptr_t)in_data % elem_size) == 0;
                 for (int i = 0; i < p.kept_in.n; ++i)
                     if (((p.kept_in.stride[i] - p.kept_out.stride[i]) * (int64_t)elem_size) % 16 != 0) same = false;
-                if (same) {
+                const int64_t nvs = (p.cols + 2 * (max_vec - 1)) / max_vec;
+                // (two-byte layernorm keeps two vectors per thread: beyond 512 threads per row it only loses)
+                if (same && nvs > ((n_norm_dims > 0 && elem_size == 2) ? 512 : 2048)) {
                     p.kind = NormKind::RowStream;
                     p.vec = max_vec;
                     p.shift = 1;
@@ -490,11 +496,17 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     p.rpb = 1;
                     return p;
                 }
+                if (same) {
+                    v = max_vec;
+                    p.vec = v;
+                    p.shift = 1;
+                }
             }
-            int64_t nv = p.cols / (v / p.sstride);
+            // vector loads per row (shifted rows: one more than the row's own length needs)
+            int64_t nv = p.shift ? (p.cols + 2 * (v - 1)) / v : p.cols / (v / p.sstride);
             // Few, very long contiguous rows: share each row among workgroups. (One workgroup per
             // row would leave a chip of 256 compute units mostly idle.)
-            if (sa == 1 && p.rows <= 128 && p.cols >= 16384 && p.cols % v == 0) {
+            if (sa == 1 && !p.shift && p.rows <= 128 && p.cols >= 16384 && p.cols % v == 0) {
                 const int64_t nvec = p.cols / v;
                 int64_t S = std::min<int64_t>(512, std::max<int64_t>(1, 1024 / p.rows));
                 S = std::min<int64_t>(S, std::max<int64_t>(1, nvec / 1024));  // at least 4 vectors per thread
@@ -508,14 +520,18 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             // A row fits the registers of a workgroup up to 8 vectors per thread; layernorm also keeps
             // gamma and beta there (the eight-vector form spills), so it stops at four and streams
             // longer rows (two sweeps; gamma / beta as vectors).
-            const int64_t reg_limit = (n_norm_dims > 0 && v > 1) ? 4096 : 8192;
+            // Two-byte types hold eight elements per vector: with gamma and beta beside the row, sixteen
+            // elements per thread is what fits 128 registers, i.e. two vectors (four of a stride-2 row).
+            const bool ln_half = n_norm_dims > 0 && v > 1 && elem_size == 2;
+            const int64_t per = ln_half ? 2 * p.sstride : 4;
+            const int64_t reg_limit = ln_half ? 1024 * per : (n_norm_dims > 0 && v > 1) ? 4096 : 8192;
             if (nv <= reg_limit) {
                 p.kind = NormKind::RowReg;
                 // about four 128-bit vectors per thread; rows that only allow single elements
                 // take eight per thread (fewer, busier threads: a 257-element row stays in one
                 // wavefront instead of four that meet in LDS)
-                p.tpr = (int)std::min<int64_t>(1024, v > 1 ? pow2_ceil((nv + 3) / 4) : pow2_ceil((nv + 7) / 8));
-                if (p.tpr > 64 && p.tpr < 256) p.tpr = 256;
+                p.tpr = (int)std::min<int64_t>(1024, v > 1 ? pow2_ceil((nv + per - 1) / per) : pow2_ceil((nv + 7) / 8));
+                if (p.tpr > 64 && p.tpr < 256 && !(ln_half && p.tpr == 128)) p.tpr = 256;
                 int64_t nc = (nv + p.tpr - 1) / p.tpr;
                 p.nchunk = std::max(1, pow2_ceil(nc));
                 int block = std::max(256, p.tpr);

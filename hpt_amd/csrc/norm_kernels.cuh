@@ -96,8 +96,16 @@ __device__ __forceinline__ A row_all_reduce(A v, int tpr, int ty, A* smem) {
 // same cache lines as a scalar gather with a fraction of the instructions. (A
 // 16-byte aligned vector that holds one valid element never leaves that element's
 // page, so the unused half of the last vector is safe to touch.)
-template <int KIND, class T, int VEC, int NCHUNK, int SS = 1>
+// SHIFT (VEC > 1, SS = 1): rows whose START is only element-aligned (odd row lengths: 197, 4097,
+// 50257). A row is covered by the 16-byte ALIGNED vectors that contain it: vector iv holds the
+// row's elements iv * VEC - m ... + VEC - 1, m = the row's misalignment in elements; positions
+// outside the row are masked, whole vectors are stored whole and the two end vectors element by
+// element. Input, output and residual rows share m (the caller checks bases and pitches mod 16
+// bytes). Layernorm keeps gamma / beta per thread, so a thread's rows must share m as well: the
+// launch makes the row step of the walk a multiple of VEC.
+template <int KIND, class T, int VEC, int NCHUNK, int SS = 1, bool SHIFT = false>
 __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
+    static_assert(!SHIFT || (VEC > 1 && SS == 1), "SHIFT is a full-vector mode");
     constexpr int UV = VEC / SS;  // useful elements per vector
     using CT = typename Elem<T>::Wide;
     using ST = typename StatType<T>::type;
@@ -107,7 +115,10 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     const int tpr = a.tpr;
     const int tx = threadIdx.x & (tpr - 1);
     const int ty = threadIdx.x >> a.tpr_log2;
-    const int nv = (int)(a.cols / UV);
+    const int nv = SHIFT ? (int)((a.cols + 2 * (VEC - 1)) / VEC) : (int)(a.cols / UV);  // SHIFT: upper bound
+    const int cols = (int)a.cols;
+    // misalignment, in elements, of a row that starts at p
+    auto shift_of = [](const T* p) -> int { return SHIFT ? (int)(((uintptr_t)p / sizeof(T)) % VEC) : 0; };
     constexpr bool kSoft = !norm_is_layer(KIND);
     constexpr bool kLog = norm_is_log(KIND);
     constexpr bool kCausal = norm_is_causal(KIND);
@@ -125,7 +136,23 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                 gam[c].v[j] = Elem<T>::narrow((CT)1);
                 bet[c].v[j] = Elem<T>::narrow((CT)0);
             }
-            if (iv < nv) {
+            if constexpr (SHIFT) {
+                // every row this thread will see has the misalignment of its first one
+                const int64_t row = (int64_t)blockIdx.x * a.rpb + ty;
+                const int m = shift_of((const T*)a.out + (row < a.rows ? row : 0) * a.cols);
+                const int e0 = iv * VEC - m;
+                if (e0 >= 0 && e0 + VEC <= cols) {
+                    if (a.gamma) gam[c] = load_pack_unaligned<T, UV>((const T*)a.gamma + e0);
+                    if (a.beta) bet[c] = load_pack_unaligned<T, UV>((const T*)a.beta + e0);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < UV; ++j)
+                        if ((unsigned)(e0 + j) < (unsigned)cols) {
+                            if (a.gamma) gam[c].v[j] = ((const T*)a.gamma)[e0 + j];
+                            if (a.beta) bet[c].v[j] = ((const T*)a.beta)[e0 + j];
+                        }
+                }
+            } else if (iv < nv) {
                 if constexpr (VEC > 1) {
                     if (a.gamma) gam[c] = load_pack<T, UV>((const T*)a.gamma + (int64_t)iv * UV);
                     if (a.beta) bet[c] = load_pack<T, UV>((const T*)a.beta + (int64_t)iv * UV);
@@ -164,7 +191,9 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
         const int64_t row = row0 + ty;
         if (row >= a.rows) return;
         const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
-        const int nv_row = kCausal ? (int)((row_limit(row) + UV - 1) / UV) : nv;
+        const int m = shift_of(in_row);
+        in_row -= m;
+        const int nv_row = (kCausal || SHIFT) ? (int)((row_limit(row) + m + UV - 1) / UV) : nv;
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int iv = c * tpr + tx;
@@ -172,7 +201,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                 if constexpr (VEC > 1) raw[c] = load_pack_stream<T, VEC>(in_row + (int64_t)iv * VEC);
                 else raw[c].v[0] = in_row[(int64_t)iv * a.sa];
                 if constexpr (kRes) {
-                    const T* res_row = (const T*)a.residual + row * a.cols;
+                    const T* res_row = (const T*)a.residual + row * a.cols - m;
                     if constexpr (VEC > 1) raw_res[c] = load_pack_stream<T, UV>(res_row + (int64_t)iv * UV);
                     else raw_res[c].v[0] = res_row[iv];
                 }
@@ -186,6 +215,12 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
         const bool valid = row < a.rows;
         T* out_row = (T*)a.out + (valid ? row * a.cols : 0);
         const int limit = valid ? (int)row_limit(row) : 0;  // cols <= 8192 vectors here
+        const int sh = shift_of(out_row);
+        // is element j of vector iv inside the row (and, for the causal kinds, kept)?
+        auto inside = [&](int iv, int j) -> bool {
+            if constexpr (SHIFT) return (unsigned)(iv * UV + j - sh) < (unsigned)limit;
+            else return iv < nv && (!kCausal || iv * UV + j < limit);
+        };
 
         CT x[NCHUNK][UV];
 #pragma unroll
@@ -193,7 +228,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
             const int iv = c * tpr + tx;
 #pragma unroll
             for (int j = 0; j < UV; ++j) {
-                const bool have = valid && iv < nv && (!kCausal || iv * UV + j < limit);
+                const bool have = valid && inside(iv, j);
                 CT e = have ? Elem<T>::widen(raw[c].v[j * SS]) : fill;
                 // the fused forms round the intermediate (in + residual, scale * in) to the tensor's
                 // dtype, as the separate add / mul_ of the unfused sequence would have stored it
@@ -217,7 +252,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                 // causal kinds: a chunk that lies wholly above the diagonal (the same for every lane
                 // of the row) is all -inf: its exponentials are 0 without computing them. A row with
                 // no key at all takes the ordinary way and comes out NaN, as -inf - -inf does.
-                if (kCausal && limit > 0 && c * tpr * UV >= limit) {
+                if (kCausal && limit > 0 && c * tpr * UV - sh >= limit) {
 #pragma unroll
                     for (int j = 0; j < UV; ++j) x[c][j] = kLog ? neg_inf<CT>() : (CT)0;
                     continue;
@@ -256,7 +291,8 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                 const bool in_row_c = (c * tpr + tx) < nv;
 #pragma unroll
                 for (int j = 0; j < UV; ++j) {
-                    const CT d = in_row_c ? (x[c][j] - mean_hi) - mean_lo : (CT)0;
+                    const bool in_row_e = SHIFT ? inside(c * tpr + tx, j) : in_row_c;
+                    const CT d = in_row_e ? (x[c][j] - mean_hi) - mean_lo : (CT)0;
                     x[c][j] = d;
                     q += d * d;
                 }
@@ -274,7 +310,21 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c) {
                 const int iv = c * tpr + tx;
-                if (iv < nv) {
+                if constexpr (SHIFT) {
+                    const int e0 = iv * VEC - sh;
+                    if (e0 + VEC > 0 && e0 < cols) {
+                        Pack<T, UV> o;
+#pragma unroll
+                        for (int j = 0; j < UV; ++j) o.v[j] = Elem<T>::narrow(x[c][j]);
+                        if (e0 >= 0 && e0 + VEC <= cols) {
+                            store_pack_stream<T, UV>(out_row + e0, o);
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < UV; ++j)
+                                if ((unsigned)(e0 + j) < (unsigned)cols) out_row[e0 + j] = o.v[j];
+                        }
+                    }
+                } else if (iv < nv) {
                     if constexpr (VEC > 1) {
                         Pack<T, UV> o;
 #pragma unroll
@@ -526,6 +576,20 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
                 }
                 if (a.gamma) g = load_pack<T, VEC>((const T*)a.gamma + iv * VEC);
                 if (a.beta) b = load_pack<T, VEC>((const T*)a.beta + iv * VEC);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    x[j] = ((x[j] - mean_hi) - mean_lo) * rstd * Elem<T>::widen(g.v[j]) + Elem<T>::widen(b.v[j]);
+            } else if (SHIFT && iv * VEC - m >= 0 && iv * VEC - m + VEC <= a.cols) {
+                // a whole vector of a shifted row: its gamma / beta run starts off a boundary by m
+                const int64_t e0 = iv * VEC - m;
+                Pack<T, VEC> g, b;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    g.v[j] = Elem<T>::narrow((CT)1);
+                    b.v[j] = Elem<T>::narrow((CT)0);
+                }
+                if (a.gamma) g = load_pack_unaligned<T, VEC>((const T*)a.gamma + e0);
+                if (a.beta) b = load_pack_unaligned<T, VEC>((const T*)a.beta + e0);
 #pragma unroll
                 for (int j = 0; j < VEC; ++j)
                     x[j] = ((x[j] - mean_hi) - mean_lo) * rstd * Elem<T>::widen(g.v[j]) + Elem<T>::widen(b.v[j]);

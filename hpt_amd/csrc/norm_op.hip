@@ -20,13 +20,13 @@ inline int ilog2(int v) {
     return l;
 }
 
-template <class T, int VEC, int SS = 1>
+template <class T, int VEC, int SS = 1, bool SHIFT = false>
 void launch_row_reg(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block, hipStream_t st) {
     switch (p.nchunk) {
-        case 1: row_reg_kernel<KIND, T, VEC, 1, SS><<<grid, block, 0, st>>>(a); break;
-        case 2: row_reg_kernel<KIND, T, VEC, 2, SS><<<grid, block, 0, st>>>(a); break;
-        case 4: row_reg_kernel<KIND, T, VEC, 4, SS><<<grid, block, 0, st>>>(a); break;
-        case 8: row_reg_kernel<KIND, T, VEC, 8, SS><<<grid, block, 0, st>>>(a); break;
+        case 1: row_reg_kernel<KIND, T, VEC, 1, SS, SHIFT><<<grid, block, 0, st>>>(a); break;
+        case 2: row_reg_kernel<KIND, T, VEC, 2, SS, SHIFT><<<grid, block, 0, st>>>(a); break;
+        case 4: row_reg_kernel<KIND, T, VEC, 4, SS, SHIFT><<<grid, block, 0, st>>>(a); break;
+        case 8: row_reg_kernel<KIND, T, VEC, 8, SS, SHIFT><<<grid, block, 0, st>>>(a); break;
         default: fail(HPT_ERR_KERNEL, "row_reg: unsupported chunk count %d", p.nchunk);
     }
 }
@@ -178,6 +178,18 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         // Layernorm workgroups walk the rows (gamma / beta stay in registers);
         // softmax has nothing to reuse across rows and runs one row per group.
         if (norm_is_layer(KIND) && grid.x > (unsigned)p.max_blocks) grid.x = (unsigned)p.max_blocks;
+        if constexpr (FULL > 1) {
+            if (p.vec == FULL && p.shift) {
+                // shifted rows: a thread's gamma / beta fit every row it walks only if those rows share
+                // their misalignment, i.e. the row step is a whole number of vectors
+                if (norm_is_layer(KIND) && (int64_t)grid.x * p.rpb < p.rows) {
+                    if (grid.x >= (unsigned)FULL) grid.x -= grid.x % FULL;
+                    else fail(HPT_ERR_KERNEL, "row_reg: shifted rows need a row step of whole vectors");
+                }
+                launch_row_reg<T, FULL, 1, true>(p, a, grid, block, st);
+                return;
+            }
+        }
         if (p.vec == FULL && p.sstride == 2 && FULL > 1) launch_row_reg<T, FULL, 2>(p, a, grid, block, st);
         else if (p.vec == FULL) launch_row_reg<T, FULL>(p, a, grid, block, st);
         else launch_row_reg<T, 1>(p, a, grid, block, st);
