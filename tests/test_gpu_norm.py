@@ -305,3 +305,58 @@ def test_few_long_rows_are_shared_by_workgroups(hpt, orc, dev, case):
         from oracle import elementwise as ew
         summed = ew.binary(ew.ADD, ac, r)
         check(t.add_layernorm(tr, [n], tg, tb, 1e-5).numpy(), orc.layernorm(summed, 1, g, b, 1e-5, acc=acc), "add_layernorm", 4e-6)
+
+
+WIDE_ROW_CASES = [
+    # more rows than the 512 workgroups launched: each walks two or three rows, the last ones fewer
+    ("f32 2050 vectors, 1024 threads per row", np.float32, [1300, 8200]),
+    ("f32 odd number of chunks", np.float32, [1100, 10000]),
+    ("f64", np.float64, [1030, 4100]),
+    ("f16 two vectors per thread", np.float16, [1100, 8192]),
+    ("f16 eight vectors per thread", np.float16, [600, 65536]),
+    ("bf16", "bf16", [1111, 16384]),
+    # odd lengths: aligned vectors, masked row ends (registers up to 2048 vectors, then streaming)
+    ("f32 rows of 4097", np.float32, [2100, 4097]),
+    ("f16 rows of 197", np.float16, [30011, 197]),
+    ("f32 rows of 257 in a 3-D tensor", np.float32, [7, 1500, 257]),
+    ("bf16 rows of 10001", "bf16", [700, 10001]),
+]
+
+
+@pytest.mark.parametrize("case", WIDE_ROW_CASES, ids=[c[0] for c in WIDE_ROW_CASES])
+def test_long_and_odd_rows_walked_with_prefetch(hpt, orc, dev, case):
+    """Rows of 512 / 1024 threads are walked by at most 512 workgroups that issue the next row's loads
+    before the current row's statistics; odd-length rows move aligned vectors with masked ends. Every
+    row must come out as from the plain kernels: first, middle and last rows of the walk alike."""
+    name, npdt, shape = case
+    rng = np.random.default_rng(209)
+    x = (rng.standard_normal(shape) * 2 + rng.uniform(-3, 3, shape[:-1] + [1])).astype(np.float32)
+    if npdt == "bf16":
+        cv, dt, odt, bits, tof, acc = hpt.f32_to_bf16_bits, hpt.bf16, orc.BF16, 8, hpt.bf16_bits_to_f32, orc.ACC_F32
+    elif npdt == np.float16:
+        cv, dt, odt, bits, tof, acc = (lambda v: v.astype(np.float16)), None, None, 11, (lambda v: v.astype(np.float32)), orc.ACC_F32
+    else:
+        cv, dt, odt, bits, tof, acc = (lambda v: v.astype(npdt)), None, None, 0, (lambda v: v), orc.ACC_F64
+    a = cv(x)
+    t = hpt.Tensor.from_numpy(a, dt).to_hip(dev)
+    n = shape[-1]
+    ax = len(shape) - 1
+    g, b = cv(rng.normal(1, 0.1, n).astype(np.float32)), cv(rng.normal(0, 0.1, n).astype(np.float32))
+    tg, tb = (hpt.Tensor.from_numpy(v, dt).to_hip(dev) for v in (g, b))
+
+    def check(got, want, what, atol32=F32_ATOL):
+        got, want = tof(got), tof(want)
+        if bits:
+            assert_close(got, want, HALF_RTOL, max(half_atol(want[np.isfinite(want)], bits), 6e-8), f"{what} {name}")
+        else:
+            assert_close(got, want, F32_RTOL, atol32, f"{what} {name}")
+
+    check(t.softmax(ax).numpy(), orc.softmax(a, ax, acc=acc, dtype=odt), "softmax")
+    check(t.log_softmax(-1).numpy(), orc.softmax(a, ax, log=True, acc=acc, dtype=odt), "log_softmax", 2e-6)
+    check(t.layernorm([n], tg, tb, 1e-5).numpy(), orc.layernorm(a, 1, g, b, 1e-5, acc=acc, dtype=odt), "layernorm", 4e-6)
+    if not bits:
+        from oracle import elementwise as ew
+        r = cv(rng.standard_normal(shape).astype(np.float32))
+        tr = hpt.Tensor.from_numpy(r, dt).to_hip(dev)
+        check(t.add_layernorm(tr, [n], tg, tb, 1e-5).numpy(), orc.layernorm(ew.binary(ew.ADD, a, r), 1, g, b, 1e-5, acc=acc),
+              "add_layernorm", 4e-6)
