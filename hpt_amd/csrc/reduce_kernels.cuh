@@ -236,6 +236,64 @@ __device__ __forceinline__ void fold_thread_rows(typename Op::Acc (&acc)[VEC], t
     }
 }
 
+// Short rows laid back to back (a contiguous [K, R] matrix, R * sizeof(T) <= 1 KiB): a workgroup
+// stages `rows_per_wg` consecutive rows (16 KiB, a multiple of VEC rows so that the tile starts
+// on a 16-byte boundary) in LDS with aligned 128-bit loads, then groups of `tpr` lanes reduce
+// the rows out of LDS. HBM sees only whole, aligned lines whatever R is.
+struct RowTileArgs {
+    const void* in;
+    void* out;
+    int64_t K;   // rows
+    double count;
+    int R;       // row length
+    int rows_per_wg;
+    int tpr, tpr_log2;
+    int init_out;
+};
+
+template <class Op, int VEC>
+__global__ void __launch_bounds__(256) row_tile_kernel(const RowTileArgs a) {
+    using T = typename Op::In;
+    using Acc = typename Op::Acc;
+    constexpr int NV = 4;  // vectors per thread: 256 * 4 * 16 bytes = 16 KiB
+    __shared__ __align__(16) unsigned char tile_raw[256 * NV * 16];
+    T* tile = reinterpret_cast<T*>(tile_raw);
+    const int t = threadIdx.x;
+    const int64_t row0 = (int64_t)blockIdx.x * a.rows_per_wg;
+    const int64_t left = a.K - row0;
+    const int nrows = left < a.rows_per_wg ? (int)left : a.rows_per_wg;
+    const int n = nrows * a.R;  // elements of this tile
+    const T* src = (const T*)a.in + row0 * a.R;
+    Pack<T, VEC> v[NV];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int e = (t + u * 256) * VEC;
+        if (e + VEC <= n) {
+            v[u] = load_pack_stream<T, VEC>(src + e);
+        } else {  // the tensor's last, partial vector
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                if (e + j < n) v[u].v[j] = src[e + j];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int e = (t + u * 256) * VEC;
+        if (e < n) store_pack<T, VEC>(tile + e, v[u]);
+    }
+    __syncthreads();
+    const int tx = t & (a.tpr - 1);
+    const int g = t >> a.tpr_log2;
+    const int groups = 256 >> a.tpr_log2;
+    for (int r = g; r < nrows; r += groups) {
+        Acc acc = Op::identity();
+        const T* row = tile + r * a.R;
+        for (int c = tx; c < a.R; c += a.tpr) fold_in<Op>(acc, row[c], c);
+        acc = group_reduce<Op>(acc, a.tpr);
+        if (tx == 0) write_out<Op>(a.out, row0 + r, acc, a.init_out, a.count);
+    }
+}
+
 // Lean form: outputs are (outer, inner) with inner the lane dim; one reduced dim.
 // out[outer * kin + inner] = reduce over r of in[outer * so + r * rs + inner * sk].
 struct ColLeanArgs {
@@ -589,6 +647,22 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
     }
     const bool vec = p.vec == FULL && FULL > 1;
     void* stage1_out = p.split > 1 ? sc.partial : out;
+    if (p.kind == ReduceKind::Row && p.row_tile > 0) {
+        if constexpr (FULL > 1) {
+            RowTileArgs a{};
+            a.in = in;
+            a.out = out;
+            a.K = p.K;
+            a.count = count;
+            a.R = (int)p.R;
+            a.rows_per_wg = p.row_tile;
+            a.tpr = p.tpr;
+            a.tpr_log2 = ilog2(p.tpr);
+            a.init_out = init_out;
+            row_tile_kernel<Op, FULL><<<dim3((unsigned)((p.K + p.row_tile - 1) / p.row_tile)), dim3(256), 0, st>>>(a);
+        }
+        return;
+    }
     if (p.kind == ReduceKind::Row) {
         dim3 grid((unsigned)((p.K + p.rpb - 1) / p.rpb), (unsigned)p.split);
         dim3 block((unsigned)(p.tpr * p.rpb));

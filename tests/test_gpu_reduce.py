@@ -239,6 +239,45 @@ def test_narrow_inner_dim_flat_walk(hpt, orc, dev):
     assert c.sum([0]).numpy().tolist() == [900001 * 2.5] * 3
 
 
+def test_short_rows_staged_through_lds(hpt, orc, dev):
+    """Contiguous [N, k] with short rows reduced over k: 16 KiB tiles of whole rows are brought in
+    with aligned vectors and reduced out of LDS. Row lengths that are / are not whole vectors, a
+    partial last tile and a partial last vector; ties for the index rule."""
+    rng = np.random.default_rng(117)
+    assert hpt.reduce_plan(hpt.Tensor.empty([1400001, 3], hpt.f32, dev), hpt.SUM, [1]).startswith("row-tile")
+    for shape, npdt in (((1400001, 3), np.float32), ((200003, 33), np.float16), ((50001, 100), np.int32),
+                        ((30001, 255), np.float32), ((300001, 17), np.uint8), ((70001, 9), np.float64),
+                        ((1100001, 8), np.float16), ((40, 30001, 5), np.float32), ((9001, 512), np.int16)):
+        if np.issubdtype(npdt, np.floating):
+            base = rng.standard_normal(shape).astype(npdt)
+        else:
+            base = rng.integers(0, 50, shape).astype(npdt)   # many ties
+        t, a = upload(hpt, base, dev=dev)
+        ax = len(shape) - 1
+        tag = f"{np.dtype(npdt).name} {shape}"
+        assert np.array_equal(t.argmax(ax).numpy(), orc.argreduce(True, a, ax)), tag
+        assert np.array_equal(t.argmin(ax).numpy(), orc.argreduce(False, a, ax)), tag
+        assert np.array_equal(t.min([ax]).numpy(), a.min(ax)), tag
+        if npdt == np.float16:
+            want = orc.reduce(orc.SUM, a, [ax], acc=orc.ACC_F32).astype(np.float32)
+            assert_close(t.sum([ax]).numpy().astype(np.float32), want, HALF_RTOL, half_atol(want, 11), tag)
+        elif np.issubdtype(npdt, np.floating):
+            assert_close(t.sum([ax]).numpy(), orc.reduce(orc.SUM, a, [ax], acc=orc.ACC_F64), F32_RTOL, F32_ATOL, tag)
+            assert_close(t.reducel2([ax]).numpy(), np.sqrt((a.astype(np.float64) ** 2).sum(ax)), F32_RTOL, F32_ATOL, tag)
+        else:
+            assert np.array_equal(t.sum([ax]).numpy(), orc.reduce(orc.SUM, a, [ax])), tag
+            assert np.array_equal(t.prod([ax]).numpy(), orc.reduce(orc.PROD, a, [ax])), tag
+    b = rng.integers(0, 2, (900001, 7)).astype(np.bool_)
+    tb, ab = upload(hpt, b, dev=dev)
+    assert np.array_equal(tb.all([1]).numpy(), ab.all(1)) and np.array_equal(tb.any([1]).numpy(), ab.any(1))
+    # accumulate into an existing output
+    x = rng.standard_normal((1200000, 3)).astype(np.float32)
+    tx, ax_ = upload(hpt, x, dev=dev)
+    out = hpt.Tensor.full(2.0, [1200000], hpt.f32, dev)
+    tx.sum_([1], False, False, out)
+    assert_close(out.numpy(), ax_.astype(np.float64).sum(1) + 2.0, F32_RTOL, F32_ATOL, "sum_ accumulate, short rows")
+
+
 def test_sum_inplace_out_and_accumulate(hpt, orc, dev):
     """sum_ with init_out: true overwrites, false adds to what `out` holds (reduce.rs:84-92)."""
     rng = np.random.default_rng(107)
