@@ -344,6 +344,133 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     }
 }
 
+// ---- short rows laid back to back: whole tiles through LDS ---------------------------------
+// A contiguous [rows, cols] matrix with short rows (cols <= 512): a workgroup brings a.rpb
+// consecutive rows (16 KiB; a multiple of VEC rows, so the tile starts on a 16-byte boundary
+// whatever cols is) into LDS with aligned 128-bit loads, groups of `tpr` lanes normalise the rows
+// in place (at most eight elements per lane, held in registers between the passes), and the tile
+// leaves with aligned 128-bit stores. HBM sees whole lines only, in both directions.
+template <int KIND, class T, int VEC>
+__global__ void __launch_bounds__(256) norm_tile_kernel(const NormArgs a) {
+    static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX || KIND == NORM_LAYERNORM, "plain kinds only");
+    using CT = typename Elem<T>::Wide;
+    using ST = typename StatType<T>::type;
+    constexpr bool kSoft = !norm_is_layer(KIND);
+    constexpr bool kLog = norm_is_log(KIND);
+    constexpr int NV = 4;   // vectors per thread: 256 * 4 * 16 bytes = 16 KiB
+    constexpr int EPL = 8;  // elements per lane at most
+    __shared__ __align__(16) unsigned char tile_raw[256 * NV * 16];
+    T* tile = reinterpret_cast<T*>(tile_raw);
+    const int t = threadIdx.x;
+    const int R = (int)a.cols;
+    const int64_t row0 = (int64_t)blockIdx.x * a.rpb;
+    const int64_t left = a.rows - row0;
+    const int nrows = left < a.rpb ? (int)left : a.rpb;
+    const int n = nrows * R;
+    const T* src = (const T*)a.in + row0 * R;
+    T* dst = (T*)a.out + row0 * R;
+    {
+        Pack<T, VEC> v[NV];
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int e = (t + u * 256) * VEC;
+            if (e + VEC <= n) {
+                v[u] = load_pack_stream<T, VEC>(src + e);
+            } else {  // the tensor's last, partial vector
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    if (e + j < n) v[u].v[j] = src[e + j];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int e = (t + u * 256) * VEC;
+            if (e < n) store_pack<T, VEC>(tile + e, v[u]);
+        }
+    }
+    __syncthreads();
+    const int tpr = a.tpr;
+    const int tx = t & (tpr - 1);
+    const int g = t >> a.tpr_log2;
+    const int groups = 256 >> a.tpr_log2;
+    const CT fill = kSoft ? neg_inf<CT>() : (CT)0;
+    // a lane keeps its columns from row to row: gamma / beta are fetched once
+    CT gam[kSoft ? 1 : EPL], bet[kSoft ? 1 : EPL];
+    if constexpr (!kSoft) {
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+            const int c = tx + i * tpr;
+            gam[i] = (a.gamma && c < R) ? Elem<T>::widen(((const T*)a.gamma)[c]) : (CT)1;
+            bet[i] = (a.beta && c < R) ? Elem<T>::widen(((const T*)a.beta)[c]) : (CT)0;
+        }
+    }
+    for (int r = g; r < nrows; r += groups) {
+        T* row = tile + r * R;
+        CT x[EPL];
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+            const int c = tx + i * tpr;
+            x[i] = c < R ? Elem<T>::widen(row[c]) : fill;
+        }
+        if constexpr (kSoft) {
+            CT m = neg_inf<CT>();
+#pragma unroll
+            for (int i = 0; i < EPL; ++i) m = MaxC<CT>::comb(m, x[i]);
+            m = group_reduce<MaxC<CT>>(m, tpr);
+            CT s = 0;
+#pragma unroll
+            for (int i = 0; i < EPL; ++i) {
+                const CT d = x[i] - m;
+                const CT e = exp_ct<T>(d);
+                s += e;
+                x[i] = kLog ? d : e;
+            }
+            s = group_reduce<SumC<CT>>(s, tpr);
+            const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
+#pragma unroll
+            for (int i = 0; i < EPL; ++i) x[i] = kLog ? x[i] - k : x[i] * k;
+        } else {
+            // (a row may be three elements: the lane's own sum is taken in the wide type too, or the
+            // mean of a row whose spread is small against its offset loses digits that matter)
+            ST s = 0;
+#pragma unroll
+            for (int i = 0; i < EPL; ++i) s += (ST)x[i];
+            const ST sum = group_reduce<SumC<ST>>(s, tpr);
+            const ST m0 = sum * (ST)a.inv_cols;
+            const ST mean = fma_ct(fma_ct(-m0, (ST)a.cols, sum), (ST)a.inv_cols, m0);
+            const CT mean_hi = (CT)mean;
+            const CT mean_lo = (CT)(mean - (ST)mean_hi);
+            CT q = 0;
+#pragma unroll
+            for (int i = 0; i < EPL; ++i) {
+                const CT d = tx + i * tpr < R ? (x[i] - mean_hi) - mean_lo : (CT)0;
+                x[i] = d;
+                q += d * d;
+            }
+            const ST var = group_reduce<SumC<ST>>((ST)q, tpr) * (ST)a.inv_cols;
+            const CT rstd = rsqrt_ct((CT)var + (CT)a.eps);
+#pragma unroll
+            for (int i = 0; i < EPL; ++i) x[i] = x[i] * rstd * gam[i] + bet[i];
+        }
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+            const int c = tx + i * tpr;
+            if (c < R) row[c] = Elem<T>::narrow(x[i]);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int e = (t + u * 256) * VEC;
+        if (e + VEC <= n) {
+            store_pack_stream<T, VEC>(dst + e, load_pack<T, VEC>(tile + e));
+        } else {
+            for (int j = 0; j < VEC; ++j)
+                if (e + j < n) dst[e + j] = tile[e + j];
+        }
+    }
+}
+
 // ---- streaming rows: online statistics, then a second sweep ------------------
 
 // running (max, sum of exp(x - max)); the sum may be carried in a wider type ST

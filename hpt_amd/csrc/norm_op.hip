@@ -177,6 +177,17 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
     if (p.kind == NormKind::RowReg) {
         // Layernorm workgroups walk the rows (gamma / beta stay in registers);
         // softmax has nothing to reuse across rows and runs one row per group.
+        if constexpr (FULL > 1 && KIND <= NORM_LAYERNORM) {
+            if (p.tile_rows > 0) {
+                a.rpb = p.tile_rows;
+                a.tpr = 1;
+                while (a.tpr < 64 && a.tpr * 8 < p.cols) a.tpr <<= 1;
+                a.tpr_log2 = ilog2(a.tpr);
+                norm_tile_kernel<KIND, T, FULL>
+                    <<<dim3((unsigned)((p.rows + p.tile_rows - 1) / p.tile_rows)), dim3(256), 0, st>>>(a);
+                return;
+            }
+        }
         if (norm_is_layer(KIND) && grid.x > (unsigned)p.max_blocks) grid.x = (unsigned)p.max_blocks;
         if constexpr (FULL > 1) {
             if (p.vec == FULL && p.shift) {

@@ -360,3 +360,63 @@ def test_long_and_odd_rows_walked_with_prefetch(hpt, orc, dev, case):
         tr = hpt.Tensor.from_numpy(r, dt).to_hip(dev)
         check(t.add_layernorm(tr, [n], tg, tb, 1e-5).numpy(), orc.layernorm(ew.binary(ew.ADD, a, r), 1, g, b, 1e-5, acc=acc),
               "add_layernorm", 4e-6)
+
+
+SHORT_ROW_CASES = [
+    ("f32 rows of 3", np.float32, [400001, 3]),
+    ("f32 rows of 8 (whole vectors)", np.float32, [140001, 8]),
+    ("f32 rows of 33 in a 3-D tensor", np.float32, [11, 3001, 33]),
+    ("f32 rows of 100", np.float32, [12001, 100]),
+    ("f64 rows of 65", np.float64, [9001, 65]),
+    ("f16 rows of 33", np.float16, [70001, 33]),
+    ("f16 rows of 64 (whole vectors)", np.float16, [40001, 64]),
+    ("bf16 rows of 197", "bf16", [12001, 197]),
+    ("f32 rows of 511", np.float32, [2501, 511]),
+]
+
+
+@pytest.mark.parametrize("case", SHORT_ROW_CASES, ids=[c[0] for c in SHORT_ROW_CASES])
+def test_short_rows_normalised_in_lds_tiles(hpt, orc, dev, case):
+    """Short rows laid back to back go through 16 KiB LDS tiles (aligned vectors in and out whatever
+    the row length). The row counts leave a partial last tile and a partial last vector; masked and
+    constant rows keep their closed forms."""
+    name, npdt, shape = case
+    rng = np.random.default_rng(210)
+    x = (rng.standard_normal(shape) * 2 + rng.uniform(-3, 3, shape[:-1] + [1])).astype(np.float32)
+    if npdt == "bf16":
+        cv, dt, odt, bits, tof, acc = hpt.f32_to_bf16_bits, hpt.bf16, orc.BF16, 8, hpt.bf16_bits_to_f32, orc.ACC_F32
+    elif npdt == np.float16:
+        cv, dt, odt, bits, tof, acc = (lambda v: v.astype(np.float16)), None, None, 11, (lambda v: v.astype(np.float32)), orc.ACC_F32
+    else:
+        cv, dt, odt, bits, tof, acc = (lambda v: v.astype(npdt)), None, None, 0, (lambda v: v), orc.ACC_F64
+    x.reshape(-1, shape[-1])[5, :] = 1.25           # a constant row
+    x.reshape(-1, shape[-1])[7, 1:] = -np.inf       # a row with one finite entry
+    a = cv(x)
+    t = hpt.Tensor.from_numpy(a, dt).to_hip(dev)
+    n = shape[-1]
+    ax = len(shape) - 1
+    assert "+tile" in hpt.normalize_plan(t, ax), hpt.normalize_plan(t, ax)
+    g, b = cv(rng.normal(1, 0.1, n).astype(np.float32)), cv(rng.normal(0, 0.1, n).astype(np.float32))
+    tg, tb = (hpt.Tensor.from_numpy(v, dt).to_hip(dev) for v in (g, b))
+
+    def check(got, want, what, atol32=F32_ATOL):
+        got, want = tof(got), tof(want)
+        if bits:
+            assert_close(got, want, HALF_RTOL, max(half_atol(want[np.isfinite(want)], bits), 6e-8), f"{what} {name}")
+        else:
+            assert_close(got, want, F32_RTOL, atol32, f"{what} {name}")
+
+    sm = t.softmax(ax).numpy()
+    check(sm, orc.softmax(a, ax, acc=acc, dtype=odt), "softmax")
+    smf = tof(sm).reshape(-1, n)
+    assert np.all(smf[7, 0] == 1.0) and np.all(smf[7, 1:] == 0.0), "one finite entry -> exactly (1, 0, 0, ...)"
+    check(t.log_softmax(-1).numpy(), orc.softmax(a, ax, log=True, acc=acc, dtype=odt), "log_softmax", 2e-6)
+    fin = np.where(np.isfinite(x), x, 0.0).astype(np.float32)   # layernorm of -inf is NaN: compare finite rows
+    af = cv(fin)
+    tf_ = hpt.Tensor.from_numpy(af, dt).to_hip(dev)
+    if "+tile" in hpt.normalize_plan(tf_, 0, 1):
+        ln = tf_.layernorm([n], tg, tb, 1e-5).numpy()
+        check(ln, orc.layernorm(af, 1, g, b, 1e-5, acc=acc, dtype=odt), "layernorm", 4e-6)
+        assert np.array_equal(tof(ln).reshape(-1, n)[5], tof(b)), "constant row -> beta exactly"
+        check(tf_.layernorm([n], None, None, 1e-5).numpy(), orc.layernorm(af, 1, None, None, 1e-5, acc=acc, dtype=odt),
+              "layernorm without gamma / beta", 4e-6)
