@@ -408,15 +408,38 @@ __global__ void __launch_bounds__(1024) col_flat_kernel(const ColFlatArgs a) {
         const int64_t whole = a.total / L;  // periods that lie wholly inside the slab
         const int split = a.split;
         int64_t it = blockIdx.z;  // periods are dealt round-robin over the workgroups of a slab
-        for (; it + 3 * split < whole; it += 4 * split) {
-            Pack<T, VEC> v[4];
+        // Batches of four vectors, two batches alternating: the next batch is in flight while the
+        // current one is folded in. (Its loads are issued unconditionally, from a repeated address
+        // on the last round: a load under a branch would make the wait before the fold a full one.)
+        auto load4 = [&](Pack<T, VEC>(&v)[4], int64_t i0) {
 #pragma unroll
-            for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(base + (it + u * split) * L + p0);
+            for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(base + (i0 + u * split) * L + p0);
+        };
+        auto fold4 = [&](const Pack<T, VEC>(&v)[4], int64_t i0) {
 #pragma unroll
             for (int u = 0; u < 4; ++u)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j)
-                    fold_in<Op>(acc[j], v[u].v[j], row[j] + (int)(it + u * split) * rows_per_period);
+                    fold_in<Op>(acc[j], v[u].v[j], row[j] + (int)(i0 + u * split) * rows_per_period);
+        };
+        const int64_t step = 4 * (int64_t)split;
+        if (it + 3 * split < whole) {
+            Pack<T, VEC> va[4], vb[4];
+            load4(va, it);
+            for (;;) {
+                int64_t nx = it + step;
+                bool more = nx + 3 * split < whole;
+                load4(vb, more ? nx : it);
+                fold4(va, it);
+                it = nx;
+                if (!more) break;
+                nx = it + step;
+                more = nx + 3 * split < whole;
+                load4(va, more ? nx : it);
+                fold4(vb, it);
+                it = nx;
+                if (!more) break;
+            }
         }
         for (; it < whole; it += split) {
             Pack<T, VEC> v = load_pack_stream<T, VEC>(base + it * L + p0);
@@ -486,14 +509,35 @@ __global__ void __launch_bounds__(1024) col_flat_wide_kernel(const ColFlatWideAr
     const int64_t whole = a.total / L;
     const int slices = a.slices;
     int64_t it = blockIdx.z;
-    for (; it + 3 * slices < whole; it += 4 * slices) {
-        Pack<T, VEC> v[4];
+    // two alternating batches of four vectors, as in col_flat_kernel
+    auto load4 = [&](Pack<T, VEC>(&v)[4], int64_t i0) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(base + (it + u * slices) * L + p0);
+        for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(base + (i0 + u * slices) * L + p0);
+    };
+    auto fold4 = [&](const Pack<T, VEC>(&v)[4], int64_t i0) {
 #pragma unroll
         for (int u = 0; u < 4; ++u)
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v[u].v[j], row[j] + (int)(it + u * slices) * a.phases);
+            for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v[u].v[j], row[j] + (int)(i0 + u * slices) * a.phases);
+    };
+    const int64_t step = 4 * (int64_t)slices;
+    if (it + 3 * slices < whole) {
+        Pack<T, VEC> va[4], vb[4];
+        load4(va, it);
+        for (;;) {
+            int64_t nx = it + step;
+            bool more = nx + 3 * slices < whole;
+            load4(vb, more ? nx : it);
+            fold4(va, it);
+            it = nx;
+            if (!more) break;
+            nx = it + step;
+            more = nx + 3 * slices < whole;
+            load4(va, more ? nx : it);
+            fold4(vb, it);
+            it = nx;
+            if (!more) break;
+        }
     }
     for (; it < whole; it += slices) {
         Pack<T, VEC> v = load_pack_stream<T, VEC>(base + it * L + p0);
@@ -608,8 +652,19 @@ __global__ void __launch_bounds__(1024) finish_cols_kernel(const void* part_, vo
     const int64_t o = (int64_t)blockIdx.x * 64 + tx;
     const bool valid = o < K;
     Acc acc = Op::identity();
-    if (valid)
-        for (int s = ty; s < split; s += by) acc = Op::comb(acc, part[(int64_t)s * K + o]);
+    if (valid) {
+        // eight partials in flight per thread (the kernel is a chain of load latencies otherwise)
+        const Acc* p = part + o;
+        int s = ty;
+        for (; s + 7 * by < split; s += 8 * by) {
+            Acc v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = p[(int64_t)(s + u * by) * K];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc = Op::comb(acc, v[u]);
+        }
+        for (; s < split; s += by) acc = Op::comb(acc, p[(int64_t)s * K]);
+    }
     if (by > 1) {
         sm[ty * 64 + tx] = acc;
         __syncthreads();
