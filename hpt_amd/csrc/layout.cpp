@@ -603,6 +603,24 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             if (!vec_ok) v = 1;
             p.kind = NormKind::ColSplit;
             p.vec = v;
+            // A narrow inner dim (or one that is not whole vectors) leaves most lanes idle: walk the
+            // contiguous [cols, L] slab as a flat array of aligned vectors instead.
+            if (max_vec > 1 && (!vec_ok || L < 64 * max_vec) && sa == L && ((uintptr_t)in_data % 16) == 0 &&
+                ((uintptr_t)out_data % 16) == 0 && p.cols * L * (int64_t)elem_size >= (8ll << 20) &&
+                (batch == 1 || (p.kept_in.stride[0] % max_vec == 0 && (p.cols * L) % max_vec == 0))) {
+                int64_t g = L, b = max_vec;
+                while (b) { int64_t t = g % b; g = b; b = t; }
+                const int64_t lp = L / g;  // threads per period
+                const int64_t tmax = std::min<int64_t>(1024, (64 << 10) / (max_vec * (elem_size == 8 ? 16 : 8)));
+                if (lp <= tmax) {
+                    p.flat_t = (int)(lp * (tmax / lp));
+                    p.vec = max_vec;
+                    const int64_t periods = p.cols * L / ((int64_t)p.flat_t * max_vec);
+                    p.tsplit = (int)std::max<int64_t>(1, std::min<int64_t>(periods / 4, std::max<int64_t>(1, 256 / batch)));
+                    p.scratch_bytes = (size_t)p.rows * p.tsplit * 16 + (size_t)p.rows * 3 * 8;
+                    return p;
+                }
+            }
             const int64_t groups = (L + 64 * v - 1) / (64 * v) * batch;
             int64_t S = std::max<int64_t>(1, std::min<int64_t>((512 + groups - 1) / groups, p.cols / 32));
             p.tsplit = (int)std::min<int64_t>(S, 64);
@@ -625,6 +643,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
 void demote_to_generic(NormPlan& p) {
     p.kind = NormKind::Generic;
     p.tile_rows = 0;
+    p.flat_t = 0;
     p.vec = 1;
     p.shift = 0;
     p.sstride = 1;
@@ -639,7 +658,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.shift ? "-shift" : ""), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.shift ? "-shift" : (p.flat_t ? "-flat" : "")), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     describe_dims(s, "rows_in", p.kept_in);

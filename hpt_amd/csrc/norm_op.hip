@@ -71,6 +71,16 @@ template <class T, int VEC> void launch_col_split(const NormPlan& p, const NormA
     t.bi = nk > 1 ? p.kept_in.stride[0] : 0;
     t.inv_cols = a.inv_cols;
     using Part = typename RowPartial<KIND, T>::type;
+    if constexpr (VEC > 1) {
+        if (p.flat_t > 0) {  // narrow inner dim: flat walk (statistics, the shared finalize, apply)
+            const unsigned block = (unsigned)((p.flat_t + 63) / 64 * 64);
+            col_flat_stats_kernel<KIND, T, VEC><<<dim3((unsigned)t.S, 1, batch), dim3(block),
+                                                  (size_t)p.flat_t * VEC * sizeof(Part), st>>>(t, p.flat_t);
+            transposed_finalize_kernel<KIND, T><<<dim3((unsigned)((t.R + 15) / 16), 1, batch), dim3(16, 16), 0, st>>>(t);
+            col_flat_apply_kernel<KIND, T, VEC><<<dim3((unsigned)t.S, 1, batch), dim3(block), 0, st>>>(t, p.flat_t, t.S);
+            return;
+        }
+    }
     const unsigned nw = (unsigned)p.tpr;
     const unsigned rg = (unsigned)((t.R + 64 * VEC - 1) / (64 * VEC));
     transposed_stats_kernel<KIND, T, VEC>

@@ -344,6 +344,146 @@ __global__ void __launch_bounds__(256) col_apply_kernel(const TransposedArgs a, 
     for (; c < c_end; c += 4) apply(load_pack<T, VEC>(in + (int64_t)c * a.sa), c);
 }
 
+// ---- the same, for a NARROW inner dim: the slab is walked as a flat array --------------------
+// softmax over axis 0 of a contiguous [cols, L] slab with L = 3, 8, 33, 100: lanes along the inner
+// dim would leave most of a wavefront idle. Thread t instead owns elements [t * VEC, t * VEC + VEC)
+// of every period of Lp = threads * VEC elements, Lp a multiple of L: each vector slot stays on ONE
+// inner index for the whole walk, all accesses are aligned 128-bit vectors, and the periods are
+// dealt round-robin over the S workgroups of a slab. Statistics: per-slot running (max, rescaled
+// sum), folded per inner index in LDS, one partial per workgroup in the layout of
+// transposed_stats_kernel (stats[b][y][L]) so that transposed_finalize_kernel serves both. Apply:
+// the same walk with the two per-index numbers of each slot in registers.
+template <int KIND, class T, int VEC>
+__global__ void __launch_bounds__(1024) col_flat_stats_kernel(const TransposedArgs a, int threads) {
+    static_assert(KIND != NORM_LAYERNORM, "a softmax pass");
+    using CT = typename Elem<T>::Wide;
+    using Part = SoftStat<CT>;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    Part* sm = (Part*)smem_raw;
+    const int t = threadIdx.x;
+    const int L = a.R;
+    const int Lp = threads * VEC;
+    const int p0 = t * VEC;
+    const int64_t total = (int64_t)a.cols * L;
+    CT m[VEC], s[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        m[k] = neg_inf<CT>();
+        s[k] = 0;
+    }
+    auto fold = [&](const Pack<T, VEC>* v, auto cnt_tag) {
+        constexpr int CNT = decltype(cnt_tag)::value;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            CT bm = neg_inf<CT>();
+#pragma unroll
+            for (int i = 0; i < CNT; ++i) bm = MaxC<CT>::comb(bm, Elem<T>::widen(v[i].v[k]));
+            if (bm > m[k]) {
+                s[k] = s[k] == (CT)0 ? (CT)0 : s[k] * exp_ct<T>(m[k] - bm);
+                m[k] = bm;
+            }
+            if (m[k] > neg_inf<CT>()) {
+#pragma unroll
+                for (int i = 0; i < CNT; ++i) s[k] += exp_ct<T>(Elem<T>::widen(v[i].v[k]) - m[k]);
+            }
+        }
+    };
+    if (t < threads) {
+        const T* base = (const T*)a.in + (int64_t)blockIdx.z * a.bi;
+        const int64_t whole = total / Lp;
+        const int S = a.S;
+        int64_t it = blockIdx.x;
+        for (; it + 3 * S < whole; it += 4 * S) {
+            Pack<T, VEC> v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = load_pack<T, VEC>(base + (it + u * S) * Lp + p0);
+            fold(v, std::integral_constant<int, 4>{});
+        }
+        for (; it < whole; it += S) {
+            Pack<T, VEC> v = load_pack<T, VEC>(base + it * Lp + p0);
+            fold(&v, std::integral_constant<int, 1>{});
+        }
+        if (it == whole) {  // the last, partial period: element by element
+            Pack<T, VEC> v;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                const int64_t pos = whole * Lp + p0 + k;
+                v.v[k] = pos < total ? base[pos] : Elem<T>::narrow(neg_inf<CT>());
+            }
+            fold(&v, std::integral_constant<int, 1>{});
+        }
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) sm[p0 + k] = Part{m[k], s[k]};
+    }
+    __syncthreads();
+    // slot p holds inner index p % L: fold the Lp / L slot rows pairwise, upper half into lower half
+    const int slot_rows = Lp / L;
+    int top = 1;
+    while (top < slot_rows) top <<= 1;
+    for (int h = top >> 1; h >= 1; h >>= 1) {
+        const int n = h * L;
+        for (int i = t; i < n; i += blockDim.x)
+            if (i + n < Lp) sm[i] = SoftStatOp<T, CT>::comb(sm[i], sm[i + n]);
+        __syncthreads();
+    }
+    Part* dst = (Part*)a.stats + ((int64_t)blockIdx.z * a.S + blockIdx.x) * L;
+    for (int c = t; c < L; c += blockDim.x) dst[c] = sm[c];
+}
+
+template <int KIND, class T, int VEC>
+__global__ void __launch_bounds__(1024) col_flat_apply_kernel(const TransposedArgs a, int threads, int slices) {
+    using CT = typename Elem<T>::Wide;
+    constexpr bool kLog = KIND == NORM_LOGSOFTMAX;
+    const int t = threadIdx.x;
+    if (t >= threads) return;
+    const int L = a.R;
+    const int Lp = threads * VEC;
+    const int p0 = t * VEC;
+    const int64_t total = (int64_t)a.cols * L;
+    const CT* pp = (const CT*)a.params + (int64_t)blockIdx.z * 3 * L;
+    CT pm[VEC], pk[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        const int c = (p0 + k) % L;
+        pm[k] = pp[c];
+        pk[k] = pp[L + c];
+    }
+    const T* in = (const T*)a.in + (int64_t)blockIdx.z * a.bi;
+    T* out = (T*)a.out + (int64_t)blockIdx.z * total;
+    auto apply1 = [&](T x, int k) -> T {
+        const CT d = Elem<T>::widen(x) - pm[k];
+        return Elem<T>::narrow(kLog ? d - pk[k] : exp_ct<T>(d) * pk[k]);
+    };
+    const int64_t whole = total / Lp;
+    int64_t it = blockIdx.x;
+    for (; it + 3 * slices < whole; it += 4 * slices) {
+        Pack<T, VEC> v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(in + (it + u * slices) * Lp + p0);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            Pack<T, VEC> o;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) o.v[k] = apply1(v[u].v[k], k);
+            store_pack_stream<T, VEC>(out + (it + u * slices) * Lp + p0, o);
+        }
+    }
+    for (; it < whole; it += slices) {
+        const Pack<T, VEC> v = load_pack_stream<T, VEC>(in + it * Lp + p0);
+        Pack<T, VEC> o;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) o.v[k] = apply1(v.v[k], k);
+        store_pack_stream<T, VEC>(out + it * Lp + p0, o);
+    }
+    if (it == whole) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            const int64_t pos = whole * Lp + p0 + k;
+            if (pos < total) out[pos] = apply1(in[pos], k);
+        }
+    }
+}
+
 // ---- single pass: the whole row block lives in registers -------------------------
 // When (16 * rgN bytes of consecutive rows) x (all columns) fits the register file of
 // one compute unit (16 vectors per thread, up to 1024 threads), a workgroup loads its

@@ -420,3 +420,57 @@ def test_short_rows_normalised_in_lds_tiles(hpt, orc, dev, case):
         assert np.array_equal(tof(ln).reshape(-1, n)[5], tof(b)), "constant row -> beta exactly"
         check(tf_.layernorm([n], None, None, 1e-5).numpy(), orc.layernorm(af, 1, None, None, 1e-5, acc=acc, dtype=odt),
               "layernorm without gamma / beta", 4e-6)
+
+
+FLAT_COLUMN_CASES = [
+    ("f32 [N, 3] axis 0", np.float32, [1000001, 3], 0),
+    ("f16 [N, 8] axis 0", np.float16, [600001, 8], 0),
+    ("f32 [N, 33] axis 0", np.float32, [70001, 33], 0),
+    ("bf16 [N, 100] axis 0", "bf16", [50001, 100], 0),
+    ("f16 [N, 257] axis 0", np.float16, [20001, 257], 0),
+    ("f32 [3, N, 5] axis 1", np.float32, [3, 500000, 5], 1),
+    ("f64 [N, 7] axis 0", np.float64, [200001, 7], 0),
+]
+
+
+@pytest.mark.parametrize("case", FLAT_COLUMN_CASES, ids=[c[0] for c in FLAT_COLUMN_CASES])
+def test_softmax_over_a_long_axis_with_a_narrow_inner_dim(hpt, orc, dev, case):
+    """softmax over axis 0 of [N, 3]: lanes along the inner dim would idle, so the slab is walked as a
+    flat array (statistics, finalize, apply). A column that is all -inf comes out NaN, a column with
+    one finite entry comes out exactly one-hot."""
+    name, npdt, shape, axis = case
+    rng = np.random.default_rng(211)
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    idx = [slice(None)] * len(shape)
+    idx[-1] = 1
+    x[tuple(idx)] = -np.inf                                   # inner index 1: nothing finite
+    idx[-1] = 2
+    x[tuple(idx)] = -np.inf
+    one = list(idx)
+    one[axis] = 12345
+    x[tuple(one)] = 0.5                                       # inner index 2: one finite entry
+    if npdt == "bf16":
+        cv, dt, odt, bits, tof, acc = hpt.f32_to_bf16_bits, hpt.bf16, orc.BF16, 8, hpt.bf16_bits_to_f32, orc.ACC_F32
+    elif npdt == np.float16:
+        cv, dt, odt, bits, tof, acc = (lambda v: v.astype(np.float16)), None, None, 11, (lambda v: v.astype(np.float32)), orc.ACC_F32
+    else:
+        cv, dt, odt, bits, tof, acc = (lambda v: v.astype(npdt)), None, None, 0, (lambda v: v), orc.ACC_F64
+    a = cv(x)
+    t = hpt.Tensor.from_numpy(a, dt).to_hip(dev)
+    assert hpt.normalize_plan(t, axis).startswith("col-split-flat"), hpt.normalize_plan(t, axis)
+    for log in (False, True):
+        got = tof((t.log_softmax(axis) if log else t.softmax(axis)).numpy())
+        want = tof(orc.softmax(a, axis, log=log, acc=acc, dtype=odt))
+        idx[-1] = 1
+        assert np.all(np.isnan(got[tuple(idx)])), f"{name}: a column without a finite entry is NaN"
+        if not log:
+            idx[-1] = 2
+            col = got[tuple(idx)]
+            assert np.count_nonzero(col) == col.size // shape[axis] and np.all(col[col != 0] == 1.0), f"{name}: one-hot"
+        keep = np.ones(shape[-1], bool)
+        keep[1] = False
+        g, w = got[..., keep], want[..., keep]
+        if bits:
+            assert_close(g, w, HALF_RTOL, max(half_atol(w[np.isfinite(w)], bits), 6e-8), f"{name} log={log}")
+        else:
+            assert_close(g, w, F32_RTOL, 2e-6 if log else F32_ATOL, f"{name} log={log}")
