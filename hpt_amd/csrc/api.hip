@@ -645,7 +645,7 @@ int32_t hpt_hip_softmax_causal(int32_t dev, void* stream, int32_t log, const hpt
         NormCall c = prepare_norm(in, out->data, in->ndim - 1, 0);
         if (c.plan.kind == NormKind::Empty) return;
         if (c.plan.kind == NormKind::Transposed || c.plan.kind == NormKind::TransposedTile ||
-            c.plan.kind == NormKind::ColSplit || c.plan.kind == NormKind::RowSplit)
+            c.plan.kind == NormKind::ColSplit || c.plan.kind == NormKind::RowSplit || c.plan.kind == NormKind::ColReg)
             demote_to_generic(c.plan);
         c.args.scale = scale;
         c.args.q_rows = in->shape[in->ndim - 2];

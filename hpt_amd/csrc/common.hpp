@@ -121,6 +121,7 @@ enum class NormKind {
     ColSplit,   // same layout, vectorisable inner dim: statistics over workgroups, finalize, apply in place
     Transposed, // input contiguous along the rows, output along the axis: statistics, then a register-tile transpose
     TransposedTile,  // same layout, a block of rows fits one compute unit's registers: one read, one write
+    ColReg,     // softmax over a SHORT strided axis (channels): each thread keeps the whole axis of its inner positions in registers
     Generic     // anything else: one block per row, per-element offset arithmetic
 };
 

@@ -597,6 +597,27 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             (nk == 1 || p.kept_in.size[0] <= 65535)) {
             const int64_t L = p.kept_in.size[nk - 1];
             const int64_t batch = nk > 1 ? p.kept_in.size[0] : 1;
+            // A SHORT axis (softmax over the channels of [B, 21, H, W]): a thread keeps the whole axis of
+            // its inner positions in registers, up to 64 registers of raw values: one read, one write.
+            // The widest vector that the axis length leaves room for and the layout allows is taken.
+            if (p.cols <= 1024 && p.rows >= 64 * 1024) {
+                // (two-byte types: vectors of at least 8 bytes, or the loads are too many and too small)
+                for (int ev = max_vec; ev >= (elem_size == 2 ? 4 : 1); ev /= 2) {
+                    const int64_t regs = std::max<int64_t>(1, ev * (int64_t)elem_size / 4);
+                    const int64_t nc_max = std::min<int64_t>(64, 64 / regs);
+                    const size_t vb = (size_t)ev * elem_size;
+                    // thread rows that share an inner position when the axis is longer than one thread holds
+                    const int64_t ty = pow2_ceil((p.cols + nc_max - 1) / nc_max);
+                    if (ty <= 16 && L % ev == 0 && sa % ev == 0 && (nk == 1 || p.kept_in.stride[0] % ev == 0) &&
+                        (p.cols * L) % ev == 0 && ((uintptr_t)in_data % vb) == 0 && ((uintptr_t)out_data % vb) == 0) {
+                        p.kind = NormKind::ColReg;
+                        p.vec = ev;
+                        p.nchunk = (int)nc_max;
+                        p.tpr = (int)ty;
+                        return p;
+                    }
+                }
+            }
             int v = max_vec;
             const bool vec_ok = v > 1 && L % v == 0 && sa % v == 0 && (nk == 1 || p.kept_in.stride[0] % v == 0) &&
                                 ((uintptr_t)in_data % 16) == 0 && ((uintptr_t)out_data % 16) == 0;
@@ -655,7 +676,7 @@ void demote_to_generic(NormPlan& p) {
 }
 
 std::string describe(const NormPlan& p) {
-    static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "generic"};
+    static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
              names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.shift ? "-shift" : (p.flat_t ? "-flat" : "")), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,

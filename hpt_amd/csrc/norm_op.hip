@@ -95,6 +95,27 @@ template <class T, int VEC> void launch_col_split(const NormPlan& p, const NormA
     col_apply_kernel<KIND, T, VEC><<<dim3(rg, (unsigned)chunks, batch), dim3(256), 0, st>>>(t, chunk);
 }
 
+// A short strided axis held in registers (softmax kinds).
+template <class T, int EV> void launch_col_reg(const NormPlan& p, const NormArgs& a, hipStream_t st) {
+    constexpr int REGS = (EV * (int)sizeof(T) + 3) / 4;
+    constexpr int NC = 64 / REGS > 64 ? 64 : 64 / REGS;
+    ColRegArgs c{};
+    const int nk = p.kept_in.n;
+    c.in = a.in;
+    c.out = a.out;
+    c.sa = a.sa;
+    c.bi = nk > 1 ? p.kept_in.stride[0] : 0;
+    c.L = p.kept_in.size[nk - 1];
+    c.nvec = c.L / EV;
+    c.total = (nk > 1 ? p.kept_in.size[0] : 1) * c.nvec;
+    c.cols = (int)p.cols;
+    c.ty_log2 = ilog2(p.tpr);  // thread rows per inner position
+    if (p.tpr > 16 || c.cols > NC * p.tpr)
+        fail(HPT_ERR_KERNEL, "col-reg: axis of %d does not fit %d thread rows of %d vectors", c.cols, p.tpr, NC);
+    const int64_t tx = 256 / p.tpr;
+    col_reg_kernel<KIND, T, EV, NC><<<dim3((unsigned)((c.total + tx - 1) / tx)), dim3(256), 0, st>>>(c);
+}
+
 // The transposed forms (kinds 0..2 only).
 template <class T> void launch_transposed(const NormPlan& p, const NormArgs& a, hipStream_t st) {
     constexpr int FULL = 16 / sizeof(T);
@@ -166,6 +187,20 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         } else {
             if (p.vec == FULL && FULL > 1) launch_row_split<T, FULL>(p, a, st);
             else launch_row_split<T, 1>(p, a, st);
+        }
+        return;
+    }
+    if (p.kind == NormKind::ColReg) {
+        if constexpr (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX) {
+            switch (p.vec) {
+                case 1: launch_col_reg<T, 1>(p, a, st); break;
+                case 2: if constexpr (FULL >= 2) launch_col_reg<T, 2>(p, a, st); break;
+                case 4: if constexpr (FULL >= 4) launch_col_reg<T, 4>(p, a, st); break;
+                case 8: if constexpr (FULL >= 8) launch_col_reg<T, 8>(p, a, st); break;
+                default: fail(HPT_ERR_KERNEL, "col-reg: unsupported vector width %d", p.vec);
+            }
+        } else {
+            fail(HPT_ERR_KERNEL, "col-reg is a softmax plan");
         }
         return;
     }

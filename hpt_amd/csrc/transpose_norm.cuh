@@ -344,6 +344,103 @@ __global__ void __launch_bounds__(256) col_apply_kernel(const TransposedArgs a, 
     for (; c < c_end; c += 4) apply(load_pack<T, VEC>(in + (int64_t)c * a.sa), c);
 }
 
+// ---- a SHORT strided axis: the whole axis in registers ---------------------------------------
+// softmax over the channels of [B, C, H, W] (segmentation logits, C = 21; feature maps, C = 128):
+// lanes run along the contiguous inner dim, EV elements each, and the threads that share an inner
+// position (one for C <= NC; 2, 4, 8 or 16 thread rows for longer axes, channels dealt round-robin)
+// load ALL C values of it: C strided vectors, every one of them in flight at once. Max, sum and
+// result come from registers (thread rows meet in LDS), and C vectors are stored: one HBM read and
+// one write. Only the raw values stay in registers (NC * EV * sizeof(T) <= 256 bytes per thread);
+// the exponentials are computed twice (for the sum, then for the result) rather than kept.
+struct ColRegArgs {
+    const void* in;
+    void* out;
+    int64_t sa;     // input stride along the axis
+    int64_t bi;     // input stride of the batch dim
+    int64_t nvec;   // vectors per batch slab along the inner dim: L / EV
+    int64_t total;  // batch * nvec
+    int64_t L;      // inner length
+    int cols;       // axis length (<= NC << ty_log2)
+    int ty_log2;    // log2 of the thread rows that share an inner position
+};
+
+template <int KIND, class T, int EV, int NC>
+__global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
+    static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX, "a softmax kernel");
+    using CT = typename Elem<T>::Wide;
+    constexpr bool kLog = KIND == NORM_LOGSOFTMAX;
+    __shared__ CT sm[256 * EV];
+    const int TY = 1 << a.ty_log2;
+    const int TX = 256 >> a.ty_log2;
+    const int tx = threadIdx.x & (TX - 1);
+    const int ty = threadIdx.x >> (8 - a.ty_log2);
+    const int64_t g = (int64_t)blockIdx.x * TX + tx;
+    const bool valid = g < a.total;
+    int64_t b = 0, q = 0;
+    if (valid) {
+        if (((uint64_t)(g | a.nvec) >> 32) == 0) {
+            b = (uint32_t)g / (uint32_t)a.nvec;
+            q = (uint32_t)g - (uint32_t)b * (uint32_t)a.nvec;
+        } else {
+            b = g / a.nvec;
+            q = g - b * a.nvec;
+        }
+    }
+    const T* in = (const T*)a.in + b * a.bi + q * EV;
+    T* out = (T*)a.out + b * a.cols * a.L + q * EV;
+    // this thread's channels: ty, ty + TY, ...
+    const int mine = valid ? (a.cols - ty + TY - 1) >> a.ty_log2 : 0;
+    Pack<T, EV> raw[NC];
+#pragma unroll
+    for (int i = 0; i < NC; ++i)
+        if (i < mine) raw[i] = load_pack_stream<T, EV>(in + (int64_t)(ty + (i << a.ty_log2)) * a.sa);
+    // all-reduce over the thread rows of an inner position
+    auto across = [&](CT(&v)[EV], auto op) {
+        if (TY == 1) return;
+#pragma unroll
+        for (int k = 0; k < EV; ++k) sm[(ty * TX + tx) * EV + k] = v[k];
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < EV; ++k) {
+            CT r = sm[tx * EV + k];
+            for (int y = 1; y < TY; ++y) r = op(r, sm[(y * TX + tx) * EV + k]);
+            v[k] = r;
+        }
+        __syncthreads();
+    };
+    CT m[EV], s[EV], kk[EV];
+#pragma unroll
+    for (int k = 0; k < EV; ++k) {
+        m[k] = neg_inf<CT>();
+        s[k] = 0;
+    }
+#pragma unroll
+    for (int i = 0; i < NC; ++i)
+        if (i < mine)
+#pragma unroll
+            for (int k = 0; k < EV; ++k) m[k] = MaxC<CT>::comb(m[k], Elem<T>::widen(raw[i].v[k]));
+    across(m, [](CT x, CT y) { return MaxC<CT>::comb(x, y); });
+#pragma unroll
+    for (int i = 0; i < NC; ++i)
+        if (i < mine)
+#pragma unroll
+            for (int k = 0; k < EV; ++k) s[k] += exp_ct<T>(Elem<T>::widen(raw[i].v[k]) - m[k]);
+    across(s, [](CT x, CT y) { return x + y; });
+#pragma unroll
+    for (int k = 0; k < EV; ++k) kk[k] = kLog ? log_ct<T>(s[k]) : (CT)1 / s[k];
+#pragma unroll
+    for (int i = 0; i < NC; ++i)
+        if (i < mine) {
+            Pack<T, EV> o;
+#pragma unroll
+            for (int k = 0; k < EV; ++k) {
+                const CT d = Elem<T>::widen(raw[i].v[k]) - m[k];
+                o.v[k] = Elem<T>::narrow(kLog ? d - kk[k] : exp_ct<T>(d) * kk[k]);
+            }
+            store_pack_stream<T, EV>(out + (int64_t)(ty + (i << a.ty_log2)) * a.L, o);
+        }
+}
+
 // ---- the same, for a NARROW inner dim: the slab is walked as a flat array --------------------
 // softmax over axis 0 of a contiguous [cols, L] slab with L = 3, 8, 33, 100: lanes along the inner
 // dim would leave most of a wavefront idle. Thread t instead owns elements [t * VEC, t * VEC + VEC)

@@ -474,3 +474,50 @@ def test_softmax_over_a_long_axis_with_a_narrow_inner_dim(hpt, orc, dev, case):
             assert_close(g, w, HALF_RTOL, max(half_atol(w[np.isfinite(w)], bits), 6e-8), f"{name} log={log}")
         else:
             assert_close(g, w, F32_RTOL, 2e-6 if log else F32_ATOL, f"{name} log={log}")
+
+
+CHANNEL_CASES = [
+    ("f32 [4, 21, 128, 128] axis 1", np.float32, [4, 21, 128, 128], 1),
+    ("f16 [2, 3, 40000] axis 1", np.float16, [2, 3, 40000], 1),
+    ("f32 [32, 70000] axis 0", np.float32, [32, 70000], 0),
+    ("bf16 [3, 64, 30000] axis 1", "bf16", [3, 64, 30000], 1),
+    ("f32 [2, 10, 33333] axis 1 (odd inner length)", np.float32, [2, 10, 33333], 1),
+    ("f64 [2, 30, 40000] axis 1", np.float64, [2, 30, 40000], 1),
+    ("f32 [60000, 16, 2] axis 1 (many batches)", np.float32, [60000, 16, 2], 1),
+    # longer axes: 2 ... 16 thread rows share an inner position and meet in LDS
+    ("f32 [24, 128, 56, 56] axis 1 (8 thread rows)", np.float32, [24, 128, 56, 56], 1),
+    ("f16 [2, 300, 40000] axis 1 (16 thread rows)", np.float16, [2, 300, 40000], 1),
+    ("f32 [600, 66001] axis 0 (single elements, 16 thread rows)", np.float32, [600, 66001], 0),
+    ("f64 [3, 100, 30000] axis 1", np.float64, [3, 100, 30000], 1),
+]
+
+
+@pytest.mark.parametrize("case", CHANNEL_CASES, ids=[c[0] for c in CHANNEL_CASES])
+def test_softmax_over_a_short_strided_axis_in_registers(hpt, orc, dev, case):
+    """softmax over the channels of [B, C, H, W], C <= 64: every thread keeps the whole axis of its
+    inner positions in registers (one read, one write)."""
+    name, npdt, shape, axis = case
+    rng = np.random.default_rng(212)
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    idx = [0] * len(shape)
+    idx[axis], idx[-1] = slice(None), 1
+    x[tuple(idx)] = -np.inf                      # one inner position without a finite entry
+    if npdt == "bf16":
+        cv, dt, odt, bits, tof, acc = hpt.f32_to_bf16_bits, hpt.bf16, orc.BF16, 8, hpt.bf16_bits_to_f32, orc.ACC_F32
+    elif npdt == np.float16:
+        cv, dt, odt, bits, tof, acc = (lambda v: v.astype(np.float16)), None, None, 11, (lambda v: v.astype(np.float32)), orc.ACC_F32
+    else:
+        cv, dt, odt, bits, tof, acc = (lambda v: v.astype(npdt)), None, None, 0, (lambda v: v), orc.ACC_F64
+    a = cv(x)
+    t = hpt.Tensor.from_numpy(a, dt).to_hip(dev)
+    assert hpt.normalize_plan(t, axis).startswith("col-reg"), hpt.normalize_plan(t, axis)
+    for log in (False, True):
+        got = tof((t.log_softmax(axis) if log else t.softmax(axis)).numpy())
+        want = tof(orc.softmax(a, axis, log=log, acc=acc, dtype=odt))
+        dead = np.isnan(want)
+        assert dead.any() and np.all(np.isnan(got[dead])), f"{name}: no finite entry -> NaN"
+        g, w = np.where(dead, 0, got), np.where(dead, 0, want)
+        if bits:
+            assert_close(g, w, HALF_RTOL, max(half_atol(w[np.isfinite(w)], bits), 6e-8), f"{name} log={log}")
+        else:
+            assert_close(g, w, F32_RTOL, 2e-6 if log else F32_ATOL, f"{name} log={log}")
