@@ -609,9 +609,7 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
         using ST = typename StatType<T>::type;
         SoftStat<CT, ST> st{neg_inf<CT>(), (ST)0};
         if (valid) {
-            for (int64_t iv = tx; iv < nv_lim; iv += tpr) {
-                CT x[VEC];
-                load(iv, x);
+            auto take = [&](int64_t iv, CT* x) {
                 if constexpr (SHIFT) {
 #pragma unroll
                     for (int j = 0; j < VEC; ++j)
@@ -630,12 +628,42 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
                     for (int j = 0; j < VEC; ++j) part += exp_ct<T>(x[j] - st.m);
                     st.s += (ST)part;
                 }
+            };
+            // four vectors in flight per thread (one per iteration left the memory pipeline mostly idle)
+            int64_t iv = tx;
+            for (; iv + 3 * tpr < nv_lim; iv += 4 * tpr) {
+                CT x[4][VEC];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) load(iv + u * tpr, x[u]);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) take(iv + u * tpr, x[u]);
+            }
+            for (; iv < nv_lim; iv += tpr) {
+                CT x[VEC];
+                load(iv, x);
+                take(iv, x);
             }
         }
         st = stat_all_reduce<SoftStatOp<T, CT, ST>>(st, tpr, (SoftStat<CT, ST>*)smem_raw);
         if (!valid) return;
         const CT k = kLog ? log_ct<T>((CT)st.s) : (CT)((ST)1 / st.s);
-        for (int64_t iv = tx; iv < nv; iv += tpr) {
+        auto finish = [&](int64_t iv, CT* x) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                CT d = x[j] - st.m;
+                x[j] = kLog ? d - k : exp_ct<T>(d) * k;
+            }
+            store(iv, x);
+        };
+        int64_t iv = tx;
+        for (; iv + 3 * tpr < nv_lim; iv += 4 * tpr) {
+            CT x[4][VEC];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) load(iv + u * tpr, x[u]);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) finish(iv + u * tpr, x[u]);
+        }
+        for (; iv < nv; iv += tpr) {
             CT x[VEC];
             if (iv < nv_lim) {
                 load(iv, x);
@@ -643,12 +671,7 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) x[j] = neg_inf<CT>();
             }
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) {
-                CT d = x[j] - st.m;
-                x[j] = kLog ? d - k : exp_ct<T>(d) * k;
-            }
-            store(iv, x);
+            finish(iv, x);
         }
     } else {
         using ST = typename StatType<T>::type;
@@ -660,9 +683,7 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
             CT k = 0, s1 = 0, s2 = 0;
             int64_t n = 0;
             bool first = true;
-            for (int64_t iv = tx; iv < nv; iv += tpr) {
-                CT x[VEC];
-                load(iv, x);
+            auto take = [&](int64_t iv, CT* x) {
                 if (first) {
                     k = x[0];  // the first element of the row this lane sees
                     if constexpr (SHIFT) {
@@ -682,6 +703,19 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
                     s2 += d * d;
                     n += in_row_j;
                 }
+            };
+            int64_t iv = tx;
+            for (; iv + 3 * tpr < nv; iv += 4 * tpr) {  // four vectors in flight per thread
+                CT x[4][VEC];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) load(iv + u * tpr, x[u]);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) take(iv + u * tpr, x[u]);
+            }
+            for (; iv < nv; iv += tpr) {
+                CT x[VEC];
+                load(iv, x);
+                take(iv, x);
             }
             if (n > 0) {
                 st.n = (ST)n;
@@ -695,9 +729,7 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
         const CT mean_hi = (CT)st.mean;
         const CT mean_lo = (CT)(st.mean - (ST)mean_hi);
         const CT rstd = rsqrt_ct((CT)(st.m2 * (ST)a.inv_cols) + (CT)a.eps);
-        for (int64_t iv = tx; iv < nv; iv += tpr) {
-            CT x[VEC];
-            load(iv, x);
+        auto finish = [&](int64_t iv, CT* x) {
             if constexpr (VEC > 1 && !SHIFT) {
                 // aligned rows: gamma / beta come as vectors too (the caller checked their alignment)
                 Pack<T, VEC> g, b;
@@ -738,6 +770,19 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
                 }
             }
             store(iv, x);
+        };
+        int64_t iv = tx;
+        for (; iv + 3 * tpr < nv; iv += 4 * tpr) {
+            CT x[4][VEC];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) load(iv + u * tpr, x[u]);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) finish(iv + u * tpr, x[u]);
+        }
+        for (; iv < nv; iv += tpr) {
+            CT x[VEC];
+            load(iv, x);
+            finish(iv, x);
         }
     }
 }
