@@ -74,6 +74,46 @@ def test_reduce_shape_and_out_dtype_match_the_oracle(hpt, orc):
             assert od.value == orc.reduce_out_dtype(op, d.code)
 
 
+def test_plans_for_shapes_off_the_benchmark_list(hpt):
+    """One plan per region of the shape space the planner distinguishes (no device needed: the views
+    only carry an address, shape and strides)."""
+    from hpt_amd.tensor import _contiguous_strides
+
+    def view(shape, dt=None):
+        return hpt.Tensor(None, 4096, list(shape), _contiguous_strides(list(shape)), dt or hpt.f32, "hip", 0)
+
+    red = [
+        # column reductions over a slab whose rows are not whole vectors: flat walk
+        ([1016800, 33], [0], "col-flat "), ([8190, 4097], [0], "col-flat-wide"),
+        # too little data for it: lanes along the inner dim
+        ([100, 33], [0], "col vec=1"),
+        # whole vectors, narrow: many thread rows and slices
+        ([4194304, 8], [0], "col vec=4 bx=2 by=256"),
+        # short rows back to back: LDS tiles; long rows: lanes along the row
+        ([1016800, 33], [1], "row-tile vec=4 tpr=8"), ([335544, 100], [1], "row-tile"),
+        ([65536, 512], [1], "row vec=4"), ([131584, 257], [1], "row-tile"),
+    ]
+    for shape, axes, want in red:
+        got = hpt.reduce_plan(view(shape), hpt.SUM, axes)
+        assert got.startswith(want), (shape, axes, got)
+    norm = [
+        # (shape, dtype, axis, n_norm_dims, plan prefix)
+        ([1016800, 33], None, 1, 0, "rowreg+tile"), ([1016800, 33], None, 0, 1, "rowreg+tile"),
+        ([262144, 128], None, 1, 0, "rowreg rows"),                 # whole vectors, 512 bytes: registers
+        ([8190, 4097], None, 1, 0, "rowreg-shift"), ([1043, 50257], None, 1, 0, "rowstream-shift"),
+        ([3355, 10000], None, 1, 0, "rowreg rows=3355 cols=10000 vec=4 tpr=1024"),
+        ([512, 65536], None, 1, 0, "rowstream"), ([32, 1048576], None, 1, 0, "rowsplit"),
+        ([32768, 1024], hpt.f16, 0, 1, "rowreg rows=32768 cols=1024 vec=8 tpr=64 rpb=4 nchunk=2"),
+        ([32768, 1024], hpt.f32, 0, 1, "rowreg rows=32768 cols=1024 vec=4 tpr=64 rpb=4 nchunk=4"),
+        # softmax over an axis that is not the last
+        ([8, 21, 512, 512], None, 1, 0, "col-reg"), ([64, 128, 56, 56], None, 1, 0, "col-reg"),
+        ([11184810, 3], None, 0, 0, "col-split-flat"), ([32768, 1024], None, 0, 0, "col-split rows"),
+    ]
+    for shape, dt, axis, nn, want in norm:
+        got = hpt.normalize_plan(view(shape, dt), axis, nn)
+        assert got.startswith(want), (shape, axis, nn, got)
+
+
 def test_plans_for_the_benchmark_configurations(hpt):
     """Which kernel family and launch shape each benchmark op gets (no device needed)."""
     f32 = lambda *s: hpt.Tensor.from_numpy(np.zeros(s, np.float32))
