@@ -160,26 +160,65 @@ __global__ void __launch_bounds__(1024) row_reduce_kernel(const RowArgs a) {
         const int64_t i0 = si * a.ichunk;
         const int64_t i1 = min(a.rin_v, i0 + a.ichunk);
         const int64_t ni = i1 - i0;
-        if (ni >= tpr || q1 - q0 <= 1) {
-            for (int64_t q = q0; q < q1; ++q) {
-                const T* p = base + offset_of(a.redo, q);
+        if (q1 - q0 <= 1) {
+            if (q0 < q1) {
+                const T* p = base + offset_of(a.redo, q0);
 #pragma unroll 4
                 for (int64_t iv = i0 + tx; iv < i1; iv += tpr) row_step<Op, VEC>(acc, p, iv, a.sr);
             }
         } else if (ni > 0) {
-            // short inner runs: spread the lanes over (outer, inner) pairs
+            // Several outer reduced indices, each with an inner run of ni vectors (the sums of a
+            // batch norm: [N, C, H*W] over N and H*W): the lanes walk the (outer, inner) pairs as ONE
+            // flat range, so a run that is not a multiple of the group size wastes no lanes, with
+            // four loads in flight per lane. The pair of a lane advances by a fixed (outer, inner)
+            // step: one division up front, none in the loop.
             const int64_t total = (q1 - q0) * ni;
-            for (int64_t t = tx; t < total; t += tpr) {
-                int64_t dq, di;
-                if (((uint64_t)total >> 32) == 0) {
-                    uint32_t d = (uint32_t)t / (uint32_t)ni;
-                    dq = d;
-                    di = (uint32_t)t - d * (uint32_t)ni;
-                } else {
-                    dq = t / ni;
-                    di = t - dq * ni;
+            int64_t dq, di;
+            if (((uint64_t)(tx | ni) >> 32) == 0) {
+                dq = (uint32_t)tx / (uint32_t)ni;
+                di = (uint32_t)tx - (uint32_t)dq * (uint32_t)ni;
+            } else {
+                dq = tx / ni;
+                di = tx - dq * ni;
+            }
+            const int64_t step_q = tpr / ni, step_i = tpr - step_q * ni;
+            auto advance = [&]() {
+                dq += step_q;
+                di += step_i;
+                if (di >= ni) {
+                    di -= ni;
+                    ++dq;
                 }
+            };
+            int64_t t = tx;
+            for (; t + 3 * (int64_t)tpr < total; t += 4 * (int64_t)tpr) {
+                const T* p[4];
+                int64_t iv[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    p[u] = base + offset_of(a.redo, q0 + dq);
+                    iv[u] = i0 + di;
+                    advance();
+                }
+                if constexpr (VEC > 1) {
+                    Pack<T, VEC> v[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(p[u] + iv[u] * VEC);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) fold_in<Op>(acc, v[u].v[j], iv[u] * VEC + j);
+                } else {
+                    T v[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) v[u] = p[u][iv[u] * a.sr];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) fold_in<Op>(acc, v[u], iv[u]);
+                }
+            }
+            for (; t < total; t += tpr) {
                 row_step<Op, VEC>(acc, base + offset_of(a.redo, q0 + dq), i0 + di, a.sr);
+                advance();
             }
         }
     }
