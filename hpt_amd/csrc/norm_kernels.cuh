@@ -655,23 +655,31 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
             }
             store(iv, x);
         };
-        int64_t iv = tx;
-        for (; iv + 3 * tpr < nv_lim; iv += 4 * tpr) {
-            CT x[4][VEC];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) load(iv + u * tpr, x[u]);
-#pragma unroll
-            for (int u = 0; u < 4; ++u) finish(iv + u * tpr, x[u]);
-        }
-        for (; iv < nv; iv += tpr) {
-            CT x[VEC];
+        // The second sweep runs BACKWARDS: the end of the row is what the first sweep read last and
+        // what the L2 still holds.
+        auto fetch = [&](int64_t iv, CT* x) {
             if (iv < nv_lim) {
                 load(iv, x);
             } else {
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) x[j] = neg_inf<CT>();
             }
-            finish(iv, x);
+        };
+        // (Shifted rows measured slower that way and keep the forward order.)
+        const int64_t cnt = tx < nv ? (nv - tx + tpr - 1) / tpr : 0;  // vectors of this thread
+        auto at = [&](int64_t i) { return tx + (SHIFT ? cnt - 1 - i : i) * tpr; };
+        int64_t left = cnt;
+        for (; left >= 4; left -= 4) {
+            CT x[4][VEC];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) fetch(at(left - 1 - u), x[u]);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) finish(at(left - 1 - u), x[u]);
+        }
+        for (; left > 0; --left) {
+            CT x[VEC];
+            fetch(at(left - 1), x);
+            finish(at(left - 1), x);
         }
     } else {
         using ST = typename StatType<T>::type;
@@ -771,18 +779,21 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
             }
             store(iv, x);
         };
-        int64_t iv = tx;
-        for (; iv + 3 * tpr < nv; iv += 4 * tpr) {
+        // backwards, as in the softmax branch: the row's end is the part the L2 still holds
+        const int64_t cnt = tx < nv ? (nv - tx + tpr - 1) / tpr : 0;
+        auto at = [&](int64_t i) { return tx + (SHIFT ? cnt - 1 - i : i) * tpr; };
+        int64_t left = cnt;
+        for (; left >= 4; left -= 4) {
             CT x[4][VEC];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) load(iv + u * tpr, x[u]);
+            for (int u = 0; u < 4; ++u) load(at(left - 1 - u), x[u]);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) finish(iv + u * tpr, x[u]);
+            for (int u = 0; u < 4; ++u) finish(at(left - 1 - u), x[u]);
         }
-        for (; iv < nv; iv += tpr) {
+        for (; left > 0; --left) {
             CT x[VEC];
-            load(iv, x);
-            finish(iv, x);
+            load(at(left - 1), x);
+            finish(at(left - 1), x);
         }
     }
 }
