@@ -521,3 +521,24 @@ def test_softmax_over_a_short_strided_axis_in_registers(hpt, orc, dev, case):
             assert_close(g, w, HALF_RTOL, max(half_atol(w[np.isfinite(w)], bits), 6e-8), f"{name} log={log}")
         else:
             assert_close(g, w, F32_RTOL, 2e-6 if log else F32_ATOL, f"{name} log={log}")
+
+
+def test_special_values_on_the_large_shape_kernels(hpt, orc, dev):
+    """+inf and NaN entries on the kernels only large shapes reach: a row / column with +inf or NaN
+    comes out NaN where the oracle says so, everything else matches."""
+    rng = np.random.default_rng(213)
+    for shape, axis, plan in (((60001, 33), 1, "rowreg+tile"), ((1100, 8200), 1, "rowreg rows"), ((500001, 5), 0, "col-split-flat"),
+                              ((4, 21, 128, 128), 1, "col-reg"), ((300, 70000), 1, "rowstream"), ((2100, 4097), 1, "rowreg-shift")):
+        x = (rng.standard_normal(shape) * 2).astype(np.float32)
+        flat = x.reshape(-1)
+        flat[rng.integers(0, flat.size, 40)] = np.inf
+        flat[rng.integers(0, flat.size, 40)] = np.nan
+        flat[rng.integers(0, flat.size, flat.size // 100)] = -np.inf
+        t = hpt.Tensor.from_numpy(x).to_hip(dev)
+        assert hpt.normalize_plan(t, axis).startswith(plan), hpt.normalize_plan(t, axis)
+        for log in (False, True):
+            got = (t.log_softmax(axis) if log else t.softmax(axis)).numpy()
+            with np.errstate(invalid="ignore", over="ignore"):
+                want = orc.softmax(x, axis, log=log, acc=orc.ACC_F64)
+            assert np.array_equal(np.isnan(got), np.isnan(want)), f"{shape} axis={axis} log={log}: NaN pattern"
+            assert_close(got, want, F32_RTOL, 2e-6, f"{shape} axis={axis} log={log}")

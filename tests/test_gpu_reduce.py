@@ -278,6 +278,44 @@ def test_short_rows_staged_through_lds(hpt, orc, dev):
     assert_close(out.numpy(), ax_.astype(np.float64).sum(1) + 2.0, F32_RTOL, F32_ATOL, "sum_ accumulate, short rows")
 
 
+def test_special_values_on_the_large_shape_kernels(hpt, orc, dev):
+    """NaN, +-inf on the kernels that only large shapes reach (LDS row tiles, the flat column walk, its
+    wide form, the flat (outer, inner) row walk): max / min skip NaN, a NaN never wins an arg
+    reduction (all-NaN -> index 0), nansum skips it, sum propagates it."""
+    rng = np.random.default_rng(118)
+    for shape, axes, plan in (((500001, 5), [1], "row-tile"), ((500001, 5), [0], "col-flat "), ((2051, 4097), [0], "col-flat-wide"),
+                              ((40, 24, 56, 56), [0, 2, 3], "row-general"), ((8192, 1024), [0], "col vec=4")):
+        x = rng.standard_normal(shape).astype(np.float32)
+        flat = x.reshape(-1)
+        flat[rng.integers(0, flat.size, flat.size // 50)] = np.nan
+        flat[rng.integers(0, flat.size, flat.size // 200)] = np.inf
+        flat[rng.integers(0, flat.size, flat.size // 200)] = -np.inf
+        if len(axes) == 1:       # one output with nothing but NaN
+            idx = [0] * len(shape)
+            idx[axes[0]] = slice(None)
+            x[tuple(idx)] = np.nan
+        t, a = upload(hpt, x, dev=dev)
+        assert hpt.reduce_plan(t, hpt.SUM, axes).startswith(plan), hpt.reduce_plan(t, hpt.SUM, axes)
+        tag = f"{shape} {axes}"
+        assert np.array_equal(t.max(axes).numpy(), orc.reduce(orc.MAX, a, axes)), tag
+        assert np.array_equal(t.min(axes).numpy(), orc.reduce(orc.MIN, a, axes)), tag
+        with np.errstate(invalid="ignore"):
+            want = orc.reduce(orc.SUM, a, axes, acc=orc.ACC_F64)
+            got = t.sum(axes).numpy()
+            assert np.array_equal(np.isnan(got), np.isnan(want)), tag
+            fin = np.isfinite(want)
+            assert np.array_equal(got[~fin & ~np.isnan(want)], want[~fin & ~np.isnan(want)]), tag
+            assert_close(got[fin], want[fin], F32_RTOL, 1e-5, "sum " + tag)
+            wn = orc.reduce(orc.NANSUM, a, axes, acc=orc.ACC_F64)
+            gn = t.nansum(axes).numpy()
+            assert np.array_equal(np.isnan(gn), np.isnan(wn)) and np.array_equal(np.isinf(gn), np.isinf(wn)), tag
+            ok = np.isfinite(wn)
+            assert_close(gn[ok], wn[ok], F32_RTOL, 1e-5, "nansum " + tag)
+        if len(axes) == 1:
+            assert np.array_equal(t.argmax(axes[0]).numpy(), orc.argreduce(True, a, axes[0])), tag
+            assert np.array_equal(t.argmin(axes[0]).numpy(), orc.argreduce(False, a, axes[0])), tag
+
+
 def test_sum_inplace_out_and_accumulate(hpt, orc, dev):
     """sum_ with init_out: true overwrites, false adds to what `out` holds (reduce.rs:84-92)."""
     rng = np.random.default_rng(107)
