@@ -636,8 +636,28 @@ __global__ void __launch_bounds__(1024) col_reduce_kernel(const ColArgs a) {
         const T* base = (const T*)a.in + offset_of(a.kept_outer, outer) + inner * a.sk;
         const int64_t r0 = (int64_t)blockIdx.y * a.chunk;
         const int64_t r1 = min(a.R, r0 + a.chunk);
-#pragma unroll 2
-        for (int64_t r = r0 + ty; r < r1; r += by) {
+        int64_t r = r0 + ty;
+        for (; r + 7 * by < r1; r += 8 * by) {  // eight reduced positions in flight per lane
+            const T* p[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) p[u] = base + offset_of(a.red, r + u * by);
+            if constexpr (VEC > 1) {
+                Pack<T, VEC> v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = load_pack_stream<T, VEC>(p[u]);
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v[u].v[j], r + u * by);
+            } else {
+                T v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = *p[u];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) fold_in<Op>(acc[0], v[u], r + u * by);
+            }
+        }
+        for (; r < r1; r += by) {
             const T* p = base + offset_of(a.red, r);
             if constexpr (VEC > 1) {
                 Pack<T, VEC> v = load_pack_stream<T, VEC>(p);
