@@ -306,6 +306,51 @@ def cases_c6(P):
     return cases
 
 
+def cases_c8(P):
+    """Shapes off the reference's list that the planner treats separately (~128 MiB each): short rows,
+    narrow and odd inner dims, long rows, channel softmax, batch-norm statistics."""
+    import hpt_amd as hpt
+    rng = np.random.default_rng(8)
+    cases = []
+
+    def up(shape, n=3):
+        base = rng.standard_normal(shape, dtype=np.float32)
+        return [hpt.Tensor.from_numpy(np.roll(base, k, 0)).to_hip(0) for k in range(n)], base.nbytes
+
+    def red(ts, nb, cfg, op, axes, label, rows):
+        run, outs = P.reduce(ts, op, axes)
+        P.keep.append(outs)
+        cases.append(Case(label, cfg, "f32", rows, nb, run, len(ts)))
+
+    def nrm(ts, nb, cfg, kind, axis, label, rows):
+        run, outs = P.norm(ts, kind, axis=axis)
+        P.keep.append(outs)
+        cases.append(Case(label, cfg, "f32", rows, 2 * nb, run, len(ts)))
+
+    ts, nb = up([1016800, 33])
+    red(ts, nb, "f32 [1016800,33] (short odd rows)", "sum", [1], "sum(axis=1)", 1016800)
+    red(ts, nb, "f32 [1016800,33]", "sum", [0], "sum(axis=0)", 33)
+    nrm(ts, nb, "f32 [1016800,33]", "softmax", 1, "softmax(axis=1)", 1016800)
+    del ts
+    ts, nb = up([8190, 4097])
+    nrm(ts, nb, "f32 [8190,4097] (odd row length)", "softmax", 1, "softmax(axis=1)", 8190)
+    red(ts, nb, "f32 [8190,4097]", "sum", [0], "sum(axis=0)", 4097)
+    del ts
+    ts, nb = up([2048, 16384])
+    nrm(ts, nb, "f32 [2048,16384] (rows of 1024 threads)", "log_softmax", 1, "log_softmax(axis=1)", 2048)
+    del ts
+    ts, nb = up([8, 21, 512, 512])
+    nrm(ts, nb, "f32 [8,21,512,512] (softmax over channels)", "softmax", 1, "softmax(axis=1)", 8 * 512 * 512)
+    del ts
+    ts, nb = up([64, 128, 56, 56])
+    red(ts, nb, "C3 f32 [64,128,56,56] (batch-norm statistics)", "sum", [0, 2, 3], "sum([0,2,3])", 128)
+    nrm(ts, nb, "C3 f32 [64,128,56,56] (softmax over channels)", "softmax", 1, "softmax(axis=1)", 64 * 56 * 56)
+    del ts
+    ts, nb = up([11184810, 3])
+    nrm(ts, nb, "f32 [11184810,3]", "softmax", 0, "softmax(axis=0)", 3)
+    return cases
+
+
 def build_cases(which: str, configs=None):
     """Synthetic inputs of the benchmark configurations, uploaded once; outputs preallocated.
     The headline (C2 layernorm) is always first; `configs` limits the others (e.g. {"c3"})."""
@@ -313,7 +358,7 @@ def build_cases(which: str, configs=None):
     cases, head = cases_c2(P, which == "headline")
     if which != "headline":
         for name, fn in (("c1", cases_c1), ("c3", cases_c3), ("c4", cases_c4), ("c5", cases_c5), ("c6", cases_c6),
-                         ("c7", cases_c7)):
+                         ("c7", cases_c7), ("c8", cases_c8)):
             if configs is None or name in configs:
                 cases += fn(P)
     return cases, P, head
@@ -358,7 +403,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--ops", choices=["all", "headline"], default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--configs", default="", help="comma list of c1,c3,c4,c5,c6 to measure besides the headline (c6 = the steps either side: contiguous / in-place affine / full)")
+    ap.add_argument("--configs", default="", help="comma list of c1,c3,c4,c5,c6,c7,c8 to measure besides the headline (c6 = the steps either side: contiguous / in-place affine / full; c7 = the fused forms; c8 = shapes off the reference's list)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region, run one plain device-to-device copy of the headline input "
                          "(134217728 bytes read + as many written): the known-size dispatch that hardware "
