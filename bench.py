@@ -384,7 +384,7 @@ def cpu_baseline(x, g, b, gpu_out, budget_s=15.0):
         port_err = float(np.abs(out[rows].astype(np.float64) - truth).max())
     times = []
     t_end = time.perf_counter() + budget_s
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 400):
         t0 = time.perf_counter()
         orc.mt_layernorm_f32(x, g, b, 1e-5, cores, out)
         times.append(time.perf_counter() - t0)
