@@ -208,6 +208,15 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
         // ---- Col: lanes walk the outputs -----------------------------------
         p.kind = ReduceKind::Col;
         const int nk = p.kept.n;
+        // Two kept dims of which the FIRST is the contiguous one (a reduction over the last axis of a
+        // permuted view): the lanes must run along that one. List it last; the kernel then scatters
+        // its (few) outputs instead of gathering its (many) inputs.
+        if (nk == 2 && p.red.n <= 1 && iabs(p.kept.stride[0]) < iabs(p.kept.stride[1]) && p.kept.size[1] <= 65535 &&
+            p.kept.size[0] <= kI32 && p.R <= kI32 && iabs(p.kept.stride[0]) <= kI32) {
+            std::swap(p.kept.size[0], p.kept.size[1]);
+            std::swap(p.kept.stride[0], p.kept.stride[1]);
+            p.kept_swapped = true;
+        }
         int64_t kin = nk ? p.kept.size[nk - 1] : 1;
         p.vec = 1;
         if (nk && p.kept.stride[nk - 1] == 1)
@@ -215,6 +224,14 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
         const int64_t outer = nk > 1 ? p.kept.size[0] : 1;
         p.lean = p.red.n <= 1 && nk <= 2 && outer <= 65535 && kin <= kI32 && p.R <= kI32 &&
                  (nk == 0 || iabs(p.kept.stride[nk - 1]) <= kI32);
+        if (p.kept_swapped && !p.lean) {  // the general kernel numbers its outputs in kept order: undo
+            std::swap(p.kept.size[0], p.kept.size[1]);
+            std::swap(p.kept.stride[0], p.kept.stride[1]);
+            p.kept_swapped = false;
+            kin = p.kept.size[nk - 1];
+            p.vec = 1;
+            if (p.kept.stride[nk - 1] == 1) p.vec = legal_vec(data, elem_size, kin, p.kept, p.red, 1, 0);
+        }
         if (p.lean && nk && p.kept.stride[nk - 1] == 2 && elem_size <= 8 &&
             legal_vec(data, elem_size, kin * 2, p.kept, p.red, 1, 0) > 1) {
             // neighbouring outputs sit at every second position: full vectors, even positions kept
@@ -222,7 +239,7 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
             p.sstride = 2;
         }
         const int full = (int)(16 / elem_size);
-        if (p.lean && nk && p.vec == 1 && p.sstride == 1 && full > 1 && p.kept.stride[nk - 1] == 1 &&
+        if (p.lean && nk && !p.kept_swapped && p.vec == 1 && p.sstride == 1 && full > 1 && p.kept.stride[nk - 1] == 1 &&
             p.red.n == 1 && p.red.stride[0] == kin && (uintptr_t)data % 16 == 0 &&
             (outer == 1 || p.kept.stride[0] % full == 0) && kin * p.R * (int64_t)elem_size >= (8ll << 20)) {
             // A contiguous [R, kin] slab whose rows are not whole vectors (kin = 3, 33, 257): walk it
@@ -341,7 +358,7 @@ std::string describe(const ReducePlan& p) {
             break;
         case ReduceKind::Col:
             snprintf(buf, sizeof buf, "col%s%s vec=%d bx=%d by=%d outs=%lld red=%lld split=%d ",
-                     p.flat_xb ? "-flat-wide" : p.flat_t ? "-flat" : p.lean ? "" : "-general",
+                     p.flat_xb ? "-flat-wide" : p.flat_t ? "-flat" : p.kept_swapped ? "-swapped" : p.lean ? "" : "-general",
                      p.sstride == 2 ? "-step2" : "", p.vec,
                      p.flat_t ? p.flat_t : p.bx, p.by,
                      (long long)p.K, (long long)p.R, p.split);

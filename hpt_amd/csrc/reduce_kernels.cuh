@@ -346,6 +346,7 @@ struct ColLeanArgs {
     int sk;          // inner kept stride in elements (1 when VEC > 1)
     int R;           // reduced length
     int split, init_out;
+    int64_t oso, osi;  // output strides of the outer / inner kept index (kin and 1 unless the kept dims were swapped)
 };
 
 template <class Op, int VEC, int SS = 1>
@@ -400,7 +401,8 @@ __global__ void __launch_bounds__(1024) col_lean_kernel(const ColLeanArgs a) {
         const int64_t o0 = ((int64_t)outer * a.kin_v + cv) * UV;
         if (a.split == 1) {
 #pragma unroll
-            for (int j = 0; j < UV; ++j) write_out<Op>(a.out, o0 + j, acc[j], a.init_out, a.count);
+            for (int j = 0; j < UV; ++j)
+                write_out<Op>(a.out, (int64_t)outer * a.oso + ((int64_t)cv * UV + j) * a.osi, acc[j], a.init_out, a.count);
         } else {
 #pragma unroll
             for (int j = 0; j < UV; ++j) ((Acc*)a.out)[(int64_t)blockIdx.z * a.K + o0 + j] = acc[j];
@@ -702,7 +704,8 @@ __global__ void __launch_bounds__(256) finish_rows_kernel(const void* part_, voi
 // loads, then folded through LDS.
 template <class Op>
 __global__ void __launch_bounds__(1024) finish_cols_kernel(const void* part_, void* out, int64_t K, int split,
-                                                           int init_out, double count) {
+                                                           int init_out, double count, int64_t kin, int64_t oso,
+                                                           int64_t osi) {
     using Acc = typename Op::Acc;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     Acc* sm = (Acc*)smem_raw;
@@ -730,7 +733,8 @@ __global__ void __launch_bounds__(1024) finish_cols_kernel(const void* part_, vo
         if (ty == 0)
             for (int y = 1; y < by; ++y) acc = Op::comb(acc, sm[y * 64 + tx]);
     }
-    if (ty == 0 && valid) write_out<Op>(out, o, acc, init_out, count);
+    // output o of the kernel's (outer, inner) numbering sits at outer * oso + inner * osi
+    if (ty == 0 && valid) write_out<Op>(out, (o / kin) * oso + (o % kin) * osi, acc, init_out, count);
 }
 
 // Fill `n` outputs with the op's identity (a reduced dim of size 0).
@@ -885,6 +889,8 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.split = p.split;
             a.init_out = init_out;
             const int64_t outer = nk > 1 ? p.kept.size[0] : 1;
+            a.oso = p.kept_swapped ? 1 : kin;
+            a.osi = p.kept_swapped ? outer : 1;
             dim3 grid((unsigned)((a.kin_v + p.bx - 1) / p.bx), (unsigned)outer, (unsigned)p.split);
             if (vec && p.sstride == 2) col_lean_kernel<Op, FULL, 2><<<grid, block, smem, st>>>(a);
             else if (vec) col_lean_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
@@ -912,9 +918,12 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
     if (p.split > 1) {
         int fy = 1;  // thread rows sharing an output's partials: about two partials per thread
         while (fy < 16 && fy * 2 < p.split) fy <<= 1;
+        // (swapped kept dims: the partials are in the kernel's numbering, the outputs in the caller's)
+        const int64_t kin = p.kept_swapped ? p.kept.size[1] : p.K;
+        const int64_t oso = p.kept_swapped ? 1 : 0, osi = p.kept_swapped ? p.kept.size[0] : 1;
         finish_cols_kernel<Op><<<dim3((unsigned)((p.K + 63) / 64)), dim3(64, (unsigned)fy),
                                  fy > 1 ? (size_t)fy * 64 * sizeof(Acc) : 0, st>>>(sc.partial, out, p.K, p.split,
-                                                                                    init_out, count);
+                                                                                    init_out, count, kin, oso, osi);
     }
 }
 

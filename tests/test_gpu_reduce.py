@@ -316,6 +316,30 @@ def test_special_values_on_the_large_shape_kernels(hpt, orc, dev):
             assert np.array_equal(t.argmin(axes[0]).numpy(), orc.argreduce(False, a, axes[0])), tag
 
 
+def test_reduction_over_the_last_axis_of_a_permuted_view(hpt, orc, dev):
+    """x.permute(2, 1, 0).sum(2): the first kept dim is the contiguous one. The lanes run along it and
+    the outputs are scattered (one launch, and the two-stage form with its second-stage remap)."""
+    rng = np.random.default_rng(119)
+    for shape, npdt in (((96, 40, 72), np.float32), ((2000, 70, 36), np.float32), ((3000, 9, 64), np.int32), ((700, 33, 24), np.float16)):
+        base = (rng.standard_normal(shape) * 3).astype(npdt) if np.issubdtype(npdt, np.floating) else rng.integers(-9, 9, shape).astype(npdt)
+        t, a = upload(hpt, base, (("permute", (2, 1, 0)),), dev=dev)
+        assert hpt.reduce_plan(t, hpt.SUM, [2]).startswith("col-swapped"), hpt.reduce_plan(t, hpt.SUM, [2])
+        tag = f"{np.dtype(npdt).name} {shape}"
+        assert np.array_equal(t.argmax(2).numpy(), orc.argreduce(True, a, 2)), tag
+        assert np.array_equal(t.max([2]).numpy(), a.max(2)), tag
+        if npdt == np.float16:
+            want = orc.reduce(orc.SUM, a, [2], acc=orc.ACC_F32).astype(np.float32)
+            assert_close(t.sum([2]).numpy().astype(np.float32), want, HALF_RTOL, half_atol(want, 11), tag)
+        elif npdt == np.float32:
+            want = orc.reduce(orc.SUM, a, [2], acc=orc.ACC_F64)
+            assert_close(t.sum([2], True).numpy(), want.reshape(want.shape + (1,)), F32_RTOL, F32_ATOL, tag)
+            out = hpt.Tensor.full(1.0, list(want.shape), hpt.f32, dev)
+            t.sum_([2], False, False, out)
+            assert_close(out.numpy(), want + 1.0, F32_RTOL, F32_ATOL, "accumulate " + tag)
+        else:
+            assert np.array_equal(t.sum([2]).numpy(), orc.reduce(orc.SUM, a, [2])), tag
+
+
 def test_sum_inplace_out_and_accumulate(hpt, orc, dev):
     """sum_ with init_out: true overwrites, false adds to what `out` holds (reduce.rs:84-92)."""
     rng = np.random.default_rng(107)
