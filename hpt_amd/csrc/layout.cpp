@@ -560,7 +560,14 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             // longer rows (two sweeps; gamma / beta as vectors).
             // Two-byte types hold eight elements per vector: with gamma and beta beside the row, sixteen
             // elements per thread is what fits 128 registers, i.e. two vectors (four of a stride-2 row).
-            const bool ln_half = n_norm_dims > 0 && v > 1 && elem_size == 2;
+            bool ln_half = n_norm_dims > 0 && v > 1 && elem_size == 2;
+            // Long two-byte layernorm rows (4096 < cols <= 16384): gamma / beta go to LDS (at most 64 KiB)
+            // and the row takes four vectors per thread like any other. Measured, f16 (TB/s): [6553, 5120]
+            // 3.5 -> 4.6, [4096, 8192] 4.7 -> 5.0, [2730, 12288] 3.2 -> 4.6, [2048, 16384] 3.8 -> 4.6.
+            if (ln_half && p.sstride == 1 && !p.shift && nv * v > 4096 && nv * v <= 16384) {
+                p.gb_lds = 1;
+                ln_half = false;
+            }
             const int64_t per = ln_half ? 2 * p.sstride : 4;
             const int64_t reg_limit = ln_half ? 1024 * per : (n_norm_dims > 0 && v > 1) ? 4096 : 8192;
             if (nv <= reg_limit) {
@@ -680,6 +687,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
 
 void demote_to_generic(NormPlan& p) {
     p.kind = NormKind::Generic;
+    p.gb_lds = 0;
     p.tile_rows = 0;
     p.flat_t = 0;
     p.vec = 1;
@@ -696,7 +704,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.shift ? "-shift" : (p.flat_t ? "-flat" : "")), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.shift ? "-shift" : (p.flat_t ? "-flat" : (p.gb_lds ? "-ldsgb" : ""))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     describe_dims(s, "rows_in", p.kept_in);

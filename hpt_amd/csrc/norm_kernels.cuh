@@ -105,8 +105,12 @@ __device__ __forceinline__ A row_all_reduce(A v, int tpr, int ty, A* smem) {
 // launch makes the row step of the walk a multiple of VEC.
 // PF: always issue the next row's loads before the current row's statistics (see kPrefetch below);
 // the launch then caps the grid so that workgroups do walk rows.
-template <int KIND, class T, int VEC, int NCHUNK, int SS = 1, bool SHIFT = false, bool PF = false>
+// GBL (layernorm of 2-byte types, long rows): gamma / beta live in LDS instead of registers (loaded
+// once per workgroup, read per row), which leaves room for four vectors of the row per thread where
+// the register form holds two: half as many threads per row, twice as many rows in flight.
+template <int KIND, class T, int VEC, int NCHUNK, int SS = 1, bool SHIFT = false, bool PF = false, bool GBL = false>
 __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
+    static_assert(!GBL || (norm_is_layer(KIND) && VEC > 1 && SS == 1 && !SHIFT), "GBL is an aligned layernorm form");
     static_assert(!SHIFT || (VEC > 1 && SS == 1), "SHIFT is a full-vector mode");
     constexpr int UV = VEC / SS;  // useful elements per vector
     using CT = typename Elem<T>::Wide;
@@ -127,9 +131,27 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     constexpr bool kRes = KIND == NORM_ADD_LAYERNORM;
     const CT fill = kSoft ? neg_inf<CT>() : (CT)0;
 
-    // this thread's columns never change: keep gamma / beta in registers
-    Pack<T, UV> gam[NCHUNK], bet[NCHUNK];
-    if constexpr (!kSoft) {
+    // this thread's columns never change: keep gamma / beta in registers (or, GBL, in LDS)
+    extern __shared__ __align__(16) unsigned char gb_raw[];
+    T* lds_gamma = reinterpret_cast<T*>(gb_raw);
+    T* lds_beta = lds_gamma + (GBL ? (size_t)nv * UV : 0);
+    if constexpr (GBL) {
+        for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+            Pack<T, UV> g, b;
+#pragma unroll
+            for (int j = 0; j < UV; ++j) {
+                g.v[j] = Elem<T>::narrow((CT)1);
+                b.v[j] = Elem<T>::narrow((CT)0);
+            }
+            if (a.gamma) g = load_pack<T, UV>((const T*)a.gamma + (int64_t)i * UV);
+            if (a.beta) b = load_pack<T, UV>((const T*)a.beta + (int64_t)i * UV);
+            store_pack<T, UV>(lds_gamma + (size_t)i * UV, g);
+            store_pack<T, UV>(lds_beta + (size_t)i * UV, b);
+        }
+        __syncthreads();
+    }
+    Pack<T, UV> gam[GBL ? 1 : NCHUNK], bet[GBL ? 1 : NCHUNK];
+    if constexpr (!kSoft && !GBL) {
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int iv = c * tpr + tx;
@@ -173,7 +195,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     // Rows that take 512 or 1024 threads leave room for one or two workgroups per compute unit, so
     // nothing else hides a row's load -> reduce -> reduce -> store chain: there (PF) the prefetch
     // pays for every type (f32 [3355, 10000] softmax: 3.2 TB/s without).
-    constexpr bool kPrefetch = ((sizeof(T) == 2 && NCHUNK * UV <= (kSoft ? 32 : 16)) || PF) && !kRes;
+    constexpr bool kPrefetch = ((sizeof(T) == 2 && NCHUNK * UV <= ((kSoft || GBL) ? 32 : 16)) || PF) && !kRes;
     const int64_t row_step = (int64_t)gridDim.x * a.rpb;
     Pack<T, VEC> raw[NCHUNK];
     Pack<T, UV> raw_res[kRes ? NCHUNK : 1];
@@ -304,11 +326,25 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
             }
             const ST var = row_all_reduce<SumC<ST>>((ST)q, tpr, ty, ssmem) * (ST)a.inv_cols;
             const CT rstd = rsqrt_ct((CT)var + (CT)a.eps);
+            if constexpr (GBL) {
 #pragma unroll
-            for (int c = 0; c < NCHUNK; ++c)
+                for (int c = 0; c < NCHUNK; ++c) {
+                    const int iv = c * tpr + tx;
+                    if (iv < nv) {
+                        const Pack<T, UV> g = load_pack<T, UV>(lds_gamma + (size_t)iv * UV);
+                        const Pack<T, UV> b = load_pack<T, UV>(lds_beta + (size_t)iv * UV);
 #pragma unroll
-                for (int j = 0; j < UV; ++j)
-                    x[c][j] = x[c][j] * rstd * Elem<T>::widen(gam[c].v[j]) + Elem<T>::widen(bet[c].v[j]);
+                        for (int j = 0; j < UV; ++j)
+                            x[c][j] = x[c][j] * rstd * Elem<T>::widen(g.v[j]) + Elem<T>::widen(b.v[j]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+                    for (int j = 0; j < UV; ++j)
+                        x[c][j] = x[c][j] * rstd * Elem<T>::widen(gam[c].v[j]) + Elem<T>::widen(bet[c].v[j]);
+            }
         }
 
         if (valid) {

@@ -246,6 +246,18 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
                 return;
             }
         }
+        if constexpr (FULL > 1 && sizeof(T) == 2 && norm_is_layer(KIND)) {
+            if (p.gb_lds && p.vec == FULL && p.sstride == 1 && !p.shift && p.nchunk == 4) {
+                const size_t smem = 2 * (size_t)p.cols * sizeof(T);
+                if (p.tpr >= 512 && KIND != NORM_ADD_LAYERNORM) {
+                    if (grid.x > 512u) grid.x = 512u;
+                    row_reg_kernel<KIND, T, FULL, 4, 1, false, true, true><<<grid, block, smem, st>>>(a);
+                } else {
+                    row_reg_kernel<KIND, T, FULL, 4, 1, false, false, true><<<grid, block, smem, st>>>(a);
+                }
+                return;
+            }
+        }
         if constexpr (FULL > 1 && KIND != NORM_ADD_LAYERNORM) {
             // Long rows: 512 large workgroups that walk the rows and prefetch the next one. Measured
             // (TB/s, without -> with): f32 [3355, 10000] layernorm 3.6 -> 5.1, softmax 3.2 -> 4.2;

@@ -97,6 +97,8 @@ ADD_LN_CASES = [
     ("rows in registers", [37, 1024], (), 1),
     ("two normalised dims", [6, 8, 96], (), 2),
     ("long rows: streaming", [3, 40000], (), 1),
+    ("rows of 8192 (two-byte types keep gamma / beta in LDS)", [1300, 8192], (), 1),
+    ("rows of 12288, more rows than workgroups", [1100, 12288], (), 1),
     ("sliced input", [20, 300], (("slice", ((2, 19, 1), (4, 260, 1))),), 1),
     ("step-2 input", [16, 512], (("slice", ((0, 16, 1), (0, 512, 2))),), 1),
     ("transposed input: demoted to the generic rows", [256, 4096], (("permute", (1, 0)),), 1),
