@@ -194,8 +194,7 @@ __global__ void __launch_bounds__(256) transposed_finalize_kernel(const Transpos
     else { acc0 = (ST)neg_inf<CT>(); acc1 = 0; }
     if (ok) {
         const Part* sp = (const Part*)a.stats + (int64_t)blockIdx.z * P * a.R + r;
-        for (int p = threadIdx.y; p < P; p += LY) {
-            const Part t = sp[(int64_t)p * a.R];
+        auto take = [&](const Part& t) {
             if constexpr (KIND == NORM_LAYERNORM) {
                 acc0 += (ST)t.s1;
                 acc1 += (ST)t.s2;
@@ -205,7 +204,16 @@ __global__ void __launch_bounds__(256) transposed_finalize_kernel(const Transpos
                 acc0 = x.m;
                 acc1 = x.s;
             }
+        };
+        int p = threadIdx.y;
+        for (; p + 3 * LY < P; p += 4 * LY) {  // four partials in flight (the kernel is a chain of load latencies)
+            Part t[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) t[u] = sp[(int64_t)(p + u * LY) * a.R];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) take(t[u]);
         }
+        for (; p < P; p += LY) take(sp[(int64_t)p * a.R]);
     }
     sm0[threadIdx.y][threadIdx.x] = acc0;
     sm1[threadIdx.y][threadIdx.x] = acc1;
