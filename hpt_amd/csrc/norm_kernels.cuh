@@ -39,27 +39,11 @@ template <class CT> struct SumC {
 };
 
 // exp / log in the compute type. Half tensors, whose results are rounded to 8 or 11 significant
-// bits anyway, use the hardware exp2 / log2 on the scaled argument. f32 tensors (tolerance 1e-5
-// against the CPU path) need more: the error of exp2(x * log2 e) grows with |x| (the product is
-// rounded before the exponential sees it). exp_reduced splits x = n ln 2 + r exactly first
-// (Cody-Waite, two fused multiply-adds), hands the hardware exp2 an argument of at most 1/2 in
-// magnitude and scales by 2^n: within about 2 ulp over the whole range (1.2 ulp from the
-// reduction and final rounding, the rest the hardware's), at a third of the library routine's
-// cost - which is what bounded the read-only statistics passes (39 -> 27 us on f32 [32768, 1024]
-// softmax(axis=0)).
-__device__ __forceinline__ float exp_reduced(float x) {
-    const float n = __builtin_rintf(x * 1.44269504f);
-    float r = __builtin_fmaf(n, -0.693145752f, x);      // ln 2, high part (exact product for |n| < 2^10)
-    r = __builtin_fmaf(n, -1.42860682e-6f, r);          // ln 2, low part
-    const float e = __builtin_amdgcn_exp2f(r * 1.44269504f);
-    const float v = __builtin_ldexpf(e, (int)n);
-    // below e^-104 the result is 0 (and -inf would make the reduction inf - inf); NaN compares
-    // false and passes through
-    return x < -104.0f ? 0.0f : v;
-}
+// bits anyway, use the hardware exp2 / log2 on the scaled argument; f32 tensors (tolerance 1e-5
+// against the CPU path) the exactly reduced form (exp_reduced, device_utils.cuh).
 template <class T> __device__ __forceinline__ float exp_ct(float x) {
     if constexpr (sizeof(T) == 2) return __expf(x);
-    else return exp_reduced(x);
+    else return exp_reduced<true>(x);  // every exponential of a softmax is of x - max <= 0
 }
 template <class T> __device__ __forceinline__ double exp_ct(double x) { return exp(x); }
 template <class T> __device__ __forceinline__ float log_ct(float x) {

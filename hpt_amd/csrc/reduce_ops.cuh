@@ -155,7 +155,7 @@ template <int OP, class T> struct FloatOp {
             return a * a * a;
         } else if constexpr (OP == HPT_LOGSUMEXP) {
             if constexpr (sizeof(OutWide) == 8) return (Acc)exp(f);
-            else return (Acc)expf(f);
+            else return (Acc)exp_reduced(f);
         } else return (Acc)f;
     }
     __device__ static __forceinline__ Acc comb(Acc a, Acc b) { return a + b; }
