@@ -241,7 +241,7 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
         const int full = (int)(16 / elem_size);
         if (p.lean && nk && !p.kept_swapped && p.vec == 1 && p.sstride == 1 && full > 1 && p.kept.stride[nk - 1] == 1 &&
             p.red.n == 1 && p.red.stride[0] == kin && (uintptr_t)data % 16 == 0 &&
-            (outer == 1 || p.kept.stride[0] % full == 0) && kin * p.R * (int64_t)elem_size >= (8ll << 20)) {
+            (outer == 1 || p.kept.stride[0] % full == 0) && outer * kin * p.R * (int64_t)elem_size >= (8ll << 20)) {
             // A contiguous [R, kin] slab whose rows are not whole vectors (kin = 3, 33, 257): walk it
             // as a FLAT array of aligned vectors. With a stride between a thread's visits that is a
             // multiple of kin, every vector slot of every thread stays on one column.
@@ -249,7 +249,8 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
             while (b) { int64_t t = g % b; g = b; b = t; }
             const int64_t kp = kin / g;  // threads per period: kp * full elements = full rows
             const int64_t tmax = std::min<int64_t>(1024, (int64_t)((64u << 10) / ((size_t)full * acc_size)));
-            if (kp <= tmax) {
+            // (each slab must be worth at least two periods of the walk)
+            if (kp <= tmax && kin * p.R >= 2 * kp * (tmax / kp) * full) {
                 p.flat_t = (int)(kp * (tmax / kp));
                 p.vec = full;
                 const int64_t per_iter = (int64_t)p.flat_t * full;
@@ -268,7 +269,7 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
             // the partials are [slice][phase][K].
             const int64_t phases = full / g;
             const int64_t xb = (kp + 1023) / 1024;
-            if (p.R >= 64 * phases && xb <= 65535 && kin * phases <= kI32) {
+            if (kp > tmax && p.R >= 16 * phases && xb <= 65535 && kin * phases <= kI32) {
                 p.flat_t = (int)(((kp + xb - 1) / xb + 63) / 64 * 64);
                 p.flat_xb = (int)xb;
                 p.flat_phases = (int)phases;
@@ -431,10 +432,12 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
     p.out_axis_stride = 1;
     if (n_norm_dims <= 0) p.out_axis_stride = ostr[axis];
     if (p.cols == 1) {
-        // one element per row: still a legal call; the generic kernel handles it
+        // one element per row: still a legal call. The axis has no extent, so neither of its strides
+        // matters: say 1 and the row plans (one lane per "row") take it, whatever the axis was.
         p.norm_in.n = 1;
         p.norm_in.size[0] = 1;
         p.norm_in.stride[0] = 1;
+        p.out_axis_stride = 1;
     }
 
     const int64_t sa = p.norm_in.n == 1 ? p.norm_in.stride[0] : 0;  // input stride along the row
@@ -624,15 +627,18 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             // A SHORT axis (softmax over the channels of [B, 21, H, W]): a thread keeps the whole axis of
             // its inner positions in registers, up to 64 registers of raw values: one read, one write.
             // The widest vector that the axis length leaves room for and the layout allows is taken.
-            if (p.cols <= 1024 && p.rows >= 64 * 1024) {
+            if (p.cols <= 1024 && p.cols > 1) {
                 // (two-byte types: vectors of at least 8 bytes, or the loads are too many and too small)
-                for (int ev = max_vec; ev >= (elem_size == 2 ? 4 : 1); ev /= 2) {
+                // (... unless the axis is so short that one thread holds it anyway)
+                for (int ev = max_vec; ev >= ((elem_size == 2 && p.cols > 16) ? 4 : 1); ev /= 2) {
                     const int64_t regs = std::max<int64_t>(1, ev * (int64_t)elem_size / 4);
                     const int64_t nc_max = std::min<int64_t>(64, 64 / regs);
                     const size_t vb = (size_t)ev * elem_size;
                     // thread rows that share an inner position when the axis is longer than one thread holds
                     const int64_t ty = pow2_ceil((p.cols + nc_max - 1) / nc_max);
-                    if (ty <= 16 && L % ev == 0 && sa % ev == 0 && (nk == 1 || p.kept_in.stride[0] % ev == 0) &&
+                    // enough threads to fill the chip: inner positions x thread rows
+                    if (ty <= 16 && p.rows / ev * ty >= 8 * 1024 && L % ev == 0 && sa % ev == 0 &&
+                        (nk == 1 || p.kept_in.stride[0] % ev == 0) &&
                         (p.cols * L) % ev == 0 && ((uintptr_t)in_data % vb) == 0 && ((uintptr_t)out_data % vb) == 0) {
                         p.kind = NormKind::ColReg;
                         p.vec = ev;
@@ -651,13 +657,14 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             // A narrow inner dim (or one that is not whole vectors) leaves most lanes idle: walk the
             // contiguous [cols, L] slab as a flat array of aligned vectors instead.
             if (max_vec > 1 && (!vec_ok || L < 64 * max_vec) && sa == L && ((uintptr_t)in_data % 16) == 0 &&
-                ((uintptr_t)out_data % 16) == 0 && p.cols * L * (int64_t)elem_size >= (8ll << 20) &&
+                ((uintptr_t)out_data % 16) == 0 && batch * p.cols * L * (int64_t)elem_size >= (8ll << 20) &&
                 (batch == 1 || (p.kept_in.stride[0] % max_vec == 0 && (p.cols * L) % max_vec == 0))) {
                 int64_t g = L, b = max_vec;
                 while (b) { int64_t t = g % b; g = b; b = t; }
                 const int64_t lp = L / g;  // threads per period
                 const int64_t tmax = std::min<int64_t>(1024, (64 << 10) / (max_vec * (elem_size == 8 ? 16 : 8)));
-                if (lp <= tmax) {
+                // (each batch slab must be worth at least two periods of the walk)
+                if (lp <= tmax && p.cols * L >= 2 * lp * (tmax / lp) * max_vec) {
                     p.flat_t = (int)(lp * (tmax / lp));
                     p.vec = max_vec;
                     const int64_t periods = p.cols * L / ((int64_t)p.flat_t * max_vec);

@@ -40,6 +40,22 @@ __device__ __forceinline__ void write_out(void* out, int64_t o, typename Op::Acc
     *p = Op::post(acc, count);
 }
 
+// N neighbouring outputs of one lane, overwritten (init_out) with 128-bit stores. `p` must be
+// aligned to min(16, N * sizeof(Out)) bytes; the caller checks the base and o is a multiple of N.
+template <class Op, int N>
+__device__ __forceinline__ void write_out_pack(void* out, int64_t o, const typename Op::Acc (&acc)[N], double count) {
+    using Out = typename Op::Out;
+    constexpr int PER = 16 / sizeof(Out) < N ? 16 / sizeof(Out) : N;  // outputs per store
+    Out* p = (Out*)out + o;
+#pragma unroll
+    for (int j0 = 0; j0 < N; j0 += PER) {
+        Pack<Out, PER> v;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) v.v[j] = Op::post(acc[j0 + j], count);
+        store_pack<Out, PER>(p + j0, v);
+    }
+}
+
 // ---- lean row kernel ---------------------------------------------------------
 // out[row] = reduce over i in [0, rin) of in[row * row_stride + i * sr].
 struct RowLeanArgs {
@@ -347,6 +363,7 @@ struct ColLeanArgs {
     int R;           // reduced length
     int split, init_out;
     int64_t oso, osi;  // output strides of the outer / inner kept index (kin and 1 unless the kept dims were swapped)
+    int vec_out;       // the outputs of a lane may be stored as vectors: overwrite mode, unit stride, aligned
 };
 
 template <class Op, int VEC, int SS = 1>
@@ -400,9 +417,16 @@ __global__ void __launch_bounds__(1024) col_lean_kernel(const ColLeanArgs a) {
     if (ty == 0 && valid) {
         const int64_t o0 = ((int64_t)outer * a.kin_v + cv) * UV;
         if (a.split == 1) {
+            if (UV > 1 && a.vec_out) {
+                // a lane's UV outputs are neighbours in memory: whole vectors (the outputs are half the
+                // traffic when few elements are reduced into each)
+                write_out_pack<Op, UV>(a.out, (int64_t)outer * a.oso + (int64_t)cv * UV, acc, a.count);
+            } else {
 #pragma unroll
-            for (int j = 0; j < UV; ++j)
-                write_out<Op>(a.out, (int64_t)outer * a.oso + ((int64_t)cv * UV + j) * a.osi, acc[j], a.init_out, a.count);
+                for (int j = 0; j < UV; ++j)
+                    write_out<Op>(a.out, (int64_t)outer * a.oso + ((int64_t)cv * UV + j) * a.osi, acc[j], a.init_out,
+                                  a.count);
+            }
         } else {
 #pragma unroll
             for (int j = 0; j < UV; ++j) ((Acc*)a.out)[(int64_t)blockIdx.z * a.K + o0 + j] = acc[j];
@@ -891,6 +915,13 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             const int64_t outer = nk > 1 ? p.kept.size[0] : 1;
             a.oso = p.kept_swapped ? 1 : kin;
             a.osi = p.kept_swapped ? outer : 1;
+            {
+                using Out = typename Op::Out;
+                const int uv = p.vec / p.sstride;
+                const size_t chunk = std::min<size_t>(16, (size_t)uv * sizeof(Out));
+                // every lane's first output index, outer * kin + cv * uv, must be a multiple of uv: kin is
+                a.vec_out = init_out && !p.kept_swapped && uv > 1 && kin % uv == 0 && ((uintptr_t)out % chunk) == 0;
+            }
             dim3 grid((unsigned)((a.kin_v + p.bx - 1) / p.bx), (unsigned)outer, (unsigned)p.split);
             if (vec && p.sstride == 2) col_lean_kernel<Op, FULL, 2><<<grid, block, smem, st>>>(a);
             else if (vec) col_lean_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
