@@ -285,7 +285,18 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
                 return p;
             }
         }
-        int64_t kv = (p.lean ? kin : p.K) / (p.vec / p.sstride);  // vector columns the lanes spread over
+        // Rows that are not whole, aligned vectors (an odd inner length, a base or pitch off 16 bytes):
+        // a lane still takes `full` neighbouring outputs, with unaligned 128-bit loads (global memory
+        // takes them; now and then one touches two lines) instead of one element at a time - eight
+        // times the bytes in flight per lane for f16. The last lane of a row loads its few elements singly.
+        // (Worth it when a row is a few wavefronts of such lanes and enough is reduced into each output
+        // that the lane's outputs, which it then writes one by one, are a small part of the traffic.)
+        if (p.lean && nk && p.vec == 1 && p.sstride == 1 && full > 1 && p.kept.stride[nk - 1] == 1 && kin >= 256 &&
+            p.R >= 256 && (uintptr_t)data % elem_size == 0) {
+            p.unaligned = true;
+            p.vec = full;
+        }
+        int64_t kv = ((p.lean ? kin : p.K) + (p.unaligned ? full - 1 : 0)) / (p.vec / p.sstride);  // vector columns the lanes spread over
         p.bx = (int)std::min<int64_t>(64, pow2_ceil(kv));
         int64_t xblocks = (kv + p.bx - 1) / p.bx * (p.lean ? outer : 1);
         // One wavefront per 64 vector columns streams best when there are enough
@@ -359,7 +370,7 @@ std::string describe(const ReducePlan& p) {
             break;
         case ReduceKind::Col:
             snprintf(buf, sizeof buf, "col%s%s vec=%d bx=%d by=%d outs=%lld red=%lld split=%d ",
-                     p.flat_xb ? "-flat-wide" : p.flat_t ? "-flat" : p.kept_swapped ? "-swapped" : p.lean ? "" : "-general",
+                     p.flat_xb ? "-flat-wide" : p.flat_t ? "-flat" : p.kept_swapped ? "-swapped" : p.unaligned ? "-unaligned" : p.lean ? "" : "-general",
                      p.sstride == 2 ? "-step2" : "", p.vec,
                      p.flat_t ? p.flat_t : p.bx, p.by,
                      (long long)p.K, (long long)p.R, p.split);

@@ -364,10 +364,14 @@ struct ColLeanArgs {
     int split, init_out;
     int64_t oso, osi;  // output strides of the outer / inner kept index (kin and 1 unless the kept dims were swapped)
     int vec_out;       // the outputs of a lane may be stored as vectors: overwrite mode, unit stride, aligned
+    int kin;           // inner kept length in elements (UA: kin_v = ceil(kin / VEC))
 };
 
-template <class Op, int VEC, int SS = 1>
+// UA: the rows are not whole, aligned vectors. A lane takes VEC neighbouring outputs all the same, with
+// unaligned 128-bit loads; the last lane of a row, which has fewer, loads them one by one.
+template <class Op, int VEC, int SS = 1, bool UA = false>
 __global__ void __launch_bounds__(1024) col_lean_kernel(const ColLeanArgs a) {
+    static_assert(!UA || (VEC > 1 && SS == 1), "UA is a full-vector mode");
     using T = typename Op::In;
     using Acc = typename Op::Acc;
     constexpr int UV = VEC / SS;  // outputs per lane (SS = 2: every second position of a vector)
@@ -376,9 +380,27 @@ __global__ void __launch_bounds__(1024) col_lean_kernel(const ColLeanArgs a) {
     const int cv = blockIdx.x * blockDim.x + tx;  // vector column in the inner dim
     const int outer = blockIdx.y;
     const bool valid = cv < a.kin_v;
+    // UA: outputs of this lane (VEC except in the last lane of a row)
+    const int cnt = UA ? (a.kin - cv * VEC < VEC ? a.kin - cv * VEC : VEC) : UV;
     Acc acc[UV];
 #pragma unroll
     for (int j = 0; j < UV; ++j) acc[j] = Op::identity();
+    auto load = [&](const T* p) {
+        Pack<T, VEC> v;
+        if constexpr (UA) {
+            if (cnt == VEC) {
+                v = load_pack_unaligned<T, VEC>(p);
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) v.v[j] = j < cnt ? p[j] : p[0];
+            }
+        } else if constexpr (VEC > 1) {
+            v = load_pack_stream<T, VEC>(p);
+        } else {
+            v.v[0] = *p;
+        }
+        return v;
+    };
     if (valid) {
         const T* base = (const T*)a.in + (int64_t)outer * a.so + (int64_t)cv * (VEC > 1 ? VEC : a.sk);
         // The reduced range is dealt out round-robin: thread row ty of workgroup z takes
@@ -392,29 +414,33 @@ __global__ void __launch_bounds__(1024) col_lean_kernel(const ColLeanArgs a) {
         for (; r + 7 * step < a.R; r += 8 * step) {
             Pack<T, VEC> v[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const T* p = base + (int64_t)(r + u * step) * a.rs;
-                if constexpr (VEC > 1) v[u] = load_pack_stream<T, VEC>(p);
-                else v[u].v[0] = *p;
-            }
+            for (int u = 0; u < 8; ++u) v[u] = load(base + (int64_t)(r + u * step) * a.rs);
 #pragma unroll
             for (int u = 0; u < 8; ++u)
 #pragma unroll
                 for (int j = 0; j < UV; ++j) fold_in<Op>(acc[j], v[u].v[j * SS], r + u * step);
         }
         for (; r < a.R; r += step) {
-            const T* p = base + (int64_t)r * a.rs;
-            if constexpr (VEC > 1) {
-                Pack<T, VEC> v = load_pack_stream<T, VEC>(p);
+            const Pack<T, VEC> v = load(base + (int64_t)r * a.rs);
 #pragma unroll
-                for (int j = 0; j < UV; ++j) fold_in<Op>(acc[j], v.v[j * SS], r);
-            } else {
-                fold_in<Op>(acc[0], *p, r);
-            }
+            for (int j = 0; j < UV; ++j) fold_in<Op>(acc[j], v.v[j * SS], r);
         }
     }
     fold_thread_rows<Op, UV>(acc, (Acc*)smem_raw);
     if (ty == 0 && valid) {
+        if constexpr (UA) {
+            // (the lanes of a row do not all have VEC outputs: element by element)
+            const int64_t ov = (int64_t)outer * a.kin + (int64_t)cv * VEC;  // in the kernel's numbering
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                if (j >= cnt) break;
+                if (a.split == 1)
+                    write_out<Op>(a.out, (int64_t)outer * a.oso + ((int64_t)cv * VEC + j) * a.osi, acc[j], a.init_out, a.count);
+                else
+                    ((Acc*)a.out)[(int64_t)blockIdx.z * a.K + ov + j] = acc[j];
+            }
+            return;
+        }
         const int64_t o0 = ((int64_t)outer * a.kin_v + cv) * UV;
         if (a.split == 1) {
             if (UV > 1 && a.vec_out) {
@@ -907,7 +933,8 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.rs = p.red.n ? p.red.stride[0] : 0;
             a.K = p.K;
             a.count = count;
-            a.kin_v = (int)(kin / (p.vec / p.sstride));
+            a.kin_v = (int)((kin + (p.unaligned ? p.vec - 1 : 0)) / (p.vec / p.sstride));
+            a.kin = (int)kin;
             a.sk = nk ? (int)p.kept.stride[nk - 1] : 1;
             a.R = (int)p.R;
             a.split = p.split;
@@ -924,7 +951,9 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             }
             dim3 grid((unsigned)((a.kin_v + p.bx - 1) / p.bx), (unsigned)outer, (unsigned)p.split);
             if (vec && p.sstride == 2) col_lean_kernel<Op, FULL, 2><<<grid, block, smem, st>>>(a);
-            else if (vec) col_lean_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
+            else if (vec && p.unaligned) {
+                if constexpr (FULL > 1) col_lean_kernel<Op, FULL, 1, true><<<grid, block, smem, st>>>(a);
+            } else if (vec) col_lean_kernel<Op, FULL><<<grid, block, smem, st>>>(a);
             else col_lean_kernel<Op, 1><<<grid, block, smem, st>>>(a);
         } else {
             ColArgs a{};

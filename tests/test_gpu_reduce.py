@@ -340,6 +340,35 @@ def test_reduction_over_the_last_axis_of_a_permuted_view(hpt, orc, dev):
             assert np.array_equal(t.sum([2]).numpy(), orc.reduce(orc.SUM, a, [2])), tag
 
 
+def test_column_reduction_over_rows_that_are_not_whole_vectors(hpt, orc, dev):
+    """Reductions over a long axis whose inner rows are odd-length or start off 16-byte boundaries:
+    a lane still takes a vector's worth of neighbouring outputs (unaligned 128-bit loads); the last
+    lane of a row, with fewer, loads them one by one."""
+    rng = np.random.default_rng(120)
+    cases = [((600, 259), (), 0, np.float32), ((5000, 301), (), 0, np.float16), ((3, 300, 1001), (), 1, np.float32),
+             ((601, 270), (("slice", ((1, 601, 1), (3, 264, 1))),), 0, np.float16), ((700, 263), (), 0, np.int32),
+             ((400, 257), (), 0, np.float64), ((2, 300, 513), (("permute", (1, 0, 2)),), 0, np.float32)]
+    for shape, ops, axis, npdt in cases:
+        base = (rng.standard_normal(shape) * 3).astype(npdt) if np.issubdtype(npdt, np.floating) else rng.integers(-9, 9, shape).astype(npdt)
+        t, a = upload(hpt, base, ops, dev=dev)
+        plan = hpt.reduce_plan(t, hpt.SUM, [axis])
+        assert "unaligned" in plan or "swapped" in plan, plan
+        tag = f"{np.dtype(npdt).name} {shape} {ops} axis={axis}"
+        assert np.array_equal(t.argmax(axis).numpy(), orc.argreduce(True, a, axis)), tag
+        assert np.array_equal(t.min([axis]).numpy(), a.min(axis)), tag
+        if npdt == np.float16:
+            want = orc.reduce(orc.SUM, a, [axis], acc=orc.ACC_F32).astype(np.float32)
+            assert_close(t.sum([axis]).numpy().astype(np.float32), want, HALF_RTOL, half_atol(want, 11), tag)
+        elif np.issubdtype(npdt, np.floating):
+            want = orc.reduce(orc.SUM, a, [axis], acc=orc.ACC_F64)
+            assert_close(t.sum([axis]).numpy(), want, F32_RTOL, F32_ATOL, tag)
+            out = hpt.Tensor.full(1.0, list(want.shape), t.dtype, dev)
+            t.sum_([axis], False, False, out)
+            assert_close(out.numpy(), want + 1.0, F32_RTOL, F32_ATOL, "accumulate " + tag)
+        else:
+            assert np.array_equal(t.sum([axis]).numpy(), orc.reduce(orc.SUM, a, [axis])), tag
+
+
 def test_sum_inplace_out_and_accumulate(hpt, orc, dev):
     """sum_ with init_out: true overwrites, false adds to what `out` holds (reduce.rs:84-92)."""
     rng = np.random.default_rng(107)

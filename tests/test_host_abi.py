@@ -85,7 +85,9 @@ def test_plans_for_shapes_off_the_benchmark_list(hpt):
     red = [
         # column reductions over a slab whose rows are not whole vectors: flat walk
         ([1016800, 33], [0], "col-flat "), ([8190, 4097], [0], "col-flat-wide"),
-        # too little data for it: lanes along the inner dim
+        # too little data for it: lanes along the inner dim, four neighbours each with unaligned vectors
+        ([300, 257], [0], "col-unaligned vec=4"),
+        # rows too short for that: one element per lane
         ([100, 33], [0], "col vec=1"),
         # whole vectors, narrow: many thread rows and slices
         ([4194304, 8], [0], "col vec=4 bx=2 by=256"),
