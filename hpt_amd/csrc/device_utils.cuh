@@ -188,6 +188,11 @@ __device__ __forceinline__ typename Elem<T>::Wide widen_fma(T x, typename Elem<T
     else return Elem<T>::widen(x) * b + c;
 }
 
+template <class T, int N>
+__device__ __forceinline__ void store_pack_unaligned(T* p, const Pack<T, N>& v) {
+    __builtin_memcpy(p, &v, sizeof(T) * N);
+}
+
 // ---- exponential ---------------------------------------------------------------
 // e^x for f32 data. The error of the hardware route exp2(x * log2 e) grows with |x| (the product
 // is rounded before the exponential sees it: |x| * 6e-8 relative). Here x = n ln 2 + r is split

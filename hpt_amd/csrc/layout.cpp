@@ -667,9 +667,11 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             p.vec = v;
             // A narrow inner dim (or one that is not whole vectors) leaves most lanes idle: walk the
             // contiguous [cols, L] slab as a flat array of aligned vectors instead.
-            if (max_vec > 1 && (!vec_ok || L < 64 * max_vec) && sa == L && ((uintptr_t)in_data % 16) == 0 &&
-                ((uintptr_t)out_data % 16) == 0 && batch * p.cols * L * (int64_t)elem_size >= (8ll << 20) &&
-                (batch == 1 || (p.kept_in.stride[0] % max_vec == 0 && (p.cols * L) % max_vec == 0))) {
+            if (max_vec > 1 && (!vec_ok || L < 64 * max_vec) && sa == L && ((uintptr_t)in_data % elem_size) == 0 &&
+                ((uintptr_t)out_data % elem_size) == 0 && batch * p.cols * L * (int64_t)elem_size >= (8ll << 20)) {
+                // (slabs that start off 16-byte boundaries take the same vectors unaligned: `shift`)
+                const bool aligned = ((uintptr_t)in_data % 16) == 0 && ((uintptr_t)out_data % 16) == 0 &&
+                                     (batch == 1 || (p.kept_in.stride[0] % max_vec == 0 && (p.cols * L) % max_vec == 0));
                 int64_t g = L, b = max_vec;
                 while (b) { int64_t t = g % b; g = b; b = t; }
                 const int64_t lp = L / g;  // threads per period
@@ -678,6 +680,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 if (lp <= tmax && p.cols * L >= 2 * lp * (tmax / lp) * max_vec) {
                     p.flat_t = (int)(lp * (tmax / lp));
                     p.vec = max_vec;
+                    p.shift = aligned ? 0 : 1;
                     const int64_t periods = p.cols * L / ((int64_t)p.flat_t * max_vec);
                     p.tsplit = (int)std::max<int64_t>(1, std::min<int64_t>(periods / 4, std::max<int64_t>(1, 256 / batch)));
                     p.scratch_bytes = (size_t)p.rows * p.tsplit * 16 + (size_t)p.rows * 3 * 8;
@@ -722,7 +725,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.shift ? "-shift" : (p.flat_t ? "-flat" : (p.gb_lds ? "-ldsgb" : ""))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? "-shift" : (p.gb_lds ? "-ldsgb" : ""))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     describe_dims(s, "rows_in", p.kept_in);

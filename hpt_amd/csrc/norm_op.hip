@@ -74,10 +74,17 @@ template <class T, int VEC> void launch_col_split(const NormPlan& p, const NormA
     if constexpr (VEC > 1) {
         if (p.flat_t > 0) {  // narrow inner dim: flat walk (statistics, the shared finalize, apply)
             const unsigned block = (unsigned)((p.flat_t + 63) / 64 * 64);
-            col_flat_stats_kernel<KIND, T, VEC><<<dim3((unsigned)t.S, 1, batch), dim3(block),
-                                                  (size_t)p.flat_t * VEC * sizeof(Part), st>>>(t, p.flat_t);
-            transposed_finalize_kernel<KIND, T><<<dim3((unsigned)((t.R + 15) / 16), 1, batch), dim3(16, 16), 0, st>>>(t);
-            col_flat_apply_kernel<KIND, T, VEC><<<dim3((unsigned)t.S, 1, batch), dim3(block), 0, st>>>(t, p.flat_t, t.S);
+            const size_t smem = (size_t)p.flat_t * VEC * sizeof(Part);
+            const dim3 grid((unsigned)t.S, 1, batch);
+            if (p.shift) {  // batch slabs off 16-byte boundaries: unaligned vectors
+                col_flat_stats_kernel<KIND, T, VEC, true><<<grid, dim3(block), smem, st>>>(t, p.flat_t);
+                transposed_finalize_kernel<KIND, T><<<dim3((unsigned)((t.R + 15) / 16), 1, batch), dim3(16, 16), 0, st>>>(t);
+                col_flat_apply_kernel<KIND, T, VEC, true><<<grid, dim3(block), 0, st>>>(t, p.flat_t, t.S);
+            } else {
+                col_flat_stats_kernel<KIND, T, VEC><<<grid, dim3(block), smem, st>>>(t, p.flat_t);
+                transposed_finalize_kernel<KIND, T><<<dim3((unsigned)((t.R + 15) / 16), 1, batch), dim3(16, 16), 0, st>>>(t);
+                col_flat_apply_kernel<KIND, T, VEC><<<grid, dim3(block), 0, st>>>(t, p.flat_t, t.S);
+            }
             return;
         }
     }

@@ -458,7 +458,8 @@ __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
 // sum), folded per inner index in LDS, one partial per workgroup in the layout of
 // transposed_stats_kernel (stats[b][y][L]) so that transposed_finalize_kernel serves both. Apply:
 // the same walk with the two per-index numbers of each slot in registers.
-template <int KIND, class T, int VEC>
+// UA: the batch slabs do not start on 16-byte boundaries; the same vectors, unaligned.
+template <int KIND, class T, int VEC, bool UA = false>
 __global__ void __launch_bounds__(1024) col_flat_stats_kernel(const TransposedArgs a, int threads) {
     static_assert(KIND != NORM_LAYERNORM, "a softmax pass");
     using CT = typename Elem<T>::Wide;
@@ -501,11 +502,12 @@ __global__ void __launch_bounds__(1024) col_flat_stats_kernel(const TransposedAr
         for (; it + 3 * S < whole; it += 4 * S) {
             Pack<T, VEC> v[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) v[u] = load_pack<T, VEC>(base + (it + u * S) * Lp + p0);
+            for (int u = 0; u < 4; ++u)
+                v[u] = UA ? load_pack_unaligned<T, VEC>(base + (it + u * S) * Lp + p0) : load_pack<T, VEC>(base + (it + u * S) * Lp + p0);
             fold(v, std::integral_constant<int, 4>{});
         }
         for (; it < whole; it += S) {
-            Pack<T, VEC> v = load_pack<T, VEC>(base + it * Lp + p0);
+            Pack<T, VEC> v = UA ? load_pack_unaligned<T, VEC>(base + it * Lp + p0) : load_pack<T, VEC>(base + it * Lp + p0);
             fold(&v, std::integral_constant<int, 1>{});
         }
         if (it == whole) {  // the last, partial period: element by element
@@ -535,7 +537,7 @@ __global__ void __launch_bounds__(1024) col_flat_stats_kernel(const TransposedAr
     for (int c = t; c < L; c += blockDim.x) dst[c] = sm[c];
 }
 
-template <int KIND, class T, int VEC>
+template <int KIND, class T, int VEC, bool UA = false>
 __global__ void __launch_bounds__(1024) col_flat_apply_kernel(const TransposedArgs a, int threads, int slices) {
     using CT = typename Elem<T>::Wide;
     constexpr bool kLog = KIND == NORM_LOGSOFTMAX;
@@ -564,21 +566,24 @@ __global__ void __launch_bounds__(1024) col_flat_apply_kernel(const TransposedAr
     for (; it + 3 * slices < whole; it += 4 * slices) {
         Pack<T, VEC> v[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(in + (it + u * slices) * Lp + p0);
+        for (int u = 0; u < 4; ++u)
+            v[u] = UA ? load_pack_unaligned<T, VEC>(in + (it + u * slices) * Lp + p0) : load_pack_stream<T, VEC>(in + (it + u * slices) * Lp + p0);
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             Pack<T, VEC> o;
 #pragma unroll
             for (int k = 0; k < VEC; ++k) o.v[k] = apply1(v[u].v[k], k);
-            store_pack_stream<T, VEC>(out + (it + u * slices) * Lp + p0, o);
+            if constexpr (UA) store_pack_unaligned<T, VEC>(out + (it + u * slices) * Lp + p0, o);
+            else store_pack_stream<T, VEC>(out + (it + u * slices) * Lp + p0, o);
         }
     }
     for (; it < whole; it += slices) {
-        const Pack<T, VEC> v = load_pack_stream<T, VEC>(in + it * Lp + p0);
+        const Pack<T, VEC> v = UA ? load_pack_unaligned<T, VEC>(in + it * Lp + p0) : load_pack_stream<T, VEC>(in + it * Lp + p0);
         Pack<T, VEC> o;
 #pragma unroll
         for (int k = 0; k < VEC; ++k) o.v[k] = apply1(v.v[k], k);
-        store_pack_stream<T, VEC>(out + it * Lp + p0, o);
+        if constexpr (UA) store_pack_unaligned<T, VEC>(out + it * Lp + p0, o);
+        else store_pack_stream<T, VEC>(out + it * Lp + p0, o);
     }
     if (it == whole) {
 #pragma unroll

@@ -430,6 +430,9 @@ FLAT_COLUMN_CASES = [
     ("f16 [N, 257] axis 0", np.float16, [20001, 257], 0),
     ("f32 [3, N, 5] axis 1", np.float32, [3, 500000, 5], 1),
     ("f64 [N, 7] axis 0", np.float64, [200001, 7], 0),
+    # batch slabs that start off 16-byte boundaries: the same walk with unaligned vectors
+    ("f16 [257, 13988, 7] axis 1 (misaligned slabs)", np.float16, [257, 13988, 7], 1),
+    ("f32 [31, 70001, 3] axis 1 (misaligned slabs)", np.float32, [31, 70001, 3], 1),
 ]
 
 
