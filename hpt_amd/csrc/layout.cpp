@@ -641,7 +641,9 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             if (p.cols <= 1024 && p.cols > 1) {
                 // (two-byte types: vectors of at least 8 bytes, or the loads are too many and too small)
                 // (... unless the axis is so short that one thread holds it anyway)
-                for (int ev = max_vec; ev >= ((elem_size == 2 && p.cols > 16) ? 4 : 1); ev /= 2) {
+                // (... or the inner dim so narrow that the alternative, lanes along it, would leave most idle:
+                // f16 [4097, 12, 96, 5] over axis 2, 0.4 -> 1.3 TB/s)
+                for (int ev = max_vec; ev >= ((elem_size == 2 && p.cols > 16 && L >= 64) ? 4 : 1); ev /= 2) {
                     const int64_t regs = std::max<int64_t>(1, ev * (int64_t)elem_size / 4);
                     const int64_t nc_max = std::min<int64_t>(64, 64 / regs);
                     const size_t vb = (size_t)ev * elem_size;
