@@ -372,6 +372,17 @@ struct ColRegArgs {
     int ty_log2;    // log2 of the thread rows that share an inner position
 };
 
+// Make the compiler forget what it knows about a pack of 2-byte elements: between two sweeps over
+// the raw values it would otherwise keep the widened (f32) copies of the first sweep alive for the
+// second, at twice the registers of the values themselves. Widening again costs one conversion.
+template <class T, int N> __device__ __forceinline__ void forget_pack(Pack<T, N>& v) {
+    if constexpr (sizeof(T) == 2) {
+        if constexpr (sizeof(T) * N == 16) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&v)));
+        else if constexpr (sizeof(T) * N == 8) asm volatile("" : "+v"(*reinterpret_cast<u32x2*>(&v)));
+        else if constexpr (sizeof(T) * N == 4) asm volatile("" : "+v"(*reinterpret_cast<uint32_t*>(&v)));
+    }
+}
+
 template <int KIND, class T, int EV, int NC>
 __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
     static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX, "a softmax kernel");
@@ -429,11 +440,15 @@ __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
             for (int k = 0; k < EV; ++k) m[k] = MaxC<CT>::comb(m[k], Elem<T>::widen(raw[i].v[k]));
     across(m, [](CT x, CT y) { return MaxC<CT>::comb(x, y); });
 #pragma unroll
+    for (int i = 0; i < NC; ++i) forget_pack(raw[i]);
+#pragma unroll
     for (int i = 0; i < NC; ++i)
         if (i < mine)
 #pragma unroll
             for (int k = 0; k < EV; ++k) s[k] += exp_ct<T>(Elem<T>::widen(raw[i].v[k]) - m[k]);
     across(s, [](CT x, CT y) { return x + y; });
+#pragma unroll
+    for (int i = 0; i < NC; ++i) forget_pack(raw[i]);
 #pragma unroll
     for (int k = 0; k < EV; ++k) kk[k] = kLog ? log_ct<T>(s[k]) : (CT)1 / s[k];
 #pragma unroll
