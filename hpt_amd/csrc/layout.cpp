@@ -582,8 +582,20 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 p.gb_lds = 1;
                 ln_half = false;
             }
+            // Two-byte softmax rows of 32769 ... 131072 elements: the raw row in registers (sixteen vectors
+            // per thread at most), one read instead of the streaming kernel's two.
+            const bool raw_rows = n_norm_dims <= 0 && elem_size == 2 && v == max_vec && p.sstride == 1 && !p.shift &&
+                                  nv > 4096 && nv <= 16384;
             const int64_t per = ln_half ? 2 * p.sstride : 4;
             const int64_t reg_limit = ln_half ? 1024 * per : (n_norm_dims > 0 && v > 1) ? 4096 : 8192;
+            if (raw_rows) {
+                p.kind = NormKind::RowReg;
+                p.raw_rows = 1;
+                p.tpr = 1024;
+                p.rpb = 1;
+                p.nchunk = nv > 8192 ? 16 : 8;
+                return p;
+            }
             if (nv <= reg_limit) {
                 p.kind = NormKind::RowReg;
                 // Short rows laid back to back: the plain kinds move whole 16 KiB tiles through LDS
@@ -710,6 +722,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
 
 void demote_to_generic(NormPlan& p) {
     p.kind = NormKind::Generic;
+    p.raw_rows = 0;
     p.gb_lds = 0;
     p.tile_rows = 0;
     p.flat_t = 0;
@@ -727,7 +740,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? "-shift" : (p.gb_lds ? "-ldsgb" : ""))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? "-shift" : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : "")))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     describe_dims(s, "rows_in", p.kept_in);

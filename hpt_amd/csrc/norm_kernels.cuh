@@ -380,6 +380,78 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     }
 }
 
+// ---- long rows of 2-byte elements: the raw row in registers ---------------------------------
+// softmax / log_softmax over rows of 32769 ... 131072 f16 / bf16 elements (a vocabulary). The row
+// kernel above keeps the widened row (f32) between its sweeps, which is 64 registers per thread at
+// eight vectors and does not fit at sixteen. Here only the RAW row stays (4 registers per vector:
+// 64 at sixteen vectors per thread, 1024 threads per row) and every sweep widens again: max, then
+// the sum of exponentials, then the result, the exponential taken twice. One HBM read and one
+// write where the streaming kernel reads twice.
+// PF (eight vectors per thread): the next row's loads are issued before the current row's sweeps;
+// there is one workgroup per compute unit, so nothing else hides a row's load -> sweeps -> store chain.
+template <int KIND, class T, int NCHUNK, bool PF = false>
+__global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
+    static_assert(sizeof(T) == 2 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX), "2-byte softmax rows");
+    constexpr int VEC = 8;
+    constexpr bool kLog = KIND == NORM_LOGSOFTMAX;
+    using CT = float;
+    __shared__ CT smem[16];
+    const int tx = threadIdx.x;
+    const int nv = (int)(a.cols / VEC);
+    Pack<T, VEC> raw[NCHUNK], nxt[PF ? NCHUNK : 1];
+    auto fetch = [&](Pack<T, VEC>* dst, int64_t row) {
+        if (row >= a.rows) return;
+        const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            const int iv = c * 1024 + tx;
+            if (iv < nv) dst[c] = load_pack_stream<T, VEC>(in_row + (int64_t)iv * VEC);
+        }
+    };
+    if constexpr (PF) fetch(raw, blockIdx.x);
+    for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
+        T* out_row = (T*)a.out + row * a.cols;
+        if constexpr (PF) fetch(nxt, row + gridDim.x);
+        else fetch(raw, row);
+        CT m = neg_inf<CT>();
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c)
+            if (c * 1024 + tx < nv)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, Elem<T>::widen(raw[c].v[j]));
+        m = row_all_reduce<MaxC<CT>>(m, 1024, 0, smem);
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&raw[c])));
+        CT s = 0;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c)
+            if (c * 1024 + tx < nv)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) s += exp_ct<T>(Elem<T>::widen(raw[c].v[j]) - m);
+        s = row_all_reduce<SumC<CT>>(s, 1024, 0, smem);
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&raw[c])));
+        const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            const int iv = c * 1024 + tx;
+            if (iv < nv) {
+                Pack<T, VEC> o;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const CT d = Elem<T>::widen(raw[c].v[j]) - m;
+                    o.v[j] = Elem<T>::narrow(kLog ? d - k : exp_ct<T>(d) * k);
+                }
+                store_pack_stream<T, VEC>(out_row + (int64_t)iv * VEC, o);
+            }
+        }
+        if constexpr (PF) {
+#pragma unroll
+            for (int c = 0; c < NCHUNK; ++c) raw[c] = nxt[c];
+        }
+    }
+}
+
 // ---- short rows laid back to back: whole tiles through LDS ---------------------------------
 // A contiguous [rows, cols] matrix with short rows (cols <= 512): a workgroup brings a.rpb
 // consecutive rows (16 KiB; a multiple of VEC rows, so the tile starts on a 16-byte boundary

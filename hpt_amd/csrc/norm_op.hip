@@ -226,6 +226,20 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         else launch_transposed<T>(p, a, st);
         return;
     }
+    if (p.kind == NormKind::RowReg && p.raw_rows) {
+        // long two-byte softmax rows: the raw row in registers; the fused kinds stream (sixteen vectors
+        // per thread) or take the ordinary register kernel (eight)
+        if constexpr (sizeof(T) == 2 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX)) {
+            if (grid.x > 512u) grid.x = 512u;
+            if (p.nchunk == 16) row_raw_kernel<KIND, T, 16><<<grid, dim3(1024), 0, st>>>(a);
+            else row_raw_kernel<KIND, T, 8, true><<<grid, dim3(1024), 0, st>>>(a);
+            return;
+        } else if (p.nchunk > 8) {
+            if (p.vec == FULL) row_stream_kernel<KIND, T, FULL><<<grid, block, 0, st>>>(a);
+            else row_stream_kernel<KIND, T, 1><<<grid, block, 0, st>>>(a);
+            return;
+        }
+    }
     if (p.kind == NormKind::RowReg) {
         // Layernorm workgroups walk the rows (gamma / beta stay in registers);
         // softmax has nothing to reuse across rows and runs one row per group.

@@ -315,6 +315,8 @@ WIDE_ROW_CASES = [
     ("f16 two vectors per thread", np.float16, [1100, 8192]),
     ("f16 eight vectors per thread", np.float16, [600, 65536]),
     ("bf16", "bf16", [1111, 16384]),
+    ("bf16 rows of 128256: the raw row in registers, sixteen vectors per thread", "bf16", [530, 128256]),
+    ("f16 rows of 100000: the same, the last chunks partly filled", np.float16, [515, 100000]),
     # odd lengths: aligned vectors, masked row ends (registers up to 2048 vectors, then streaming)
     ("f32 rows of 4097", np.float32, [2100, 4097]),
     ("f16 rows of 197", np.float16, [30011, 197]),
