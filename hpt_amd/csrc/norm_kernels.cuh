@@ -391,14 +391,18 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
 // there is one workgroup per compute unit, so nothing else hides a row's load -> sweeps -> store chain.
 template <int KIND, class T, int NCHUNK, bool PF = false>
 __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
-    static_assert(sizeof(T) == 2 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX), "2-byte softmax rows");
-    constexpr int VEC = 8;
+    static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX, "a softmax kernel");
+    constexpr int VEC = 16 / sizeof(T);
     constexpr bool kLog = KIND == NORM_LOGSOFTMAX;
-    using CT = float;
+    using CT = typename Elem<T>::Wide;
     __shared__ CT smem[16];
     const int tx = threadIdx.x;
     const int nv = (int)(a.cols / VEC);
     Pack<T, VEC> raw[NCHUNK], nxt[PF ? NCHUNK : 1];
+    // (2-byte types: keep the compiler from holding the widened copies of one sweep for the next)
+    auto forget = [](Pack<T, VEC>& v) {
+        if constexpr (sizeof(T) == 2) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&v)));
+    };
     auto fetch = [&](Pack<T, VEC>* dst, int64_t row) {
         if (row >= a.rows) return;
         const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
@@ -421,7 +425,7 @@ __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
                 for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, Elem<T>::widen(raw[c].v[j]));
         m = row_all_reduce<MaxC<CT>>(m, 1024, 0, smem);
 #pragma unroll
-        for (int c = 0; c < NCHUNK; ++c) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&raw[c])));
+        for (int c = 0; c < NCHUNK; ++c) forget(raw[c]);
         CT s = 0;
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c)
@@ -430,7 +434,7 @@ __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
                 for (int j = 0; j < VEC; ++j) s += exp_ct<T>(Elem<T>::widen(raw[c].v[j]) - m);
         s = row_all_reduce<SumC<CT>>(s, 1024, 0, smem);
 #pragma unroll
-        for (int c = 0; c < NCHUNK; ++c) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&raw[c])));
+        for (int c = 0; c < NCHUNK; ++c) forget(raw[c]);
         const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
