@@ -174,6 +174,14 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
                 return p;
             }
         }
+        if (p.lean && p.vec == 1 && full > 1 && p.sstride == 1 && p.red.stride[0] == 1 && rin >= 64 * full &&
+            (uintptr_t)data % elem_size == 0) {
+            // Long contiguous rows whose length, pitch or base is off the 16-byte grid (the sum of a
+            // whole array of odd length): the kernel peels each row's first elements up to a 16-byte
+            // boundary and its last ones, and reads everything between as aligned vectors.
+            p.ragged = true;
+            p.vec = full;
+        }
         int64_t nv = p.R / (p.vec / p.sstride);  // vector loads per output
         // About 8 vector loads per lane; groups of one or two wavefronts per row
         // stream best (each wavefront walks its own long run of the row), and
@@ -365,7 +373,7 @@ std::string describe(const ReducePlan& p) {
         case ReduceKind::Identity: return "identity";
         case ReduceKind::Row:
             snprintf(buf, sizeof buf, "row%s%s vec=%d tpr=%d rpb=%d rows=%lld cols=%lld split=%d(%dx%d) ",
-                     p.row_tile ? "-tile" : p.lean ? "" : "-general", p.sstride == 2 ? "-step2" : "", p.vec, p.tpr, p.rpb,
+                     p.row_tile ? "-tile" : p.ragged ? "-ragged" : p.lean ? "" : "-general", p.sstride == 2 ? "-step2" : "", p.vec, p.tpr, p.rpb,
                      (long long)p.K, (long long)p.R, p.split, p.split_q, p.split_i);
             break;
         case ReduceKind::Col:

@@ -65,6 +65,7 @@ struct RowLeanArgs {
     double count;
     int K;           // rows
     int rin_v;       // row length in vectors
+    int rin;         // row length in elements (RAG)
     int sr;          // element stride along the row (1 when VEC > 1)
     int ichunk;      // vectors per split
     int tpr, tpr_log2, rpb, split, init_out;
@@ -72,7 +73,10 @@ struct RowLeanArgs {
 
 // SS = 2: the row's elements sit at every second position; full vectors are
 // loaded and the odd positions dropped (see row_reg_kernel).
-template <class Op, int VEC, int SS = 1>
+// RAG: contiguous rows of any length that start anywhere. A row's elements before its first
+// 16-byte boundary and after its last whole vector are folded one by one (by the first split's
+// lanes); the vectors between are aligned.
+template <class Op, int VEC, int SS = 1, bool RAG = false>
 __global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
     using T = typename Op::In;
     using Acc = typename Op::Acc;
@@ -86,8 +90,17 @@ __global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
     Acc acc = Op::identity();
     if (valid) {
         const T* p = (const T*)a.in + (int64_t)row * a.row_stride;
+        int nvec = a.rin_v, head = 0;
+        if constexpr (RAG) {
+            head = min((int)(((16 - ((uintptr_t)p & 15)) & 15) / sizeof(T)), a.rin);
+            nvec = (a.rin - head) / VEC;
+            // (a lane meets its indices in growing order: head, vectors, tail)
+            if (blockIdx.y == 0)
+                for (int i = tx; i < head; i += tpr) fold_in<Op>(acc, p[i], i);
+            p += head;
+        }
         const int i0 = blockIdx.y * a.ichunk;
-        const int i1 = min(a.rin_v, i0 + a.ichunk);
+        const int i1 = min(nvec, i0 + a.ichunk);
         int iv = i0 + tx;
         if constexpr (VEC > 1) {
             // batches of four loads in flight per lane before any is consumed
@@ -99,16 +112,20 @@ __global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
                 for (int u = 0; u < 4; ++u)
 #pragma unroll
                     for (int j = 0; j < UV; ++j)
-                        fold_in<Op>(acc, v[u].v[j * SS], (iv + u * tpr) * UV + j);
+                        fold_in<Op>(acc, v[u].v[j * SS], head + (iv + u * tpr) * UV + j);
             }
             for (; iv < i1; iv += tpr) {
                 Pack<T, VEC> v = load_pack_stream<T, VEC>(p + (int64_t)iv * VEC);
 #pragma unroll
-                for (int j = 0; j < UV; ++j) fold_in<Op>(acc, v.v[j * SS], iv * UV + j);
+                for (int j = 0; j < UV; ++j) fold_in<Op>(acc, v.v[j * SS], head + iv * UV + j);
             }
         } else {
 #pragma unroll 4
             for (; iv < i1; iv += tpr) fold_in<Op>(acc, p[(int64_t)iv * a.sr], iv);
+        }
+        if constexpr (RAG) {
+            if (blockIdx.y == 0)
+                for (int i = nvec * VEC + tx; i < a.rin - head; i += tpr) fold_in<Op>(acc, p[i], head + i);
         }
     }
     acc = group_reduce<Op>(acc, tpr < 64 ? tpr : 64);
@@ -843,6 +860,7 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.count = count;
             a.K = (int)p.K;
             a.rin_v = (int)(rin / (p.vec / p.sstride));
+            a.rin = (int)rin;
             a.sr = (int)p.red.stride[0];
             a.ichunk = (a.rin_v + p.split - 1) / p.split;
             a.tpr = p.tpr;
@@ -851,6 +869,7 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.split = p.split;
             a.init_out = init_out;
             if (vec && p.sstride == 2) row_lean_kernel<Op, FULL, 2><<<grid, block, 0, st>>>(a);
+            else if (vec && p.ragged) row_lean_kernel<Op, FULL, 1, true><<<grid, block, 0, st>>>(a);
             else if (vec) row_lean_kernel<Op, FULL><<<grid, block, 0, st>>>(a);
             else row_lean_kernel<Op, 1><<<grid, block, 0, st>>>(a);
         } else {

@@ -316,6 +316,48 @@ def test_special_values_on_the_large_shape_kernels(hpt, orc, dev):
             assert np.array_equal(t.argmin(axes[0]).numpy(), orc.argreduce(False, a, axes[0])), tag
 
 
+def test_long_rows_off_the_vector_grid(hpt, orc, dev):
+    """Long contiguous rows whose length, pitch or start is not a whole number of 128-bit vectors (the
+    sum of a whole array of odd length, a slice that drops the first element): the first and last
+    elements of each row are folded one by one, the rest as aligned vectors. Ties check the index rule
+    across the peeled ends; a row shorter than its own peel and the two-stage form are included."""
+    rng = np.random.default_rng(121)
+    assert hpt.reduce_plan(hpt.Tensor.empty([3000001], hpt.u8, dev), hpt.SUM, [0]).startswith("row-ragged")
+    for shape, view, npdt in (((3000001,), (), np.uint8), ((1000003,), (("slice", ((3, 1000000, 1),)),), np.float32),
+                              ((2000001,), (("slice", ((1, 2000001, 1),)),), np.int16), ((7, 300001), (), np.float16),
+                              ((300, 5001), (), np.float32), ((33, 40007), (("slice", ((0, 33, 1), (5, 40000, 1))),), np.int32),
+                              ((5001, 1100), (("slice", ((0, 5001, 1), (1, 1040, 1))),), np.uint8), ((4000003,), (), np.bool_), ((12, 100003), (), np.float64)):
+        if npdt == np.bool_:
+            base = rng.integers(0, 2, shape).astype(npdt)
+        elif np.issubdtype(npdt, np.floating):
+            base = rng.standard_normal(shape).astype(npdt)
+        else:
+            base = rng.integers(0, 60, shape).astype(npdt)   # many ties
+        t, a = upload(hpt, base, view, dev=dev)
+        ax = len(shape) - 1
+        tag = f"{np.dtype(npdt).name} {shape} {view}"
+        assert hpt.reduce_plan(t, hpt.SUM, [ax]).startswith("row-ragged"), hpt.reduce_plan(t, hpt.SUM, [ax])
+        assert np.array_equal(t.argmax(ax).numpy(), orc.argreduce(True, a, ax)), tag
+        assert np.array_equal(t.argmin(ax).numpy(), orc.argreduce(False, a, ax)), tag
+        if npdt == np.bool_:
+            assert np.array_equal(t.all([ax]).numpy().reshape(-1), a.all(ax).reshape(-1)) and np.array_equal(t.any([ax]).numpy().reshape(-1), a.any(ax).reshape(-1)), tag
+            continue
+        assert np.array_equal(t.max([ax]).numpy(), orc.reduce(orc.MAX, a, [ax])), tag
+        if npdt == np.float16:
+            want = orc.reduce(orc.SUM, a, [ax], acc=orc.ACC_F32).astype(np.float32)
+            assert_close(t.sum([ax]).numpy().astype(np.float32), want, HALF_RTOL, half_atol(want, 11), tag)
+        elif np.issubdtype(npdt, np.floating):
+            assert_close(t.sum([ax]).numpy(), orc.reduce(orc.SUM, a, [ax], acc=orc.ACC_F64), F32_RTOL, 2e-5, tag)
+        else:
+            assert np.array_equal(t.sum([ax]).numpy(), orc.reduce(orc.SUM, a, [ax])), tag
+    # the extreme value sits in a peeled end: first element, last element
+    for pos in (0, 1000002):
+        x = np.zeros(1000003, np.float32)
+        x[pos] = 7.0
+        t, a = upload(hpt, x, dev=dev)
+        assert int(t.argmax(0).numpy()) == pos and float(t.max([0]).numpy()) == 7.0 and float(t.sum([0]).numpy()) == 7.0
+
+
 def test_reduction_over_the_last_axis_of_a_permuted_view(hpt, orc, dev):
     """x.permute(2, 1, 0).sum(2): the first kept dim is the contiguous one. The lanes run along it and
     the outputs are scattered (one launch, and the two-stage form with its second-stage remap)."""

@@ -139,9 +139,10 @@ def test_plans_for_the_benchmark_configurations(hpt):
     assert hpt.normalize_plan(c5[:, ::2], 1).startswith("rowreg-step2") and "norm_in=[64:2]" in hpt.normalize_plan(c5[:, ::2], 1)
     assert hpt.reduce_plan(c5[:, ::2], hpt.SUM, [0]).startswith("col-step2 vec=8")
     assert hpt.reduce_plan(c5[:, 1::2], hpt.SUM, [0]).startswith("col vec=1")   # odd start: vectors would be misaligned
-    # misaligned base pointer or odd row length: scalar loads
-    assert hpt.reduce_plan(f32(7, 1023), hpt.SUM, [1]).startswith("row vec=1")
-    assert hpt.reduce_plan(f32(8, 1024)[:, 1:], hpt.SUM, [1]).startswith("row vec=1")
+    # misaligned base pointer or odd row length: long rows peel their ends, short ones take scalar loads
+    assert hpt.reduce_plan(f32(7, 1023), hpt.SUM, [1]).startswith("row-ragged vec=4")
+    assert hpt.reduce_plan(f32(8, 1024)[:, 1:], hpt.SUM, [1]).startswith("row-ragged vec=4")
+    assert hpt.reduce_plan(f32(7, 103), hpt.SUM, [1]).startswith("row vec=1")
 
 
 def test_coalescing_matches_brute_force_offsets(hpt):
