@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 # (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, with --copy-calibration), each counter scaled
 # by what it reads for the plain 134217728-byte copy in the same run: fetch 131395.9 KiB +
 # write 131093.8 KiB. A measured constant, not something this script can read live.
-HEADLINE_TRAFFIC_BYTES = 268789487
+HEADLINE_TRAFFIC_BYTES = 268783485
 
 
 # ---- HIP events on the launch stream (the null stream: the library is called with stream=NULL) ----
@@ -469,7 +469,7 @@ def main():
         "rows_per_s": round(8192 * args.steps / wall, 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": HEADLINE_TRAFFIC_BYTES,
-                     "kernel": "hpt::row_reg_kernel<2, float, 4, 4, 1, false, false>", "kernel_us": round(kernel_us, 2)},
+                     "kernel": "hpt::row_reg_kernel<2, float, 4, 4, 1, false, false, false>", "kernel_us": round(kernel_us, 2)},
         "cpu_baseline": cpu,
         "ops": ops,
     }
