@@ -98,7 +98,7 @@ struct ReducePlan {
     int sstride = 1;    // lean kernels: 2 = elements along the lane dim sit at every second position
     bool lean = false;  // the layout fits the lean kernels (one reduced dim, <= 2 kept dims, 32-bit extents)
     bool ragged = false;        // Row (lean): rows of any length and alignment; aligned 128-bit loads over the body, the two ends element-wise
-    bool unaligned = false;     // Col (lean): rows are not whole / aligned vectors; lanes still take VEC neighbours with unaligned 128-bit loads
+    bool unaligned = false;     // Col (lean): rows are not whole / aligned vectors; lanes still take VEC neighbours with unaligned 128-bit loads. Row: runs off the 16-byte grid read with unaligned 128-bit loads
     bool kept_swapped = false;  // Col (lean): the two kept dims are listed inner-most-in-memory last, not in output order
     int row_tile = 0;   // Row, > 0: short contiguous rows staged through LDS, this many rows per workgroup
     int flat_t = 0;     // Col, > 0: contiguous [R, kin] slab walked as a flat array by this many threads

@@ -182,7 +182,14 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
             p.ragged = true;
             p.vec = full;
         }
-        int64_t nv = p.R / (p.vec / p.sstride);  // vector loads per output
+        if (p.vec == 1 && full > 1 && p.sstride == 1 && p.red.stride[p.red.n - 1] == 1 && rin >= full &&
+            (uintptr_t)data % elem_size == 0) {
+            // Shorter contiguous runs off the grid (the batch-norm sums of [N, C, 7, 7]: runs of 49):
+            // unaligned 128-bit loads from the run's start on, the last one taken from the run's end.
+            p.unaligned = true;
+            p.vec = full;
+        }
+        int64_t nv = p.unaligned ? (p.R / rin) * ((rin + full - 1) / full) : p.R / (p.vec / p.sstride);  // vector loads per output
         // About 8 vector loads per lane; groups of one or two wavefronts per row
         // stream best (each wavefront walks its own long run of the row), and
         // only very long rows get a whole workgroup.
@@ -193,11 +200,17 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
         int64_t blocks = (p.K + p.rpb - 1) / p.rpb;
         p.split = p.split_q = p.split_i = 1;
         if (blocks < kBlocksToFill / 4) {
-            // Too few outputs to fill the chip: several workgroups of 256 threads
+            // Too few outputs to fill the chip: a whole workgroup per output when that leaves
+            // each thread 8 loads or more, then several workgroups of 256 threads
             // per output, each with a long contiguous share (>= 16 loads per
-            // thread); about 512 workgroups in all is the measured sweet spot.
+            // thread, 8 when there are many outputs to amortise the second stage over); about
+            // 512 workgroups in all is the measured sweet spot.
+            if (p.tpr < 256 && nv >= 256 * 8) {
+                p.tpr = 256;
+                p.rpb = 1;
+            }
             int64_t want = (512 + p.K - 1) / p.K;
-            int64_t can = nv / (256 * 16);
+            int64_t can = nv / (256 * (p.K >= 64 ? 8 : 16));
             int64_t split = std::min<int64_t>(std::min(want, can), 4096);
             if (split > 1) {
                 p.tpr = 256;
@@ -373,7 +386,7 @@ std::string describe(const ReducePlan& p) {
         case ReduceKind::Identity: return "identity";
         case ReduceKind::Row:
             snprintf(buf, sizeof buf, "row%s%s vec=%d tpr=%d rpb=%d rows=%lld cols=%lld split=%d(%dx%d) ",
-                     p.row_tile ? "-tile" : p.ragged ? "-ragged" : p.lean ? "" : "-general", p.sstride == 2 ? "-step2" : "", p.vec, p.tpr, p.rpb,
+                     p.row_tile ? "-tile" : p.ragged ? "-ragged" : p.lean ? "" : "-general", p.sstride == 2 ? "-step2" : p.unaligned ? "-unaligned" : "", p.vec, p.tpr, p.rpb,
                      (long long)p.K, (long long)p.R, p.split, p.split_q, p.split_i);
             break;
         case ReduceKind::Col:

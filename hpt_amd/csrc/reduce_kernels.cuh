@@ -76,8 +76,12 @@ struct RowLeanArgs {
 // RAG: contiguous rows of any length that start anywhere. A row's elements before its first
 // 16-byte boundary and after its last whole vector are folded one by one (by the first split's
 // lanes); the vectors between are aligned.
-template <class Op, int VEC, int SS = 1, bool RAG = false>
+// UA: short or strided-pitch rows off the grid: unaligned 128-bit loads from the row start on; the
+// last vector of a row is taken from the row's END backwards and the elements it shares with the
+// vector before are skipped, so no load leaves the row.
+template <class Op, int VEC, int SS = 1, bool RAG = false, bool UA = false>
 __global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
+    static_assert(!UA || (VEC > 1 && SS == 1 && !RAG), "UA is a full-vector mode of its own");
     using T = typename Op::In;
     using Acc = typename Op::Acc;
     constexpr int UV = VEC / SS;
@@ -103,22 +107,30 @@ __global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
         const int i1 = min(nvec, i0 + a.ichunk);
         int iv = i0 + tx;
         if constexpr (VEC > 1) {
+            auto load = [&](int i) {
+                if constexpr (UA) return load_pack_unaligned<T, VEC>(p + min(i * VEC, a.rin - VEC));
+                else return load_pack_stream<T, VEC>(p + (int64_t)i * VEC);
+            };
+            auto fold = [&](const Pack<T, VEC>& v, int i) {
+                if constexpr (UA) {
+                    const int e = i * VEC, from = min(e, a.rin - VEC);
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        if (from + j >= e) fold_in<Op>(acc, v.v[j], from + j);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < UV; ++j) fold_in<Op>(acc, v.v[j * SS], head + i * UV + j);
+                }
+            };
             // batches of four loads in flight per lane before any is consumed
             for (; iv + 3 * tpr < i1; iv += 4 * tpr) {
                 Pack<T, VEC> v[4];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(p + (int64_t)(iv + u * tpr) * VEC);
+                for (int u = 0; u < 4; ++u) v[u] = load(iv + u * tpr);
 #pragma unroll
-                for (int u = 0; u < 4; ++u)
-#pragma unroll
-                    for (int j = 0; j < UV; ++j)
-                        fold_in<Op>(acc, v[u].v[j * SS], head + (iv + u * tpr) * UV + j);
+                for (int u = 0; u < 4; ++u) fold(v[u], iv + u * tpr);
             }
-            for (; iv < i1; iv += tpr) {
-                Pack<T, VEC> v = load_pack_stream<T, VEC>(p + (int64_t)iv * VEC);
-#pragma unroll
-                for (int j = 0; j < UV; ++j) fold_in<Op>(acc, v.v[j * SS], head + iv * UV + j);
-            }
+            for (; iv < i1; iv += tpr) fold(load(iv), iv);
         } else {
 #pragma unroll 4
             for (; iv < i1; iv += tpr) fold_in<Op>(acc, p[(int64_t)iv * a.sr], iv);
@@ -151,6 +163,7 @@ struct RowArgs {
     int64_t K;       // outputs
     int64_t rout;    // product of redo sizes
     int64_t rin_v;   // innermost reduced length, in vectors
+    int64_t rin;     // innermost reduced length, in elements (UA)
     int64_t sr;      // innermost reduced stride in elements (1 when VEC > 1)
     int64_t qchunk;  // outer reduced indices per split
     int64_t ichunk;  // inner vectors per split
@@ -158,21 +171,34 @@ struct RowArgs {
     int tpr, tpr_log2, rpb, split_q, split_i, init_out;
 };
 
-template <class Op, int VEC>
-__device__ __forceinline__ void row_step(typename Op::Acc& acc, const typename Op::In* p, int64_t iv,
-                                         int64_t sr) {
-    using T = typename Op::In;
-    if constexpr (VEC > 1) {
-        Pack<T, VEC> v = load_pack_stream<T, VEC>(p + iv * VEC);
+// Vector iv of a run of `rin` contiguous elements at p. UA (runs that are not whole, aligned
+// vectors): an unaligned load; the run's last vector is taken from its end backwards and the
+// elements it shares with the vector before are skipped.
+template <class T, int VEC, bool UA>
+__device__ __forceinline__ Pack<T, VEC> row_vec_load(const T* p, int64_t iv, int64_t rin) {
+    if constexpr (UA) return load_pack_unaligned<T, VEC>(p + min(iv * VEC, rin - VEC));
+    else return load_pack_stream<T, VEC>(p + iv * VEC);
+}
+template <class Op, int VEC, bool UA>
+__device__ __forceinline__ void row_vec_fold(typename Op::Acc& acc, const Pack<typename Op::In, VEC>& v, int64_t iv,
+                                             int64_t rin) {
+    const int64_t e = iv * VEC, from = UA ? min(e, rin - VEC) : e;
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) fold_in<Op>(acc, v.v[j], iv * VEC + j);
-    } else {
-        fold_in<Op>(acc, p[iv * sr], iv);
-    }
+    for (int j = 0; j < VEC; ++j)
+        if (!UA || from + j >= e) fold_in<Op>(acc, v.v[j], from + j);
 }
 
-template <class Op, int VEC>
+template <class Op, int VEC, bool UA>
+__device__ __forceinline__ void row_step(typename Op::Acc& acc, const typename Op::In* p, int64_t iv,
+                                         int64_t sr, int64_t rin) {
+    using T = typename Op::In;
+    if constexpr (VEC > 1) row_vec_fold<Op, VEC, UA>(acc, row_vec_load<T, VEC, UA>(p, iv, rin), iv, rin);
+    else fold_in<Op>(acc, p[iv * sr], iv);
+}
+
+template <class Op, int VEC, bool UA = false>
 __global__ void __launch_bounds__(1024) row_reduce_kernel(const RowArgs a) {
+    static_assert(!UA || VEC > 1, "UA is a full-vector mode");
     using T = typename Op::In;
     using Acc = typename Op::Acc;
     __shared__ Acc smem[16];
@@ -197,7 +223,7 @@ __global__ void __launch_bounds__(1024) row_reduce_kernel(const RowArgs a) {
             if (q0 < q1) {
                 const T* p = base + offset_of(a.redo, q0);
 #pragma unroll 4
-                for (int64_t iv = i0 + tx; iv < i1; iv += tpr) row_step<Op, VEC>(acc, p, iv, a.sr);
+                for (int64_t iv = i0 + tx; iv < i1; iv += tpr) row_step<Op, VEC, UA>(acc, p, iv, a.sr, a.rin);
             }
         } else if (ni > 0) {
             // Several outer reduced indices, each with an inner run of ni vectors (the sums of a
@@ -236,11 +262,9 @@ __global__ void __launch_bounds__(1024) row_reduce_kernel(const RowArgs a) {
                 if constexpr (VEC > 1) {
                     Pack<T, VEC> v[4];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(p[u] + iv[u] * VEC);
+                    for (int u = 0; u < 4; ++u) v[u] = row_vec_load<T, VEC, UA>(p[u], iv[u], a.rin);
 #pragma unroll
-                    for (int u = 0; u < 4; ++u)
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) fold_in<Op>(acc, v[u].v[j], iv[u] * VEC + j);
+                    for (int u = 0; u < 4; ++u) row_vec_fold<Op, VEC, UA>(acc, v[u], iv[u], a.rin);
                 } else {
                     T v[4];
 #pragma unroll
@@ -250,7 +274,7 @@ __global__ void __launch_bounds__(1024) row_reduce_kernel(const RowArgs a) {
                 }
             }
             for (; t < total; t += tpr) {
-                row_step<Op, VEC>(acc, base + offset_of(a.redo, q0 + dq), i0 + di, a.sr);
+                row_step<Op, VEC, UA>(acc, base + offset_of(a.redo, q0 + dq), i0 + di, a.sr, a.rin);
                 advance();
             }
         }
@@ -859,7 +883,7 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.row_stride = p.kept.n ? p.kept.stride[0] : 0;
             a.count = count;
             a.K = (int)p.K;
-            a.rin_v = (int)(rin / (p.vec / p.sstride));
+            a.rin_v = (int)((rin + (p.unaligned ? p.vec - 1 : 0)) / (p.vec / p.sstride));
             a.rin = (int)rin;
             a.sr = (int)p.red.stride[0];
             a.ichunk = (a.rin_v + p.split - 1) / p.split;
@@ -870,6 +894,7 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.init_out = init_out;
             if (vec && p.sstride == 2) row_lean_kernel<Op, FULL, 2><<<grid, block, 0, st>>>(a);
             else if (vec && p.ragged) row_lean_kernel<Op, FULL, 1, true><<<grid, block, 0, st>>>(a);
+            else if (vec && p.unaligned) row_lean_kernel<Op, FULL, 1, false, true><<<grid, block, 0, st>>>(a);
             else if (vec) row_lean_kernel<Op, FULL><<<grid, block, 0, st>>>(a);
             else row_lean_kernel<Op, 1><<<grid, block, 0, st>>>(a);
         } else {
@@ -881,7 +906,8 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.redo.n = p.red.n - 1;
             a.K = p.K;
             a.rout = p.R / rin;
-            a.rin_v = rin / p.vec;
+            a.rin_v = (rin + (p.unaligned ? p.vec - 1 : 0)) / p.vec;
+            a.rin = rin;
             a.sr = p.red.stride[p.red.n - 1];
             a.qchunk = (a.rout + p.split_q - 1) / p.split_q;
             a.ichunk = (a.rin_v + p.split_i - 1) / p.split_i;
@@ -892,7 +918,8 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.split_q = p.split_q;
             a.split_i = p.split_i;
             a.init_out = init_out;
-            if (vec) row_reduce_kernel<Op, FULL><<<grid, block, 0, st>>>(a);
+            if (vec && p.unaligned) row_reduce_kernel<Op, FULL, true><<<grid, block, 0, st>>>(a);
+            else if (vec) row_reduce_kernel<Op, FULL><<<grid, block, 0, st>>>(a);
             else row_reduce_kernel<Op, 1><<<grid, block, 0, st>>>(a);
         }
         if (p.split > 1)

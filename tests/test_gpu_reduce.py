@@ -358,6 +358,47 @@ def test_long_rows_off_the_vector_grid(hpt, orc, dev):
         assert int(t.argmax(0).numpy()) == pos and float(t.max([0]).numpy()) == 7.0 and float(t.sum([0]).numpy()) == 7.0
 
 
+def test_short_runs_off_the_vector_grid(hpt, orc, dev):
+    """Contiguous runs that are not whole, aligned vectors and too short to peel (the batch-norm sums of
+    [N, C, 7, 7]: runs of 49; rows of 103 at an odd pitch): unaligned 128-bit loads, the last vector of
+    a run taken from its end backwards with the shared elements skipped. Runs barely longer than a
+    vector, exactly one vector, and ties for the index rule."""
+    rng = np.random.default_rng(122)
+    for shape, view, axes, npdt in (((64, 96, 7, 7), (), [0, 2, 3], np.float32), ((64, 96, 7, 7), (), [0, 2, 3], np.float16),
+                                    ((40, 30, 14, 14), (), [0, 2, 3], np.float16), ((33, 17, 5, 3), (), [0, 2, 3], np.int32),
+                                    ((16, 8, 57, 57), (), [0, 2, 3], np.uint8), ((300, 103), (), [1], np.float32),
+                                    ((300, 120), (("slice", ((0, 300, 1), (3, 106, 1))),), [1], np.int16),
+                                    ((5000, 17), (("slice", ((0, 5000, 1), (1, 17, 1))),), [1], np.uint8),
+                                    ((9, 4, 6, 9), (), [1, 3], np.float32), ((12, 5, 3, 2, 11), (), [0, 2, 4], np.float64),
+                                    ((50, 9), (), [1], np.float16), ((50, 8), (("slice", ((0, 50, 1), (0, 8, 1))),), [1], np.float16)):
+        if np.issubdtype(npdt, np.floating):
+            base = rng.standard_normal(shape).astype(npdt)
+        else:
+            base = rng.integers(0, 40, shape).astype(npdt)   # many ties
+        t, a = upload(hpt, base, view, dev=dev)
+        tag = f"{np.dtype(npdt).name} {shape} {view} {axes}"
+        plan = hpt.reduce_plan(t, hpt.SUM, axes)
+        if (shape, view) != ((50, 8), (("slice", ((0, 50, 1), (0, 8, 1))),)):
+            assert "-unaligned" in plan and plan.startswith("row"), plan
+        assert np.array_equal(t.max(axes).numpy(), orc.reduce(orc.MAX, a, axes)), tag
+        assert np.array_equal(t.min(axes).numpy(), orc.reduce(orc.MIN, a, axes)), tag
+        if len(axes) == 1:
+            assert np.array_equal(t.argmax(axes[0]).numpy(), orc.argreduce(True, a, axes[0])), tag
+            assert np.array_equal(t.argmin(axes[0]).numpy(), orc.argreduce(False, a, axes[0])), tag
+        if npdt == np.float16:
+            want = orc.reduce(orc.SUM, a, axes, acc=orc.ACC_F32).astype(np.float32)
+            assert_close(t.sum(axes).numpy().astype(np.float32), want, HALF_RTOL, half_atol(want, 11), tag)
+        elif np.issubdtype(npdt, np.floating):
+            assert_close(t.sum(axes).numpy(), orc.reduce(orc.SUM, a, axes, acc=orc.ACC_F64), F32_RTOL, 2e-5, tag)
+            assert_close(t.mean(axes).numpy(), a.astype(np.float64).mean(tuple(axes)), F32_RTOL, F32_ATOL, tag)
+        else:
+            assert np.array_equal(t.sum(axes).numpy(), orc.reduce(orc.SUM, a, axes)), tag
+    # a view that ends on the buffer's last element: the last vector must not reach past it
+    x = rng.integers(0, 9, (64, 3, 7, 7)).astype(np.int32)
+    t, a = upload(hpt, x, dev=dev)
+    assert np.array_equal(t.sum([0, 2, 3]).numpy(), orc.reduce(orc.SUM, a, [0, 2, 3]))
+
+
 def test_reduction_over_the_last_axis_of_a_permuted_view(hpt, orc, dev):
     """x.permute(2, 1, 0).sum(2): the first kept dim is the contiguous one. The lanes run along it and
     the outputs are scattered (one launch, and the two-stage form with its second-stage remap)."""

@@ -139,10 +139,13 @@ def test_plans_for_the_benchmark_configurations(hpt):
     assert hpt.normalize_plan(c5[:, ::2], 1).startswith("rowreg-step2") and "norm_in=[64:2]" in hpt.normalize_plan(c5[:, ::2], 1)
     assert hpt.reduce_plan(c5[:, ::2], hpt.SUM, [0]).startswith("col-step2 vec=8")
     assert hpt.reduce_plan(c5[:, 1::2], hpt.SUM, [0]).startswith("col vec=1")   # odd start: vectors would be misaligned
-    # misaligned base pointer or odd row length: long rows peel their ends, short ones take scalar loads
+    # misaligned base pointer or odd row length: long rows peel their ends, shorter ones take unaligned
+    # vectors, rows shorter than a vector scalar loads
     assert hpt.reduce_plan(f32(7, 1023), hpt.SUM, [1]).startswith("row-ragged vec=4")
     assert hpt.reduce_plan(f32(8, 1024)[:, 1:], hpt.SUM, [1]).startswith("row-ragged vec=4")
-    assert hpt.reduce_plan(f32(7, 103), hpt.SUM, [1]).startswith("row vec=1")
+    assert hpt.reduce_plan(f32(7, 103), hpt.SUM, [1]).startswith("row-unaligned vec=4")
+    assert hpt.reduce_plan(f32(16, 8, 7, 7), hpt.SUM, [0, 2, 3]).startswith("row-general-unaligned vec=4")
+    assert hpt.reduce_plan(f32(7, 3), hpt.SUM, [1]).startswith("row vec=1")
 
 
 def test_coalescing_matches_brute_force_offsets(hpt):
