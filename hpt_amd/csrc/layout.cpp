@@ -580,14 +580,24 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             // Few, very long contiguous rows: share each row among workgroups. (One workgroup per
             // row would leave a chip of 256 compute units mostly idle.)
             if (sa == 1 && !p.shift && p.rows <= 128 && p.cols >= 16384 && p.cols % v == 0) {
-                const int64_t nvec = p.cols / v;
+                if (v == 1 && max_vec > 1 && ((uintptr_t)in_data % elem_size) == 0 && ((uintptr_t)out_data % elem_size) == 0) {
+                    // rows off the 16-byte grid: unaligned vectors, the last one from the row's end backwards
+                    v = max_vec;
+                    p.vec = v;
+                    p.shift = 1;
+                }
+                const int64_t nvec = (p.cols + v - 1) / v;
                 int64_t S = std::min<int64_t>(512, std::max<int64_t>(1, 1024 / p.rows));
                 S = std::min<int64_t>(S, std::max<int64_t>(1, nvec / 1024));  // at least 4 vectors per thread
                 if (S >= 2) {
                     p.kind = NormKind::RowSplit;
                     p.tsplit = (int)S;
-                    p.scratch_bytes = (size_t)p.rows * S * 16 + (size_t)p.rows * 3 * 8;
+                    p.scratch_bytes = (size_t)p.rows * S * 16;
                     return p;
+                }
+                if (p.shift) {  // not worth splitting: back to element-wise rows
+                    p.shift = 0;
+                    p.vec = v = 1;
                 }
             }
             // A row fits the registers of a workgroup up to 8 vectors per thread; layernorm also keeps
@@ -762,7 +772,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? "-shift" : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : "")))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? (p.kind == NormKind::RowSplit ? "-unaligned" : "-shift") : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : "")))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     describe_dims(s, "rows_in", p.kept_in);

@@ -915,9 +915,8 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
 // units (a batch of 32 rows of 131072 logits). Here S workgroups take a slice of the row each:
 //   row_split_stats_kernel     partial statistics of a slice: softmax (max, sum of exp(x - max)),
 //                              layernorm sums of (x - k), (x - k)^2 with k the row's first element
-//   row_split_finalize_kernel  folds the S partials of a row into (max, 1/sum or ln sum) or
-//                              (mean_hi, mean_lo, rstd)
-//   row_split_apply_kernel     re-reads the slice and writes the result
+//   row_split_apply_kernel     folds the S partials of its row into (max, 1/sum or ln sum) or
+//                              (mean_hi, mean_lo, rstd), re-reads the slice and writes the result
 // Input rows are contiguous along the axis (any row offsets), the output is contiguous.
 struct RowSplitArgs {
     const void* in;
@@ -926,7 +925,6 @@ struct RowSplitArgs {
     const void* beta;
     const void* residual;  // NORM_ADD_LAYERNORM
     void* part;            // [rows][S] partials (16 bytes each at most)
-    void* params;          // [rows][3] numbers for the last pass
     Dims kept_in;
     int64_t rows, cols;
     int64_t chunk_v;       // vectors per slice
@@ -941,36 +939,55 @@ template <class ST> struct SumPairOp {
     __device__ static __forceinline__ SumPair<ST> comb(SumPair<ST> x, SumPair<ST> y) { return SumPair<ST>{x.a + y.a, x.b + y.b}; }
 };
 
-// element `j` of vector `iv` of a row, with the residual added where the kind says so
-template <int KIND, class T, int VEC>
-__device__ __forceinline__ void row_split_load(const RowSplitArgs& a, const T* in_row, int64_t row, int64_t iv,
+// UA: rows whose length or start is off the 16-byte grid. The vectors are unaligned, and a row's last
+// vector is taken from the row's end backwards: it shares its first `skip` elements with the vector
+// before (the statistics leave them out, the last pass does not store them).
+template <int VEC, bool UA> __device__ __forceinline__ int64_t row_split_vectors(int64_t cols) {
+    return UA ? (cols + VEC - 1) / VEC : cols / VEC;
+}
+template <int VEC, bool UA> __device__ __forceinline__ int64_t row_split_start(int64_t iv, int64_t cols) {
+    return UA ? min(iv * VEC, cols - VEC) : iv * VEC;
+}
+template <class T, int VEC, bool UA> __device__ __forceinline__ Pack<T, VEC> row_split_pack(const T* p) {
+    if constexpr (UA) return load_pack_unaligned<T, VEC>(p);
+    else return load_pack<T, VEC>(p);
+}
+
+// the VEC elements of a row from element e0 on, with the residual added where the kind says so
+template <int KIND, class T, int VEC, bool UA>
+__device__ __forceinline__ void row_split_load(const RowSplitArgs& a, const T* in_row, int64_t row, int64_t e0,
                                                typename Elem<T>::Wide (&x)[VEC]) {
-    using CT = typename Elem<T>::Wide;
-    const Pack<T, VEC> v = load_pack<T, VEC>(in_row + iv * VEC);
+    const Pack<T, VEC> v = row_split_pack<T, VEC, UA>(in_row + e0);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) x[j] = Elem<T>::widen(v.v[j]);
     if constexpr (KIND == NORM_ADD_LAYERNORM) {
-        const Pack<T, VEC> r = load_pack<T, VEC>((const T*)a.residual + row * a.cols + iv * VEC);
+        const Pack<T, VEC> r = row_split_pack<T, VEC, UA>((const T*)a.residual + row * a.cols + e0);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) x[j] = Elem<T>::widen(Elem<T>::narrow(x[j] + Elem<T>::widen(r.v[j])));
     }
-    (void)sizeof(CT);
 }
 
-template <int KIND, class T, int VEC>
+template <int KIND, class T, int VEC, bool UA>
 __global__ void __launch_bounds__(256) row_split_stats_kernel(const RowSplitArgs a) {
     using CT = typename Elem<T>::Wide;
     using ST = typename StatType<T>::type;
     __shared__ __align__(16) unsigned char smem_raw[16 * 2 * sizeof(double)];
     const int64_t row = blockIdx.y;
     const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
-    const int64_t nv = a.cols / VEC;
+    const int64_t nv = row_split_vectors<VEC, UA>(a.cols);
     const int64_t v0 = (int64_t)blockIdx.x * a.chunk_v, v1 = min(nv, v0 + a.chunk_v);
     if constexpr (!norm_is_layer(KIND)) {
         SoftStat<CT, ST> st{neg_inf<CT>(), (ST)0};
         for (int64_t iv = v0 + threadIdx.x; iv < v1; iv += 256) {
             CT x[VEC];
-            row_split_load<KIND, T, VEC>(a, in_row, row, iv, x);
+            const int64_t e0 = row_split_start<VEC, UA>(iv, a.cols);
+            row_split_load<KIND, T, VEC, UA>(a, in_row, row, e0, x);
+            if constexpr (UA) {
+                const int skip = (int)(iv * VEC - e0);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    if (j < skip) x[j] = neg_inf<CT>();
+            }
             CT cm = x[0];
 #pragma unroll
             for (int j = 1; j < VEC; ++j) cm = MaxC<CT>::comb(cm, x[j]);
@@ -992,16 +1009,18 @@ __global__ void __launch_bounds__(256) row_split_stats_kernel(const RowSplitArgs
         CT k;
         {
             CT x0[VEC];
-            row_split_load<KIND, T, VEC>(a, in_row, row, 0, x0);
+            row_split_load<KIND, T, VEC, UA>(a, in_row, row, 0, x0);
             k = x0[0];
         }
         CT s1 = 0, s2 = 0;
         for (int64_t iv = v0 + threadIdx.x; iv < v1; iv += 256) {
             CT x[VEC];
-            row_split_load<KIND, T, VEC>(a, in_row, row, iv, x);
+            const int64_t e0 = row_split_start<VEC, UA>(iv, a.cols);
+            row_split_load<KIND, T, VEC, UA>(a, in_row, row, e0, x);
+            const int skip = UA ? (int)(iv * VEC - e0) : 0;
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
-                const CT d = x[j] - k;
+                const CT d = (!UA || j >= skip) ? x[j] - k : (CT)0;
                 s1 += d;
                 s2 += d * d;
             }
@@ -1012,55 +1031,44 @@ __global__ void __launch_bounds__(256) row_split_stats_kernel(const RowSplitArgs
     }
 }
 
-// one wavefront per row folds its S partials
-template <int KIND, class T, int VEC>
-__global__ void __launch_bounds__(64) row_split_finalize_kernel(const RowSplitArgs a) {
-    using CT = typename Elem<T>::Wide;
-    using ST = typename StatType<T>::type;
-    const int64_t row = blockIdx.x;
-    const int lane = threadIdx.x;
-    CT* p = (CT*)a.params + row * 3;
-    if constexpr (!norm_is_layer(KIND)) {
-        SoftStat<CT, ST> st{neg_inf<CT>(), (ST)0};
-        for (int i = lane; i < a.S; i += 64) st = SoftStatOp<T, CT, ST>::comb(st, ((const SoftStat<CT, ST>*)a.part)[row * a.S + i]);
-        st = group_reduce<SoftStatOp<T, CT, ST>>(st, 64);
-        if (lane == 0) {
-            p[0] = st.m;
-            p[1] = norm_is_log(KIND) ? log_ct<T>((CT)st.s) : (CT)((ST)1 / st.s);
-            p[2] = 0;
-        }
-    } else {
-        SumPair<ST> sp{(ST)0, (ST)0};
-        for (int i = lane; i < a.S; i += 64) sp = SumPairOp<ST>::comb(sp, ((const SumPair<ST>*)a.part)[row * a.S + i]);
-        sp = group_reduce<SumPairOp<ST>>(sp, 64);
-        if (lane == 0) {
-            const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
-            CT x0[VEC];
-            row_split_load<KIND, T, VEC>(a, in_row, row, 0, x0);
-            const ST mean = (ST)x0[0] + sp.a * (ST)a.inv_cols;
-            ST m2 = sp.b - sp.a * sp.a * (ST)a.inv_cols;
-            if (m2 < (ST)0) m2 = 0;
-            const CT hi = (CT)mean;
-            p[0] = hi;
-            p[1] = (CT)(mean - (ST)hi);
-            p[2] = rsqrt_ct((CT)(m2 * (ST)a.inv_cols) + (CT)a.eps);
-        }
-    }
-}
-
-template <int KIND, class T, int VEC>
+// The last pass: every workgroup of a row folds the row's S partials itself (at most 512, in the same
+// order, so all of them arrive at the same bits; a launch of its own for that would cost more than the
+// few hundred loads), then re-reads its slice and writes the result.
+template <int KIND, class T, int VEC, bool UA>
 __global__ void __launch_bounds__(256) row_split_apply_kernel(const RowSplitArgs a) {
     using CT = typename Elem<T>::Wide;
+    using ST = typename StatType<T>::type;
+    __shared__ __align__(16) unsigned char smem_raw[16 * 2 * sizeof(double)];
     const int64_t row = blockIdx.y;
     const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
     T* out_row = (T*)a.out + row * a.cols;
-    const CT* p = (const CT*)a.params + row * 3;
-    const CT p0 = p[0], p1 = p[1], p2 = p[2];
-    const int64_t nv = a.cols / VEC;
+    CT p0, p1, p2;
+    if constexpr (!norm_is_layer(KIND)) {
+        SoftStat<CT, ST> st{neg_inf<CT>(), (ST)0};
+        for (int i = threadIdx.x; i < a.S; i += 256) st = SoftStatOp<T, CT, ST>::comb(st, ((const SoftStat<CT, ST>*)a.part)[row * a.S + i]);
+        st = block_reduce<SoftStatOp<T, CT, ST>>(st, (SoftStat<CT, ST>*)smem_raw);
+        p0 = st.m;
+        p1 = norm_is_log(KIND) ? log_ct<T>((CT)st.s) : (CT)((ST)1 / st.s);
+        p2 = 0;
+    } else {
+        SumPair<ST> sp{(ST)0, (ST)0};
+        for (int i = threadIdx.x; i < a.S; i += 256) sp = SumPairOp<ST>::comb(sp, ((const SumPair<ST>*)a.part)[row * a.S + i]);
+        sp = block_reduce<SumPairOp<ST>>(sp, (SumPair<ST>*)smem_raw);
+        CT x0[VEC];
+        row_split_load<KIND, T, VEC, UA>(a, in_row, row, 0, x0);
+        const ST mean = (ST)x0[0] + sp.a * (ST)a.inv_cols;
+        ST m2 = sp.b - sp.a * sp.a * (ST)a.inv_cols;
+        if (m2 < (ST)0) m2 = 0;
+        p0 = (CT)mean;
+        p1 = (CT)(mean - (ST)p0);
+        p2 = rsqrt_ct((CT)(m2 * (ST)a.inv_cols) + (CT)a.eps);
+    }
+    const int64_t nv = row_split_vectors<VEC, UA>(a.cols);
     const int64_t v0 = (int64_t)blockIdx.x * a.chunk_v, v1 = min(nv, v0 + a.chunk_v);
     for (int64_t iv = v0 + threadIdx.x; iv < v1; iv += 256) {
         CT x[VEC];
-        row_split_load<KIND, T, VEC>(a, in_row, row, iv, x);
+        const int64_t e0 = row_split_start<VEC, UA>(iv, a.cols);
+        row_split_load<KIND, T, VEC, UA>(a, in_row, row, e0, x);
         Pack<T, VEC> o;
         if constexpr (norm_is_layer(KIND)) {
             Pack<T, VEC> g, b;
@@ -1069,8 +1077,8 @@ __global__ void __launch_bounds__(256) row_split_apply_kernel(const RowSplitArgs
                 g.v[j] = Elem<T>::narrow((CT)1);
                 b.v[j] = Elem<T>::narrow((CT)0);
             }
-            if (a.gamma) g = load_pack<T, VEC>((const T*)a.gamma + iv * VEC);
-            if (a.beta) b = load_pack<T, VEC>((const T*)a.beta + iv * VEC);
+            if (a.gamma) g = row_split_pack<T, VEC, UA>((const T*)a.gamma + e0);
+            if (a.beta) b = row_split_pack<T, VEC, UA>((const T*)a.beta + e0);
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
                 o.v[j] = Elem<T>::narrow(((x[j] - p0) - p1) * p2 * Elem<T>::widen(g.v[j]) + Elem<T>::widen(b.v[j]));
@@ -1081,8 +1089,17 @@ __global__ void __launch_bounds__(256) row_split_apply_kernel(const RowSplitArgs
                 o.v[j] = Elem<T>::narrow(norm_is_log(KIND) ? d - p1 : exp_ct<T>(d) * p1);
             }
         }
-        if constexpr (VEC > 1) store_pack_stream<T, VEC>(out_row + iv * VEC, o);
-        else out_row[iv] = o.v[0];
+        if constexpr (UA) {
+            const int skip = (int)(iv * VEC - e0);
+            if (skip == 0) {
+                store_pack_unaligned<T, VEC>(out_row + e0, o);
+            } else {  // the row's last vector: only the elements that are its own
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    if (j >= skip) out_row[e0 + j] = o.v[j];
+            }
+        } else if constexpr (VEC > 1) store_pack_stream<T, VEC>(out_row + e0, o);
+        else out_row[e0] = o.v[0];
     }
 }
 

@@ -32,7 +32,7 @@ void launch_row_reg(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block,
 }
 
 // Few, very long rows: several workgroups per row.
-template <class T, int VEC> void launch_row_split(const NormPlan& p, const NormArgs& a, hipStream_t st) {
+template <class T, int VEC, bool UA> void launch_row_split(const NormPlan& p, const NormArgs& a, hipStream_t st) {
     RowSplitArgs r{};
     r.in = a.in;
     r.out = a.out;
@@ -45,14 +45,12 @@ template <class T, int VEC> void launch_row_split(const NormPlan& p, const NormA
     r.eps = a.eps;
     r.inv_cols = a.inv_cols;
     r.S = p.tsplit;
-    const int64_t nv = a.cols / VEC;
+    const int64_t nv = UA ? (a.cols + VEC - 1) / VEC : a.cols / VEC;
     r.chunk_v = (nv + r.S - 1) / r.S;
     r.part = a.scratch;
-    r.params = (char*)a.scratch + (size_t)a.rows * r.S * 16;
     const dim3 grid((unsigned)r.S, (unsigned)a.rows);
-    row_split_stats_kernel<KIND, T, VEC><<<grid, dim3(256), 0, st>>>(r);
-    row_split_finalize_kernel<KIND, T, VEC><<<dim3((unsigned)a.rows), dim3(64), 0, st>>>(r);
-    row_split_apply_kernel<KIND, T, VEC><<<grid, dim3(256), 0, st>>>(r);
+    row_split_stats_kernel<KIND, T, VEC, UA><<<grid, dim3(256), 0, st>>>(r);
+    row_split_apply_kernel<KIND, T, VEC, UA><<<grid, dim3(256), 0, st>>>(r);
 }
 
 // Softmax / log_softmax over an axis that is strided in the output too: three passes.
@@ -192,8 +190,9 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         if constexpr (norm_is_causal(KIND)) {
             fail(HPT_ERR_KERNEL, "row-split has no causal form");
         } else {
-            if (p.vec == FULL && FULL > 1) launch_row_split<T, FULL>(p, a, st);
-            else launch_row_split<T, 1>(p, a, st);
+            if (p.vec == FULL && FULL > 1 && p.shift) launch_row_split<T, FULL, true>(p, a, st);
+            else if (p.vec == FULL && FULL > 1) launch_row_split<T, FULL, false>(p, a, st);
+            else launch_row_split<T, 1, false>(p, a, st);
         }
         return;
     }

@@ -261,7 +261,11 @@ def test_log_softmax_long_columns_keep_the_absolute_tolerance(hpt, orc, dev):
 ROW_SPLIT_CASES = [
     ("a decode batch of logits", np.float32, [32, 131072], ()),
     ("one row", np.float32, [1, 65544], ()),
-    ("odd length: one element per access", np.float32, [7, 20001], ()),
+    ("odd length: unaligned vectors, the last one from the row's end", np.float32, [7, 20001], ()),
+    ("odd length, f16 (vocabulary of 50257)", np.float16, [32, 50257], ()),
+    ("odd length, bf16, one row", "bf16", [1, 128257], ()),
+    ("rows at an odd offset of a wider buffer", np.float32, [6, 70001], (("slice", ((1, 6, 1), (3, 65539, 1))),)),
+    ("f64 odd length", np.float64, [3, 100003], ()),
     ("rows of a wider buffer", np.float32, [12, 40000], (("slice", ((1, 11, 1), (64, 32832, 1))),)),
     ("f64", np.float64, [5, 33000], ()),
     ("f16", np.float16, [16, 65536], ()),
