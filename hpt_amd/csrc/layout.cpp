@@ -561,6 +561,19 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     if (((p.kept_in.stride[i] - p.kept_out.stride[i]) * (int64_t)elem_size) % 16 != 0) same = false;
                 const int64_t nvs = (p.cols + 2 * (max_vec - 1)) / max_vec;
                 // (two-byte layernorm keeps two vectors per thread: beyond 512 threads per row it only loses)
+                if (same && n_norm_dims <= 0 && elem_size == 2 && nvs > 4096 && nvs <= 8192) {
+                    // two-byte softmax rows of 32769 ... 65521 elements (a vocabulary of 50257): the raw row
+                    // in registers (see below), f16 [4096, 50257] log_softmax 3.1 -> 4.0 TB/s. The
+                    // sixteen-vector form spills with the masks of the shifted walk and only matches streaming.
+                    p.kind = NormKind::RowReg;
+                    p.raw_rows = 1;
+                    p.vec = max_vec;
+                    p.shift = 1;
+                    p.tpr = 1024;
+                    p.rpb = 1;
+                    p.nchunk = 8;
+                    return p;
+                }
                 if (same && nvs > ((n_norm_dims > 0 && elem_size == 2) ? 512 : 2048)) {
                     p.kind = NormKind::RowStream;
                     p.vec = max_vec;
@@ -772,7 +785,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? (p.kind == NormKind::RowSplit ? "-unaligned" : "-shift") : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : "")))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? (p.kind == NormKind::RowSplit ? "-unaligned" : (p.raw_rows ? "-raw-shift" : "-shift")) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : "")))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     describe_dims(s, "rows_in", p.kept_in);

@@ -389,7 +389,10 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
 // write where the streaming kernel reads twice.
 // PF (eight vectors per thread): the next row's loads are issued before the current row's sweeps;
 // there is one workgroup per compute unit, so nothing else hides a row's load -> sweeps -> store chain.
-template <int KIND, class T, int NCHUNK, bool PF = false>
+// SHIFT: rows that start off 16-byte boundaries (a vocabulary of 50257): a row is covered by the
+// aligned vectors that contain it, as in row_reg_kernel; positions outside the row count as -inf and
+// the two end vectors are stored element by element. Input and output rows share their misalignment.
+template <int KIND, class T, int NCHUNK, bool PF = false, bool SHIFT = false>
 __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
     static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX, "a softmax kernel");
     constexpr int VEC = 16 / sizeof(T);
@@ -397,7 +400,10 @@ __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
     using CT = typename Elem<T>::Wide;
     __shared__ CT smem[16];
     const int tx = threadIdx.x;
-    const int nv = (int)(a.cols / VEC);
+    const int cols = (int)a.cols;
+    auto shift_of = [](const T* p) -> int { return SHIFT ? (int)(((uintptr_t)p / sizeof(T)) % VEC) : 0; };
+    // vectors that cover a row which starts sh elements after a 16-byte boundary
+    auto vectors = [&](int sh) -> int { return SHIFT ? (cols + sh + VEC - 1) / VEC : cols / VEC; };
     Pack<T, VEC> raw[NCHUNK], nxt[PF ? NCHUNK : 1];
     // (2-byte types: keep the compiler from holding the widened copies of one sweep for the next)
     auto forget = [](Pack<T, VEC>& v) {
@@ -406,23 +412,41 @@ __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
     auto fetch = [&](Pack<T, VEC>* dst, int64_t row) {
         if (row >= a.rows) return;
         const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
+        const int sh = shift_of(in_row);
+        const int nv = vectors(sh);
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int iv = c * 1024 + tx;
-            if (iv < nv) dst[c] = load_pack_stream<T, VEC>(in_row + (int64_t)iv * VEC);
+            if (iv < nv) dst[c] = load_pack_stream<T, VEC>(in_row - sh + (int64_t)iv * VEC);
         }
     };
     if constexpr (PF) fetch(raw, blockIdx.x);
     for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
         T* out_row = (T*)a.out + row * a.cols;
+        const int sh = shift_of(out_row);
+        const int nv = vectors(sh);
         if constexpr (PF) fetch(nxt, row + gridDim.x);
         else fetch(raw, row);
+        if constexpr (SHIFT) {
+            // the row's two end vectors: positions outside the row become -inf once, here, and the
+            // sweeps below need no masks
+#pragma unroll
+            for (int c = 0; c < NCHUNK; ++c) {
+                const int iv = c * 1024 + tx;
+                if (iv == 0 || iv == nv - 1) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        if ((unsigned)(iv * VEC + j - sh) >= (unsigned)cols) raw[c].v[j] = Elem<T>::narrow(neg_inf<CT>());
+                }
+            }
+        }
+        auto elem = [&](const Pack<T, VEC>& v, int, int j) -> CT { return Elem<T>::widen(v.v[j]); };
         CT m = neg_inf<CT>();
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c)
             if (c * 1024 + tx < nv)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, Elem<T>::widen(raw[c].v[j]));
+                for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, elem(raw[c], c * 1024 + tx, j));
         m = row_all_reduce<MaxC<CT>>(m, 1024, 0, smem);
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) forget(raw[c]);
@@ -431,7 +455,7 @@ __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
         for (int c = 0; c < NCHUNK; ++c)
             if (c * 1024 + tx < nv)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) s += exp_ct<T>(Elem<T>::widen(raw[c].v[j]) - m);
+                for (int j = 0; j < VEC; ++j) s += exp_ct<T>(elem(raw[c], c * 1024 + tx, j) - m);
         s = row_all_reduce<SumC<CT>>(s, 1024, 0, smem);
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) forget(raw[c]);
@@ -446,7 +470,14 @@ __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
                     const CT d = Elem<T>::widen(raw[c].v[j]) - m;
                     o.v[j] = Elem<T>::narrow(kLog ? d - k : exp_ct<T>(d) * k);
                 }
-                store_pack_stream<T, VEC>(out_row + (int64_t)iv * VEC, o);
+                const int e0 = iv * VEC - sh;
+                if (!SHIFT || (e0 >= 0 && e0 + VEC <= cols)) {
+                    store_pack_stream<T, VEC>(out_row + e0, o);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        if ((unsigned)(e0 + j) < (unsigned)cols) out_row[e0 + j] = o.v[j];
+                }
             }
         }
         if constexpr (PF) {

@@ -230,8 +230,15 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         // per thread) or take the ordinary register kernel (eight)
         if constexpr (sizeof(T) == 2 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX)) {
             if (grid.x > 512u) grid.x = 512u;
-            if (p.nchunk == 16) row_raw_kernel<KIND, T, 16><<<grid, dim3(1024), 0, st>>>(a);
-            else row_raw_kernel<KIND, T, 8, true><<<grid, dim3(1024), 0, st>>>(a);
+            if (p.shift) {
+                row_raw_kernel<KIND, T, 8, true, true><<<grid, dim3(1024), 0, st>>>(a);
+            } else {
+                if (p.nchunk == 16) row_raw_kernel<KIND, T, 16><<<grid, dim3(1024), 0, st>>>(a);
+                else row_raw_kernel<KIND, T, 8, true><<<grid, dim3(1024), 0, st>>>(a);
+            }
+            return;
+        } else if (p.shift) {  // the fused kinds stream shifted rows this long
+            if constexpr (FULL > 1) row_stream_kernel<KIND, T, FULL, true><<<grid, block, 0, st>>>(a);
             return;
         } else if (p.nchunk > 8) {
             if (p.vec == FULL) row_stream_kernel<KIND, T, FULL><<<grid, block, 0, st>>>(a);

@@ -326,6 +326,10 @@ WIDE_ROW_CASES = [
     ("f16 rows of 197", np.float16, [30011, 197]),
     ("f32 rows of 257 in a 3-D tensor", np.float32, [7, 1500, 257]),
     ("bf16 rows of 10001", "bf16", [700, 10001]),
+    # odd lengths of two-byte rows beyond 32768: the raw row in registers over aligned vectors, masked ends
+    ("f16 rows of 50257: raw row, eight vectors per thread, shifted", np.float16, [523, 50257]),
+    ("bf16 rows of 65521: the longest shifted raw row", "bf16", [517, 65521]),
+    ("f16 rows of 65537: streamed again", np.float16, [130, 65537]),
 ]
 
 
