@@ -574,6 +574,17 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     p.nchunk = 8;
                     return p;
                 }
+                if (same && n_norm_dims <= 0 && elem_size == 4 && nvs > 8192 && nvs <= 16384) {
+                    // four-byte softmax rows of 32769 ... 65530 elements: registers and LDS (see below)
+                    p.kind = NormKind::RowReg;
+                    p.lds_rows = 1;
+                    p.vec = max_vec;
+                    p.shift = 1;
+                    p.tpr = 1024;
+                    p.rpb = 1;
+                    p.nchunk = 16;
+                    return p;
+                }
                 if (same && nvs > ((n_norm_dims > 0 && elem_size == 2) ? 512 : 2048)) {
                     p.kind = NormKind::RowStream;
                     p.vec = max_vec;
@@ -639,6 +650,16 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 p.tpr = 1024;
                 p.rpb = 1;
                 p.nchunk = nv > 8192 ? 16 : 8;
+                return p;
+            }
+            // Four-byte softmax rows of 32769 ... 65536 elements: eight vectors per thread in registers and
+            // up to eight more in LDS, one read instead of the streaming kernel's two.
+            if (n_norm_dims <= 0 && elem_size == 4 && v == max_vec && p.sstride == 1 && !p.shift && nv > 8192 && nv <= 16384) {
+                p.kind = NormKind::RowReg;
+                p.lds_rows = 1;
+                p.tpr = 1024;
+                p.rpb = 1;
+                p.nchunk = 16;
                 return p;
             }
             if (nv <= reg_limit) {
@@ -768,6 +789,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
 void demote_to_generic(NormPlan& p) {
     p.kind = NormKind::Generic;
     p.raw_rows = 0;
+    p.lds_rows = 0;
     p.gb_lds = 0;
     p.tile_rows = 0;
     p.flat_t = 0;
@@ -785,7 +807,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? (p.kind == NormKind::RowSplit ? "-unaligned" : (p.raw_rows ? "-raw-shift" : "-shift")) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : "")))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? (p.kind == NormKind::RowSplit ? "-unaligned" : (p.raw_rows ? "-raw-shift" : (p.lds_rows ? "-lds-shift" : "-shift"))) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     describe_dims(s, "rows_in", p.kept_in);

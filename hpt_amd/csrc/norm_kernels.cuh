@@ -487,6 +487,130 @@ __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
     }
 }
 
+// ---- long rows of 4-byte elements: the row in registers AND LDS ------------------------------
+// softmax / log_softmax over f32 rows of 32769 ... 65536 elements (logits of a 50257 / 50304 / 65536
+// vocabulary in f32). Eight vectors per thread live in registers, up to eight more in LDS (128 KiB
+// of the compute unit's 160; every thread reads back only the slots it wrote, so the LDS part needs
+// no barrier: it is a second register file). One HBM read and one write where the streaming
+// kernel reads twice. The summing sweep overwrites the held row with exp(x - max) (softmax) or
+// x - max (log_softmax), so the exponential is taken once per element either way.
+// SHIFT: as in row_raw_kernel.
+template <int KIND, class T, bool SHIFT = false>
+__global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
+    static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX, "a softmax kernel");
+    static_assert(sizeof(T) == 4, "rows of 4-byte elements");
+    constexpr int VEC = 4, NREG = 8, NLDS = 8;
+    constexpr bool kLog = KIND == NORM_LOGSOFTMAX;
+    using CT = typename Elem<T>::Wide;
+    __shared__ CT smem[16];
+    __shared__ __align__(16) unsigned char lds_raw[NLDS * 1024 * 16];
+    Pack<T, VEC>* lds = reinterpret_cast<Pack<T, VEC>*>(lds_raw);
+    const int tx = threadIdx.x;
+    const int cols = (int)a.cols;
+    auto shift_of = [](const T* p) -> int { return SHIFT ? (int)(((uintptr_t)p / sizeof(T)) % VEC) : 0; };
+    for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
+        const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
+        T* out_row = (T*)a.out + row * a.cols;
+        const int sh = shift_of(out_row);
+        const int nv = SHIFT ? (cols + sh + VEC - 1) / VEC : cols / VEC;
+        auto mask_ends = [&](Pack<T, VEC>& v, int iv) {
+            if constexpr (SHIFT) {
+                if (iv == 0 || iv == nv - 1) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        if ((unsigned)(iv * VEC + j - sh) >= (unsigned)cols) v.v[j] = Elem<T>::narrow(neg_inf<CT>());
+                }
+            }
+        };
+        Pack<T, VEC> reg[NREG];
+        {
+            Pack<T, VEC> tmp[NLDS];
+#pragma unroll
+            for (int c = 0; c < NLDS; ++c) {
+                const int iv = (NREG + c) * 1024 + tx;
+                if (iv < nv) tmp[c] = load_pack_stream<T, VEC>(in_row - sh + (int64_t)iv * VEC);
+            }
+#pragma unroll
+            for (int c = 0; c < NREG; ++c) {
+                const int iv = c * 1024 + tx;
+                if (iv < nv) reg[c] = load_pack_stream<T, VEC>(in_row - sh + (int64_t)iv * VEC);
+            }
+#pragma unroll
+            for (int c = 0; c < NLDS; ++c) {
+                const int iv = (NREG + c) * 1024 + tx;
+                if (iv < nv) {
+                    mask_ends(tmp[c], iv);
+                    lds[c * 1024 + tx] = tmp[c];
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < NREG; ++c) mask_ends(reg[c], c * 1024 + tx);
+        CT m = neg_inf<CT>();
+#pragma unroll
+        for (int c = 0; c < NREG; ++c)
+            if (c * 1024 + tx < nv)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, Elem<T>::widen(reg[c].v[j]));
+#pragma unroll
+        for (int c = 0; c < NLDS; ++c)
+            if ((NREG + c) * 1024 + tx < nv) {
+                const Pack<T, VEC> v = lds[c * 1024 + tx];
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, Elem<T>::widen(v.v[j]));
+            }
+        m = row_all_reduce<MaxC<CT>>(m, 1024, 0, smem);
+        CT s = 0;
+#pragma unroll
+        for (int c = 0; c < NREG; ++c)
+            if (c * 1024 + tx < nv)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const CT d = Elem<T>::widen(reg[c].v[j]) - m;
+                    const CT e = exp_ct<T>(d);
+                    s += e;
+                    reg[c].v[j] = Elem<T>::narrow(kLog ? d : e);
+                }
+#pragma unroll
+        for (int c = 0; c < NLDS; ++c)
+            if ((NREG + c) * 1024 + tx < nv) {
+                Pack<T, VEC> v = lds[c * 1024 + tx];
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const CT d = Elem<T>::widen(v.v[j]) - m;
+                    const CT e = exp_ct<T>(d);
+                    s += e;
+                    v.v[j] = Elem<T>::narrow(kLog ? d : e);
+                }
+                lds[c * 1024 + tx] = v;
+            }
+        s = row_all_reduce<SumC<CT>>(s, 1024, 0, smem);
+        const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
+        auto finish = [&](Pack<T, VEC> v, int iv) {
+            Pack<T, VEC> o;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const CT x = Elem<T>::widen(v.v[j]);
+                o.v[j] = Elem<T>::narrow(kLog ? x - k : x * k);
+            }
+            const int e0 = iv * VEC - sh;
+            if (!SHIFT || (e0 >= 0 && e0 + VEC <= cols)) {
+                store_pack_stream<T, VEC>(out_row + e0, o);
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    if ((unsigned)(e0 + j) < (unsigned)cols) out_row[e0 + j] = o.v[j];
+            }
+        };
+#pragma unroll
+        for (int c = 0; c < NREG; ++c)
+            if (c * 1024 + tx < nv) finish(reg[c], c * 1024 + tx);
+#pragma unroll
+        for (int c = 0; c < NLDS; ++c)
+            if ((NREG + c) * 1024 + tx < nv) finish(lds[c * 1024 + tx], (NREG + c) * 1024 + tx);
+    }
+}
+
 // ---- short rows laid back to back: whole tiles through LDS ---------------------------------
 // A contiguous [rows, cols] matrix with short rows (cols <= 512): a workgroup brings a.rpb
 // consecutive rows (16 KiB; a multiple of VEC rows, so the tile starts on a 16-byte boundary

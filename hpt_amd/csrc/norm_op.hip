@@ -225,6 +225,17 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         else launch_transposed<T>(p, a, st);
         return;
     }
+    if (p.kind == NormKind::RowReg && p.lds_rows) {
+        // long four-byte softmax rows: registers + LDS; the fused kinds stream
+        if constexpr (sizeof(T) == 4 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX)) {
+            if (p.shift) row_lds_kernel<KIND, T, true><<<grid, dim3(1024), 0, st>>>(a);
+            else row_lds_kernel<KIND, T, false><<<grid, dim3(1024), 0, st>>>(a);
+        } else if constexpr (FULL > 1) {
+            if (p.shift) row_stream_kernel<KIND, T, FULL, true><<<grid, block, 0, st>>>(a);
+            else row_stream_kernel<KIND, T, FULL><<<grid, block, 0, st>>>(a);
+        }
+        return;
+    }
     if (p.kind == NormKind::RowReg && p.raw_rows) {
         // long two-byte softmax rows: the raw row in registers; the fused kinds stream (sixteen vectors
         // per thread) or take the ordinary register kernel (eight)

@@ -326,6 +326,12 @@ WIDE_ROW_CASES = [
     ("f16 rows of 197", np.float16, [30011, 197]),
     ("f32 rows of 257 in a 3-D tensor", np.float32, [7, 1500, 257]),
     ("bf16 rows of 10001", "bf16", [700, 10001]),
+    # f32 rows of 32769 ... 65536: half the row in registers, half in LDS; odd lengths shifted
+    ("f32 rows of 50304: registers and LDS", np.float32, [300, 50304]),
+    ("f32 rows of 50257: registers and LDS, shifted", np.float32, [270, 50257]),
+    ("f32 rows of 65536: every LDS slot in use", np.float32, [140, 65536]),
+    ("f32 rows of 32772: one vector beyond the registers", np.float32, [200, 32772]),
+    ("f32 rows of 65530: the longest shifted row", np.float32, [131, 65530]),
     # odd lengths of two-byte rows beyond 32768: the raw row in registers over aligned vectors, masked ends
     ("f16 rows of 50257: raw row, eight vectors per thread, shifted", np.float16, [523, 50257]),
     ("bf16 rows of 65521: the longest shifted raw row", "bf16", [517, 65521]),
