@@ -574,8 +574,9 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     p.nchunk = 8;
                     return p;
                 }
-                if (same && n_norm_dims <= 0 && elem_size == 4 && nvs > 8192 && nvs <= 16384) {
-                    // four-byte softmax rows of 32769 ... 65530 elements: registers and LDS (see below)
+                if (same && n_norm_dims <= 0 && elem_size == 4 && nvs > 8192 && p.cols <= 65536 - 34) {
+                    // four-byte softmax rows of 32769 ... 65502 elements: registers and LDS (see below; the
+                    // kernel's vector grid starts up to 31 elements before the row)
                     p.kind = NormKind::RowReg;
                     p.lds_rows = 1;
                     p.vec = max_vec;

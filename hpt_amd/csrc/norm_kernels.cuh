@@ -505,9 +505,13 @@ __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
     __shared__ CT smem[16];
     __shared__ __align__(16) unsigned char lds_raw[NLDS * 1024 * 16];
     Pack<T, VEC>* lds = reinterpret_cast<Pack<T, VEC>*>(lds_raw);
+    __shared__ Pack<T, VEC> ends[SHIFT ? 2 : 1];
     const int tx = threadIdx.x;
     const int cols = (int)a.cols;
-    auto shift_of = [](const T* p) -> int { return SHIFT ? (int)(((uintptr_t)p / sizeof(T)) % VEC) : 0; };
+    // SHIFT: the vector grid starts on the 128-byte line that holds the row's first element, so a
+    // wavefront's 1 KiB of loads or stores covers eight whole lines, not nine partial ones
+    constexpr int LINE = 128 / sizeof(T);
+    auto shift_of = [](const T* p) -> int { return SHIFT ? (int)(((uintptr_t)p / sizeof(T)) % LINE) : 0; };
     for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
         const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
         T* out_row = (T*)a.out + row * a.cols;
@@ -515,25 +519,28 @@ __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
         const int nv = SHIFT ? (cols + sh + VEC - 1) / VEC : cols / VEC;
         auto mask_ends = [&](Pack<T, VEC>& v, int iv) {
             if constexpr (SHIFT) {
-                if (iv == 0 || iv == nv - 1) {
+                if (iv * VEC < sh || iv == nv - 1) {
 #pragma unroll
                     for (int j = 0; j < VEC; ++j)
                         if ((unsigned)(iv * VEC + j - sh) >= (unsigned)cols) v.v[j] = Elem<T>::narrow(neg_inf<CT>());
                 }
             }
         };
+        // (a vector that lies wholly before the row is not loaded: only a vector that holds an element of
+        // the row is sure to stay on that element's page)
+        auto touches = [&](int iv) { return !SHIFT || (iv + 1) * VEC > sh; };
         Pack<T, VEC> reg[NREG];
         {
             Pack<T, VEC> tmp[NLDS];
 #pragma unroll
             for (int c = 0; c < NLDS; ++c) {
                 const int iv = (NREG + c) * 1024 + tx;
-                if (iv < nv) tmp[c] = load_pack_stream<T, VEC>(in_row - sh + (int64_t)iv * VEC);
+                if (iv < nv && touches(iv)) tmp[c] = load_pack_stream<T, VEC>(in_row - sh + (int64_t)iv * VEC);
             }
 #pragma unroll
             for (int c = 0; c < NREG; ++c) {
                 const int iv = c * 1024 + tx;
-                if (iv < nv) reg[c] = load_pack_stream<T, VEC>(in_row - sh + (int64_t)iv * VEC);
+                if (iv < nv && touches(iv)) reg[c] = load_pack_stream<T, VEC>(in_row - sh + (int64_t)iv * VEC);
             }
 #pragma unroll
             for (int c = 0; c < NLDS; ++c) {
@@ -594,13 +601,8 @@ __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
                 o.v[j] = Elem<T>::narrow(kLog ? x - k : x * k);
             }
             const int e0 = iv * VEC - sh;
-            if (!SHIFT || (e0 >= 0 && e0 + VEC <= cols)) {
-                store_pack_stream<T, VEC>(out_row + e0, o);
-            } else {
-#pragma unroll
-                for (int j = 0; j < VEC; ++j)
-                    if ((unsigned)(e0 + j) < (unsigned)cols) out_row[e0 + j] = o.v[j];
-            }
+            if (!SHIFT || (e0 >= 0 && e0 + VEC <= cols)) store_pack_stream<T, VEC>(out_row + e0, o);
+            else if (e0 + VEC > 0) ends[e0 < 0 ? 0 : 1] = o;  // the row's two end vectors leave element by element below
         };
 #pragma unroll
         for (int c = 0; c < NREG; ++c)
@@ -608,6 +610,16 @@ __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
 #pragma unroll
         for (int c = 0; c < NLDS; ++c)
             if ((NREG + c) * 1024 + tx < nv) finish(lds[c * 1024 + tx], (NREG + c) * 1024 + tx);
+        if constexpr (SHIFT) {
+            __syncthreads();
+            if (tx < 2 * VEC) {
+                const int which = tx / VEC, j = tx % VEC;
+                const int e = (which == 0 ? sh / VEC : nv - 1) * VEC - sh + j;
+                const bool partial = which == 0 ? sh % VEC != 0 : nv * VEC - sh > cols;
+                if (partial && (unsigned)e < (unsigned)cols) out_row[e] = ends[which].v[j];
+            }
+            __syncthreads();  // before the next row's end vectors
+        }
     }
 }
 

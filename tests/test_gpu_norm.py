@@ -331,7 +331,8 @@ WIDE_ROW_CASES = [
     ("f32 rows of 50257: registers and LDS, shifted", np.float32, [270, 50257]),
     ("f32 rows of 65536: every LDS slot in use", np.float32, [140, 65536]),
     ("f32 rows of 32772: one vector beyond the registers", np.float32, [200, 32772]),
-    ("f32 rows of 65530: the longest shifted row", np.float32, [131, 65530]),
+    ("f32 rows of 65501: the longest shifted row", np.float32, [131, 65501]),
+    ("f32 rows of 32771 in a view that starts 29 elements into a line", np.float32, [135, 32771]),
     # odd lengths of two-byte rows beyond 32768: the raw row in registers over aligned vectors, masked ends
     ("f16 rows of 50257: raw row, eight vectors per thread, shifted", np.float16, [523, 50257]),
     ("bf16 rows of 65521: the longest shifted raw row", "bf16", [517, 65521]),
