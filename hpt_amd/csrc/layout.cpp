@@ -574,6 +574,18 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     p.nchunk = 8;
                     return p;
                 }
+                if (same && n_norm_dims <= 0 && elem_size == 2 && nvs > 8192 && p.cols <= 131072 - 70) {
+                    // two-byte softmax rows of 65522 ... 131002 elements: registers and LDS (see below; the
+                    // kernel's vector grid starts up to 63 elements before the row)
+                    p.kind = NormKind::RowReg;
+                    p.lds_rows = 1;
+                    p.vec = max_vec;
+                    p.shift = 1;
+                    p.tpr = 1024;
+                    p.rpb = 1;
+                    p.nchunk = 16;
+                    return p;
+                }
                 if (same && n_norm_dims <= 0 && elem_size == 4 && nvs > 8192 && p.cols <= 65536 - 34) {
                     // four-byte softmax rows of 32769 ... 65502 elements: registers and LDS (see below; the
                     // kernel's vector grid starts up to 31 elements before the row)
@@ -654,7 +666,8 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 return p;
             }
             // Four-byte softmax rows of 32769 ... 65536 elements: eight vectors per thread in registers and
-            // up to eight more in LDS, one read instead of the streaming kernel's two.
+            // up to eight more in LDS, one read instead of the streaming kernel's two. (Twelve and eight, for
+            // two-byte rows up to 163840 elements, has twenty loads in flight per thread and spills 40 registers.)
             if (n_norm_dims <= 0 && elem_size == 4 && v == max_vec && p.sstride == 1 && !p.shift && nv > 8192 && nv <= 16384) {
                 p.kind = NormKind::RowReg;
                 p.lds_rows = 1;

@@ -487,19 +487,22 @@ __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
     }
 }
 
-// ---- long rows of 4-byte elements: the row in registers AND LDS ------------------------------
+// ---- the longest rows that stay on chip: the row in registers AND LDS -------------------------
 // softmax / log_softmax over f32 rows of 32769 ... 65536 elements (logits of a 50257 / 50304 / 65536
-// vocabulary in f32). Eight vectors per thread live in registers, up to eight more in LDS (128 KiB
-// of the compute unit's 160; every thread reads back only the slots it wrote, so the LDS part needs
-// no barrier: it is a second register file). One HBM read and one write where the streaming
-// kernel reads twice. The summing sweep overwrites the held row with exp(x - max) (softmax) or
-// x - max (log_softmax), so the exponential is taken once per element either way.
+// vocabulary in f32) and two-byte rows of odd length from 65522 to 131002 elements.
+// NREG vectors per thread live in registers, up to NLDS more in LDS (NLDS * 16 KiB of the compute
+// unit's 160; every thread reads back only the slots it wrote, so the LDS part needs no barrier: it
+// is a second register file). One HBM read and one write where the streaming kernel reads twice.
+// Four-byte types: the summing sweep overwrites the held row with exp(x - max) (softmax) or x - max
+// (log_softmax), so the exponential is taken once per element either way. Two-byte types keep the
+// raw row (rounding the intermediate to 16 bits would cost accuracy) and take the exponential twice.
 // SHIFT: as in row_raw_kernel.
-template <int KIND, class T, bool SHIFT = false>
+template <int KIND, class T, int NREG, int NLDS, bool SHIFT = false>
 __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
     static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX, "a softmax kernel");
-    static_assert(sizeof(T) == 4, "rows of 4-byte elements");
-    constexpr int VEC = 4, NREG = 8, NLDS = 8;
+    static_assert(NLDS * 16 <= 144, "LDS of a compute unit");
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr bool kKeep = sizeof(T) >= 4;  // the held row may be overwritten with intermediates
     constexpr bool kLog = KIND == NORM_LOGSOFTMAX;
     using CT = typename Elem<T>::Wide;
     __shared__ CT smem[16];
@@ -512,6 +515,10 @@ __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
     // wavefront's 1 KiB of loads or stores covers eight whole lines, not nine partial ones
     constexpr int LINE = 128 / sizeof(T);
     auto shift_of = [](const T* p) -> int { return SHIFT ? (int)(((uintptr_t)p / sizeof(T)) % LINE) : 0; };
+    // (2-byte types: keep the compiler from holding the widened copies of one sweep for the next)
+    auto forget = [](Pack<T, VEC>& v) {
+        if constexpr (sizeof(T) == 2) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&v)));
+    };
     for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
         const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
         T* out_row = (T*)a.out + row * a.cols;
@@ -567,6 +574,8 @@ __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
                 for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, Elem<T>::widen(v.v[j]));
             }
         m = row_all_reduce<MaxC<CT>>(m, 1024, 0, smem);
+#pragma unroll
+        for (int c = 0; c < NREG; ++c) forget(reg[c]);
         CT s = 0;
 #pragma unroll
         for (int c = 0; c < NREG; ++c)
@@ -576,7 +585,7 @@ __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
                     const CT d = Elem<T>::widen(reg[c].v[j]) - m;
                     const CT e = exp_ct<T>(d);
                     s += e;
-                    reg[c].v[j] = Elem<T>::narrow(kLog ? d : e);
+                    if constexpr (kKeep) reg[c].v[j] = Elem<T>::narrow(kLog ? d : e);
                 }
 #pragma unroll
         for (int c = 0; c < NLDS; ++c)
@@ -587,18 +596,21 @@ __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
                     const CT d = Elem<T>::widen(v.v[j]) - m;
                     const CT e = exp_ct<T>(d);
                     s += e;
-                    v.v[j] = Elem<T>::narrow(kLog ? d : e);
+                    if constexpr (kKeep) v.v[j] = Elem<T>::narrow(kLog ? d : e);
                 }
-                lds[c * 1024 + tx] = v;
+                if constexpr (kKeep) lds[c * 1024 + tx] = v;
             }
         s = row_all_reduce<SumC<CT>>(s, 1024, 0, smem);
+#pragma unroll
+        for (int c = 0; c < NREG; ++c) forget(reg[c]);
         const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
         auto finish = [&](Pack<T, VEC> v, int iv) {
             Pack<T, VEC> o;
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
                 const CT x = Elem<T>::widen(v.v[j]);
-                o.v[j] = Elem<T>::narrow(kLog ? x - k : x * k);
+                if constexpr (kKeep) o.v[j] = Elem<T>::narrow(kLog ? x - k : x * k);
+                else o.v[j] = Elem<T>::narrow(kLog ? (x - m) - k : exp_ct<T>(x - m) * k);
             }
             const int e0 = iv * VEC - sh;
             if (!SHIFT || (e0 >= 0 && e0 + VEC <= cols)) store_pack_stream<T, VEC>(out_row + e0, o);

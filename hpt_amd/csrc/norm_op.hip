@@ -226,11 +226,15 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         return;
     }
     if (p.kind == NormKind::RowReg && p.lds_rows) {
-        // long four-byte softmax rows: registers + LDS; the fused kinds stream
-        if constexpr (sizeof(T) == 4 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX)) {
-            if (p.shift) row_lds_kernel<KIND, T, true><<<grid, dim3(1024), 0, st>>>(a);
-            else row_lds_kernel<KIND, T, false><<<grid, dim3(1024), 0, st>>>(a);
-        } else if constexpr (FULL > 1) {
+        // the longest rows that stay on chip: registers + LDS; the fused kinds stream
+        if constexpr (FULL > 1 && sizeof(T) <= 4 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX)) {
+            if (p.nchunk == 16) {
+                if (p.shift) row_lds_kernel<KIND, T, 8, 8, true><<<grid, dim3(1024), 0, st>>>(a);
+                else row_lds_kernel<KIND, T, 8, 8, false><<<grid, dim3(1024), 0, st>>>(a);
+                return;
+            }
+        }
+        if constexpr (FULL > 1) {
             if (p.shift) row_stream_kernel<KIND, T, FULL, true><<<grid, block, 0, st>>>(a);
             else row_stream_kernel<KIND, T, FULL><<<grid, block, 0, st>>>(a);
         }

@@ -336,7 +336,9 @@ WIDE_ROW_CASES = [
     # odd lengths of two-byte rows beyond 32768: the raw row in registers over aligned vectors, masked ends
     ("f16 rows of 50257: raw row, eight vectors per thread, shifted", np.float16, [523, 50257]),
     ("bf16 rows of 65521: the longest shifted raw row", "bf16", [517, 65521]),
-    ("f16 rows of 65537: streamed again", np.float16, [130, 65537]),
+    ("f16 rows of 65537: registers and LDS, shifted", np.float16, [130, 65537]),
+    ("bf16 rows of 131001: the longest shifted two-byte row on chip", "bf16", [133, 131001]),
+    ("f16 rows of 131003: streamed", np.float16, [131, 131003]),
 ]
 
 
