@@ -666,7 +666,9 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 return p;
             }
             // Four-byte softmax rows of 32769 ... 65536 elements: eight vectors per thread in registers and
-            // up to eight more in LDS, one read instead of the streaming kernel's two. (Twelve and eight, for
+            // up to eight more in LDS, one read instead of the streaming kernel's two. (Layernorm in that kernel,
+            // with gamma / beta from L2 in the last sweep, spilled 60 to 130 registers and ran at 1.6-3.3 TB/s:
+            // such rows stream, at 3.0-3.4.) (Twelve and eight, for
             // two-byte rows up to 163840 elements, has twenty loads in flight per thread and spills 40 registers.)
             if (n_norm_dims <= 0 && elem_size == 4 && v == max_vec && p.sstride == 1 && !p.shift && nv > 8192 && nv <= 16384) {
                 p.kind = NormKind::RowReg;

@@ -333,6 +333,11 @@ WIDE_ROW_CASES = [
     ("f32 rows of 32772: one vector beyond the registers", np.float32, [200, 32772]),
     ("f32 rows of 65501: the longest shifted row", np.float32, [131, 65501]),
     ("f32 rows of 32771 in a view that starts 29 elements into a line", np.float32, [135, 32771]),
+    # layernorm rows beyond 16384 elements stream (softmax of the same rows: registers and LDS)
+    ("f32 rows of 20480", np.float32, [300, 20480]),
+    ("f32 rows of 16385, shifted", np.float32, [290, 16385]),
+    ("f16 rows of 20480", np.float16, [300, 20480]),
+    ("bf16 rows of 40001, shifted", "bf16", [280, 40001]),
     # odd lengths of two-byte rows beyond 32768: the raw row in registers over aligned vectors, masked ends
     ("f16 rows of 50257: raw row, eight vectors per thread, shifted", np.float16, [523, 50257]),
     ("bf16 rows of 65521: the longest shifted raw row", "bf16", [517, 65521]),
