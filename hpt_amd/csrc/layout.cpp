@@ -269,9 +269,11 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
             int64_t g = kin, b = full;
             while (b) { int64_t t = g % b; g = b; b = t; }
             const int64_t kp = kin / g;  // threads per period: kp * full elements = full rows
-            const int64_t tmax = std::min<int64_t>(1024, (int64_t)((64u << 10) / ((size_t)full * acc_size)));
-            // (each slab must be worth at least two periods of the walk)
-            if (kp <= tmax && kin * p.R >= 2 * kp * (tmax / kp) * full) {
+            int64_t tmax = std::min<int64_t>(1024, (int64_t)((64u << 10) / ((size_t)full * acc_size)));
+            // (each slab must be worth at least two periods of the walk: small slabs, of which there are
+            // many, take fewer threads each)
+            tmax = std::min(tmax, kin * p.R / (2 * full));
+            if (kp <= tmax && tmax >= 64) {
                 p.flat_t = (int)(kp * (tmax / kp));
                 p.vec = full;
                 const int64_t per_iter = (int64_t)p.flat_t * full;
@@ -771,9 +773,11 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 int64_t g = L, b = max_vec;
                 while (b) { int64_t t = g % b; g = b; b = t; }
                 const int64_t lp = L / g;  // threads per period
-                const int64_t tmax = std::min<int64_t>(1024, (64 << 10) / (max_vec * (elem_size == 8 ? 16 : 8)));
-                // (each batch slab must be worth at least two periods of the walk)
-                if (lp <= tmax && p.cols * L >= 2 * lp * (tmax / lp) * max_vec) {
+                int64_t tmax = std::min<int64_t>(1024, (64 << 10) / (max_vec * (elem_size == 8 ? 16 : 8)));
+                // (each batch slab must be worth at least two periods of the walk: small slabs, of which there
+                // are many, take fewer threads each)
+                tmax = std::min(tmax, p.cols * L / (2 * max_vec));
+                if (lp <= tmax && tmax >= 64) {
                     p.flat_t = (int)(lp * (tmax / lp));
                     p.vec = max_vec;
                     p.shift = aligned ? 0 : 1;
