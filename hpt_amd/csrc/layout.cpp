@@ -746,11 +746,21 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     // thread rows that share an inner position when the axis is longer than one thread holds
                     const int64_t ty = pow2_ceil((p.cols + nc_max - 1) / nc_max);
                     // enough threads to fill the chip: inner positions x thread rows
-                    if (ty <= 16 && p.rows / ev * ty >= 8 * 1024 && L % ev == 0 && sa % ev == 0 &&
-                        (nk == 1 || p.kept_in.stride[0] % ev == 0) &&
+                    if (!(ty <= 16 && p.rows / ev * ty >= 8 * 1024)) continue;
+                    if (L % ev == 0 && sa % ev == 0 && (nk == 1 || p.kept_in.stride[0] % ev == 0) &&
                         (p.cols * L) % ev == 0 && ((uintptr_t)in_data % vb) == 0 && ((uintptr_t)out_data % vb) == 0) {
                         p.kind = NormKind::ColReg;
                         p.vec = ev;
+                        p.nchunk = (int)nc_max;
+                        p.tpr = (int)ty;
+                        return p;
+                    }
+                    // an inner dim that is not whole, aligned vectors of this width (odd L, odd strides): the
+                    // same vectors unaligned beat narrower aligned ones
+                    if (ev > 1 && L >= 8 * ev && ((uintptr_t)in_data % elem_size) == 0 && ((uintptr_t)out_data % elem_size) == 0) {
+                        p.kind = NormKind::ColReg;
+                        p.vec = ev;
+                        p.shift = 1;
                         p.nchunk = (int)nc_max;
                         p.tpr = (int)ty;
                         return p;
@@ -827,7 +837,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? (p.kind == NormKind::RowSplit ? "-unaligned" : (p.raw_rows ? "-raw-shift" : (p.lds_rows ? "-lds-shift" : "-shift"))) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg) ? "-unaligned" : (p.raw_rows ? "-raw-shift" : (p.lds_rows ? "-lds-shift" : "-shift"))) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     describe_dims(s, "rows_in", p.kept_in);

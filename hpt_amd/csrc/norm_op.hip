@@ -111,14 +111,21 @@ template <class T, int EV> void launch_col_reg(const NormPlan& p, const NormArgs
     c.sa = a.sa;
     c.bi = nk > 1 ? p.kept_in.stride[0] : 0;
     c.L = p.kept_in.size[nk - 1];
-    c.nvec = c.L / EV;
+    c.nvec = p.shift ? (c.L + EV - 1) / EV : c.L / EV;
     c.total = (nk > 1 ? p.kept_in.size[0] : 1) * c.nvec;
     c.cols = (int)p.cols;
     c.ty_log2 = ilog2(p.tpr);  // thread rows per inner position
     if (p.tpr > 16 || c.cols > NC * p.tpr)
         fail(HPT_ERR_KERNEL, "col-reg: axis of %d does not fit %d thread rows of %d vectors", c.cols, p.tpr, NC);
     const int64_t tx = 256 / p.tpr;
-    col_reg_kernel<KIND, T, EV, NC><<<dim3((unsigned)((c.total + tx - 1) / tx)), dim3(256), 0, st>>>(c);
+    const dim3 grid((unsigned)((c.total + tx - 1) / tx));
+    if constexpr (EV > 1) {
+        if (p.shift) {
+            col_reg_kernel<KIND, T, EV, NC, true><<<grid, dim3(256), 0, st>>>(c);
+            return;
+        }
+    }
+    col_reg_kernel<KIND, T, EV, NC><<<grid, dim3(256), 0, st>>>(c);
 }
 
 // The transposed forms (kinds 0..2 only).

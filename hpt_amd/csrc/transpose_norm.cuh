@@ -365,7 +365,7 @@ struct ColRegArgs {
     void* out;
     int64_t sa;     // input stride along the axis
     int64_t bi;     // input stride of the batch dim
-    int64_t nvec;   // vectors per batch slab along the inner dim: L / EV
+    int64_t nvec;   // vectors per batch slab along the inner dim: L / EV (UA: rounded up)
     int64_t total;  // batch * nvec
     int64_t L;      // inner length
     int cols;       // axis length (<= NC << ty_log2)
@@ -383,7 +383,10 @@ template <class T, int N> __device__ __forceinline__ void forget_pack(Pack<T, N>
     }
 }
 
-template <int KIND, class T, int EV, int NC>
+// UA: the inner dim is not whole, aligned vectors (an odd length, odd strides): unaligned vectors all the
+// same; the last vector of an inner row is taken from the row's end backwards and stores only the
+// elements that the vector before it does not cover.
+template <int KIND, class T, int EV, int NC, bool UA = false>
 __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
     static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX, "a softmax kernel");
     using CT = typename Elem<T>::Wide;
@@ -405,14 +408,19 @@ __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
             q = g - b * a.nvec;
         }
     }
-    const T* in = (const T*)a.in + b * a.bi + q * EV;
-    T* out = (T*)a.out + b * a.cols * a.L + q * EV;
+    const int64_t e0 = UA ? min(q * EV, a.L - EV) : q * EV;
+    const int skip = (int)(q * EV - e0);  // UA: leading elements that belong to the vector before
+    const T* in = (const T*)a.in + b * a.bi + e0;
+    T* out = (T*)a.out + b * a.cols * a.L + e0;
     // this thread's channels: ty, ty + TY, ...
     const int mine = valid ? (a.cols - ty + TY - 1) >> a.ty_log2 : 0;
     Pack<T, EV> raw[NC];
 #pragma unroll
     for (int i = 0; i < NC; ++i)
-        if (i < mine) raw[i] = load_pack_stream<T, EV>(in + (int64_t)(ty + (i << a.ty_log2)) * a.sa);
+        if (i < mine) {
+            if constexpr (UA) raw[i] = load_pack_unaligned<T, EV>(in + (int64_t)(ty + (i << a.ty_log2)) * a.sa);
+            else raw[i] = load_pack_stream<T, EV>(in + (int64_t)(ty + (i << a.ty_log2)) * a.sa);
+        }
     // all-reduce over the thread rows of an inner position
     auto across = [&](CT(&v)[EV], auto op) {
         if (TY == 1) return;
@@ -460,7 +468,18 @@ __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
                 const CT d = Elem<T>::widen(raw[i].v[k]) - m[k];
                 o.v[k] = Elem<T>::narrow(kLog ? d - kk[k] : exp_ct<T>(d) * kk[k]);
             }
-            store_pack_stream<T, EV>(out + (int64_t)(ty + (i << a.ty_log2)) * a.L, o);
+            T* dst = out + (int64_t)(ty + (i << a.ty_log2)) * a.L;
+            if constexpr (UA) {
+                if (skip == 0) {
+                    store_pack_unaligned<T, EV>(dst, o);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < EV; ++k)
+                        if (k >= skip) dst[k] = o.v[k];
+                }
+            } else {
+                store_pack_stream<T, EV>(dst, o);
+            }
         }
 }
 

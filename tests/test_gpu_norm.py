@@ -519,6 +519,12 @@ CHANNEL_CASES = [
     ("f16 [2, 300, 40000] axis 1 (16 thread rows)", np.float16, [2, 300, 40000], 1),
     ("f32 [600, 66001] axis 0 (single elements, 16 thread rows)", np.float32, [600, 66001], 0),
     ("f64 [3, 100, 30000] axis 1", np.float64, [3, 100, 30000], 1),
+    # inner dims that are not whole vectors: unaligned vectors, the last one of a row from its end
+    ("f16 [3, 7, 33, 1361] axis 1 (odd inner length 44913)", np.float16, [3, 7, 33, 1361], 1),
+    ("bf16 [21, 33, 3631] axis 0 (two thread rows)", "bf16", [21, 33, 3631], 0),
+    ("f32 [2, 21, 213, 211] axis 1", np.float32, [2, 21, 213, 211], 1),
+    ("f64 [2, 9, 70001] axis 1", np.float64, [2, 9, 70001], 1),
+    ("f16 [300, 70001] axis 0 (16 thread rows)", np.float16, [300, 70001], 0),
 ]
 
 
