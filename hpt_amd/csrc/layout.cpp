@@ -261,8 +261,10 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
         }
         const int full = (int)(16 / elem_size);
         if (p.lean && nk && !p.kept_swapped && p.vec == 1 && p.sstride == 1 && full > 1 && p.kept.stride[nk - 1] == 1 &&
-            p.red.n == 1 && p.red.stride[0] == kin && (uintptr_t)data % 16 == 0 &&
-            (outer == 1 || p.kept.stride[0] % full == 0) && outer * kin * p.R * (int64_t)elem_size >= (8ll << 20)) {
+            p.red.n == 1 && p.red.stride[0] == kin && (uintptr_t)data % elem_size == 0 &&
+            outer * kin * p.R * (int64_t)elem_size >= (8ll << 20)) {
+            // (slabs that start off 16-byte boundaries take the same vectors unaligned)
+            const bool slabs_aligned = (uintptr_t)data % 16 == 0 && (outer == 1 || p.kept.stride[0] % full == 0);
             // A contiguous [R, kin] slab whose rows are not whole vectors (kin = 3, 33, 257): walk it
             // as a FLAT array of aligned vectors. With a stride between a thread's visits that is a
             // multiple of kin, every vector slot of every thread stays on one column.
@@ -276,6 +278,7 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
             if (kp <= tmax && tmax >= 64) {
                 p.flat_t = (int)(kp * (tmax / kp));
                 p.vec = full;
+                p.unaligned = !slabs_aligned;
                 const int64_t per_iter = (int64_t)p.flat_t * full;
                 const int64_t iters = (kin * p.R + per_iter - 1) / per_iter;
                 int64_t cap = std::max<int64_t>(1, (int64_t)((64ll << 20) / acc_size) / p.K);
@@ -292,7 +295,7 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
             // the partials are [slice][phase][K].
             const int64_t phases = full / g;
             const int64_t xb = (kp + 1023) / 1024;
-            if (kp > tmax && p.R >= 16 * phases && xb <= 65535 && kin * phases <= kI32) {
+            if (slabs_aligned && kp > tmax && p.R >= 16 * phases && xb <= 65535 && kin * phases <= kI32) {
                 p.flat_t = (int)(((kp + xb - 1) / xb + 63) / 64 * 64);
                 p.flat_xb = (int)xb;
                 p.flat_phases = (int)phases;
@@ -393,7 +396,7 @@ std::string describe(const ReducePlan& p) {
             break;
         case ReduceKind::Col:
             snprintf(buf, sizeof buf, "col%s%s vec=%d bx=%d by=%d outs=%lld red=%lld split=%d ",
-                     p.flat_xb ? "-flat-wide" : p.flat_t ? "-flat" : p.kept_swapped ? "-swapped" : p.unaligned ? "-unaligned" : p.lean ? "" : "-general",
+                     p.flat_xb ? "-flat-wide" : p.flat_t ? (p.unaligned ? "-flat-unaligned" : "-flat") : p.kept_swapped ? "-swapped" : p.unaligned ? "-unaligned" : p.lean ? "" : "-general",
                      p.sstride == 2 ? "-step2" : "", p.vec,
                      p.flat_t ? p.flat_t : p.bx, p.by,
                      (long long)p.K, (long long)p.R, p.split);

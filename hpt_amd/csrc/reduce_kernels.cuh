@@ -517,12 +517,17 @@ struct ColFlatArgs {
     int split, init_out;
 };
 
-template <class Op, int VEC>
+// UA: the slabs do not start on 16-byte boundaries (an odd slab size): the same vectors, unaligned.
+template <class Op, int VEC, bool UA = false>
 __global__ void __launch_bounds__(1024) col_flat_kernel(const ColFlatArgs a) {
     using T = typename Op::In;
     using Acc = typename Op::Acc;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     Acc* smem = (Acc*)smem_raw;
+    auto flat_load = [](const T* p) {
+        if constexpr (UA) return load_pack_unaligned<T, VEC>(p);
+        else return load_pack_stream<T, VEC>(p);
+    };
     const int t = threadIdx.x;
     const int outer = blockIdx.y;
     const int L = a.threads * VEC;
@@ -545,7 +550,7 @@ __global__ void __launch_bounds__(1024) col_flat_kernel(const ColFlatArgs a) {
         // on the last round: a load under a branch would make the wait before the fold a full one.)
         auto load4 = [&](Pack<T, VEC>(&v)[4], int64_t i0) {
 #pragma unroll
-            for (int u = 0; u < 4; ++u) v[u] = load_pack_stream<T, VEC>(base + (i0 + u * split) * L + p0);
+            for (int u = 0; u < 4; ++u) v[u] = flat_load(base + (i0 + u * split) * L + p0);
         };
         auto fold4 = [&](const Pack<T, VEC>(&v)[4], int64_t i0) {
 #pragma unroll
@@ -574,7 +579,7 @@ __global__ void __launch_bounds__(1024) col_flat_kernel(const ColFlatArgs a) {
             }
         }
         for (; it < whole; it += split) {
-            Pack<T, VEC> v = load_pack_stream<T, VEC>(base + it * L + p0);
+            Pack<T, VEC> v = flat_load(base + it * L + p0);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v.v[j], row[j] + (int)it * rows_per_period);
         }
@@ -962,7 +967,9 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.threads = p.flat_t;
             a.split = p.split;
             a.init_out = init_out;
-            col_flat_kernel<Op, FULL><<<dim3(1, (unsigned)outer, (unsigned)p.split), dim3((unsigned)p.bx),
+if (p.unaligned)             col_flat_kernel<Op, FULL, true><<<dim3(1, (unsigned)outer, (unsigned)p.split), dim3((unsigned)p.bx),
+                                        (size_t)p.flat_t * FULL * sizeof(Acc), st>>>(a);
+            else             col_flat_kernel<Op, FULL><<<dim3(1, (unsigned)outer, (unsigned)p.split), dim3((unsigned)p.bx),
                                         (size_t)p.flat_t * FULL * sizeof(Acc), st>>>(a);
         }
     } else {

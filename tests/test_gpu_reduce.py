@@ -211,6 +211,7 @@ def test_narrow_inner_dim_flat_walk(hpt, orc, dev):
     for shape, axis, npdt in (((700001, 3), 0, np.float32), ((70003, 33), 0, np.float32), ((4, 500000, 5), 1, np.float32),
                               ((140001, 33), 0, np.float16), ((20001, 257), 0, np.float16), ((1100003, 1, 3), 0, np.float64),
                               ((700, 2048, 3), 1, np.float32), ((900, 1031, 5), 1, np.float16),   # many small slabs
+                              ((257, 4097, 23), 1, np.float16), ((31, 70001, 3), 1, np.float32),    # slabs off 16-byte boundaries
                               ((2100001, 3), 0, np.int32), ((3000001, 3), 0, np.uint8), ((600011, 7), 0, np.int16),
                               # rows wider than a workgroup: the period spans several workgroups ("flat-wide")
                               ((2051, 4097), 0, np.float32), ((1031, 5003), 0, np.float16), ((2, 1028, 2051), 1, np.float32),
