@@ -260,7 +260,7 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
             p.sstride = 2;
         }
         const int full = (int)(16 / elem_size);
-        if (p.lean && nk && !p.kept_swapped && p.vec == 1 && p.sstride == 1 && full > 1 && p.kept.stride[nk - 1] == 1 &&
+        if (p.lean && nk && !p.kept_swapped && p.vec < full && p.sstride == 1 && full > 1 && p.kept.stride[nk - 1] == 1 &&
             p.red.n == 1 && p.red.stride[0] == kin && (uintptr_t)data % elem_size == 0 &&
             outer * kin * p.R * (int64_t)elem_size >= (8ll << 20)) {
             // (slabs that start off 16-byte boundaries take the same vectors unaligned)
@@ -778,7 +778,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             p.vec = v;
             // A narrow inner dim (or one that is not whole vectors) leaves most lanes idle: walk the
             // contiguous [cols, L] slab as a flat array of aligned vectors instead.
-            if (max_vec > 1 && (!vec_ok || L < 64 * max_vec) && sa == L && ((uintptr_t)in_data % elem_size) == 0 &&
+            if (max_vec > 1 && (!vec_ok || L <= 1024 * max_vec) && sa == L && ((uintptr_t)in_data % elem_size) == 0 &&
                 ((uintptr_t)out_data % elem_size) == 0 && batch * p.cols * L * (int64_t)elem_size >= (8ll << 20)) {
                 // (slabs that start off 16-byte boundaries take the same vectors unaligned: `shift`)
                 const bool aligned = ((uintptr_t)in_data % 16) == 0 && ((uintptr_t)out_data % 16) == 0 &&

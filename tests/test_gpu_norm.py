@@ -244,6 +244,24 @@ def test_transposed_tile_masked_and_constant_rows(hpt, dev):
     assert np.array_equal(out, np.broadcast_to(b, out.shape))
 
 
+def test_softmax_over_axis_0_with_a_wide_inner_dim(hpt, orc, dev):
+    """Inner dims wider than a workgroup's period (more than 1024 vectors) keep lanes along the inner dim:
+    statistics over the axis dealt to wavefronts and workgroups, finalize, apply."""
+    rng = np.random.default_rng(213)
+    for npdt, shape in ((np.float32, (1500, 5000)), (np.float16, (1100, 8200)), (np.float32, (3, 1100, 4100))):
+        base = (rng.standard_normal(shape) * 3).astype(npdt)
+        t, a = upload(hpt, base, dev=dev)
+        ax = len(shape) - 2
+        assert hpt.normalize_plan(t, ax).startswith("col-split rows"), hpt.normalize_plan(t, ax)
+        for log in (False, True):
+            got = (t.log_softmax(ax) if log else t.softmax(ax)).numpy().astype(np.float32)
+            if npdt == np.float16:
+                want = orc.softmax(a, ax, log=log, acc=orc.ACC_F32).astype(np.float32)
+                assert_close(got, want, HALF_RTOL, max(half_atol(want, 11), 6e-8), f"f16 {shape} log={log}")
+            else:
+                assert_close(got, orc.softmax(a, ax, log=log, acc=orc.ACC_F64), F32_RTOL, 2e-6 if log else F32_ATOL, f"f32 {shape} log={log}")
+
+
 def test_log_softmax_long_columns_keep_the_absolute_tolerance(hpt, orc, dev):
     """Column softmax where one lane sums a whole column (1012 terms one after the other): the entry at the
     column's maximum is -ln(sum) ~ -0.004, so the sum must be right to better than 1e-6 relative for the

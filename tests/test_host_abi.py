@@ -109,7 +109,7 @@ def test_plans_for_shapes_off_the_benchmark_list(hpt):
         ([32768, 1024], hpt.f32, 0, 1, "rowreg rows=32768 cols=1024 vec=4 tpr=64 rpb=4 nchunk=4"),
         # softmax over an axis that is not the last
         ([8, 21, 512, 512], None, 1, 0, "col-reg"), ([64, 128, 56, 56], None, 1, 0, "col-reg"),
-        ([11184810, 3], None, 0, 0, "col-split-flat"), ([32768, 1024], None, 0, 0, "col-split rows"),
+        ([11184810, 3], None, 0, 0, "col-split-flat"), ([32768, 1024], None, 0, 0, "col-split-flat"), ([4096, 8192], None, 0, 0, "col-split rows"),
     ]
     for shape, dt, axis, nn, want in norm:
         got = hpt.normalize_plan(view(shape, dt), axis, nn)
