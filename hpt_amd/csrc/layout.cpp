@@ -260,6 +260,28 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
             p.sstride = 2;
         }
         const int full = (int)(16 / elem_size);
+        {
+            // Small groups laid back to back ([outer, R, kin] with R * kin elements of at most 2 KiB and
+            // rows of kin shorter than a wavefront of vectors): 16 KiB tiles of whole groups through LDS.
+            const int64_t G = p.R * kin;
+            if (nk == 2 && !p.kept_swapped && p.red.n == 1 && full > 1 && p.sstride == 1 && p.kept.stride[1] == 1 &&
+                p.red.stride[0] == kin && p.kept.stride[0] == G && (uintptr_t)data % 16 == 0 &&
+                G * (int64_t)elem_size <= 2048 && kin * (int64_t)elem_size < 1024 && p.R >= 2 && p.R <= 256 &&
+                p.K * p.R * (int64_t)elem_size >= (4ll << 20) && p.kept.size[0] >= 1024) {
+                int64_t groups = (16 << 10) / (G * (int64_t)elem_size);
+                groups -= groups % full;  // tiles start on 16-byte boundaries
+                if (groups >= full) {
+                    p.group_tile = (int)groups;
+                    p.vec = full;
+                    p.lean = true;
+                    p.split = 1;
+                    p.bx = 256;
+                    p.by = 1;
+                    p.chunk = 0;
+                    return p;
+                }
+            }
+        }
         if (p.lean && nk && !p.kept_swapped && p.vec < full && p.sstride == 1 && full > 1 && p.kept.stride[nk - 1] == 1 &&
             p.red.n == 1 && p.red.stride[0] == kin && (uintptr_t)data % elem_size == 0 &&
             outer * kin * p.R * (int64_t)elem_size >= (8ll << 20)) {
@@ -396,7 +418,7 @@ std::string describe(const ReducePlan& p) {
             break;
         case ReduceKind::Col:
             snprintf(buf, sizeof buf, "col%s%s vec=%d bx=%d by=%d outs=%lld red=%lld split=%d ",
-                     p.flat_xb ? "-flat-wide" : p.flat_t ? (p.unaligned ? "-flat-unaligned" : "-flat") : p.kept_swapped ? "-swapped" : p.unaligned ? "-unaligned" : p.lean ? "" : "-general",
+                     p.group_tile ? "-group-tile" : p.flat_xb ? "-flat-wide" : p.flat_t ? (p.unaligned ? "-flat-unaligned" : "-flat") : p.kept_swapped ? "-swapped" : p.unaligned ? "-unaligned" : p.lean ? "" : "-general",
                      p.sstride == 2 ? "-step2" : "", p.vec,
                      p.flat_t ? p.flat_t : p.bx, p.by,
                      (long long)p.K, (long long)p.R, p.split);

@@ -390,6 +390,62 @@ __global__ void __launch_bounds__(256) row_tile_kernel(const RowTileArgs a) {
     }
 }
 
+// Small groups laid back to back (a contiguous [outer, R, kin] tensor reduced over R with R * kin
+// small: [N, 2, 3], [N, 3, 16], [N, 4, 12]): lanes along kin would leave most of a wavefront idle and a
+// lane per output reads single elements at a stride. As in row_tile_kernel a workgroup stages 16 KiB of
+// whole groups in LDS with aligned 128-bit loads; then one lane per output folds its R elements out of LDS.
+struct GroupTileArgs {
+    const void* in;
+    void* out;
+    int64_t groups;  // outer
+    double count;
+    int R, kin;
+    int groups_per_wg;
+    int init_out;
+};
+
+template <class Op, int VEC>
+__global__ void __launch_bounds__(256) group_tile_kernel(const GroupTileArgs a) {
+    using T = typename Op::In;
+    using Acc = typename Op::Acc;
+    constexpr int NV = 4;  // vectors per thread: 256 * 4 * 16 bytes = 16 KiB
+    __shared__ __align__(16) unsigned char tile_raw[256 * NV * 16];
+    T* tile = reinterpret_cast<T*>(tile_raw);
+    const int t = threadIdx.x;
+    const int G = a.R * a.kin;
+    const int64_t g0 = (int64_t)blockIdx.x * a.groups_per_wg;
+    const int64_t left = a.groups - g0;
+    const int ngroups = left < a.groups_per_wg ? (int)left : a.groups_per_wg;
+    const int n = ngroups * G;  // elements of this tile
+    const T* src = (const T*)a.in + g0 * G;
+    Pack<T, VEC> v[NV];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int e = (t + u * 256) * VEC;
+        if (e + VEC <= n) {
+            v[u] = load_pack_stream<T, VEC>(src + e);
+        } else {  // the tensor's last, partial vector
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                if (e + j < n) v[u].v[j] = src[e + j];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int e = (t + u * 256) * VEC;
+        if (e < n) store_pack<T, VEC>(tile + e, v[u]);
+    }
+    __syncthreads();
+    const int nout = ngroups * a.kin;
+    for (int o = t; o < nout; o += 256) {
+        const int g = o / a.kin, i = o - g * a.kin;
+        const T* p = tile + g * G + i;
+        Acc acc = Op::identity();
+        for (int r = 0; r < a.R; ++r) fold_in<Op>(acc, p[r * a.kin], r);
+        write_out<Op>(a.out, g0 * a.kin + o, acc, a.init_out, a.count);
+    }
+}
+
 // Lean form: outputs are (outer, inner) with inner the lane dim; one reduced dim.
 // out[outer * kin + inner] = reduce over r of in[outer * so + r * rs + inner * sk].
 struct ColLeanArgs {
@@ -861,6 +917,21 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
     }
     const bool vec = p.vec == FULL && FULL > 1;
     void* stage1_out = p.split > 1 ? sc.partial : out;
+    if (p.kind == ReduceKind::Col && p.group_tile > 0) {
+        if constexpr (FULL > 1) {
+            GroupTileArgs a{};
+            a.in = in;
+            a.out = out;
+            a.groups = p.kept.size[0];
+            a.count = count;
+            a.R = (int)p.R;
+            a.kin = (int)p.kept.size[1];
+            a.groups_per_wg = p.group_tile;
+            a.init_out = init_out;
+            group_tile_kernel<Op, FULL><<<dim3((unsigned)((a.groups + p.group_tile - 1) / p.group_tile)), dim3(256), 0, st>>>(a);
+        }
+        return;
+    }
     if (p.kind == ReduceKind::Row && p.row_tile > 0) {
         if constexpr (FULL > 1) {
             RowTileArgs a{};

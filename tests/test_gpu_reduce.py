@@ -401,6 +401,66 @@ def test_short_runs_off_the_vector_grid(hpt, orc, dev):
     assert np.array_equal(t.sum([0, 2, 3]).numpy(), orc.reduce(orc.SUM, a, [0, 2, 3]))
 
 
+def test_small_groups_staged_through_lds(hpt, orc, dev):
+    """Contiguous [outer, R, k] reduced over the short middle axis with small R * k ([N, 2, 3], [N, 3, 16],
+    [N, 4, 12]): 16 KiB tiles of whole groups are brought into LDS with aligned vectors and one lane
+    per output folds its R elements from there. Partial last tiles and vectors, ties for the index rule,
+    NaN handling, the accumulate form."""
+    rng = np.random.default_rng(123)
+    assert "group-tile" in hpt.reduce_plan(hpt.Tensor.empty([700001, 2, 3], hpt.f32, dev), hpt.SUM, [1])
+    for shape, ax, npdt in (((700001, 2, 3), 1, np.float32), ((300001, 3, 16), 1, np.float16), ((5, 70001, 4, 12), 2, np.float16),
+                            ((150001, 7, 33), 1, np.uint8), ((40001, 50, 9), 1, np.int32), ((60001, 16, 8), 1, np.float64),
+                            ((90001, 2, 255), 1, np.int16), ((3, 11, 20001, 16, 2), 3, np.float32)):
+        if np.issubdtype(npdt, np.floating):
+            base = rng.standard_normal(shape).astype(npdt)
+        else:
+            base = rng.integers(0, 40, shape).astype(npdt)   # many ties
+        t, a = upload(hpt, base, dev=dev)
+        tag = f"{np.dtype(npdt).name} {shape}"
+        assert "group-tile" in hpt.reduce_plan(t, hpt.SUM, [ax]), hpt.reduce_plan(t, hpt.SUM, [ax])
+        assert np.array_equal(t.argmax(ax).numpy(), orc.argreduce(True, a, ax)), tag
+        assert np.array_equal(t.argmin(ax).numpy(), orc.argreduce(False, a, ax)), tag
+        assert np.array_equal(t.max([ax]).numpy(), a.max(ax)), tag
+        if npdt == np.float16:
+            want = orc.reduce(orc.SUM, a, [ax], acc=orc.ACC_F32).astype(np.float32)
+            assert_close(t.sum([ax]).numpy().astype(np.float32), want, HALF_RTOL, half_atol(want, 11), tag)
+        elif np.issubdtype(npdt, np.floating):
+            assert_close(t.sum([ax]).numpy(), orc.reduce(orc.SUM, a, [ax], acc=orc.ACC_F64), F32_RTOL, F32_ATOL, tag)
+            assert_close(t.mean([ax]).numpy(), a.astype(np.float64).mean(ax), F32_RTOL, F32_ATOL, tag)
+        else:
+            assert np.array_equal(t.sum([ax]).numpy(), orc.reduce(orc.SUM, a, [ax])), tag
+            assert np.array_equal(t.prod([ax]).numpy(), orc.reduce(orc.PROD, a, [ax])), tag
+    # NaN / inf: max skips NaN, a NaN never wins an arg reduction, sum propagates, nansum skips
+    x = rng.standard_normal((400001, 3, 4)).astype(np.float32)
+    flat = x.reshape(-1)
+    flat[rng.integers(0, flat.size, flat.size // 20)] = np.nan
+    flat[rng.integers(0, flat.size, flat.size // 100)] = np.inf
+    x[7] = np.nan
+    t, a = upload(hpt, x, dev=dev)
+    assert np.array_equal(t.max([1]).numpy(), orc.reduce(orc.MAX, a, [1]))
+    assert np.array_equal(t.argmax(1).numpy(), orc.argreduce(True, a, 1))
+    with np.errstate(invalid="ignore"):
+        want = orc.reduce(orc.SUM, a, [1], acc=orc.ACC_F64)
+        got = t.sum([1]).numpy()
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        ok = np.isfinite(want)
+        assert_close(got[ok], want[ok], F32_RTOL, 1e-5, "sum with special values")
+        wn = orc.reduce(orc.NANSUM, a, [1], acc=orc.ACC_F64)
+        gn = t.nansum([1]).numpy()
+        ok = np.isfinite(wn)
+        assert np.array_equal(np.isinf(gn), np.isinf(wn))
+        assert_close(gn[ok], wn[ok], F32_RTOL, 1e-5, "nansum with special values")
+    # accumulate into an existing output
+    y = rng.standard_normal((500000, 2, 3)).astype(np.float32)
+    ty, ay = upload(hpt, y, dev=dev)
+    out = hpt.Tensor.full(2.0, [500000, 3], hpt.f32, dev)
+    ty.sum_([1], False, False, out)
+    assert_close(out.numpy(), ay.astype(np.float64).sum(1) + 2.0, F32_RTOL, F32_ATOL, "sum_ accumulate, small groups")
+    b = rng.integers(0, 2, (900001, 3, 5)).astype(np.bool_)
+    tb, ab = upload(hpt, b, dev=dev)
+    assert np.array_equal(tb.all([1]).numpy(), ab.all(1)) and np.array_equal(tb.any([1]).numpy(), ab.any(1))
+
+
 def test_reduction_over_the_last_axis_of_a_permuted_view(hpt, orc, dev):
     """x.permute(2, 1, 0).sum(2): the first kept dim is the contiguous one. The lanes run along it and
     the outputs are scattered (one launch, and the two-stage form with its second-stage remap)."""
