@@ -751,6 +751,26 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
         // When it is in the input too, three passes spread over the whole chip: partial statistics
         // (lanes along the inner dim, the axis dealt over wavefronts and workgroups), finalize, apply.
         const int nk = p.kept_in.n;
+        // Small groups laid back to back (a contiguous [batch, cols, L] tensor with cols * L elements of at
+        // most 2 KiB: softmax over 4 heads of 64, over the 2 of [N, 2, 3]): lanes along L would idle and a
+        // lane per (batch, inner) pair reads single elements at a stride. A workgroup stages 16 KiB of whole
+        // groups in LDS with aligned vectors, one lane per pair normalises its column there, and the
+        // tile leaves as it came.
+        if (nk == 2 && max_vec > 1 && p.cols >= 2 && sa == p.kept_in.size[1] && p.kept_in.stride[1] == 1 &&
+            p.kept_out.stride[1] == 1 && p.kept_in.size[1] == p.out_axis_stride &&
+            p.kept_in.stride[0] == p.cols * sa && p.kept_out.stride[0] == p.cols * sa &&
+            p.cols * sa * (int64_t)elem_size <= 2048 && sa * (int64_t)elem_size < 512 && p.kept_in.size[0] >= 1024 &&
+            p.rows * p.cols * (int64_t)elem_size >= (4ll << 20) && (((uintptr_t)in_data | (uintptr_t)out_data) & 15) == 0) {
+            int64_t groups = (16 << 10) / (p.cols * sa * (int64_t)elem_size);
+            groups -= groups % max_vec;  // tiles start on 16-byte boundaries
+            if (groups >= max_vec) {
+                p.kind = NormKind::Col;
+                p.inner = p.out_axis_stride;
+                p.group_tile = (int)groups;
+                p.vec = max_vec;
+                return p;
+            }
+        }
         if (nk >= 1 && nk <= 2 && p.kept_in.stride[nk - 1] == 1 && p.kept_out.stride[nk - 1] == 1 &&
             p.kept_in.size[nk - 1] == p.out_axis_stride && p.kept_in.size[nk - 1] <= (1 << 30) && p.cols <= (1 << 30) &&
             (nk == 1 || p.kept_in.size[0] <= 65535)) {
@@ -845,6 +865,7 @@ void demote_to_generic(NormPlan& p) {
     p.kind = NormKind::Generic;
     p.raw_rows = 0;
     p.lds_rows = 0;
+    p.group_tile = 0;
     p.gb_lds = 0;
     p.tile_rows = 0;
     p.flat_t = 0;
@@ -862,7 +883,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg) ? "-unaligned" : (p.raw_rows ? "-raw-shift" : (p.lds_rows ? "-lds-shift" : "-shift"))) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : "", (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg) ? "-unaligned" : (p.raw_rows ? "-raw-shift" : (p.lds_rows ? "-lds-shift" : "-shift"))) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.group_tile ? "-group-tile" : ""), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     describe_dims(s, "rows_in", p.kept_in);

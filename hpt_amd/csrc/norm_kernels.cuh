@@ -762,6 +762,100 @@ __global__ void __launch_bounds__(256) norm_tile_kernel(const NormArgs a) {
     }
 }
 
+// ---- small [cols, L] groups laid back to back: softmax over the middle axis through LDS --------
+// A contiguous [batch, cols, L] tensor with cols * L small ([N, 4, 64], [N, 2, 3], [B, T, 4, 12]),
+// softmax over cols: a workgroup brings a.rpb whole groups (16 KiB, a multiple of VEC groups) into
+// LDS with aligned 128-bit loads, one lane per (group, inner position) normalises its column of
+// `cols` elements at stride L in place, and the tile leaves with aligned 128-bit stores.
+template <int KIND, class T, int VEC, bool PADDED>
+__global__ void __launch_bounds__(256) norm_group_tile_kernel(const NormArgs a, int L, int64_t batch) {
+    constexpr bool padded = PADDED;
+    static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX, "a softmax kernel");
+    using CT = typename Elem<T>::Wide;
+    constexpr bool kLog = norm_is_log(KIND);
+    constexpr int NV = 4;  // vectors per thread: 256 * 4 * 16 bytes = 16 KiB
+    // The tile is kept with one pad slot of 4 bytes (one 8-byte element) after every 128 bytes: the lanes
+    // of a wavefront walk columns whose starts are a whole group apart, and a group of 128 bytes or a
+    // multiple would put them all on the same LDS bank.
+    constexpr int PER = 128 / sizeof(T);                     // elements between pad slots
+    constexpr int PAD = sizeof(T) >= 4 ? 1 : 4 / sizeof(T);  // elements per pad slot
+    // (PADDED only where the groups' starts would collide: the pad costs the vector LDS accesses)
+    auto pad = [](int e) { return PADDED ? e + e / PER * PAD : e; };
+    __shared__ __align__(16) unsigned char tile_raw[256 * NV * 16 + (256 * NV * 16 / 128) * 8];
+    T* tile = reinterpret_cast<T*>(tile_raw);
+    const int t = threadIdx.x;
+    const int C = (int)a.cols;
+    const int G = C * L;
+    const int64_t g0 = (int64_t)blockIdx.x * a.rpb;
+    const int64_t left = batch - g0;
+    const int ngroups = left < a.rpb ? (int)left : a.rpb;
+    const int n = ngroups * G;
+    const T* src = (const T*)a.in + g0 * G;
+    T* dst = (T*)a.out + g0 * G;
+    {
+        Pack<T, VEC> v[NV];
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int e = (t + u * 256) * VEC;
+            if (e + VEC <= n) {
+                v[u] = load_pack_stream<T, VEC>(src + e);
+            } else {  // the tensor's last, partial vector
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    if (e + j < n) v[u].v[j] = src[e + j];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int e = (t + u * 256) * VEC;
+            if (e < n) {
+                if constexpr (!padded) {
+                    store_pack<T, VEC>(tile + e, v[u]);
+                } else {
+                    T* q = tile + pad(e);  // a 16-byte vector never straddles a pad slot
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) q[j] = v[u].v[j];
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const int npos = ngroups * L;
+    for (int o = t; o < npos; o += 256) {
+        const int g = o / L, i = o - g * L;
+        const int base = g * G + i;
+        CT m = neg_inf<CT>();
+        for (int c = 0; c < C; ++c) m = MaxC<CT>::comb(m, Elem<T>::widen(tile[pad(base + c * L)]));
+        CT s = 0;
+        for (int c = 0; c < C; ++c) s += exp_ct<T>(Elem<T>::widen(tile[pad(base + c * L)]) - m);
+        const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
+        for (int c = 0; c < C; ++c) {
+            T* q = tile + pad(base + c * L);
+            const CT d = Elem<T>::widen(*q) - m;
+            *q = Elem<T>::narrow(kLog ? d - k : exp_ct<T>(d) * k);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int e = (t + u * 256) * VEC;
+        if (e + VEC <= n) {
+            Pack<T, VEC> o;
+            if constexpr (!padded) {
+                o = load_pack<T, VEC>(tile + e);
+            } else {
+                const T* q = tile + pad(e);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) o.v[j] = q[j];
+            }
+            store_pack_stream<T, VEC>(dst + e, o);
+        } else {
+            for (int j = 0; j < VEC; ++j)
+                if (e + j < n) dst[e + j] = tile[pad(e + j)];
+        }
+    }
+}
+
 // ---- streaming rows: online statistics, then a second sweep ------------------
 
 // running (max, sum of exp(x - max)); the sum may be carried in a wider type ST

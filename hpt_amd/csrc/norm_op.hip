@@ -193,6 +193,20 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
     a.inv_cols = 1.0 / (double)p.cols;
     dim3 grid((unsigned)((p.rows + p.rpb - 1) / p.rpb));
     dim3 block((unsigned)(p.tpr * p.rpb));
+    if (p.kind == NormKind::Col && p.group_tile > 0) {
+        if constexpr (FULL > 1 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX)) {
+            const int64_t batch = p.kept_in.size[0];
+            a.rpb = p.group_tile;
+            // a very narrow inner dim with groups of a multiple of 128 bytes: the lanes' group starts collide in LDS
+            const bool padded = p.kept_in.size[1] * (int64_t)sizeof(T) <= 16 && (p.cols * p.kept_in.size[1] * (int64_t)sizeof(T)) % 128 == 0;
+            const dim3 ggrid((unsigned)((batch + p.group_tile - 1) / p.group_tile));
+            if (padded) norm_group_tile_kernel<KIND, T, FULL, true><<<ggrid, dim3(256), 0, st>>>(a, (int)p.kept_in.size[1], batch);
+            else norm_group_tile_kernel<KIND, T, FULL, false><<<ggrid, dim3(256), 0, st>>>(a, (int)p.kept_in.size[1], batch);
+        } else {
+            fail(HPT_ERR_KERNEL, "group tiles are a softmax plan");
+        }
+        return;
+    }
     if (p.kind == NormKind::RowSplit) {
         if constexpr (norm_is_causal(KIND)) {
             fail(HPT_ERR_KERNEL, "row-split has no causal form");

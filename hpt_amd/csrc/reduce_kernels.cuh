@@ -404,12 +404,20 @@ struct GroupTileArgs {
     int init_out;
 };
 
-template <class Op, int VEC>
+template <class Op, int VEC, bool PADDED>
 __global__ void __launch_bounds__(256) group_tile_kernel(const GroupTileArgs a) {
+    constexpr bool padded = PADDED;
     using T = typename Op::In;
     using Acc = typename Op::Acc;
     constexpr int NV = 4;  // vectors per thread: 256 * 4 * 16 bytes = 16 KiB
-    __shared__ __align__(16) unsigned char tile_raw[256 * NV * 16];
+    // One pad slot of 4 bytes (one 8-byte element) after every 128 bytes of the tile: the lanes of a
+    // wavefront start whole groups apart, and a group of 128 bytes or a multiple would put them all on
+    // the same LDS bank.
+    constexpr int PER = 128 / sizeof(T);                     // elements between pad slots
+    constexpr int PAD = sizeof(T) >= 4 ? 1 : 4 / sizeof(T);  // elements per pad slot
+    // (PADDED only where the groups' starts would collide: the pad costs the vector LDS accesses)
+    auto pad = [](int e) { return PADDED ? e + e / PER * PAD : e; };
+    __shared__ __align__(16) unsigned char tile_raw[256 * NV * 16 + (256 * NV * 16 / 128) * 8];
     T* tile = reinterpret_cast<T*>(tile_raw);
     const int t = threadIdx.x;
     const int G = a.R * a.kin;
@@ -433,15 +441,23 @@ __global__ void __launch_bounds__(256) group_tile_kernel(const GroupTileArgs a) 
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
         const int e = (t + u * 256) * VEC;
-        if (e < n) store_pack<T, VEC>(tile + e, v[u]);
+        if (e < n) {
+            if constexpr (!padded) {
+                store_pack<T, VEC>(tile + e, v[u]);
+            } else {
+                T* q = tile + pad(e);  // a 16-byte vector never straddles a pad slot
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) q[j] = v[u].v[j];
+            }
+        }
     }
     __syncthreads();
     const int nout = ngroups * a.kin;
     for (int o = t; o < nout; o += 256) {
         const int g = o / a.kin, i = o - g * a.kin;
-        const T* p = tile + g * G + i;
+        const int base = g * G + i;
         Acc acc = Op::identity();
-        for (int r = 0; r < a.R; ++r) fold_in<Op>(acc, p[r * a.kin], r);
+        for (int r = 0; r < a.R; ++r) fold_in<Op>(acc, tile[pad(base + r * a.kin)], r);
         write_out<Op>(a.out, g0 * a.kin + o, acc, a.init_out, a.count);
     }
 }
@@ -928,7 +944,14 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.kin = (int)p.kept.size[1];
             a.groups_per_wg = p.group_tile;
             a.init_out = init_out;
-            group_tile_kernel<Op, FULL><<<dim3((unsigned)((a.groups + p.group_tile - 1) / p.group_tile)), dim3(256), 0, st>>>(a);
+            // a narrow inner dim with groups of a multiple of 32 bytes: the lanes' group starts collide in LDS
+            // (a very narrow inner dim with groups of a multiple of 128 bytes: 16 or more of a wavefront's lanes
+            // would start on the same LDS bank. Measured: f32 [N, 16, 2] softmax 2.2 -> 5.8 TB/s padded; wider inner
+            // dims or other group sizes lose up to a quarter to the pad's scalar LDS accesses.)
+            const bool padded = a.kin * (int)sizeof(T) <= 16 && (a.R * a.kin * (int)sizeof(T)) % 128 == 0;
+            const dim3 grid((unsigned)((a.groups + p.group_tile - 1) / p.group_tile));
+            if (padded) group_tile_kernel<Op, FULL, true><<<grid, dim3(256), 0, st>>>(a);
+            else group_tile_kernel<Op, FULL, false><<<grid, dim3(256), 0, st>>>(a);
         }
         return;
     }

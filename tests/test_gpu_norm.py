@@ -531,7 +531,6 @@ CHANNEL_CASES = [
     ("bf16 [3, 64, 30000] axis 1", "bf16", [3, 64, 30000], 1),
     ("f32 [2, 10, 33333] axis 1 (odd inner length)", np.float32, [2, 10, 33333], 1),
     ("f64 [2, 30, 40000] axis 1", np.float64, [2, 30, 40000], 1),
-    ("f32 [60000, 16, 2] axis 1 (many batches)", np.float32, [60000, 16, 2], 1),
     # longer axes: 2 ... 16 thread rows share an inner position and meet in LDS
     ("f32 [24, 128, 56, 56] axis 1 (8 thread rows)", np.float32, [24, 128, 56, 56], 1),
     ("f16 [2, 300, 40000] axis 1 (16 thread rows)", np.float16, [2, 300, 40000], 1),
@@ -546,10 +545,22 @@ CHANNEL_CASES = [
 ]
 
 
-@pytest.mark.parametrize("case", CHANNEL_CASES, ids=[c[0] for c in CHANNEL_CASES])
+GROUP_CASES = [
+    ("f32 [60000, 16, 2] axis 1", np.float32, [60000, 16, 2], 1),
+    ("f16 [600, 128, 4, 64] axis 2 (heads)", np.float16, [600, 128, 4, 64], 2),
+    ("f16 [3, 65537, 4, 12] axis 2", np.float16, [3, 65537, 4, 12], 2),
+    ("bf16 [8191, 129, 8, 3] axis 2", "bf16", [8191, 129, 8, 3], 2),
+    ("f32 [700001, 2, 3] axis 1", np.float32, [700001, 2, 3], 1),
+    ("f16 [4097, 12, 96, 5] axis 2 (a long axis in a small group)", np.float16, [4097, 12, 96, 5], 2),
+    ("f64 [90001, 5, 7] axis 1", np.float64, [90001, 5, 7], 1),
+]
+
+
+@pytest.mark.parametrize("case", CHANNEL_CASES + GROUP_CASES, ids=[c[0] for c in CHANNEL_CASES + GROUP_CASES])
 def test_softmax_over_a_short_strided_axis_in_registers(hpt, orc, dev, case):
     """softmax over the channels of [B, C, H, W], C <= 64: every thread keeps the whole axis of its
-    inner positions in registers (one read, one write)."""
+    inner positions in registers (one read, one write). Small [C, L] groups laid back to back go
+    through LDS tiles instead (one lane per inner position of a group)."""
     name, npdt, shape, axis = case
     rng = np.random.default_rng(212)
     x = (rng.standard_normal(shape) * 3).astype(np.float32)
@@ -564,7 +575,8 @@ def test_softmax_over_a_short_strided_axis_in_registers(hpt, orc, dev, case):
         cv, dt, odt, bits, tof, acc = (lambda v: v.astype(npdt)), None, None, 0, (lambda v: v), orc.ACC_F64
     a = cv(x)
     t = hpt.Tensor.from_numpy(a, dt).to_hip(dev)
-    assert hpt.normalize_plan(t, axis).startswith("col-reg"), hpt.normalize_plan(t, axis)
+    want_plan = "col-group-tile" if case in GROUP_CASES else "col-reg"
+    assert hpt.normalize_plan(t, axis).startswith(want_plan), hpt.normalize_plan(t, axis)
     for log in (False, True):
         got = tof((t.log_softmax(axis) if log else t.softmax(axis)).numpy())
         want = tof(orc.softmax(a, axis, log=log, acc=acc, dtype=odt))
