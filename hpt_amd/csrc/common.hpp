@@ -144,6 +144,7 @@ struct NormPlan {
     int64_t inner = 1;  // Col: size of the contiguous inner dim the lanes walk
     int sstride = 1;    // RowReg: 2 = the row's elements sit at every second position of full vectors
     int flat_t = 0;     // ColSplit, > 0: a narrow inner dim; the slab is walked as a flat array by this many threads
+    int slab_tile = 0;  // Col softmax over the middle axis of mid-sized contiguous [cols, L] slabs with a narrow L: one workgroup per slab through LDS (the value: lanes per column)
     int group_tile = 0; // Col softmax over a short middle axis of small contiguous [cols, L] groups: this many groups per workgroup through LDS
     int lds_rows = 0;   // RowReg softmax of 4-byte types, 32769 ... 65536 elements per row: half the row in registers, half in LDS
     int raw_rows = 0;   // RowReg softmax of 2-byte types, 32769 ... 131072 elements per row: only the raw row stays in registers

@@ -771,6 +771,24 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 return p;
             }
         }
+        // Mid-sized slabs with a very narrow inner dim ([B, 1000, 3], [B, 2048, 5]): one workgroup per slab through LDS.
+        // (From 16 bytes of inner dim on the register kernel, which serves axes up to 1024, is as fast or faster:
+        // f32 [2048, 1024, 8] 4.0 against 2.6 TB/s; beyond 1024 the alternative is the three-pass flat walk.)
+        if (nk == 2 && max_vec > 1 && p.cols > 64 && sa == p.kept_in.size[1] && p.kept_in.stride[1] == 1 &&
+            p.kept_out.stride[1] == 1 && p.kept_in.size[1] == p.out_axis_stride &&
+            p.kept_in.stride[0] == p.cols * sa && p.kept_out.stride[0] == p.cols * sa &&
+            p.cols * sa * (int64_t)elem_size <= (64 << 10) && sa * (int64_t)elem_size <= (p.cols > 1024 ? 32 : 12) && p.kept_in.size[0] >= 256 &&
+            p.rows * p.cols * (int64_t)elem_size >= (4ll << 20) && ((uintptr_t)in_data % elem_size) == 0 &&
+            ((uintptr_t)out_data % elem_size) == 0) {
+            p.kind = NormKind::Col;
+            p.inner = p.out_axis_stride;
+            // lanes per column: as many as 256 threads leave for each of the L columns, a wavefront at most
+            int64_t tpc = 64;
+            while (tpc > 1 && tpc * sa > 256) tpc >>= 1;
+            p.slab_tile = (int)tpc;
+            p.vec = max_vec;
+            return p;
+        }
         if (nk >= 1 && nk <= 2 && p.kept_in.stride[nk - 1] == 1 && p.kept_out.stride[nk - 1] == 1 &&
             p.kept_in.size[nk - 1] == p.out_axis_stride && p.kept_in.size[nk - 1] <= (1 << 30) && p.cols <= (1 << 30) &&
             (nk == 1 || p.kept_in.size[0] <= 65535)) {
@@ -866,6 +884,7 @@ void demote_to_generic(NormPlan& p) {
     p.raw_rows = 0;
     p.lds_rows = 0;
     p.group_tile = 0;
+    p.slab_tile = 0;
     p.gb_lds = 0;
     p.tile_rows = 0;
     p.flat_t = 0;
@@ -883,7 +902,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg) ? "-unaligned" : (p.raw_rows ? "-raw-shift" : (p.lds_rows ? "-lds-shift" : "-shift"))) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.group_tile ? "-group-tile" : ""), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg) ? "-unaligned" : (p.raw_rows ? "-raw-shift" : (p.lds_rows ? "-lds-shift" : "-shift"))) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.group_tile ? "-group-tile" : (p.slab_tile ? "-slab" : "")), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     describe_dims(s, "rows_in", p.kept_in);

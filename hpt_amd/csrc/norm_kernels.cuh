@@ -856,6 +856,51 @@ __global__ void __launch_bounds__(256) norm_group_tile_kernel(const NormArgs a, 
     }
 }
 
+// ---- mid-sized [cols, L] slabs with a narrow inner dim: one workgroup per slab, through LDS -----
+// softmax over the middle axis of a contiguous [batch, cols, L] with L narrow (3 ... 64 elements) and
+// slabs of 2 ... 64 KiB ([B, 1000, 3], [B, 768, 60], [B, 1024, 33]: attention pooling over a
+// sequence with a few heads). Lanes along L idle, a lane per inner position holds up to 64 values
+// and reads 2-byte pieces. Here a workgroup brings its whole slab into LDS with 128-bit loads
+// (unaligned when the slab starts off a 16-byte boundary), groups of `tpc` lanes share a column
+// and walk it at stride L, and the slab leaves with 128-bit stores.
+template <int KIND, class T, int VEC>
+__global__ void __launch_bounds__(256) norm_slab_kernel(const NormArgs a, int L, int tpc_log2) {
+    static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX, "a softmax kernel");
+    using CT = typename Elem<T>::Wide;
+    constexpr bool kLog = norm_is_log(KIND);
+    extern __shared__ __align__(16) unsigned char slab_raw[];
+    T* tile = reinterpret_cast<T*>(slab_raw);
+    const int t = threadIdx.x;
+    const int C = (int)a.cols;
+    const int n = C * L;
+    const T* src = (const T*)a.in + (int64_t)blockIdx.x * n;
+    T* dst = (T*)a.out + (int64_t)blockIdx.x * n;
+    const int nvec = n / VEC;
+    for (int iv = t; iv < nvec; iv += 256) store_pack<T, VEC>(tile + iv * VEC, load_pack_unaligned<T, VEC>(src + iv * VEC));
+    for (int e = nvec * VEC + t; e < n; e += 256) tile[e] = src[e];
+    __syncthreads();
+    const int tpc = 1 << tpc_log2;
+    const int lane = t & (tpc - 1);
+    const int ngrp = 256 >> tpc_log2;
+    for (int i = t >> tpc_log2; i < L; i += ngrp) {
+        T* p = tile + i;
+        CT m = neg_inf<CT>();
+        for (int c = lane; c < C; c += tpc) m = MaxC<CT>::comb(m, Elem<T>::widen(p[c * L]));
+        m = group_reduce<MaxC<CT>>(m, tpc);
+        CT s = 0;
+        for (int c = lane; c < C; c += tpc) s += exp_ct<T>(Elem<T>::widen(p[c * L]) - m);
+        s = group_reduce<SumC<CT>>(s, tpc);
+        const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
+        for (int c = lane; c < C; c += tpc) {
+            const CT d = Elem<T>::widen(p[c * L]) - m;
+            p[c * L] = Elem<T>::narrow(kLog ? d - k : exp_ct<T>(d) * k);
+        }
+    }
+    __syncthreads();
+    for (int iv = t; iv < nvec; iv += 256) store_pack_unaligned<T, VEC>(dst + iv * VEC, load_pack<T, VEC>(tile + iv * VEC));
+    for (int e = nvec * VEC + t; e < n; e += 256) dst[e] = tile[e];
+}
+
 // ---- streaming rows: online statistics, then a second sweep ------------------
 
 // running (max, sum of exp(x - max)); the sum may be carried in a wider type ST

@@ -193,6 +193,16 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
     a.inv_cols = 1.0 / (double)p.cols;
     dim3 grid((unsigned)((p.rows + p.rpb - 1) / p.rpb));
     dim3 block((unsigned)(p.tpr * p.rpb));
+    if (p.kind == NormKind::Col && p.slab_tile > 0) {
+        if constexpr (FULL > 1 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX)) {
+            const int L = (int)p.kept_in.size[1];
+            const size_t bytes = ((size_t)p.cols * L * sizeof(T) + 15) / 16 * 16;
+            norm_slab_kernel<KIND, T, FULL><<<dim3((unsigned)p.kept_in.size[0]), dim3(256), bytes, st>>>(a, L, ilog2(p.slab_tile));
+        } else {
+            fail(HPT_ERR_KERNEL, "slab tiles are a softmax plan");
+        }
+        return;
+    }
     if (p.kind == NormKind::Col && p.group_tile > 0) {
         if constexpr (FULL > 1 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX)) {
             const int64_t batch = p.kept_in.size[0];

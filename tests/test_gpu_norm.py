@@ -476,8 +476,8 @@ FLAT_COLUMN_CASES = [
     ("f16 [257, 13988, 7] axis 1 (misaligned slabs)", np.float16, [257, 13988, 7], 1),
     ("f32 [31, 70001, 3] axis 1 (misaligned slabs)", np.float32, [31, 70001, 3], 1),
     # many small slabs: fewer threads per slab, so that each is still worth two periods
-    ("f32 [700, 2048, 3] axis 1 (24 KiB slabs)", np.float32, [700, 2048, 3], 1),
-    ("f16 [600, 1031, 7] axis 1 (small misaligned slabs)", np.float16, [600, 1031, 7], 1),
+    ("f32 [300, 6000, 3] axis 1 (72 KiB slabs)", np.float32, [300, 6000, 3], 1),
+    ("f16 [200, 5031, 7] axis 1 (small misaligned slabs)", np.float16, [200, 5031, 7], 1),
 ]
 
 
@@ -556,11 +556,22 @@ GROUP_CASES = [
 ]
 
 
-@pytest.mark.parametrize("case", CHANNEL_CASES + GROUP_CASES, ids=[c[0] for c in CHANNEL_CASES + GROUP_CASES])
+SLAB_CASES = [
+    ("f16 [900, 1000, 3] axis 1", np.float16, [900, 1000, 3], 1),
+    ("f32 [300, 1092, 5] axis 1 (slabs off 16-byte boundaries)", np.float32, [300, 1092, 5], 1),
+    ("bf16 [260, 2047, 16] axis 1 (64 KiB slabs)", "bf16", [260, 2047, 16], 1),
+    ("f32 [1200, 500, 2] axis 1", np.float32, [1200, 500, 2], 1),
+    ("f64 [300, 1100, 3] axis 1", np.float64, [300, 1100, 3], 1),
+    ("f16 [2, 300, 2049, 7] axis 2 (odd slab size)", np.float16, [2, 300, 2049, 7], 2),
+]
+
+
+@pytest.mark.parametrize("case", CHANNEL_CASES + GROUP_CASES + SLAB_CASES, ids=[c[0] for c in CHANNEL_CASES + GROUP_CASES + SLAB_CASES])
 def test_softmax_over_a_short_strided_axis_in_registers(hpt, orc, dev, case):
     """softmax over the channels of [B, C, H, W], C <= 64: every thread keeps the whole axis of its
     inner positions in registers (one read, one write). Small [C, L] groups laid back to back go
-    through LDS tiles instead (one lane per inner position of a group)."""
+    through LDS tiles instead (one lane per inner position of a group), mid-sized slabs with a narrow
+    inner dim one workgroup per slab (groups of lanes per column)."""
     name, npdt, shape, axis = case
     rng = np.random.default_rng(212)
     x = (rng.standard_normal(shape) * 3).astype(np.float32)
@@ -575,7 +586,7 @@ def test_softmax_over_a_short_strided_axis_in_registers(hpt, orc, dev, case):
         cv, dt, odt, bits, tof, acc = (lambda v: v.astype(npdt)), None, None, 0, (lambda v: v), orc.ACC_F64
     a = cv(x)
     t = hpt.Tensor.from_numpy(a, dt).to_hip(dev)
-    want_plan = "col-group-tile" if case in GROUP_CASES else "col-reg"
+    want_plan = "col-group-tile" if case in GROUP_CASES else "col-slab" if case in SLAB_CASES else "col-reg"
     assert hpt.normalize_plan(t, axis).startswith(want_plan), hpt.normalize_plan(t, axis)
     for log in (False, True):
         got = tof((t.log_softmax(axis) if log else t.softmax(axis)).numpy())
