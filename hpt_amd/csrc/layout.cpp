@@ -810,6 +810,12 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     const int64_t ty = pow2_ceil((p.cols + nc_max - 1) / nc_max);
                     // enough threads to fill the chip: inner positions x thread rows
                     if (!(ty <= 16 && p.rows / ev * ty >= 8 * 1024)) continue;
+                    // (a long axis of two-byte elements that only fits with sixteen thread rows of 4-byte pieces: the
+                    // three-pass flat walk is faster, f16 [512, 768, 60] 1.3 -> 2.1 TB/s, [768, 1024, 33] 1.0 -> 2.3;
+                    // f32 single elements are not: [2048, 1024, 8] 4.0 against 2.3)
+                    if (ty == 16 && elem_size == 2 && ev <= 2 && sa == L && L <= 1024 * max_vec &&
+                        batch * p.cols * L * (int64_t)elem_size >= (8ll << 20))
+                        continue;
                     if (L % ev == 0 && sa % ev == 0 && (nk == 1 || p.kept_in.stride[0] % ev == 0) &&
                         (p.cols * L) % ev == 0 && ((uintptr_t)in_data % vb) == 0 && ((uintptr_t)out_data % vb) == 0) {
                         p.kind = NormKind::ColReg;
