@@ -308,7 +308,8 @@ def cases_c6(P):
 
 def cases_c8(P):
     """Shapes off the reference's list that the planner treats separately (~128 MiB each): short rows,
-    narrow and odd inner dims, long rows, channel softmax, batch-norm statistics."""
+    narrow and odd inner dims, long rows, channel softmax, batch-norm statistics, vocabulary rows held on
+    chip, small groups and slabs."""
     import hpt_amd as hpt
     rng = np.random.default_rng(8)
     cases = []
@@ -348,6 +349,22 @@ def cases_c8(P):
     del ts
     ts, nb = up([11184810, 3])
     nrm(ts, nb, "f32 [11184810,3]", "softmax", 0, "softmax(axis=0)", 3)
+    del ts
+    # long vocabulary rows held on chip (registers + LDS), small groups and slabs through LDS tiles
+    ts, nb = up([640, 50304])
+    nrm(ts, nb, "f32 [640,50304] (rows in registers + LDS)", "log_softmax", 1, "log_softmax(axis=1)", 640)
+    del ts
+    ts, nb = up([640, 50257])
+    nrm(ts, nb, "f32 [640,50257] (the same, odd length)", "log_softmax", 1, "log_softmax(axis=1)", 640)
+    del ts
+    ts, nb = up([131072, 8, 32])
+    red(ts, nb, "f32 [131072,8,32] (small groups)", "sum", [1], "sum(axis=1)", 131072 * 32)
+    nrm(ts, nb, "f32 [131072,8,32] (small groups)", "softmax", 1, "softmax(axis=1)", 131072 * 32)
+    del ts
+    ts, nb = up([8192, 2048, 2])
+    nrm(ts, nb, "f32 [8192,2048,2] (slabs with a narrow inner dim)", "softmax", 1, "softmax(axis=1)", 8192 * 2)
+    ts1, nb1 = up([33554403])
+    red(ts1, nb1, "f32 [33554403] (odd length)", "sum", [0], "sum(all)", 1)
     return cases
 
 
