@@ -730,6 +730,11 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 // wavefront instead of four that meet in LDS)
                 p.tpr = (int)std::min<int64_t>(1024, v > 1 ? pow2_ceil((nv + per - 1) / per) : pow2_ceil((nv + 7) / 8));
                 if (p.tpr > 64 && p.tpr < 256 && !(ln_half && p.tpr == 128)) p.tpr = 256;
+                // A row just over a power of two (4097: 1026 vectors) would take twice the threads with half of
+                // them idle: softmax (no gamma / beta beside the row) of 4-byte types takes half the threads and five
+                // vectors each. Measured (TB/s): f32 [8190, 4097] 4.6 -> 5.1, [8192, 4100] 4.6 -> 5.7, [4096, 8200]
+                // 4.1 -> 4.9, [4000, 10000] 4.7 -> 5.1; f16 [8192, 8200] loses (4.7 -> 3.0: eight widened vectors spill).
+                if (n_norm_dims <= 0 && v > 1 && elem_size >= 4 && p.tpr >= 512 && nv <= (p.tpr / 2) * 5) p.tpr /= 2;
                 int64_t nc = (nv + p.tpr - 1) / p.tpr;
                 p.nchunk = std::max(1, pow2_ceil(nc));
                 int block = std::max(256, p.tpr);

@@ -103,7 +103,7 @@ def test_plans_for_shapes_off_the_benchmark_list(hpt):
         ([1016800, 33], None, 1, 0, "rowreg+tile"), ([1016800, 33], None, 0, 1, "rowreg+tile"),
         ([262144, 128], None, 1, 0, "rowreg rows"),                 # whole vectors, 512 bytes: registers
         ([8190, 4097], None, 1, 0, "rowreg-shift"), ([1043, 50257], None, 1, 0, "rowreg-lds-shift"), ([1043, 70001], None, 1, 0, "rowstream-shift"),
-        ([3355, 10000], None, 1, 0, "rowreg rows=3355 cols=10000 vec=4 tpr=1024"),
+        ([3355, 10000], None, 1, 0, "rowreg rows=3355 cols=10000 vec=4 tpr=512 rpb=1 nchunk=8"), ([3355, 12000], None, 1, 0, "rowreg rows=3355 cols=12000 vec=4 tpr=1024"),
         ([512, 65536], None, 1, 0, "rowreg-lds"), ([512, 65540], None, 1, 0, "rowstream"), ([32, 1048576], None, 1, 0, "rowsplit"),
         ([32768, 1024], hpt.f16, 0, 1, "rowreg rows=32768 cols=1024 vec=8 tpr=64 rpb=4 nchunk=2"),
         ([32768, 1024], hpt.f32, 0, 1, "rowreg rows=32768 cols=1024 vec=4 tpr=64 rpb=4 nchunk=4"),
