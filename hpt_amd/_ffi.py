@@ -79,6 +79,8 @@ SIGNATURES = {
     "hpt_hip_normalize_plan": (C.c_int32, [C.POINTER(View), C.c_int64, C.c_int32, C.c_char_p, C.c_size_t]),
     "hpt_hip_reduce": (C.c_int32, [C.c_int32, C.c_void_p, C.c_int32, C.POINTER(View), C.POINTER(C.c_int64),
                                    C.c_int32, C.c_int32, C.POINTER(View)]),
+    "hpt_hip_reduce_static": (C.c_int32, [C.c_int32, C.c_void_p, C.c_int32, C.POINTER(View), C.POINTER(C.c_int64),
+                                          C.c_int32, C.c_int32, C.POINTER(View)]),
     "hpt_hip_argreduce": (C.c_int32, [C.c_int32, C.c_void_p, C.c_int32, C.POINTER(View), C.c_int64,
                                       C.POINTER(View)]),
     "hpt_hip_softmax": (C.c_int32, [C.c_int32, C.c_void_p, C.c_int32, C.POINTER(View), C.c_int64,

@@ -182,6 +182,29 @@ size_t scratch_need(const ReducePlan& p, size_t acc_size) {
     return p.split > 1 ? (size_t)p.K * p.split * acc_size : 0;
 }
 
+// ---- scratch that is never allocated (hpt_hip_reduce_static) ------------------------
+// Part of the library's image on every device it runs on. In host code the array's name
+// is only a handle for hipGetSymbolAddress: the device address is looked up once per
+// device, with that device current, and only that address is ever handed to a kernel.
+constexpr size_t kStaticScratchBytes = HPT_HIP_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+static std::mutex g_static_scratch_mu;
+static std::map<int, void*> g_static_scratch_ptr;
+
+// Requires `dev` to be the current device.
+static void* static_scratch_of(int dev) {
+    std::lock_guard<std::mutex> g(g_static_scratch_mu);
+    auto it = g_static_scratch_ptr.find(dev);
+    if (it != g_static_scratch_ptr.end()) return it->second;
+    void* ptr = nullptr;
+    hip_check(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)), HPT_ERR_DEVICE,
+              "hipGetSymbolAddress(scratch)");
+    if (!ptr) fail(HPT_ERR_DEVICE, "hipGetSymbolAddress(scratch) returned a null address");
+    g_static_scratch_ptr.emplace(dev, ptr);
+    return ptr;
+}
+
 // ---- dispatch tables -----------------------------------------------------------
 
 const ReduceEntry& reduce_entry_for(int e) {
@@ -292,8 +315,10 @@ static ReduceCall prepare_reduce(int entry_id, const hpt_view* in, const int64_t
     return c;
 }
 
+// use_static: the partials go to the library's static device array instead of allocated
+// scratch; a plan that needs more than the array holds is refused.
 static void run_reduce(int dev, void* stream, int entry_id, const hpt_view* in, const int64_t* axes,
-                       int naxes, int init_out, hpt_view* out) {
+                       int naxes, int init_out, hpt_view* out, bool use_static = false) {
     ReduceCall c = prepare_reduce(entry_id, in, axes, naxes);
     check_out(out, c.out_dtype, c.plan.K, "reduce output");
     if (c.plan.kind == ReduceKind::Empty) return;
@@ -301,11 +326,21 @@ static void run_reduce(int dev, void* stream, int entry_id, const hpt_view* in, 
         fail(HPT_ERR_PARAM, "reduce input: data pointer is null");
     if (!init_out && !(entry_id == HPT_SUM || entry_id == HPT_NANSUM))
         fail(HPT_ERR_PARAM, "init_out = 0 (accumulate into out) is only defined for sum and nansum");
+    const size_t pbytes = scratch_need(c.plan, c.entry->acc_size[in->dtype]);
+    if (use_static && pbytes > kStaticScratchBytes)
+        fail(HPT_ERR_MEMORY,
+             "reduce_static: this reduction needs %zu bytes of scratch, the static scratch holds %zu; "
+             "use hpt_hip_reduce",
+             pbytes, kStaticScratchBytes);
     use_device(dev);
     hipStream_t st = (hipStream_t)stream;
     ReduceLaunchFn fn = c.entry->launch[in->dtype];
-    const size_t pbytes = scratch_need(c.plan, c.entry->acc_size[in->dtype]);
-    if (pbytes) {
+    if (pbytes && use_static) {
+        ReduceScratch sc;
+        sc.partial = static_scratch_of(dev);
+        fn(c.plan, in->data, out->data, sc, st, init_out);
+        check_launch("reduce_static");
+    } else if (pbytes) {
         std::lock_guard<std::mutex> g(g_scratch_mu);
         ReduceScratch sc = scratch_for(dev, st, pbytes);
         fn(c.plan, in->data, out->data, sc, st, init_out);
@@ -540,6 +575,14 @@ int32_t hpt_hip_reduce(int32_t dev, void* stream, int32_t op, const hpt_view* in
     return guarded([&] {
         if (op < 0 || op >= HPT_REDUCE_OP_COUNT) fail(HPT_ERR_PARAM, "invalid reduce op %d", op);
         run_reduce(dev, stream, op, in, axes, naxes, init_out, out);
+    });
+}
+
+int32_t hpt_hip_reduce_static(int32_t dev, void* stream, int32_t op, const hpt_view* in, const int64_t* axes,
+                              int32_t naxes, int32_t init_out, hpt_view* out) {
+    return guarded([&] {
+        if (op < 0 || op >= HPT_REDUCE_OP_COUNT) fail(HPT_ERR_PARAM, "invalid reduce op %d", op);
+        run_reduce(dev, stream, op, in, axes, naxes, init_out, out, true);
     });
 }
 

@@ -307,7 +307,9 @@ class Tensor:
         return [out[i] for i in range(n.value)]
 
     def _reduce(self, op: int, axes, keep_dims: bool, init_out: bool = True, out: "Tensor" = None,
-                stream=None) -> "Tensor":
+                stream=None, static_scratch: bool = False) -> "Tensor":
+        """static_scratch: go through hpt_hip_reduce_static (no device allocation inside the call;
+        pass `out` as well to keep this wrapper from allocating the result)."""
         self._require_hip("reduce")
         l = _ffi.lib()
         axes = _as_axes(axes)
@@ -329,7 +331,8 @@ class Tensor:
         vin, k1 = self._c_view()
         vout, k2 = res._c_view()
         ax = _ffi.i64_array(axes)
-        check(l.hpt_hip_reduce(self.device, stream, op, C.byref(vin), ax, len(axes), int(init_out), C.byref(vout)))
+        entry = l.hpt_hip_reduce_static if static_scratch else l.hpt_hip_reduce
+        check(entry(self.device, stream, op, C.byref(vin), ax, len(axes), int(init_out), C.byref(vout)))
         del k1, k2
         return Tensor(res._storage, res.ptr, final_shape, _contiguous_strides(final_shape), res.dtype, "hip",
                       self.device)

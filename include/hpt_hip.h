@@ -183,6 +183,23 @@ int32_t hpt_hip_normalize_plan(const hpt_view* in, int64_t axis, int32_t n_norm_
 int32_t hpt_hip_reduce(int32_t dev, void* stream, int32_t op, const hpt_view* in,
                        const int64_t* axes, int32_t naxes, int32_t init_out, hpt_view* out);
 
+/* hpt_hip_reduce for callers that cannot allocate device memory. It has no counterpart in
+ * the reference: it is for code under HIP graph capture, tight serving loops and
+ * harnesses that forbid hipMalloc. Same arguments and results as hpt_hip_reduce (the
+ * same kernels run), but the partial accumulators of a reduction that is split over
+ * workgroups go to a static device array of HPT_HIP_STATIC_SCRATCH_BYTES that is part
+ * of the library's image on every device, and the call makes no allocation of any kind.
+ * A reduction whose partials need more than that is refused with HPT_ERR_MEMORY before
+ * anything is launched (hpt_hip_reduce_plan shows the split: outputs x split x
+ * accumulator size). Every call on one device shares that device's array, and nothing in
+ * it has to start from a known value (each call writes what it reads): calls on
+ * different streams of one device that overlap in time race; calls ordered by a
+ * stream or by the host do not. The array's address is looked up on the first call on a
+ * device: make that call outside any graph capture. */
+#define HPT_HIP_STATIC_SCRATCH_BYTES (4u << 20)
+int32_t hpt_hip_reduce_static(int32_t dev, void* stream, int32_t op, const hpt_view* in,
+                              const int64_t* axes, int32_t naxes, int32_t init_out, hpt_view* out);
+
 /* IndexReduce::argmax / argmin (hpt-traits/src/ops/reduce.rs:26,41; CPU
  * hpt/src/backends/cpu/utils/reduce/reduce.rs:45-170, 348-364 and
  * hpt/src/backends/cpu/kernels/argreduce_kernels.rs:2-71; device
