@@ -63,6 +63,7 @@ SIGNATURES = {
     "hpt_hip_device_count": (C.c_int32, [C.POINTER(C.c_int32)]),
     "hpt_hip_alloc": (C.c_int32, [C.c_int32, C.c_size_t, C.c_size_t, C.c_int32, C.POINTER(C.c_void_p)]),
     "hpt_hip_free": (C.c_int32, [C.c_int32, C.c_void_p, C.c_size_t, C.c_size_t]),
+    "hpt_hip_forget": (C.c_int32, [C.c_int32, C.c_void_p]),
     "hpt_hip_cache_resize": (C.c_int32, [C.c_int32, C.c_size_t]),
     "hpt_hip_cache_clear": (C.c_int32, [C.c_int32]),
     "hpt_hip_alloc_stats": (C.c_int32, [C.c_int32, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),

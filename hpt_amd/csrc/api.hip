@@ -2,7 +2,9 @@
 // caching allocator, per-stream scratch, and dispatch into the kernel tables.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstring>
+#include <memory>
 #include <list>
 #include <map>
 #include <mutex>
@@ -40,11 +42,21 @@ static void hip_check(hipError_t e, int code, const char* what) {
     if (e != hipSuccess) fail(code, "%s: %s", what, hipGetErrorString(e));
 }
 
+// Make `dev` the calling thread's device. The device count is asked for once per process and
+// hipSetDevice is skipped when the thread is already there (hipGetDevice reads a thread-local of the
+// runtime): on launch-bound calls the two runtime calls this saves are a measurable part of the
+// host time.
 static void use_device(int dev) {
-    int n = 0;
-    hip_check(hipGetDeviceCount(&n), HPT_ERR_DEVICE, "hipGetDeviceCount");
+    static std::atomic<int> count{-1};
+    int n = count.load(std::memory_order_relaxed);
+    if (n < 0) {
+        hip_check(hipGetDeviceCount(&n), HPT_ERR_DEVICE, "hipGetDeviceCount");
+        count.store(n, std::memory_order_relaxed);
+    }
     if (dev < 0 || dev >= n) fail(HPT_ERR_DEVICE, "device %d does not exist (%d visible)", dev, n);
-    hip_check(hipSetDevice(dev), HPT_ERR_DEVICE, "hipSetDevice");
+    int cur = -1;
+    if (hipGetDevice(&cur) != hipSuccess || cur != dev)
+        hip_check(hipSetDevice(dev), HPT_ERR_DEVICE, "hipSetDevice");
 }
 
 // ---- device caching allocator ------------------------------------------------
@@ -69,6 +81,7 @@ struct DeviceAllocator {
     std::map<LayoutKey, std::pair<std::list<LayoutKey>::iterator, std::vector<void*>>> cache;
     std::unordered_map<void*, LayoutKey> live;
     uint64_t device_mallocs = 0;
+    size_t internal_blocks = 0;  // live blocks the library itself holds (scratch), not a caller
 
     size_t cached_blocks() const {
         size_t n = 0;
@@ -136,6 +149,8 @@ struct DeviceAllocator {
             lru.splice(lru.begin(), lru, c->second.first);
         }
     }
+    // The caller takes the block over: it leaves the table of live blocks and is not cached.
+    bool forget(void* p) { return live.erase(p) != 0; }
     void clear() {
         while (!cache.empty()) evict_one();
     }
@@ -152,30 +167,69 @@ static DeviceAllocator& allocator_of(int dev) {
 }
 
 // ---- scratch of the multi-workgroup reductions -----------------------------------
+// One buffer per (device, stream), taken from the device's caching allocator (so that
+// hpt_hip_cache_clear and the evict-and-retry path see it) and guarded by a lock of its own:
+// calls on different streams do not wait for each other. It grows geometrically; the buffer it
+// outgrows is not handed back while work that uses it may still be queued, but parked until
+// hpt_hip_cache_clear, which waits for the device first. No call on the hot path frees device
+// memory.
+
+constexpr size_t kScratchAlign = 256;
 
 struct StreamScratch {
-    void* partial = nullptr;
-    size_t partial_bytes = 0;
+    std::mutex mu;  // held from lookup to launch by the call that uses the buffer
+    void* base = nullptr;
+    size_t bytes = 0;
+    std::vector<std::pair<void*, size_t>> retired;
 };
 
-static std::mutex g_scratch_mu;  // held from lookup to launch
-static std::map<std::pair<int, hipStream_t>, StreamScratch> g_scratch;
+static std::mutex g_scratch_table_mu;  // guards the map only
+static std::map<std::pair<int, hipStream_t>, std::unique_ptr<StreamScratch>> g_scratch;
 
-// Requires g_scratch_mu. Grows the scratch of (dev, stream); growing frees the
-// old buffer, which waits for the device to go idle first.
-static ReduceScratch scratch_for(int dev, hipStream_t st, size_t partial_bytes) {
-    StreamScratch& s = g_scratch[{dev, st}];
-    if (partial_bytes > s.partial_bytes) {
-        if (s.partial) hip_check(hipFree(s.partial), HPT_ERR_MEMORY, "hipFree(scratch)");
-        s.partial = nullptr;
-        s.partial_bytes = 0;
-        size_t want = std::max<size_t>(partial_bytes, 1u << 20);
-        hip_check(hipMalloc(&s.partial, want), HPT_ERR_MEMORY, "hipMalloc(scratch)");
-        s.partial_bytes = want;
+static StreamScratch& scratch_entry(int dev, hipStream_t st) {
+    std::lock_guard<std::mutex> g(g_scratch_table_mu);
+    auto& e = g_scratch[{dev, st}];
+    if (!e) e.reset(new StreamScratch());
+    return *e;
+}
+
+// Requires s.mu. Returns a buffer of at least `bytes`. Nothing in it has to start from a known
+// value: every kernel that reads a scratch slot runs after the kernel that wrote it, on this stream.
+static void* scratch_reserve(int dev, StreamScratch& s, size_t bytes) {
+    if (!s.base || bytes > s.bytes) {
+        const size_t want = std::max<size_t>({bytes, s.bytes * 2, (size_t)1 << 20});
+        DeviceAllocator& a = allocator_of(dev);
+        void* p;
+        {
+            std::lock_guard<std::mutex> g(a.mu);
+            p = a.allocate(want, kScratchAlign);
+            ++a.internal_blocks;
+        }
+        if (s.base) s.retired.emplace_back(s.base, s.bytes);
+        s.base = p;
+        s.bytes = want;
     }
-    ReduceScratch r;
-    r.partial = s.partial;
-    return r;
+    return s.base;
+}
+
+// Give every scratch buffer of `dev` back to its allocator. The caller has made the device idle.
+static void scratch_release_all(int dev) {
+    std::lock_guard<std::mutex> gt(g_scratch_table_mu);
+    DeviceAllocator& a = allocator_of(dev);
+    for (auto& kv : g_scratch) {
+        if (kv.first.first != dev) continue;
+        StreamScratch& s = *kv.second;
+        std::lock_guard<std::mutex> gs(s.mu);
+        std::lock_guard<std::mutex> ga(a.mu);
+        if (s.base) s.retired.emplace_back(s.base, s.bytes);
+        for (auto& r : s.retired) {
+            a.deallocate(r.first, r.second, kScratchAlign);
+            --a.internal_blocks;
+        }
+        s.retired.clear();
+        s.base = nullptr;
+        s.bytes = 0;
+    }
 }
 
 size_t scratch_need(const ReducePlan& p, size_t acc_size) {
@@ -289,6 +343,39 @@ static void check_out(const hpt_view* out, int dtype, int64_t count, const char*
              (long long)view_size(out));
 }
 
+// The bytes a view can touch: [lo, hi) around its data pointer.
+static void view_extent(const hpt_view* v, const char** lo, const char** hi) {
+    const int64_t es = (int64_t)dtype_size(v->dtype);
+    int64_t below = 0, above = 0;
+    for (int i = 0; i < v->ndim; ++i) {
+        const int64_t span = (v->shape[i] - 1) * v->strides[i];
+        if (span < 0) below += span;
+        else above += span;
+    }
+    *lo = (const char*)v->data + below * es;
+    *hi = (const char*)v->data + (above + 1) * es;
+}
+
+// `out` must not share memory with `in`. With allow_same, `out` may be `in` itself: the same
+// pointer, dtype and contiguous layout, where every element is read before it is written by the
+// thread that writes it. Anything else (a permuted, sliced, stepped or shifted view of out's
+// buffer) would be read and written in different orders by different workgroups.
+static void check_alias(const hpt_view* in, const hpt_view* out, bool allow_same, const char* what,
+                        const char* in_name) {
+    if (!in || !in->data || !out->data) return;
+    if (view_size(in) == 0 || view_size(out) == 0) return;
+    const char *ilo, *ihi, *olo, *ohi;
+    view_extent(in, &ilo, &ihi);
+    view_extent(out, &olo, &ohi);
+    if (!(ilo < ohi && olo < ihi)) return;
+    bool same = allow_same && in->data == out->data && in->dtype == out->dtype && in->ndim == out->ndim &&
+                view_contiguous(in);
+    for (int i = 0; same && i < in->ndim; ++i) same = in->shape[i] == out->shape[i];
+    if (!same)
+        fail(HPT_ERR_PARAM, "%s: out overlaps %s%s", what, in_name,
+             allow_same ? " without being that very tensor (same pointer and contiguous layout)" : "");
+}
+
 static void check_launch(const char* what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) fail(HPT_ERR_KERNEL, "%s: kernel launch failed: %s", what, hipGetErrorString(e));
@@ -321,6 +408,7 @@ static void run_reduce(int dev, void* stream, int entry_id, const hpt_view* in, 
                        int naxes, int init_out, hpt_view* out, bool use_static = false) {
     ReduceCall c = prepare_reduce(entry_id, in, axes, naxes);
     check_out(out, c.out_dtype, c.plan.K, "reduce output");
+    check_alias(in, out, false, "reduce", "the input");
     if (c.plan.kind == ReduceKind::Empty) return;
     if (!in->data && c.plan.kind != ReduceKind::Identity)
         fail(HPT_ERR_PARAM, "reduce input: data pointer is null");
@@ -341,8 +429,10 @@ static void run_reduce(int dev, void* stream, int entry_id, const hpt_view* in, 
         fn(c.plan, in->data, out->data, sc, st, init_out);
         check_launch("reduce_static");
     } else if (pbytes) {
-        std::lock_guard<std::mutex> g(g_scratch_mu);
-        ReduceScratch sc = scratch_for(dev, st, pbytes);
+        StreamScratch& s = scratch_entry(dev, st);
+        std::lock_guard<std::mutex> g(s.mu);
+        ReduceScratch sc;
+        sc.partial = scratch_reserve(dev, s, pbytes);
         fn(c.plan, in->data, out->data, sc, st, init_out);
         check_launch("reduce");
     } else {
@@ -391,8 +481,9 @@ static NormCall prepare_norm(const hpt_view* in, const void* out_data, int64_t a
 // the per-stream buffer, held under its lock from lookup to launch.
 static void launch_norm(int dev, hipStream_t st, NormLaunchFn fn, NormCall& c, const char* what) {
     if (c.plan.scratch_bytes) {
-        std::lock_guard<std::mutex> g(g_scratch_mu);
-        c.args.scratch = scratch_for(dev, st, c.plan.scratch_bytes).partial;
+        StreamScratch& s = scratch_entry(dev, st);
+        std::lock_guard<std::mutex> g(s.mu);
+        c.args.scratch = scratch_reserve(dev, s, c.plan.scratch_bytes);
         fn(c.plan, c.args, st);
         check_launch(what);
     } else {
@@ -449,6 +540,15 @@ int32_t hpt_hip_free(int32_t dev, void* p, size_t bytes, size_t align) {
     });
 }
 
+int32_t hpt_hip_forget(int32_t dev, void* p) {
+    return guarded([&] {
+        if (!p) return;
+        DeviceAllocator& a = allocator_of(dev);
+        std::lock_guard<std::mutex> g(a.mu);
+        (void)a.forget(p);  // a pointer the allocator does not know is left alone, as in the reference
+    });
+}
+
 int32_t hpt_hip_cache_resize(int32_t dev, size_t entries) {
     return guarded([&] {
         use_device(dev);
@@ -462,6 +562,9 @@ int32_t hpt_hip_cache_resize(int32_t dev, size_t entries) {
 int32_t hpt_hip_cache_clear(int32_t dev) {
     return guarded([&] {
         use_device(dev);
+        // the scratch buffers go back first; work that uses them may still be queued
+        hip_check(hipDeviceSynchronize(), HPT_ERR_KERNEL, "hipDeviceSynchronize");
+        scratch_release_all(dev);
         DeviceAllocator& a = allocator_of(dev);
         std::lock_guard<std::mutex> g(a.mu);
         a.clear();
@@ -473,7 +576,7 @@ int32_t hpt_hip_alloc_stats(int32_t dev, uint64_t* live_blocks, uint64_t* cached
     return guarded([&] {
         DeviceAllocator& a = allocator_of(dev);
         std::lock_guard<std::mutex> g(a.mu);
-        if (live_blocks) *live_blocks = a.live.size();
+        if (live_blocks) *live_blocks = a.live.size() - a.internal_blocks;
         if (cached_blocks) *cached_blocks = a.cached_blocks();
         if (device_mallocs) *device_mallocs = a.device_mallocs;
     });
@@ -604,6 +707,7 @@ int32_t hpt_hip_softmax(int32_t dev, void* stream, int32_t log, const hpt_view* 
     return guarded([&] {
         check_view(in, "softmax input", true);
         check_out(out, in->dtype, view_size(in), "softmax output");
+        check_alias(in, out, true, "softmax", "the input");
         NormCall c = prepare_norm(in, out->data, axis, 0);
         if (c.plan.kind == NormKind::Empty) return;
         NormLaunchFn fn = norm_launcher_for(log ? NORM_LOGSOFTMAX : NORM_SOFTMAX, in->dtype);
@@ -619,6 +723,7 @@ static void run_layernorm(int dev, void* stream, const hpt_view* in, const hpt_v
     check_view(in, "layernorm input", true);
     if (n_norm_dims <= 0) fail(HPT_ERR_SHAPE, "layernorm: normalized_shape must not be empty");
     check_out(out, in->dtype, view_size(in), "layernorm output");
+    check_alias(in, out, true, "layernorm", "the input");
     NormCall c = prepare_norm(in, out->data, 0, n_norm_dims);
     const hpt_view* gb[2] = {gamma, beta};
     const char* names[2] = {"layernorm gamma", "layernorm beta"};
@@ -629,6 +734,7 @@ static void run_layernorm(int dev, void* stream, const hpt_view* in, const hpt_v
             fail(HPT_ERR_DTYPE, "%s: dtype is %s, expected %s", names[k], dtype_name(gb[k]->dtype),
                  dtype_name(in->dtype));
         if (!view_contiguous(gb[k])) fail(HPT_ERR_SHAPE, "%s: must be contiguous", names[k]);
+        check_alias(gb[k], out, false, "layernorm", k == 0 ? "gamma" : "beta");
         // shape must equal the normalised dims (leading 1s aside)
         if (view_size(gb[k]) != c.plan.cols && c.plan.kind != NormKind::Empty)
             fail(HPT_ERR_SHAPE, "%s: Size mismatch: expected %lld, got %lld", names[k],
@@ -643,6 +749,7 @@ static void run_layernorm(int dev, void* stream, const hpt_view* in, const hpt_v
         bool same = residual->ndim == in->ndim;
         for (int i = 0; same && i < in->ndim; ++i) same = residual->shape[i] == in->shape[i];
         if (!same) fail(HPT_ERR_SHAPE, "layernorm residual: shape differs from the input's");
+        check_alias(residual, out, true, "layernorm", "the residual");
     }
     if (c.plan.kind == NormKind::Empty) return;
     c.args.gamma = gamma ? gamma->data : nullptr;
@@ -684,6 +791,7 @@ int32_t hpt_hip_softmax_causal(int32_t dev, void* stream, int32_t log, const hpt
     return guarded([&] {
         check_view(in, "softmax_causal input", true);
         check_out(out, in->dtype, view_size(in), "softmax_causal output");
+        check_alias(in, out, true, "softmax_causal", "the input");
         if (in->ndim < 2) fail(HPT_ERR_SHAPE, "softmax_causal: needs at least 2 dims (queries x keys)");
         NormCall c = prepare_norm(in, out->data, in->ndim - 1, 0);
         if (c.plan.kind == NormKind::Empty) return;
@@ -712,6 +820,7 @@ static EwPlan prepare_copy(const hpt_view* in, const hpt_view* out) {
     check_view(in, "contiguous input", true);
     check_out(out, in->dtype, view_size(in), "contiguous output");
     check_same_shape(in, out, "contiguous");
+    check_alias(in, out, false, "contiguous", "the input");
     const void* datas[1] = {in->data};
     const int64_t* strides[1] = {in->strides};
     return plan_elementwise(out->data, in->shape, in->ndim, 1, datas, strides, dtype_size(in->dtype), true);
@@ -740,6 +849,7 @@ int32_t hpt_hip_cast(int32_t dev, void* stream, const hpt_view* in, hpt_view* ou
         check_view(out, "cast output", true);
         if (!view_contiguous(out)) fail(HPT_ERR_SHAPE, "cast output: output tensor must be contiguous");
         check_same_shape(in, out, "cast");
+        check_alias(in, out, false, "cast", "the input");
         if (in->dtype == out->dtype) {
             const EwPlan p = prepare_copy(in, out);
             if (p.kind == EwKind::Empty) return;
@@ -786,24 +896,8 @@ int32_t hpt_hip_binary(int32_t dev, void* stream, int32_t op, const hpt_view* lh
         // The output may be one of the operands (in place) but must not overlap one otherwise:
         // every element is read before it is written only when the two walk the same addresses.
         const size_t es = dtype_size(out->dtype);
-        const char* ob = (const char*)out->data;
-        const char* oe = ob + view_size(out) * es;
-        const hpt_view* ops[2] = {lhs, rhs};
-        for (const hpt_view* v : ops) {
-            // extent of the operand in memory
-            int64_t lo = 0, hi = 0;
-            for (int i = 0; i < v->ndim; ++i) {
-                const int64_t span = (v->shape[i] - 1) * v->strides[i];
-                if (span < 0) lo += span;
-                else hi += span;
-            }
-            const char* vb = (const char*)v->data + lo * (int64_t)es;
-            const char* ve = (const char*)v->data + (hi + 1) * (int64_t)es;
-            const bool overlap = view_size(out) > 0 && vb < oe && ob < ve;
-            const bool same = v->data == out->data && view_contiguous(v);
-            if (overlap && !same)
-                fail(HPT_ERR_PARAM, "binary: out overlaps an operand without being that operand");
-        }
+        check_alias(lhs, out, true, "binary", "lhs");
+        check_alias(rhs, out, true, "binary", "rhs");
         const void* datas[2] = {lhs->data, rhs->data};
         const int64_t* strides[2] = {lhs->strides, rhs->strides};
         const EwPlan p = plan_elementwise(out->data, out->shape, out->ndim, 2, datas, strides, es, false);

@@ -79,7 +79,35 @@ class _HostStorage:
         self.ptr = arr.ctypes.data
 
 
-class _DeviceStorage:
+def _stream_key(stream) -> int:
+    """A hipStream_t given as None / int / ctypes pointer -> its address (0 = the default stream)."""
+    if stream is None:
+        return 0
+    if isinstance(stream, int):
+        return stream
+    return int(getattr(stream, "value", None) or 0)
+
+
+class _StreamTracked:
+    """Which streams have work queued that reads or writes this memory. The library's free hands a
+    block to the next caller at once (include/hpt_hip.h), and the synchronous copies only wait for
+    the default stream, so the owner waits for these streams itself before it frees or copies."""
+
+    device = 0
+
+    def _init_streams(self):
+        self.pending = set()
+
+    def touch(self, stream) -> None:
+        self.pending.add(_stream_key(stream))
+
+    def wait(self) -> None:
+        while self.pending:
+            k = self.pending.pop()
+            check(_ffi.lib().hpt_hip_stream_synchronize(self.device, C.c_void_p(k) if k else None))
+
+
+class _DeviceStorage(_StreamTracked):
     """A block owned through the library's caching allocator (hpt-allocator's Backend<B>)."""
 
     def __init__(self, device: int, nbytes: int, zeroed: bool = False):
@@ -87,14 +115,25 @@ class _DeviceStorage:
         check(_ffi.lib().hpt_hip_alloc(device, nbytes, ALIGN, int(zeroed), C.byref(p)))
         self.ptr = p.value or 0
         self.nbytes, self.device = nbytes, device
+        self._init_streams()
 
     def __del__(self):
         try:
             if self.ptr:
+                self.wait()  # kernels still queued on a caller's stream may use the block
                 _ffi.lib().hpt_hip_free(self.device, C.c_void_p(self.ptr), self.nbytes, ALIGN)
                 self.ptr = 0
         except Exception:
             pass
+
+
+class _RawStorage(_StreamTracked):
+    """Device memory somebody else owns (Tensor.from_raw): never freed here (`should_drop = false`,
+    hpt/src/backends/cuda/tensor_impls.rs; hpt-allocator/src/backend.rs:12-168)."""
+
+    def __init__(self, device: int, ptr: int, nbytes: int):
+        self.ptr, self.nbytes, self.device = ptr, nbytes, device
+        self._init_streams()
 
 
 def _contiguous_strides(shape: Sequence[int]):
@@ -109,6 +148,14 @@ def _tdiv(a: int, b: int) -> int:
     """Integer division truncating toward zero (Rust's `/`)."""
     q = abs(a) // abs(b)
     return q if (a < 0) == (b < 0) else -q
+
+
+def _touch(stream, *tensors) -> None:
+    """Record that work on `stream` now uses the storage of these device tensors."""
+    for t in tensors:
+        st = getattr(t, "_storage", None) if t is not None else None
+        if isinstance(st, _StreamTracked):
+            st.touch(stream)
 
 
 def _as_axes(axes) -> list:
@@ -152,6 +199,67 @@ class Tensor:
         st = _DeviceStorage(device, n * dtype.size, zeroed)
         return cls(st, st.ptr, shape, _contiguous_strides(shape), dtype, "hip", device)
 
+    @classmethod
+    def from_raw(cls, ptr: int, shape, dtype: DType, device: int = 0, strides=None) -> "Tensor":
+        """Tensor::from_raw (hpt/src/backends/cpu/tensor_impls.rs:123-147, :269): a tensor over device
+        memory the caller owns; dropping the tensor frees nothing. The reference takes a contiguous
+        shape and asserts 64-byte alignment; here `strides` (elements) may describe any view and the
+        pointer only has to be aligned to the element size: the kernels take unaligned rows."""
+        if not ptr:
+            raise ParamError(_ffi.ERR_PARAM, "data is null")
+        if ptr % dtype.size:
+            raise ParamError(_ffi.ERR_PARAM, f"data is not aligned, it must be aligned to {dtype.size}")
+        shape = [int(s) for s in shape]
+        strides = _contiguous_strides(shape) if strides is None else [int(s) for s in strides]
+        if len(strides) != len(shape):
+            raise ShapeError(_ffi.ERR_SHAPE, f"from_raw: {len(shape)} dims but {len(strides)} strides")
+        lo = sum((d - 1) * s for d, s in zip(shape, strides) if s < 0 and d > 0)
+        hi = sum((d - 1) * s for d, s in zip(shape, strides) if s > 0 and d > 0)
+        n = 0 if 0 in shape else (hi - lo + 1)
+        st = _RawStorage(device, ptr + lo * dtype.size, n * dtype.size)
+        return cls(st, ptr, shape, strides, dtype, "hip", device)
+
+    def forget(self):
+        """Tensor::forget (hpt/src/backends/cuda/tensor_impls.rs:277-306): give the allocation up. Returns
+        (pointer, (bytes, align)); the allocator stops tracking the block (Allocator::forget,
+        hpt-allocator/src/allocators/cuda.rs:140-146) and the caller releases it with hipFree. Fails, as the
+        reference does, for a view and while another tensor shares the storage; the tensor is empty after."""
+        import sys
+        self._require_hip("forget")
+        if self.parent is not None:
+            raise ParamError(_ffi.ERR_PARAM, "Can't forget tensor: tensor is a view, cannot forget")
+        st = self._storage
+        refs = sys.getrefcount(st) - 2  # the local name and getrefcount's own argument
+        if refs > 1:
+            raise ParamError(_ffi.ERR_PARAM, f"Can't forget tensor: ref_count: {refs}")
+        st.wait()
+        ptr, nbytes = st.ptr, st.nbytes
+        if isinstance(st, _DeviceStorage):
+            check(_ffi.lib().hpt_hip_forget(self.device, C.c_void_p(ptr)))
+            st.ptr = 0  # its __del__ must not hand the block back to the cache
+        self._storage, self.ptr, self.shape, self.strides = None, 0, [0], [1]
+        return ptr, (nbytes, ALIGN)
+
+    def allclose(self, other: "Tensor", rtol: float = 1e-5, atol: float = 1e-8) -> bool:
+        """allclose of the reference (hpt/src/backends/cuda/tensor_impls.rs:259-271: both sides go to the
+        host; hpt/src/backends/cpu/tensor_impls.rs:218-248: shapes must match, NaN equals NaN, infinities by
+        sign, else |a - b| <= atol + rtol * |b|)."""
+        if self.shape != other.shape:
+            return False
+        a, b = self._host_f64(), other._host_f64()
+        both_nan = np.isnan(a) & np.isnan(b)
+        inf = np.isinf(a) & np.isinf(b)
+        with np.errstate(invalid="ignore"):
+            ok = np.abs(a - b) <= atol + rtol * np.abs(b)
+        ok = np.where(inf, np.sign(a) == np.sign(b), ok) | both_nan
+        return bool(ok.all())
+
+    def _host_f64(self) -> np.ndarray:
+        h = self.to_cpu().numpy() if self.backend == "hip" else self.numpy()
+        if self.dtype is bf16:
+            h = bf16_bits_to_f32(h)
+        return h.astype(np.float64)
+
     def size(self) -> int:
         return int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
 
@@ -188,6 +296,7 @@ class Tensor:
         src = self if (self.is_contiguous() and self.parent is None) else self.contiguous()
         arr = np.empty(self.shape, self.dtype.np_dtype)
         if arr.nbytes:
+            src._storage.wait()
             check(_ffi.lib().hpt_hip_stream_synchronize(self.device, None))
             check(_ffi.lib().hpt_hip_memcpy_d2h_sync(self.device, C.c_void_p(arr.ctypes.data),
                                                      C.c_void_p(src.ptr), arr.nbytes))
@@ -203,6 +312,7 @@ class Tensor:
         else:
             # device: copy the whole allocation once, then gather through the strides
             raw = np.empty(st.nbytes, np.uint8)
+            st.wait()
             check(_ffi.lib().hpt_hip_stream_synchronize(self.device, None))
             check(_ffi.lib().hpt_hip_memcpy_d2h_sync(self.device, C.c_void_p(raw.ctypes.data),
                                                      C.c_void_p(st.ptr), st.nbytes))
@@ -333,6 +443,7 @@ class Tensor:
         ax = _ffi.i64_array(axes)
         entry = l.hpt_hip_reduce_static if static_scratch else l.hpt_hip_reduce
         check(entry(self.device, stream, op, C.byref(vin), ax, len(axes), int(init_out), C.byref(vout)))
+        _touch(stream, self, res)
         del k1, k2
         return Tensor(res._storage, res.ptr, final_shape, _contiguous_strides(final_shape), res.dtype, "hip",
                       self.device)
@@ -349,6 +460,7 @@ class Tensor:
         vin, k1 = self._c_view()
         vout, k2 = res._c_view()
         check(l.hpt_hip_argreduce(self.device, stream, int(is_max), C.byref(vin), axes[0], C.byref(vout)))
+        _touch(stream, self, res)
         del k1, k2
         return Tensor(res._storage, res.ptr, final_shape, _contiguous_strides(final_shape), i64, "hip", self.device)
 
@@ -411,16 +523,25 @@ class Tensor:
         return self._argreduce(False, axis, keep_dims, **kw)
 
     # ---- NormalizationOps (hpt-traits/src/ops/normalization.rs:6-64) ------------
-    def _softmax(self, log: bool, axis: int, stream=None) -> "Tensor":
+    def _norm_out(self, out: Optional["Tensor"], dtype: DType) -> "Tensor":
+        """The result tensor of a normalisation: fresh, or the caller's `out` (which may be `self`: the
+        ABI allows a normalisation in place over one contiguous tensor)."""
+        if out is None:
+            return Tensor.empty(self.shape, dtype, self.device)
+        out._require_hip("out")
+        return out
+
+    def _softmax(self, log: bool, axis: int, stream=None, out: Optional["Tensor"] = None) -> "Tensor":
         self._require_hip("softmax")
         ft = self._float_binary_type()
         if ft is not self.dtype:
             # NormalizationOps::Output = Tensor<FloatBinaryType<T>>: a non-float input is cast first
-            return self.astype(ft, stream=stream)._softmax(log, axis, stream=stream)
-        res = Tensor.empty(self.shape, self.dtype, self.device)
+            return self.astype(ft, stream=stream)._softmax(log, axis, stream=stream, out=out)
+        res = self._norm_out(out, self.dtype)
         vin, k1 = self._c_view()
         vout, k2 = res._c_view()
         check(_ffi.lib().hpt_hip_softmax(self.device, stream, int(log), C.byref(vin), int(axis), C.byref(vout)))
+        _touch(stream, self, res)
         del k1, k2
         return res
 
@@ -431,7 +552,8 @@ class Tensor:
         return self._softmax(True, axis, **kw)
 
     def layernorm(self, normalized_shape, gamma: Optional["Tensor"] = None, beta: Optional["Tensor"] = None,
-                  eps: float = 1e-5, stream=None, residual: Optional["Tensor"] = None) -> "Tensor":
+                  eps: float = 1e-5, stream=None, residual: Optional["Tensor"] = None,
+                  out: Optional["Tensor"] = None) -> "Tensor":
         self._require_hip("layernorm")
         ns = [int(s) for s in (normalized_shape if isinstance(normalized_shape, Iterable) else [normalized_shape])]
         if len(ns) > self.ndim or (ns and self.shape[self.ndim - len(ns):] != ns) or not ns:
@@ -442,8 +564,8 @@ class Tensor:
         ft = self._float_binary_type()
         if ft is not self.dtype:
             return self.astype(ft, stream=stream).layernorm(normalized_shape, gamma, beta, eps, stream=stream,
-                                                            residual=residual)
-        res = Tensor.empty(self.shape, self.dtype, self.device)
+                                                            residual=residual, out=out)
+        res = self._norm_out(out, self.dtype)
         vin, k1 = self._c_view()
         vout, k2 = res._c_view()
         keep = [k1, k2]
@@ -467,6 +589,7 @@ class Tensor:
         else:
             check(_ffi.lib().hpt_hip_layernorm(self.device, stream, C.byref(vin), len(ns), gp, bp, float(eps),
                                                C.byref(vout)))
+        _touch(stream, self, res, gamma, beta, residual)
         del keep
         return res
 
@@ -481,6 +604,7 @@ class Tensor:
         vout, k2 = res._c_view()
         check(_ffi.lib().hpt_hip_softmax_causal(self.device, stream, int(log), C.byref(vin), float(scale),
                                                 int(causal_offset), C.byref(vout)))
+        _touch(stream, self, res)
         del k1, k2
         return res
 
@@ -497,6 +621,7 @@ class Tensor:
         vin, k1 = self._c_view()
         vout, k2 = res._c_view()
         check(_ffi.lib().hpt_hip_cast(self.device, stream, C.byref(vin), C.byref(vout)))
+        _touch(stream, self, res)
         del k1, k2
         return res
 
@@ -514,6 +639,7 @@ class Tensor:
         vin, k1 = self._c_view()
         vout, k2 = res._c_view()
         check(_ffi.lib().hpt_hip_contiguous(self.device, stream, C.byref(vin), C.byref(vout)))
+        _touch(stream, self, res)
         del k1, k2
         return res
 
@@ -528,6 +654,7 @@ class Tensor:
             host = np.array([value]).astype(dtype.np_dtype)
         v, k = res._c_view()
         check(_ffi.lib().hpt_hip_fill(device, stream, C.byref(v), C.c_void_p(host.ctypes.data)))
+        _touch(stream, res)
         del k
         return res
 
@@ -575,6 +702,7 @@ class Tensor:
         vb, k2 = b._c_view()
         vo, k3 = res._c_view()
         check(_ffi.lib().hpt_hip_binary(self.device, stream, op, C.byref(va), C.byref(vb), C.byref(vo)))
+        _touch(stream, self, rhs, res)
         del k1, k2, k3
         return res
 

@@ -13,7 +13,8 @@
  *   - Output tensors are allocated by the caller (through hpt_hip_alloc, i.e.
  *     the Hip allocator) and must be contiguous; the library never allocates or
  *     frees user-visible tensors. Scratch for multi-stage reductions is owned
- *     by the library, cached per (device, stream).
+ *     by the library: one buffer per (device, stream), taken from the same caching
+ *     allocator, grown on demand, released by hpt_hip_cache_clear.
  *   - Kernels are enqueued on `stream` (a hipStream_t passed as void*; NULL =
  *     the device's default stream) and are NOT synchronised; the *_sync copy
  *     functions block until the copy is complete.
@@ -117,9 +118,17 @@ int32_t hpt_hip_alloc(int32_t dev, size_t bytes, size_t align, int32_t zeroed, v
  * The block may be handed out again at once: free it only after the stream that
  * last used it has finished with it. */
 int32_t hpt_hip_free(int32_t dev, void* p, size_t bytes, size_t align);
+/* Allocator::forget (hpt-allocator/src/allocators/cuda.rs:140-146; called by Tensor::forget,
+ * hpt/src/backends/cuda/tensor_impls.rs:277-306): the allocator stops tracking `p`, which the
+ * caller owns from now on (it came from hipMalloc: release it with hipFree). A pointer the
+ * allocator does not know is ignored. The opposite direction, Tensor::from_raw
+ * (hpt/src/backends/cpu/tensor_impls.rs:123-147), needs no call: every entry point takes any
+ * device pointer, whoever allocated it, at any element-aligned address. */
+int32_t hpt_hip_forget(int32_t dev, void* p);
 /* resize_cuda_lru_cache (hpt/src/lib.rs:449-450). Evicted blocks are released. */
 int32_t hpt_hip_cache_resize(int32_t dev, size_t entries);
-/* Allocator::clear (hpt-allocator/src/traits.rs:55): release every cached block. */
+/* Allocator::clear (hpt-allocator/src/traits.rs:55): release every cached block, and the
+ * library's own scratch buffers of this device (after waiting for the device to go idle). */
 int32_t hpt_hip_cache_clear(int32_t dev);
 /* Counters for tests and leak checks: blocks handed out and not yet freed,
  * blocks sitting in the cache, and hipMalloc calls made so far. */

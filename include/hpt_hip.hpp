@@ -7,6 +7,9 @@
 //   Tensor::from_host / to_host         Tensor::new(..).to_cuda() / to_cpu()
 //                                       (hpt/src/backends/cpu/tensor_impls.rs:295-313,
 //                                        hpt/src/backends/cuda/tensor_impls.rs:142-169)
+//   Tensor::from_raw / forget / allclose
+//                                       (hpt/src/backends/cpu/tensor_impls.rs:123-147, 218-248;
+//                                        hpt/src/backends/cuda/tensor_impls.rs:259-306)
 //   permute / transpose / t / slice / expand
 //                                       ShapeManipulate, Slice (hpt/src/backends/common/
 //                                       shape_manipulate.rs:19-52, hpt-common/src/slice.rs:20-95)
@@ -21,6 +24,7 @@
 // would return (hpt-common/src/error/base.rs:8-45) and whose text is the library's.
 #pragma once
 
+#include <cmath>
 #include <cstdint>
 #include <cstring>
 #include <initializer_list>
@@ -164,6 +168,60 @@ template <class T> class Tensor {
                                                     std::to_string(t.size()));
         if (!data.empty()) check(hpt_hip_memcpy_h2d_sync(device, t.data_, data.data(), data.size() * sizeof(T)));
         return t;
+    }
+    // Tensor::from_raw: a tensor over device memory the caller owns; dropping it frees nothing. The
+    // reference takes a contiguous shape and asserts 64-byte alignment; here any element-aligned
+    // pointer is taken (the kernels read unaligned rows) and `strides` may describe any view.
+    static Tensor from_raw(T* data, const Shape& shape, int device = 0) { return from_raw(data, shape, contiguous_strides(shape), device); }
+    static Tensor from_raw(T* data, const Shape& shape, const Shape& strides, int device = 0) {
+        if (!data) throw TensorError(ErrorKind::Param, "data is null");
+        if ((uintptr_t)data % sizeof(T)) throw TensorError(ErrorKind::Param, "data is not aligned to its element size");
+        if (shape.size() != strides.size()) throw TensorError(ErrorKind::Shape, "from_raw: shape and strides differ in length");
+        Tensor t;
+        t.data_ = data;
+        t.shape_ = shape;
+        t.strides_ = strides;
+        t.device_ = device;
+        return t;
+    }
+    // Tensor::forget: give the allocation up. The allocator stops tracking the block and the caller
+    // releases it (hipFree). Fails for a view and while another tensor shares the storage.
+    struct Forgotten { void* ptr; size_t bytes, align; };
+    Forgotten forget() {
+        if (is_view_) throw TensorError(ErrorKind::Param, "Can't forget tensor: tensor is a view, cannot forget");
+        if (block_ && block_.use_count() > 1)
+            throw TensorError(ErrorKind::Param, "Can't forget tensor: ref_count: " + std::to_string(block_.use_count()));
+        Forgotten f{(void*)data_, block_ ? block_->bytes : (size_t)size() * sizeof(T), kAlign};
+        if (block_) {
+            check(hpt_hip_stream_synchronize(device_, nullptr));
+            check(hpt_hip_forget(device_, block_->ptr));
+            block_->ptr = nullptr;
+            block_.reset();
+        }
+        data_ = nullptr;
+        shape_ = {0};
+        strides_ = {1};
+        return f;
+    }
+    // allclose: both sides go to the host; shapes must match, NaN equals NaN, infinities by sign,
+    // else |a - b| <= atol + rtol * |b|.
+    bool allclose(const Tensor& other, double rtol, double atol) const {
+        if (shape_ != other.shape_) return false;
+        const auto a = to_host(), b = other.to_host();
+        auto val = [](HostElem<T> v) -> double {
+            if constexpr (std::is_same<T, f16>::value || std::is_same<T, bf16>::value) return (double)to_float(v);
+            else return (double)v;
+        };
+        for (size_t i = 0; i < a.size(); ++i) {
+            const double x = val(a[i]), y = val(b[i]);
+            if (std::isnan(x) && std::isnan(y)) continue;
+            if (std::isinf(x) && std::isinf(y)) {
+                if ((x > 0) != (y > 0)) return false;
+                continue;
+            }
+            if (!(std::fabs(x - y) <= atol + rtol * std::fabs(y))) return false;
+        }
+        return true;
     }
     static Tensor full(T value, const Shape& shape, int device = 0) {
         Tensor t = empty(shape, device);

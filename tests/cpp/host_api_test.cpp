@@ -4,6 +4,8 @@
 // against a plain host loop over the same strides (hpt-tests/src/hpt/cpu/reduce.rs:63-291), closed
 // forms for softmax / layernorm, and the error texts of hpt-common/src/axis/axis.rs:38-73.
 // Prints one line per failure; exit status 0 when all pass.
+#include <dlfcn.h>
+
 #include <cmath>
 #include <cstdio>
 #include <functional>
@@ -210,6 +212,87 @@ static void error_behaviour() {
     EXPECT(a.sum({-1}).to_host() == std::vector<float>({3, 7}), "negative axis wraps");
 }
 
+// Tensor::forget / from_raw / allclose (hpt/src/backends/cuda/tensor_impls.rs:259-306,
+// hpt/src/backends/cpu/tensor_impls.rs:123-147, 218-248): a block given up by the library becomes
+// the caller's raw device memory; tensors adopted over it - at an address that is only
+// element-aligned - compute like any other and free nothing when they go.
+static void foreign_memory() {
+    uint64_t live0 = 0, live1 = 0, live2 = 0;
+    std::vector<float> data(1000);
+    std::mt19937 rng(5);
+    std::normal_distribution<float> nd(0.f, 2.f);
+    for (auto& x : data) x = nd(rng);
+    auto t = Tensor<float>::from_host(data, {1000});
+    hpt_hip_alloc_stats(0, &live0, nullptr, nullptr);
+    expect_error(hpt::ErrorKind::Param, "tensor is a view", [&] { auto v = t.slice({{1, 1000, 1}}); v.forget(); }, "forget of a view");
+    {
+        auto shared = t.reshape({1000});  // a second owner of the block
+        (void)shared;
+    }
+    {
+        Tensor<float> second = t;
+        expect_error(hpt::ErrorKind::Param, "ref_count: 2", [&] { t.forget(); }, "forget of a shared block");
+    }
+    const auto f = t.forget();
+    hpt_hip_alloc_stats(0, &live1, nullptr, nullptr);
+    EXPECT(live1 + 1 == live0, "forget: live blocks %llu -> %llu", (unsigned long long)live0, (unsigned long long)live1);
+    EXPECT(f.bytes == 4000 && f.align == 64 && t.size() == 0, "forget: layout (%zu, %zu)", f.bytes, f.align);
+    EXPECT(hpt_hip_free(0, f.ptr, f.bytes, f.align) == HPT_ERR_MEMORY, "the allocator must not know a forgotten block");
+    {
+        // 999 floats from the second element on: 4 bytes past a 64-byte boundary
+        auto raw = Tensor<float>::from_raw((float*)f.ptr + 1, {37, 27});
+        auto sums = raw.sum({1}).to_host();
+        bool ok = true;
+        for (int r = 0; r < 37; ++r) {
+            double want = 0;
+            for (int c = 0; c < 27; ++c) want += data[1 + r * 27 + c];
+            ok = ok && close(sums[r], want, 1e-5, 1e-5);
+        }
+        EXPECT(ok, "sum over rows of a raw, odd-aligned tensor");
+        auto am = raw.argmax(1).to_host();
+        ok = true;
+        for (int r = 0; r < 37; ++r) {
+            int best = 0;
+            for (int c = 1; c < 27; ++c)
+                if (data[1 + r * 27 + c] > data[1 + r * 27 + best]) best = c;
+            ok = ok && am[r] == best;
+        }
+        EXPECT(ok, "argmax of a raw tensor");
+        auto sm = raw.softmax(1);
+        auto rows = sm.sum({1}).to_host();
+        ok = true;
+        for (float v : rows) ok = ok && close(v, 1.0, 1e-5, 1e-6);
+        EXPECT(ok, "softmax rows of a raw tensor sum to one");
+        auto ln = raw.layernorm({27}, nullptr, nullptr, 1e-5);
+        auto means = ln.mean({1}).to_host();
+        ok = true;
+        for (float v : means) ok = ok && std::fabs(v) < 1e-5;
+        EXPECT(ok, "layernorm rows of a raw tensor have mean zero");
+        // a strided view of the raw memory: every second column, and the same numbers gathered on the host
+        auto stepped = Tensor<float>::from_raw((float*)f.ptr + 1, {37, 14}, {27, 2});
+        std::vector<float> gathered;
+        for (int r = 0; r < 37; ++r)
+            for (int c = 0; c < 27; c += 2) gathered.push_back(data[1 + r * 27 + c]);
+        auto copy = Tensor<float>::from_host(gathered, {37, 14});
+        EXPECT(stepped.allclose(copy, 0.0, 0.0), "allclose: a raw stepped view against its gathered copy");
+        EXPECT(!stepped.allclose(copy.reshape({14, 37}), 1.0, 1.0), "allclose: shapes differ");
+        auto shifted = copy + Tensor<float>::full(1e-3f, {1});
+        EXPECT(!stepped.allclose(shifted, 0.0, 1e-4) && stepped.allclose(shifted, 0.0, 2e-3), "allclose: absolute tolerance");
+        auto nan1 = Tensor<float>::from_host({NAN, INFINITY, 1.f}, {3}), nan2 = Tensor<float>::from_host({NAN, INFINITY, 1.f}, {3});
+        auto inf2 = Tensor<float>::from_host({NAN, -INFINITY, 1.f}, {3});
+        EXPECT(nan1.allclose(nan2, 0.0, 0.0) && !nan1.allclose(inf2, 1.0, 1.0), "allclose: NaN equals NaN, infinities by sign");
+    }
+    hpt::synchronize();
+    hpt_hip_alloc_stats(0, &live2, nullptr, nullptr);
+    EXPECT(live2 == live1, "tensors over raw memory changed the live block count: %llu -> %llu", (unsigned long long)live1,
+           (unsigned long long)live2);
+    // the memory is the caller's now: release it with the runtime's own free
+    using hipFree_t = int (*)(void*);
+    auto hip_free = (hipFree_t)dlsym(RTLD_DEFAULT, "hipFree");
+    EXPECT(hip_free != nullptr && hip_free(f.ptr) == 0, "hipFree of the forgotten block");
+    expect_error(hpt::ErrorKind::Param, "data is null", [&] { Tensor<float>::from_raw(nullptr, {4}); }, "from_raw(null)");
+}
+
 int main() {
     if (hpt::device_count() < 1) {
         printf("no HIP device\n");
@@ -219,6 +302,7 @@ int main() {
     views_against_host_loops();
     normalisation_closed_forms();
     error_behaviour();
+    foreign_memory();
     hpt::synchronize();
     printf("%d checks, %d failures\n", checks, failures);
     return failures ? 1 : 0;

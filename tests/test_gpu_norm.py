@@ -619,3 +619,42 @@ def test_special_values_on_the_large_shape_kernels(hpt, orc, dev):
                 want = orc.softmax(x, axis, log=log, acc=orc.ACC_F64)
             assert np.array_equal(np.isnan(got), np.isnan(want)), f"{shape} axis={axis} log={log}: NaN pattern"
             assert_close(got, want, F32_RTOL, 2e-6, f"{shape} axis={axis} log={log}")
+
+
+def test_half_rows_of_millions_of_elements_against_the_f64_truth(hpt, orc, dev):
+    """f16 layernorm over all four dims of [63, 50, 53, 37] permuted (1, 2, 0, 3) — one strided row of
+    6 177 150 elements, the case a randomised run once flagged — and its bf16 twin, plus softmax and a
+    full sum of the same row. Rows this long are checked against the f64 accumulation rounded once:
+    the sequential-f32 oracle mode is itself ~0.4 % off here (shown on the host in
+    tests/test_oracle_numerics.py::test_sequential_f32_accumulation_is_no_truth_for_long_half_rows)."""
+    from util import half_acc
+    rng = np.random.default_rng(0)
+    shape = [63, 50, 53, 37]
+    x = (rng.standard_normal(shape) * 2).astype(np.float32)
+    gf = rng.normal(1, 0.1, [50, 53, 63, 37]).astype(np.float32)
+    bf = rng.normal(0, 0.1, [50, 53, 63, 37]).astype(np.float32)
+    for bits in (11, 8):
+        if bits == 8:
+            cv, dt, odt, tof = hpt.f32_to_bf16_bits, hpt.bf16, orc.BF16, hpt.bf16_bits_to_f32
+        else:
+            cv, dt, odt, tof = (lambda v: v.astype(np.float16)), None, None, (lambda v: v.astype(np.float32))
+        base, g, b = cv(x), cv(gf), cv(bf)
+        t = hpt.Tensor.from_numpy(base, dt).to_hip(dev).permute([1, 2, 0, 3])
+        a = base.transpose(1, 2, 0, 3)
+        acc = half_acc(orc, a.size)
+        assert acc == orc.ACC_F64
+        tg, tb = hpt.Tensor.from_numpy(g, dt).to_hip(dev), hpt.Tensor.from_numpy(b, dt).to_hip(dev)
+        got = tof(t.layernorm(list(a.shape), tg, tb, 1e-5).numpy())
+        want = tof(orc.layernorm(a, 4, g, b, 1e-5, acc=acc, dtype=odt))
+        # one rounding of the result apart from the oracle: an ulp of the half type, nowhere more
+        assert_close(got, want, 2.0 ** -(bits - 1), 2.0 ** -bits * 2.0 ** -6, f"layernorm of one 6M-element row, {bits} bits")
+        # and the row's own statistics, which is where a drifting accumulation would show
+        m = float(tof(t.mean([0, 1, 2, 3]).numpy())[0])
+        xd = tof(a).astype(np.float64)
+        assert abs(m - xd.mean()) < 2.0 ** -bits * max(abs(xd.mean()), 2.0 ** -14) + 1e-6
+        if bits == 8:   # (2.5e7 is beyond f16's range)
+            ss = float(tof(t.sum_square([0, 1, 2, 3]).numpy())[0])
+            assert abs(ss / (xd * xd).sum() - 1) < 2.0 ** -bits
+        got = tof(t.softmax(3).numpy())
+        want = tof(orc.softmax(a, 3, acc=orc.ACC_F32, dtype=odt))
+        assert_close(got, want, HALF_RTOL, max(half_atol(want, bits), 6e-8), f"softmax(3), {bits} bits")

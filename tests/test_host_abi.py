@@ -190,6 +190,67 @@ def test_argument_errors_without_a_device(hpt):
         t.softmax(1)
 
 
+def test_outputs_that_overlap_an_input_are_refused_before_any_launch(hpt):
+    """`out` may be the input itself (same pointer, contiguous) for the normalisations and the binary
+    ops and nothing else: a permuted / stepped / shifted view of out's buffer is HPT_ERR_PARAM, found on
+    the host before a device is touched (the pointers here are made up)."""
+    from hpt_amd import _ffi
+    from hpt_amd.tensor import Tensor, _contiguous_strides
+    l = hpt.lib()
+    BASE = 1 << 20
+
+    def fake(shape, dt=hpt.f32, strides=None, off=0):
+        return Tensor(None, BASE + off * dt.size, shape, strides or _contiguous_strides(shape), dt, "hip", 0)
+
+    def call(fn, *views, pre=(), mid=()):
+        cv = [v._c_view() for v in views]
+        args = list(pre) + [C.byref(cv[0][0])] + list(mid) + [C.byref(c[0]) for c in cv[1:]]
+        return fn(0, None, *args)
+
+    out = fake((64, 64))
+    cases = {
+        "permuted": fake((64, 64), strides=[1, 64]),
+        "stepped": fake((64, 64), strides=[128, 2]),
+        "shifted": fake((64, 64), off=8),
+        "reversed": fake((64, 64), strides=[-64, 1], off=63 * 64),
+    }
+    for name, vin in cases.items():
+        st = call(l.hpt_hip_softmax, vin, out, pre=(0,), mid=(1,))
+        assert st == _ffi.ERR_PARAM, name
+        assert "overlaps" in l.hpt_hip_last_error().decode()
+        cin, cout = vin._c_view(), out._c_view()
+        assert l.hpt_hip_layernorm(0, None, C.byref(cin[0]), 1, None, None, 1e-5, C.byref(cout[0])) == _ffi.ERR_PARAM, name
+        assert l.hpt_hip_softmax_causal(0, None, 0, C.byref(cin[0]), 1.0, 0, C.byref(cout[0])) == _ffi.ERR_PARAM, name
+        assert l.hpt_hip_contiguous(0, None, C.byref(cin[0]), C.byref(cout[0])) == _ffi.ERR_PARAM, name
+        assert l.hpt_hip_cast(0, None, C.byref(cin[0]), C.byref(cout[0])) == _ffi.ERR_PARAM, name
+    # the very same tensor: refused for copy / cast / reduce (nothing is in place there)
+    cin, cout = out._c_view(), out._c_view()
+    assert l.hpt_hip_contiguous(0, None, C.byref(cin[0]), C.byref(cout[0])) == _ffi.ERR_PARAM
+    assert l.hpt_hip_cast(0, None, C.byref(cin[0]), C.byref(cout[0])) == _ffi.ERR_PARAM
+    # a reduction whose output lies inside its input
+    red_out = fake((64,), off=64)
+    cin, cout = out._c_view(), red_out._c_view()
+    ax = _ffi.i64_array([1])
+    assert l.hpt_hip_reduce(0, None, hpt.SUM, C.byref(cin[0]), ax, 1, 1, C.byref(cout[0])) == _ffi.ERR_PARAM
+    assert l.hpt_hip_reduce_static(0, None, hpt.SUM, C.byref(cin[0]), ax, 1, 1, C.byref(cout[0])) == _ffi.ERR_PARAM
+    iout = fake((64,), dt=hpt.i64, off=16)
+    cout = iout._c_view()
+    assert l.hpt_hip_argreduce(0, None, 1, C.byref(cin[0]), 1, C.byref(cout[0])) == _ffi.ERR_PARAM
+    # gamma / beta inside the output
+    g = fake((64,), off=128)
+    cg = g._c_view()
+    far = Tensor(None, 1 << 30, (64, 64), _contiguous_strides((64, 64)), hpt.f32, "hip", 0)
+    cin, cout = far._c_view(), out._c_view()
+    assert l.hpt_hip_layernorm(0, None, C.byref(cin[0]), 1, C.byref(cg[0]), None, 1e-5, C.byref(cout[0])) == _ffi.ERR_PARAM
+    assert "gamma" in l.hpt_hip_last_error().decode()
+    # a neighbour that only touches is fine as far as this check goes: the next failure is a different one
+    # (there is no device 99)
+    nb = fake((64, 64), off=64 * 64)
+    cin = nb._c_view()
+    st = l.hpt_hip_softmax(99, None, 0, C.byref(cin[0]), 1, C.byref(cout[0]))
+    assert st == _ffi.ERR_DEVICE, l.hpt_hip_last_error().decode()
+
+
 def test_views_follow_the_reference_slice_rules(hpt, orc):
     BIG = 0x7FFFFFFFFFFFFFFF
     a = np.arange(3 * 4 * 5, dtype=np.float32).reshape(3, 4, 5)

@@ -121,6 +121,49 @@ def test_integer_wraparound_bit_exact(orc, npdt):
                 assert np.array_equal(orc.reduce(orc.SUM_SQUARE, v, axes).reshape(-1), np.atleast_1d((v * v).sum(axis=tuple(axes), dtype=npdt)).reshape(-1))
 
 
+@pytest.mark.parametrize("npdt", [np.float32, np.float64, np.float16])
+def test_float_prod_nansum_nanprod_all_any_against_numpy_float64(orc, npdt):
+    """The float branches of prod / nansum / nanprod / all / any against numpy in float64 on the same three
+    layouts (contiguous, permuted, sliced with a step). Values near 1 keep a product of 50 terms in range;
+    NaNs are planted so that nansum / nanprod have something to skip, zeros so that all / any see both answers.
+    A dropped NaN test, a sum where a product belongs or a wrong identity (0 for prod) fails here."""
+    rng = np.random.default_rng(33)
+    a = (1.0 + 0.2 * rng.standard_normal((7, 50, 9))).astype(npdt)
+    withnan = a.copy()
+    withnan[rng.random(a.shape) < 0.1] = np.nan
+    withnan[3, :, 4] = np.nan                    # one output with nothing but NaN: the identities show
+    zeros = a.copy()
+    zeros[rng.random(a.shape) < 0.3] = 0
+    zeros[2, :, :] = 0                           # all-zero outputs for `any`
+    zeros[5, :, 1::2] = 1                        # all-nonzero outputs for `all`
+    zeros[0, 0, 0] = np.nan                      # NaN is not zero: it counts as true
+    half = npdt == np.float16
+    acc = orc.ACC_F32 if half else orc.ACC_F64
+    rtol = 2e-3 if half else (1e-6 if npdt == np.float32 else 1e-12)
+    patol = 6e-8 if half else 0   # f16 products of many terms reach the subnormals (spacing 2^-24)
+    for axes in ([0], [1], [2], [0, 2], [0, 1, 2]):
+        ax = tuple(axes)
+        for mk in (lambda v: v, lambda v: v.transpose(2, 0, 1), lambda v: v[:, ::3, 1:]):
+            v, vn, vz = mk(a), mk(withnan), mk(zeros)
+            v64, vn64 = v.astype(np.float64), vn.astype(np.float64)
+            flat = lambda r: np.atleast_1d(r).reshape(-1)
+            assert_close(flat(orc.reduce(orc.PROD, v, axes, acc=acc)), flat(v64.prod(axis=ax)), rtol, patol, f"prod {axes}")
+            assert_close(flat(orc.reduce(orc.NANSUM, vn, axes, acc=acc)), flat(np.nansum(vn64, axis=ax)), rtol, 1e-3 if half else 1e-6,
+                         f"nansum {axes}")
+            assert_close(flat(orc.reduce(orc.NANPROD, vn, axes, acc=acc)), flat(np.nanprod(vn64, axis=ax)), rtol, patol,
+                         f"nanprod {axes}")
+            # a NaN poisons the plain forms
+            assert np.isnan(flat(orc.reduce(orc.PROD, vn, axes, acc=acc))).tolist() == np.isnan(flat(vn64.prod(axis=ax))).tolist()
+            assert np.isnan(flat(orc.reduce(orc.SUM, vn, axes, acc=acc))).tolist() == np.isnan(flat(vn64.sum(axis=ax))).tolist()
+            got_all, got_any = orc.reduce(orc.ALL, vz, axes), orc.reduce(orc.ANY, vz, axes)
+            assert got_all.dtype == np.bool_ and got_any.dtype == np.bool_
+            assert np.array_equal(flat(got_all), flat(np.all(vz, axis=ax)))
+            assert np.array_equal(flat(got_any), flat(np.any(vz, axis=ax)))
+    # the identities: nothing but NaN -> nansum 0, nanprod 1
+    col = withnan[3, :, 4]
+    assert orc.reduce(orc.NANSUM, col, [0], acc=acc)[0] == 0 and orc.reduce(orc.NANPROD, col, [0], acc=acc)[0] == 1
+
+
 def test_argmax_strict_compare_rules(orc):
     # ties -> first; NaN never wins; an all -inf / all MIN row -> 0 (argreduce_kernels.rs:13-21)
     a = np.array([[1, 5, 5, 2], [7, 7, 7, 7], [-3, -9, -3, -9]], np.int32)
@@ -211,6 +254,38 @@ def test_lane_structure_and_rounding_modes(orc):
     onesb = orc.f32_to_bf16(np.ones((1, 1024), np.float32))
     assert orc.bf16_to_f32(orc.reduce(orc.SUM, onesb, [1], acc=orc.ACC_NATIVE, dtype=orc.BF16))[0] == 256
     assert orc.bf16_to_f32(orc.reduce(orc.SUM, onesb, [1], acc=orc.ACC_F32, dtype=orc.BF16))[0] == 1024
+
+
+def test_sequential_f32_accumulation_is_no_truth_for_long_half_rows(orc):
+    """f16 layernorm over ALL dims of a [63, 50, 53, 37] tensor permuted (1, 2, 0, 3): one row of
+    6 177 150 elements. A randomised device run once disagreed with the oracle's ACC_F32 mode here on
+    4 elements (outputs next to zero, where a relative tolerance does not help). Which side was off is
+    decided on the host: the f64-accumulating mode agrees with numpy's float64 statistics to f16
+    rounding; the sequential-f32 mode does not, because its running sum of (x - mean)^2 passes 2^24,
+    where f32 moves in steps of 2 and terms below 1 vanish: it ends ~0.8 % low, the reciprocal
+    standard deviation ~0.4 % high. So long half rows are checked against ACC_F64 (tests/util.py half_acc)."""
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal([63, 50, 53, 37]) * 2).astype(np.float16)
+    a = x.transpose(1, 2, 0, 3)
+    g = rng.normal(1, 0.1, a.shape).astype(np.float16)
+    b = rng.normal(0, 0.1, a.shape).astype(np.float16)
+    xd = a.astype(np.float64)
+    ref = (xd - xd.mean()) / np.sqrt(xd.var() + 1e-5) * g.astype(np.float64) + b.astype(np.float64)
+    w64 = orc.layernorm(a, 4, g, b, 1e-5, acc=orc.ACC_F64).astype(np.float64)
+    w32 = orc.layernorm(a, 4, g, b, 1e-5, acc=orc.ACC_F32).astype(np.float64)
+    big = np.abs(ref) > 0.5
+    # f64 mode: half an ulp of f16 (2^-11 relative) and nothing more
+    assert (np.abs(w64 - ref)[big] / np.abs(ref)[big]).max() < 2.0 ** -11 * 1.01
+    assert np.abs(w64 - ref).max() < 2.0 ** -9 * 1.01            # |y| < 8: half an ulp is 2^-9
+    # sequential f32 mode: off by several parts in a thousand, everywhere
+    rel32 = (np.abs(w32 - ref)[big] / np.abs(ref)[big])
+    assert np.median(rel32) > 2e-3 and rel32.max() < 1e-2
+    # the cause, in isolation: the same running sum of squares in numpy's sequential f32 cumsum
+    xf = a.astype(np.float32).reshape(-1)
+    sq = ((xf - np.float32(xd.mean())) ** 2).astype(np.float32)
+    seq = float(np.cumsum(sq, dtype=np.float32)[-1])
+    true = float(sq.astype(np.float64).sum())
+    assert seq > 2.0 ** 24 and 0.990 < seq / true < 0.995
 
 
 def test_timed_restatement_equals_oracle(orc):

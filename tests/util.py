@@ -6,6 +6,19 @@ F32_RTOL, F32_ATOL = 1e-5, 1e-6     # f32 against the f64-accumulating oracle
 HALF_RTOL = 1e-2                    # f16 / bf16 against the f32-accumulating oracle
 
 
+LONG_ROW = 65536
+
+
+def half_acc(orc, n_reduced):
+    """Which oracle mode is the truth for an f16 / bf16 row of `n_reduced` elements. The sequential f32
+    sum (ACC_F32) restates "accumulated in f32" literally, but its own error grows with the row: beyond
+    2^24 a running sum of squares moves in steps of 2 and comes out low by about a percent on millions
+    of elements (see test_sequential_f32_accumulation_is_no_truth_for_long_half_rows). From 65536 elements
+    on the truth is the f64 accumulation rounded once, which any f32 scheme with bounded error (the
+    kernels' trees, pairwise sums) agrees with to half-precision rounding."""
+    return orc.ACC_F64 if n_reduced > LONG_ROW else orc.ACC_F32
+
+
 def half_atol(want, bits):
     """Absolute floor for half types: half an ulp (2^-bits relative) of the output's scale."""
     w = np.asarray(want, np.float64)
