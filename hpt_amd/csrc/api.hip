@@ -295,6 +295,15 @@ NormLaunchFn norm_launcher_for(int kind, int dtype) {
     }
 }
 
+NormLaunchFn norm_promoting_launcher_for(int kind, int in_dtype) {
+    switch (kind) {
+        case NORM_SOFTMAX: return norm_promoting_launcher<NORM_SOFTMAX>(in_dtype);
+        case NORM_LOGSOFTMAX: return norm_promoting_launcher<NORM_LOGSOFTMAX>(in_dtype);
+        case NORM_LAYERNORM: return norm_promoting_launcher<NORM_LAYERNORM>(in_dtype);
+        default: return nullptr;  // the fused kinds take float inputs only
+    }
+}
+
 // ---- view validation -------------------------------------------------------------
 
 static void check_view(const hpt_view* v, const char* name, bool need_data) {
@@ -446,11 +455,16 @@ struct NormCall {
     NormArgs args;
 };
 
-static NormCall prepare_norm(const hpt_view* in, const void* out_data, int64_t axis, int n_norm_dims) {
+// Output dtype of the normalisations: FloatBinaryType<T> (the input's own dtype for floats).
+static int norm_out_dtype(int in_dtype) { return reduce_out_dtype(HPT_MEAN, in_dtype); }
+
+// A non-float input is promoted inside the kernel; the plan is made for the output's element size and
+// cut down to what the promoting kernel runs. `float_only`: the fused kinds.
+static NormCall prepare_norm(const hpt_view* in, const void* out_data, int64_t axis, int n_norm_dims,
+                             bool float_only = false) {
     check_view(in, "normalize input", false);
-    if (!is_float_dtype(in->dtype))
-        fail(HPT_ERR_DTYPE, "softmax/log_softmax/layernorm need a float dtype, got %s",
-             dtype_name(in->dtype));
+    if (float_only && !is_float_dtype(in->dtype))
+        fail(HPT_ERR_DTYPE, "this fused normalisation needs a float dtype, got %s", dtype_name(in->dtype));
     if (in->ndim == 0) fail(HPT_ERR_SHAPE, "normalize: input has no dimensions");
     if (n_norm_dims <= 0) {
         int64_t a = axis;
@@ -462,7 +476,8 @@ static NormCall prepare_norm(const hpt_view* in, const void* out_data, int64_t a
     }
     NormCall c;
     c.plan = plan_normalize(in->data, out_data, in->shape, in->strides, in->ndim, axis, n_norm_dims,
-                            dtype_size(in->dtype));
+                            dtype_size(norm_out_dtype(in->dtype)));
+    if (!is_float_dtype(in->dtype)) restrict_to_row_stream(c.plan);
     NormArgs& a = c.args;
     memset(&a, 0, sizeof a);
     a.in = in->data;
@@ -706,11 +721,13 @@ int32_t hpt_hip_softmax(int32_t dev, void* stream, int32_t log, const hpt_view* 
                         hpt_view* out) {
     return guarded([&] {
         check_view(in, "softmax input", true);
-        check_out(out, in->dtype, view_size(in), "softmax output");
+        check_out(out, norm_out_dtype(in->dtype), view_size(in), "softmax output");
         check_alias(in, out, true, "softmax", "the input");
         NormCall c = prepare_norm(in, out->data, axis, 0);
         if (c.plan.kind == NormKind::Empty) return;
-        NormLaunchFn fn = norm_launcher_for(log ? NORM_LOGSOFTMAX : NORM_SOFTMAX, in->dtype);
+        const int kind = log ? NORM_LOGSOFTMAX : NORM_SOFTMAX;
+        NormLaunchFn fn = is_float_dtype(in->dtype) ? norm_launcher_for(kind, in->dtype)
+                                                    : norm_promoting_launcher_for(kind, in->dtype);
         if (!fn) fail(HPT_ERR_DTYPE, "softmax: unsupported dtype %s", dtype_name(in->dtype));
         use_device(dev);
         launch_norm(dev, (hipStream_t)stream, fn, c, "softmax");
@@ -722,17 +739,18 @@ static void run_layernorm(int dev, void* stream, const hpt_view* in, const hpt_v
                           const hpt_view* gamma, const hpt_view* beta, double eps, hpt_view* out) {
     check_view(in, "layernorm input", true);
     if (n_norm_dims <= 0) fail(HPT_ERR_SHAPE, "layernorm: normalized_shape must not be empty");
-    check_out(out, in->dtype, view_size(in), "layernorm output");
+    const int odt = norm_out_dtype(in->dtype);
+    check_out(out, odt, view_size(in), "layernorm output");
     check_alias(in, out, true, "layernorm", "the input");
-    NormCall c = prepare_norm(in, out->data, 0, n_norm_dims);
+    NormCall c = prepare_norm(in, out->data, 0, n_norm_dims, residual != nullptr);
     const hpt_view* gb[2] = {gamma, beta};
     const char* names[2] = {"layernorm gamma", "layernorm beta"};
     for (int k = 0; k < 2; ++k) {
         if (!gb[k]) continue;
         check_view(gb[k], names[k], true);
-        if (gb[k]->dtype != in->dtype)
+        if (gb[k]->dtype != odt)
             fail(HPT_ERR_DTYPE, "%s: dtype is %s, expected %s", names[k], dtype_name(gb[k]->dtype),
-                 dtype_name(in->dtype));
+                 dtype_name(odt));
         if (!view_contiguous(gb[k])) fail(HPT_ERR_SHAPE, "%s: must be contiguous", names[k]);
         check_alias(gb[k], out, false, "layernorm", k == 0 ? "gamma" : "beta");
         // shape must equal the normalised dims (leading 1s aside)
@@ -766,7 +784,9 @@ static void run_layernorm(int dev, void* stream, const hpt_view* in, const hpt_v
     if (c.plan.vec > 1 && !c.plan.shift &&
         (((uintptr_t)c.args.gamma | (uintptr_t)c.args.beta | (uintptr_t)c.args.residual) % 16) != 0)
         demote_to_generic(c.plan);
-    NormLaunchFn fn = norm_launcher_for(residual ? NORM_ADD_LAYERNORM : NORM_LAYERNORM, in->dtype);
+    NormLaunchFn fn = is_float_dtype(in->dtype)
+                          ? norm_launcher_for(residual ? NORM_ADD_LAYERNORM : NORM_LAYERNORM, in->dtype)
+                          : norm_promoting_launcher_for(NORM_LAYERNORM, in->dtype);
     if (!fn) fail(HPT_ERR_DTYPE, "layernorm: unsupported dtype %s", dtype_name(in->dtype));
     use_device(dev);
     launch_norm(dev, (hipStream_t)stream, fn, c, "layernorm");
@@ -793,7 +813,7 @@ int32_t hpt_hip_softmax_causal(int32_t dev, void* stream, int32_t log, const hpt
         check_out(out, in->dtype, view_size(in), "softmax_causal output");
         check_alias(in, out, true, "softmax_causal", "the input");
         if (in->ndim < 2) fail(HPT_ERR_SHAPE, "softmax_causal: needs at least 2 dims (queries x keys)");
-        NormCall c = prepare_norm(in, out->data, in->ndim - 1, 0);
+        NormCall c = prepare_norm(in, out->data, in->ndim - 1, 0, true);
         if (c.plan.kind == NormKind::Empty) return;
         if (c.plan.kind == NormKind::Transposed || c.plan.kind == NormKind::TransposedTile ||
             c.plan.kind == NormKind::ColSplit || c.plan.kind == NormKind::RowSplit || c.plan.kind == NormKind::ColReg)

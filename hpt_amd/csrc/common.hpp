@@ -166,6 +166,10 @@ std::string describe(const NormPlan& p);
 // what the caller falls back to when an operand rules the specialised kernels out.
 void demote_to_generic(NormPlan& p);
 
+// Keep of a plan what the streaming row kernel can run: rows that are contiguous along the axis and
+// on the vector grid keep their vector width, everything else becomes the generic row form.
+void restrict_to_row_stream(NormPlan& p);
+
 // ---- elementwise: strided copy (contiguous()), fill, binary ops with broadcasting ----
 
 enum class EwKind {

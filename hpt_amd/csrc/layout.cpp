@@ -909,6 +909,21 @@ void demote_to_generic(NormPlan& p) {
     p.rpb = std::max(1, 256 / p.tpr);
 }
 
+void restrict_to_row_stream(NormPlan& p) {
+    if (p.kind == NormKind::Empty) return;
+    const bool rows_on_grid = (p.kind == NormKind::RowReg || p.kind == NormKind::RowStream) && p.vec > 1 &&
+                              p.sstride == 1 && !p.shift && p.norm_in.n == 1 && p.norm_in.stride[0] == 1 &&
+                              p.out_axis_stride == 1;
+    const int vec = rows_on_grid ? p.vec : 1;
+    demote_to_generic(p);
+    if (!rows_on_grid) return;
+    p.kind = NormKind::RowStream;
+    p.vec = vec;
+    p.tpr = (int)std::min<int64_t>(1024, pow2_ceil((p.cols / vec + 3) / 4));
+    if (p.tpr > 64 && p.tpr < 256) p.tpr = 256;
+    p.rpb = std::max(1, 256 / p.tpr);
+}
+
 std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];

@@ -50,4 +50,11 @@ template <int KIND> NormLaunchFn norm_launcher(int dtype);
 
 NormLaunchFn norm_launcher_for(int kind, int dtype);
 
+// Launcher for an INTEGER (or bool) input dtype whose result has the dtype's FloatBinaryType: the
+// promotion is fused into the load of the streaming row kernel. Plain kinds only (softmax,
+// log_softmax, layernorm); the plan must have been passed through restrict_to_row_stream.
+template <int KIND> NormLaunchFn norm_promoting_launcher(int in_dtype);
+
+NormLaunchFn norm_promoting_launcher_for(int kind, int in_dtype);
+
 }  // namespace hpt

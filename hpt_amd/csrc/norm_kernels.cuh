@@ -952,9 +952,29 @@ template <class Op, class S> __device__ __forceinline__ S stat_all_reduce(S v, i
 // and positions outside 0 .. cols - 1 are masked. (An aligned vector that holds one valid
 // element lies in that element's page, so the over-read at both ends is safe.) Input, output
 // and residual rows share m: the caller checks that their bases and row pitches agree mod 16 bytes.
-template <int KIND, class T, int VEC, bool SHIFT = false>
+//
+// TI: the INPUT's element type when it is not the output's. NormalizationOps promote a non-float input to
+// FloatBinaryType<T> inside the op (hpt/src/backends/cpu/tensor_internal/normalization.rs:205-221); here the
+// conversion is part of the load - TI -> T with one rounding, exactly what a separate `astype` would
+// have stored, then widened to the compute type - so an integer tensor is normalised in one launch
+// and no promoted copy goes through HBM.
+template <class T, class TI> __device__ __forceinline__ typename Elem<T>::Wide promoted_input(TI x) {
+    using CT = typename Elem<T>::Wide;
+    if constexpr (std::is_same<T, TI>::value) {
+        return Elem<T>::widen(x);
+    } else {
+        static_assert(!Elem<TI>::is_float && Elem<T>::is_float, "promotion is integer -> float");
+        const CT f = (CT)Elem<TI>::cmp(x);  // (bool: 0 or 1)
+        if constexpr (sizeof(T) < sizeof(CT)) return Elem<T>::widen(Elem<T>::narrow(f));
+        else return f;
+    }
+}
+
+template <int KIND, class T, int VEC, bool SHIFT = false, class TI = T>
 __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
     static_assert(!SHIFT || VEC > 1, "SHIFT is a vector mode");
+    static_assert(std::is_same<T, TI>::value || (!SHIFT && KIND <= NORM_LAYERNORM),
+                  "promoted inputs: plain kinds, rows on the vector grid");
     using CT = typename Elem<T>::Wide;
     __shared__ __align__(16) unsigned char smem_raw[16 * 3 * sizeof(double)];
     const int tpr = a.tpr;
@@ -962,7 +982,7 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
     const int ty = threadIdx.x >> a.tpr_log2;
     const int64_t row = (int64_t)blockIdx.x * a.rpb + ty;
     const bool valid = row < a.rows;
-    const T* in_row = (const T*)a.in + (valid ? offset_of(a.kept_in, row) : 0);
+    const TI* in_row = (const TI*)a.in + (valid ? offset_of(a.kept_in, row) : 0);
     T* out_row = (T*)a.out + (valid ? offset_of(a.kept_out, row) : 0);
     const int m = SHIFT ? (int)(((uintptr_t)in_row / sizeof(T)) % VEC) : 0;
     const int64_t nv = SHIFT ? (a.cols + m + VEC - 1) / VEC : a.cols / VEC;
@@ -991,9 +1011,9 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
     // the separate add / mul_ of the unfused sequence would have stored it.
     auto load = [&](int64_t iv, CT* x) {
         if constexpr (VEC > 1) {
-            Pack<T, VEC> v = load_pack<T, VEC>(in_row - m + iv * VEC);
+            Pack<TI, VEC> v = load_pack<TI, VEC>(in_row - m + iv * VEC);
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) x[j] = Elem<T>::widen(v.v[j]);
+            for (int j = 0; j < VEC; ++j) x[j] = promoted_input<T, TI>(v.v[j]);
             if constexpr (kRes) {
                 Pack<T, VEC> r = load_pack<T, VEC>(res_row - m + iv * VEC);
 #pragma unroll
@@ -1001,7 +1021,7 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
             }
         } else {
             const int64_t off = one_dim ? iv * a.sa : offset_of(a.norm_in, iv);
-            x[0] = Elem<T>::widen(in_row[off]);
+            x[0] = promoted_input<T, TI>(in_row[off]);
             if constexpr (kRes) x[0] = Elem<T>::widen(Elem<T>::narrow(x[0] + Elem<T>::widen(res_row[iv])));
         }
         if constexpr (kCausal) {

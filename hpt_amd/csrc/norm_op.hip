@@ -359,7 +359,49 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
     else row_stream_kernel<KIND, T, 1><<<grid, block, 0, st>>>(a);
 }
 
+// FloatBinaryType<TI> of the integer types (hpt-types/src/type_promote.rs)
+template <class TI> struct PromotedOf { using type = f16_t; };  // bool, i8, i16, u8, u16
+template <> struct PromotedOf<int32_t> { using type = float; };
+template <> struct PromotedOf<uint32_t> { using type = float; };
+template <> struct PromotedOf<int64_t> { using type = double; };
+template <> struct PromotedOf<uint64_t> { using type = double; };
+
+template <class TI> void launch_promoting_t(const NormPlan& p, NormArgs a, hipStream_t st) {
+    using T = typename PromotedOf<TI>::type;
+    constexpr int FULL = 16 / sizeof(T);
+    if (p.kind == NormKind::Empty) return;
+    if constexpr (KIND > NORM_LAYERNORM) {
+        fail(HPT_ERR_DTYPE, "fused normalisation: the input must have a float dtype");
+    } else {
+        if (p.kind != NormKind::RowStream && p.kind != NormKind::Generic)
+            fail(HPT_ERR_KERNEL, "promoted input: the plan was not restricted to the streaming row kernel");
+        a.tpr = p.tpr;
+        a.tpr_log2 = ilog2(p.tpr);
+        a.rpb = p.rpb;
+        a.inv_cols = 1.0 / (double)p.cols;
+        const dim3 grid((unsigned)((p.rows + p.rpb - 1) / p.rpb));
+        const dim3 block((unsigned)(p.tpr * p.rpb));
+        if (p.vec == FULL && FULL > 1) row_stream_kernel<KIND, T, FULL, false, TI><<<grid, block, 0, st>>>(a);
+        else row_stream_kernel<KIND, T, 1, false, TI><<<grid, block, 0, st>>>(a);
+    }
+}
+
 }  // namespace
+
+template <> NormLaunchFn norm_promoting_launcher<HPT_NORM_KIND>(int in_dtype) {
+    switch (in_dtype) {
+        case HPT_BOOL: return &launch_promoting_t<bool8>;
+        case HPT_I8: return &launch_promoting_t<int8_t>;
+        case HPT_I16: return &launch_promoting_t<int16_t>;
+        case HPT_I32: return &launch_promoting_t<int32_t>;
+        case HPT_I64: return &launch_promoting_t<int64_t>;
+        case HPT_U8: return &launch_promoting_t<uint8_t>;
+        case HPT_U16: return &launch_promoting_t<uint16_t>;
+        case HPT_U32: return &launch_promoting_t<uint32_t>;
+        case HPT_U64: return &launch_promoting_t<uint64_t>;
+        default: return nullptr;
+    }
+}
 
 template <> NormLaunchFn norm_launcher<HPT_NORM_KIND>(int dtype) {
     switch (dtype) {

@@ -533,11 +533,9 @@ class Tensor:
 
     def _softmax(self, log: bool, axis: int, stream=None, out: Optional["Tensor"] = None) -> "Tensor":
         self._require_hip("softmax")
-        ft = self._float_binary_type()
-        if ft is not self.dtype:
-            # NormalizationOps::Output = Tensor<FloatBinaryType<T>>: a non-float input is cast first
-            return self.astype(ft, stream=stream)._softmax(log, axis, stream=stream, out=out)
-        res = self._norm_out(out, self.dtype)
+        # NormalizationOps::Output = Tensor<FloatBinaryType<T>>: a non-float input is promoted inside the
+        # kernel (one launch, no promoted copy), as the reference promotes inside the op
+        res = self._norm_out(out, self._float_binary_type())
         vin, k1 = self._c_view()
         vout, k2 = res._c_view()
         check(_ffi.lib().hpt_hip_softmax(self.device, stream, int(log), C.byref(vin), int(axis), C.byref(vout)))
@@ -562,10 +560,11 @@ class Tensor:
                              "normalized dims must match last dims of input tensor, "
                              f"shape: {self.shape}, normalized_shape: {ns}")
         ft = self._float_binary_type()
-        if ft is not self.dtype:
+        if ft is not self.dtype and residual is not None:
+            # (the fused add + layernorm takes float tensors; the promoted copy is kept alive by `_touch`)
             return self.astype(ft, stream=stream).layernorm(normalized_shape, gamma, beta, eps, stream=stream,
                                                             residual=residual, out=out)
-        res = self._norm_out(out, self.dtype)
+        res = self._norm_out(out, ft)
         vin, k1 = self._c_view()
         vout, k2 = res._c_view()
         keep = [k1, k2]

@@ -357,9 +357,9 @@ template <class T> class Tensor {
         for (size_t i = 0; ok && i < normalized_shape.size(); ++i)
             ok = shape_[ndim() - normalized_shape.size() + i] == normalized_shape[i];
         if (!ok) throw TensorError(ErrorKind::Shape, "normalized dims must match last dims of input tensor");
-        const FloatOut src = as_float();
+        // a non-float input is promoted to FloatBinaryType<T> inside the kernel: one call, no copy
         FloatOut res = FloatOut::empty(shape_, device_);
-        hpt_view vin = src.view(), vout = res.view(), vg{}, vb{};
+        hpt_view vin = view(), vout = res.view(), vg{}, vb{};
         if (gamma) vg = gamma->view();
         if (beta) vb = beta->view();
         check(hpt_hip_layernorm(device_, nullptr, &vin, (int32_t)normalized_shape.size(), gamma ? &vg : nullptr,
@@ -439,15 +439,10 @@ template <class T> class Tensor {
         check(hpt_hip_argreduce(device_, nullptr, is_max ? 1 : 0, &vin, axis, &vout));
         return keep_dims ? res.reshape(reduced_shape(ax, true)) : res;
     }
-    // a non-float input is cast to FloatBinaryType<T> first (the entries' Output type)
-    FloatOut as_float() const {
-        if constexpr (std::is_same<FloatBinaryType<T>, T>::value) return *this;
-        else return astype<FloatBinaryType<T>>();
-    }
+    // (a non-float input is promoted to FloatBinaryType<T>, the entries' Output type, inside the kernel)
     FloatOut softmax_impl(bool log, int64_t axis) const {
-        const FloatOut src = as_float();
         FloatOut res = FloatOut::empty(shape_, device_);
-        hpt_view vin = src.view(), vout = res.view();
+        hpt_view vin = view(), vout = res.view();
         check(hpt_hip_softmax(device_, nullptr, log ? 1 : 0, &vin, axis, &vout));
         return res;
     }

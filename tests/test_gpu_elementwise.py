@@ -262,3 +262,77 @@ def test_integer_inputs_of_softmax_and_layernorm_promote(hpt, orc, dev):
     s64 = hpt.Tensor.from_numpy(x64).to_hip(dev).permute([2, 0, 1]).softmax(0)
     assert s64.dtype is hpt.f64
     assert_close(s64.numpy(), orc.softmax(x64.astype(np.float64).transpose(2, 0, 1), 0, acc=orc.ACC_F64), 1e-12, 1e-14, "softmax of i64")
+
+
+PROMOTED = [(np.bool_, np.float16), (np.int8, np.float16), (np.int16, np.float16), (np.uint8, np.float16), (np.uint16, np.float16),
+            (np.int32, np.float32), (np.uint32, np.float32), (np.int64, np.float64), (np.uint64, np.float64)]
+
+
+@pytest.mark.parametrize("npin,npout", PROMOTED, ids=[p[0].__name__ for p in PROMOTED])
+def test_integer_inputs_are_promoted_inside_one_call(hpt, orc, dev, npin, npout):
+    """softmax / log_softmax / layernorm of an integer tensor through ONE C-ABI call each (no astype
+    first): the result must equal the op applied to the input cast to FloatBinaryType<T> - including
+    values the cast rounds (i16 / u16 beyond 2048 in f16, i32 beyond 2^24 in f32, u16 beyond 65504 -> inf) -
+    on contiguous rows (vector loads of the integer type), permuted, sliced and stepped views."""
+    import ctypes as C
+    from conftest import assert_close
+    from util import layouts_for, upload
+    rng = np.random.default_rng(77)
+    half = npout == np.float16
+    for shape in ([33, 256], [5, 6, 40], [260, 1024]):
+        if npin == np.bool_:
+            base = rng.random(shape) < 0.4
+        else:
+            info = np.iinfo(npin)
+            base = rng.integers(max(info.min, -9), min(info.max, 9) + 1, shape).astype(npin)
+            # a few values that do not survive the cast exactly
+            flat = base.reshape(-1)
+            big = {np.int16: [2049, -4099, 30001], np.uint16: [2051, 65519, 65535], np.int32: [(1 << 24) + 1, -(1 << 25) - 3],
+                   np.uint32: [(1 << 24) + 1, 4294967295], np.int64: [(1 << 53) + 1], np.uint64: [(1 << 53) + 1]}.get(npin, [])
+            for k, v in enumerate(big):
+                flat[(k * 37) % flat.size] = v
+        for lname, ops in layouts_for(shape, rng):
+            t, a = upload(hpt, base, ops, dev=dev)
+            if a.size == 0:
+                continue
+            with np.errstate(over="ignore"):
+                af = a.astype(npout)      # what `astype` would have stored
+            nd = a.ndim
+            for axis in (nd - 1, 0):
+                for log in (False, True):
+                    # straight through the ABI: integer view in, float tensor out
+                    res = hpt.Tensor.empty(a.shape, hpt.DTYPES[orc.reduce_out_dtype(orc.MEAN, t.dtype.code)], dev)
+                    vin, k1 = t._c_view()
+                    vout, k2 = res._c_view()
+                    hpt._ffi.check(hpt.lib().hpt_hip_softmax(dev, None, int(log), C.byref(vin), axis, C.byref(vout)))
+                    got = res.numpy()
+                    assert got.dtype == npout
+                    with np.errstate(invalid="ignore", over="ignore"):
+                        want = orc.softmax(af, axis, log=log, acc=orc.ACC_F32 if half else orc.ACC_F64)
+                    assert np.array_equal(np.isnan(got), np.isnan(want)), f"{npin.__name__} {shape} {lname} axis={axis} log={log}: NaN pattern"
+                    if half:
+                        assert_close(got, want, 1e-2, 1e-3 if log else 6e-8 + 1e-3 * float(np.nanmax(want)), f"softmax {npin.__name__} {shape} {lname} axis={axis} log={log}")
+                    elif npout == np.float32:
+                        assert_close(got, want, 1e-5, 2e-6, f"softmax {npin.__name__} {shape} {lname} axis={axis} log={log}")
+                    else:
+                        assert_close(got, want, 1e-12, 1e-13, f"softmax {npin.__name__} {shape} {lname} axis={axis} log={log}")
+            n = a.shape[-1]
+            g = rng.normal(1, 0.1, n).astype(npout)
+            b = rng.normal(0, 0.1, n).astype(npout)
+            tg, tb = hpt.Tensor.from_numpy(g).to_hip(dev), hpt.Tensor.from_numpy(b).to_hip(dev)
+            got = t.layernorm([n], tg, tb, 1e-5).numpy()
+            assert got.dtype == npout
+            fin = np.isfinite(af).all(axis=-1)
+            with np.errstate(invalid="ignore", over="ignore"):
+                want = orc.layernorm(af, 1, g, b, 1e-5, acc=orc.ACC_F32 if half else orc.ACC_F64)
+            tol = (1e-2, 4e-3) if half else ((1e-5, 4e-6) if npout == np.float32 else (1e-12, 1e-12))
+            assert_close(got[fin], want[fin], tol[0], tol[1], f"layernorm {npin.__name__} {shape} {lname}")
+            # gamma / beta must have the OUTPUT's dtype
+            if npin != np.bool_ and lname == "contiguous":
+                wrong = hpt.Tensor.from_numpy(np.ones(n, npin)).to_hip(dev)
+                with pytest.raises(hpt.DTypeError, match="gamma"):
+                    t.layernorm([n], wrong, None, 1e-5)
+    # the fused kinds take float tensors only
+    ti = hpt.Tensor.from_numpy(np.ones((4, 8), npin)).to_hip(dev)
+    with pytest.raises(hpt.DTypeError):
+        ti.softmax_causal(1.0)

@@ -182,8 +182,14 @@ def test_argument_errors_without_a_device(hpt):
         hpt.reduce_plan(t, hpt.SUM, [5])
     with pytest.raises(hpt.ParamError):
         hpt.reduce_plan(t, 99, [0])
-    with pytest.raises(hpt.DTypeError):
-        hpt.normalize_plan(hpt.Tensor.from_numpy(np.zeros((3, 4), np.int32)), 1)
+    # an integer input is promoted inside the kernel: it plans as the streaming row form of its float type
+    assert hpt.normalize_plan(hpt.Tensor.from_numpy(np.zeros((3, 4), np.int32)), 1).startswith("rowstream rows=3 cols=4 vec=4 ")
+    from hpt_amd.tensor import Tensor, _contiguous_strides
+    big = Tensor(None, 4096, [4096, 4096], _contiguous_strides([4096, 4096]), hpt.i32, "hip", 0)
+    assert hpt.normalize_plan(big, 1).startswith("rowstream rows=4096 cols=4096 vec=4 "), hpt.normalize_plan(big, 1)
+    assert hpt.normalize_plan(big.permute([1, 0]), 1).startswith("generic"), hpt.normalize_plan(big.permute([1, 0]), 1)
+    small = Tensor(None, 4096, [4096, 4096], _contiguous_strides([4096, 4096]), hpt.u8, "hip", 0)
+    assert hpt.normalize_plan(small, 1).startswith("rowstream rows=4096 cols=4096 vec=8 "), hpt.normalize_plan(small, 1)
     with pytest.raises(NotImplementedError, match="Hip backend only"):
         t.sum([0])
     with pytest.raises(NotImplementedError):
