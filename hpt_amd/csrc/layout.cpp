@@ -739,6 +739,16 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 p.nchunk = std::max(1, pow2_ceil(nc));
                 int block = std::max(256, p.tpr);
                 p.rpb = block / p.tpr;
+                // Layernorm workgroups walk the rows; how many of them is best depends on how many a compute unit
+                // can hold. f32 rows of four vectors per thread (gamma and beta beside them: ~100 registers, four
+                // workgroups of 256 threads per compute unit) do best with THREE per compute unit, rows of two vectors
+                // with six. Measured, us (768 / 1024 / 1536 workgroups): [8192, 4096] 45.7 / 47.6 / 47.5, [32768, 1024]
+                // 45.1 / 46.2 / 47.1, [65536, 512] 45.0 / 46.4 / 47.4; [16384, 2048] 52.9 / 47.5 / 46.3, [8192, 2048]
+                // 29.1 / 26.2 / 25.2, [8192, 1536] 26.9 / 23.1 / 20.3. Two-byte rows prefetch their next row and stay at 1024.
+                if (n_norm_dims > 0 && elem_size == 4 && v > 1 && p.tpr <= 256) {
+                    if (p.nchunk >= 4) p.max_blocks = 768;
+                    else if (p.nchunk == 2) p.max_blocks = 1536;
+                }
             } else {
                 p.kind = NormKind::RowStream;
                 p.tpr = 1024;
