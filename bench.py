@@ -13,9 +13,20 @@ from HBM.
 Prints ONE JSON line. `value` is algorithmic GB/s (every logical input element read once +
 every output element written once + gamma/beta once, per step) over the wall-clock time of
 exactly K steps. `roofline.achieved` uses the same bytes over the kernel's average duration
-measured with HIP events on the launch stream. `ops` lists the same measurement for every
-op of the five benchmark configurations. `cpu_baseline` is the CPU restatement of Hpt's
-layernorm (oracle/, test infrastructure) timed on the host cores of this box.
+measured with HIP events on the launch stream; `roofline.kernel`, `traffic` and the profiler's
+own duration come from profiles/headline.json (written when the rocprofv3 summaries under
+profiles/ are regenerated), and the plan the library reports for the headline call is printed
+beside the plan recorded there, so a planner change that makes the profile stale shows.
+
+`ops` lists every op of the five benchmark configurations (and the groups c6-c8), each timed
+the same way whatever --steps says: 10 warm-up launches, then 13 groups of 8 back-to-back
+launches, every group bracketed by a pair of HIP events; `us_per_launch` is the median over the
+groups of (group time / 8) - 104 timed launches. (Bracketing every single launch instead adds
+about 3 us of event handling per launch, which is a sixth of a 17 us reduction.) Where the
+restated Hpt CPU path has the op (contiguous f32 rows: softmax, log_softmax, layernorm, sum, max)
+it is timed on this box's host cores and reported beside it as `cpu_GBps`.
+`cpu_baseline` is the headline's: the CPU restatement of Hpt's layernorm (oracle/, test
+infrastructure).
 """
 from __future__ import annotations
 
@@ -33,11 +44,11 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
-# HBM bytes one headline launch moves, from two hardware-counter runs of this script
-# (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, with --copy-calibration), each counter scaled
-# by what it reads for the plain 134217728-byte copy in the same run: fetch 131395.9 KiB +
-# write 131093.8 KiB. A measured constant, not something this script can read live.
-HEADLINE_TRAFFIC_BYTES = 268783485
+# What the profiler saw for the headline launch (kernel name, average duration, HBM bytes from
+# FETCH_SIZE / WRITE_SIZE scaled by a plain copy of known size) and the plan the library
+# reported in that run. Measured constants, not something this script can read live.
+HEADLINE_PROFILE = ROOT / "profiles" / "headline.json"
+GROUPS, PER_GROUP, OP_WARMUP = 13, 8, 10  # per-op timing: 104 launches in 13 event-bracketed groups
 
 
 # ---- HIP events on the launch stream (the null stream: the library is called with stream=NULL) ----
@@ -81,9 +92,11 @@ def gen_c2(seed=1):
 class Case:
     """One op on one configuration: `run(i)` enqueues one step on buffer set i % nbuf."""
 
-    def __init__(self, name, cfg, dtype, rows, algo_bytes, run, nbuf, check=None):
+    def __init__(self, name, cfg, dtype, rows, algo_bytes, run, nbuf, check=None, plan=None, cpu=None):
         self.name, self.cfg, self.dtype, self.rows = name, cfg, dtype, rows
         self.bytes, self.run, self.nbuf, self.check = algo_bytes, run, nbuf, check
+        self.plan = plan  # what the library's planner says it launches for this call
+        self.cpu = cpu    # () -> seconds per pass of the restated Hpt CPU path on the same input, or None
 
 
 def time_case(ev: HipEvents, case: Case, steps: int, warmup: int):
@@ -101,6 +114,51 @@ def time_case(ev: HipEvents, case: Case, steps: int, warmup: int):
     wall = time.perf_counter() - t0
     dev_ms = ev.elapsed_ms(e0, e1)
     return wall, dev_ms
+
+
+def time_groups(ev: HipEvents, case: Case, groups: int = GROUPS, per: int = PER_GROUP, warmup: int = OP_WARMUP):
+    """Microseconds per launch of each of `groups` event-bracketed runs of `per` back-to-back launches."""
+    import hpt_amd as hpt
+    for i in range(warmup):
+        case.run(i)
+    hpt.synchronize(0)
+    marks = [ev.event() for _ in range(groups + 1)]
+    ev.record(marks[0])
+    k = warmup
+    for g in range(groups):
+        for _ in range(per):
+            case.run(k)
+            k += 1
+        ev.record(marks[g + 1])
+    hpt.synchronize(0)
+    return [ev.elapsed_ms(marks[g], marks[g + 1]) * 1e3 / per for g in range(groups)]
+
+
+def cpu_seconds(fn, budget_s=1.5, min_passes=3, max_passes=200):
+    """Median seconds per call of `fn` (one warm-up call first), for about `budget_s` seconds."""
+    fn()
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < min_passes or (time.perf_counter() < t_end and len(times) < max_passes):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return float(np.median(times)), len(times)
+
+
+def cpu_rows(op, x):
+    """The restated Hpt CPU path for a row op on the contiguous f32 matrix `x`: a callable that runs one
+    pass on this box's physical cores (rows split as Hpt's thread pool splits them)."""
+    def call():
+        from oracle import oracle as orc
+        cores = orc.physical_cores()
+        if op in ("softmax", "log_softmax"):
+            out = np.empty_like(x)
+            return lambda: orc.mt_softmax_f32(x, op == "log_softmax", cores, out)
+        out = np.empty(x.shape[0], np.float32)
+        code = orc.SUM if op == "sum" else orc.MAX
+        return lambda: orc.mt_reduce_rows_f32(x, code, cores, out)
+    return call
 
 
 class Prepared:
@@ -123,6 +181,7 @@ class Prepared:
         outs = [hpt.Tensor.empty(t.shape, t.dtype, 0) for t in ins]
         vi, vo = [self.view(t) for t in ins], [self.view(t) for t in outs]
         n = len(ins)
+        self.last_plan = hpt.normalize_plan(ins[0], axis, n_norm if kind == "layernorm" else 0).split(" rows_in=")[0]
         if kind == "layernorm":
             vg, vb = self.view(gamma), self.view(beta)
             return lambda i: check(l.hpt_hip_layernorm(0, None, vi[i % n], n_norm, vg, vb, eps, vo[i % n])), outs
@@ -137,8 +196,11 @@ class Prepared:
         vi, vo = [self.view(t) for t in ins], [self.view(t) for t in outs]
         n = len(ins)
         if arg is not None:
+            # (the arg-reductions are entries 14 / 15 of the planner's op table)
+            self.last_plan = hpt.reduce_plan(ins[0], 15 if arg else 14, [axes]).split(" kept=")[0]
             return lambda i: check(l.hpt_hip_argreduce(0, None, int(arg), vi[i % n], axes, vo[i % n])), outs
         code = getattr(hpt, op.upper())
+        self.last_plan = hpt.reduce_plan(ins[0], code, axes).split(" kept=")[0]
         ax = self.ffi.i64_array(axes)
         self.keep.append(ax)
         na = len(axes)
@@ -154,10 +216,11 @@ def cases_c2(P, headline_only):
     tg, tb = hpt.Tensor.from_numpy(g).to_hip(0), hpt.Tensor.from_numpy(b).to_hip(0)
     ln_bytes = 2 * x.nbytes + g.nbytes + b.nbytes
     run, ln_outs = P.norm(xs, "layernorm", n_norm=1, gamma=tg, beta=tb)
-    cases = [Case("layernorm", "C2 f32 [8192,4096] gamma,beta eps=1e-5", "f32", 8192, ln_bytes, run, nbuf)]
+    cases = [Case("layernorm", "C2 f32 [8192,4096] gamma,beta eps=1e-5", "f32", 8192, ln_bytes, run, nbuf, plan=P.last_plan)]
     if not headline_only:
         run, _ = P.norm(xs, "log_softmax", axis=1)
-        cases.append(Case("log_softmax", "C2 f32 [8192,4096] axis=1", "f32", 8192, 2 * x.nbytes, run, nbuf))
+        cases.append(Case("log_softmax", "C2 f32 [8192,4096] axis=1", "f32", 8192, 2 * x.nbytes, run, nbuf, plan=P.last_plan,
+                          cpu=cpu_rows("log_softmax", x)))
     return cases, (x, g, b, ln_outs[0])
 
 
@@ -169,11 +232,14 @@ def cases_c1(P):
     c1s = [hpt.Tensor.from_numpy(np.roll(c1, k, 0)).to_hip(0) for k in range(64)]
     cases = []
     run, _ = P.norm(c1s, "softmax", axis=1)
-    cases.append(Case("softmax", "C1 f32 [1024,1024] axis=1", "f32", 1024, 2 * c1.nbytes, run, 64))
+    cases.append(Case("softmax", "C1 f32 [1024,1024] axis=1", "f32", 1024, 2 * c1.nbytes, run, 64, plan=P.last_plan,
+                      cpu=cpu_rows("softmax", c1)))
     run, _ = P.reduce(c1s, "sum", [1])
-    cases.append(Case("sum(axis=1)", "C1 f32 [1024,1024]", "f32", 1024, c1.nbytes + 4096, run, 64))
+    cases.append(Case("sum(axis=1)", "C1 f32 [1024,1024]", "f32", 1024, c1.nbytes + 4096, run, 64, plan=P.last_plan,
+                      cpu=cpu_rows("sum", c1)))
     run, _ = P.reduce(c1s, "max", [1])
-    cases.append(Case("max(axis=1)", "C1 f32 [1024,1024]", "f32", 1024, c1.nbytes + 4096, run, 64))
+    cases.append(Case("max(axis=1)", "C1 f32 [1024,1024]", "f32", 1024, c1.nbytes + 4096, run, 64, plan=P.last_plan,
+                      cpu=cpu_rows("max", c1)))
     return cases
 
 
@@ -193,11 +259,13 @@ def cases_c3(P):
                                        ("max(axis=1)", "max", [1], 200704, 200704 * 4),
                                        ("sum(all)", "sum", [0, 1, 2, 3], 1, 4)):
         run, _ = P.reduce(c3s, op, axes)
-        cases.append(Case(name, "C3 f32 [64,128,56,56]", "f32", rows, nb + outb, run, 6))
+        # sum / mean over [2, 3] are row reductions of the contiguous [8192, 3136] matrix on the CPU path too
+        cpu = cpu_rows("sum", c3.reshape(8192, 3136)) if axes == [2, 3] else None
+        cases.append(Case(name, "C3 f32 [64,128,56,56]", "f32", rows, nb + outb, run, 6, plan=P.last_plan, cpu=cpu))
     run, _ = P.reduce(c3is, "sum", [1])
-    cases.append(Case("sum(axis=1)", "C3 i32 [64,128,56,56]", "i32", 200704, nb + 200704 * 4, run, 6))
+    cases.append(Case("sum(axis=1)", "C3 i32 [64,128,56,56]", "i32", 200704, nb + 200704 * 4, run, 6, plan=P.last_plan))
     run, _ = P.reduce(c3is, "argmax", 1, arg=True)
-    cases.append(Case("argmax(axis=1)", "C3 i32 [64,128,56,56]", "i32", 200704, nb + 200704 * 8, run, 6))
+    cases.append(Case("argmax(axis=1)", "C3 i32 [64,128,56,56]", "i32", 200704, nb + 200704 * 8, run, 6, plan=P.last_plan))
     return cases
 
 
@@ -214,7 +282,7 @@ def cases_c4(P):
            hpt.Tensor.from_numpy(np.roll(c4b, 2048, 0), hpt.bf16).to_hip(0)]
     run, _ = P.norm(c4s, "softmax", axis=1)
     return [Case("softmax", "C4 bf16 [65536,2048] causal mask as data, axis=1", "bf16", 65536,
-                 2 * c4b.nbytes, run, 2)]
+                 2 * c4b.nbytes, run, 2, plan=P.last_plan)]
 
 
 def cases_c5(P):
@@ -231,17 +299,17 @@ def cases_c5(P):
     c5h = [t[:, ::2] for t in c5s]
     cases = []
     run, _ = P.norm(c5t, "layernorm", n_norm=1, gamma=tg5, beta=tb5)
-    cases.append(Case("layernorm", "C5a f16 [4096,8192].permute(1,0) -> [8192,4096]", "f16", 8192, 2 * n5 + 16384, run, 6))
+    cases.append(Case("layernorm", "C5a f16 [4096,8192].permute(1,0) -> [8192,4096]", "f16", 8192, 2 * n5 + 16384, run, 6, plan=P.last_plan))
     run, _ = P.norm(c5t, "softmax", axis=1)
-    cases.append(Case("softmax", "C5a f16 [4096,8192].permute(1,0) axis=1", "f16", 8192, 2 * n5, run, 6))
+    cases.append(Case("softmax", "C5a f16 [4096,8192].permute(1,0) axis=1", "f16", 8192, 2 * n5, run, 6, plan=P.last_plan))
     run, _ = P.reduce(c5t, "sum", [0])
-    cases.append(Case("sum(axis=0)", "C5a f16 [4096,8192].permute(1,0)", "f16", 4096, n5 + 8192, run, 6))
+    cases.append(Case("sum(axis=0)", "C5a f16 [4096,8192].permute(1,0)", "f16", 4096, n5 + 8192, run, 6, plan=P.last_plan))
     run, _ = P.norm(c5h, "layernorm", n_norm=1, gamma=tg5, beta=tb5)
-    cases.append(Case("layernorm", "C5b f16 [4096,8192][:, ::2] -> [4096,4096]", "f16", 4096, n5 + 16384, run, 6))
+    cases.append(Case("layernorm", "C5b f16 [4096,8192][:, ::2] -> [4096,4096]", "f16", 4096, n5 + 16384, run, 6, plan=P.last_plan))
     run, _ = P.norm(c5h, "softmax", axis=1)
-    cases.append(Case("softmax", "C5b f16 [4096,8192][:, ::2] axis=1", "f16", 4096, n5, run, 6))
+    cases.append(Case("softmax", "C5b f16 [4096,8192][:, ::2] axis=1", "f16", 4096, n5, run, 6, plan=P.last_plan))
     run, _ = P.reduce(c5h, "sum", [0])
-    cases.append(Case("sum(axis=0)", "C5b f16 [4096,8192][:, ::2]", "f16", 4096, n5 // 2 + 8192, run, 6))
+    cases.append(Case("sum(axis=0)", "C5b f16 [4096,8192][:, ::2]", "f16", 4096, n5 // 2 + 8192, run, 6, plan=P.last_plan))
     return cases
 
 
@@ -321,12 +389,12 @@ def cases_c8(P):
     def red(ts, nb, cfg, op, axes, label, rows):
         run, outs = P.reduce(ts, op, axes)
         P.keep.append(outs)
-        cases.append(Case(label, cfg, "f32", rows, nb, run, len(ts)))
+        cases.append(Case(label, cfg, "f32", rows, nb, run, len(ts), plan=P.last_plan))
 
     def nrm(ts, nb, cfg, kind, axis, label, rows):
         run, outs = P.norm(ts, kind, axis=axis)
         P.keep.append(outs)
-        cases.append(Case(label, cfg, "f32", rows, 2 * nb, run, len(ts)))
+        cases.append(Case(label, cfg, "f32", rows, 2 * nb, run, len(ts), plan=P.last_plan))
 
     ts, nb = up([1016800, 33])
     red(ts, nb, "f32 [1016800,33] (short odd rows)", "sum", [1], "sum(axis=1)", 1016800)
@@ -449,17 +517,22 @@ def main():
 
     ops = []
     for c in cases:
-        if c is head:
-            w, d = wall, dev_ms
-            n = args.steps
-        else:
-            n = max(20, min(args.steps, 100))
-            w, d = time_case(ev, c, n, min(args.warmup, 10))
-        ops.append({"config": c.cfg, "op": c.name, "dtype": c.dtype, "algorithmic_bytes": c.bytes,
-                    "us_per_launch": round(d * 1e3 / n, 2),
-                    "GBps": round(c.bytes / (d / n * 1e-3) / 1e9, 1),
-                    "pct_of_hbm_peak": round(100 * c.bytes / (d / n * 1e-3) / 1e9 / HBM_PEAK_GBS, 1),
-                    "rows_per_s": round(c.rows / (d / n * 1e-3), 1)})
+        per = time_groups(ev, c)
+        med = float(np.median(per))
+        o = {"config": c.cfg, "op": c.name, "dtype": c.dtype, "algorithmic_bytes": c.bytes,
+             "us_per_launch": round(med, 2), "us_min": round(min(per), 2), "us_max": round(max(per), 2),
+             "launches_timed": GROUPS * PER_GROUP,
+             "GBps": round(c.bytes / (med * 1e-6) / 1e9, 1),
+             "pct_of_hbm_peak": round(100 * c.bytes / (med * 1e-6) / 1e9 / HBM_PEAK_GBS, 1),
+             "rows_per_s": round(c.rows / (med * 1e-6), 1), "plan": c.plan}
+        if c.cpu is not None and not args.no_cpu:
+            from oracle import oracle as orc
+            sec, passes = cpu_seconds(c.cpu())
+            o["cpu_GBps"] = round(c.bytes / sec / 1e9, 2)
+            o["cpu_ms_per_pass"] = round(sec * 1e3, 3)
+            o["cpu_cores"] = orc.physical_cores()
+            o["cpu_kind"] = "port"
+        ops.append(o)
 
     if args.copy_calibration:
         src, dst = prepared.keep[0][0], head_out
@@ -473,6 +546,23 @@ def main():
     if not args.no_cpu:
         cpu = cpu_baseline(x, g, b, head_out.numpy())
 
+    # The dominant kernel, its HBM traffic and the profiler's own duration come from the committed profile
+    # summary; the plan the library reports NOW is set beside the plan recorded THERE.
+    plan_now = head.plan
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": None,
+                "kernel_us": round(kernel_us, 2), "plan": plan_now}
+    if HEADLINE_PROFILE.exists():
+        prof = json.loads(HEADLINE_PROFILE.read_text())
+        same = prof.get("plan") == plan_now
+        roofline.update({"kernel": prof.get("kernel"), "profile_plan": prof.get("plan"), "profile_matches_plan": same,
+                         "profiler_kernel_us": prof.get("profiler_avg_us"),
+                         # a stale profile says nothing about the kernel that ran: no traffic figure then
+                         "traffic": prof.get("traffic_bytes") if same else None})
+        if not same:
+            print(f"bench.py: profiles/headline.json was recorded for plan '{prof.get('plan')}', the library now plans "
+                  f"'{plan_now}': regenerate the profile", file=sys.stderr)
+
     line = {
         "metric": "achieved HBM GB/s (% of MI355X peak) + rows/s for softmax/layernorm/reduce",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -484,15 +574,14 @@ def main():
                    "buffers_rotated": head.nbuf},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1),
         "rows_per_s": round(8192 * args.steps / wall, 1),
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": HEADLINE_TRAFFIC_BYTES,
-                     "kernel": "hpt::row_reg_kernel<2, float, 4, 4, 1, false, false, false>", "kernel_us": round(kernel_us, 2)},
+        "roofline": roofline,
         "cpu_baseline": cpu,
         "ops": ops,
     }
     for o in ops:
+        cpu = f"  cpu {o['cpu_GBps']:.1f} GB/s on {o['cpu_cores']} cores" if "cpu_GBps" in o else ""
         print(f"  {o['config']:<58} {o['op']:<16} {o['us_per_launch']:>9.2f} us  {o['GBps']:>8.1f} GB/s "
-              f"{o['pct_of_hbm_peak']:>5.1f}%  {o['rows_per_s']:.3g} rows/s", file=sys.stderr)
+              f"{o['pct_of_hbm_peak']:>5.1f}%  {o['rows_per_s']:.3g} rows/s{cpu}", file=sys.stderr)
     print(json.dumps(line))
 
 

@@ -48,7 +48,7 @@ def units():
 
 
 def _newest_header() -> float:
-    hs = list(CSRC.glob("*.hpp")) + list(CSRC.glob("*.cuh")) + list(INCLUDE.glob("*.h"))
+    hs = list(CSRC.glob("*.hpp")) + list(INCLUDE.glob("*.h"))
     return max(h.stat().st_mtime for h in hs)
 
 

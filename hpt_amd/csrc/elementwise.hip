@@ -8,7 +8,7 @@
 // All are HBM-bound: the work is in keeping both sides of the copy on whole cache lines.
 #include <cstring>
 
-#include "device_utils.cuh"
+#include "device_utils.hpp"
 #include "elementwise_entry.hpp"
 
 namespace hpt {

@@ -941,6 +941,7 @@ std::string describe(const NormPlan& p) {
              names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg) ? "-unaligned" : (p.raw_rows ? "-raw-shift" : (p.lds_rows ? "-lds-shift" : "-shift"))) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.group_tile ? "-group-tile" : (p.slab_tile ? "-slab" : "")), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
+    if (p.kind == NormKind::RowReg) s += "max_blocks=" + std::to_string(p.max_blocks) + " ";  // (layernorm walks its rows)
     describe_dims(s, "rows_in", p.kept_in);
     s += " ";
     describe_dims(s, "norm_in", p.norm_in);

@@ -23,7 +23,7 @@
 // reciprocal per row replaces the per-element division.
 #pragma once
 
-#include "device_utils.cuh"
+#include "device_utils.hpp"
 #include "norm_entry.hpp"
 
 namespace hpt {
@@ -40,7 +40,7 @@ template <class CT> struct SumC {
 
 // exp / log in the compute type. Half tensors, whose results are rounded to 8 or 11 significant
 // bits anyway, use the hardware exp2 / log2 on the scaled argument; f32 tensors (tolerance 1e-5
-// against the CPU path) the exactly reduced form (exp_reduced, device_utils.cuh).
+// against the CPU path) the exactly reduced form (exp_reduced, device_utils.hpp).
 template <class T> __device__ __forceinline__ float exp_ct(float x) {
     if constexpr (sizeof(T) == 2) return __expf(x);
     else return exp_reduced<true>(x);  // every exponential of a softmax is of x - max <= 0

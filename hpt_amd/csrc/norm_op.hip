@@ -2,7 +2,7 @@
 // float dtypes. Compiled once per kind with -DHPT_NORM_KIND=<0...5>.
 #include <algorithm>
 
-#include "transpose_norm.cuh"
+#include "transpose_norm.hpp"
 
 #ifndef HPT_NORM_KIND
 #error "compile with -DHPT_NORM_KIND=<kind>"

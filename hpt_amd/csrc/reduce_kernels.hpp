@@ -23,12 +23,12 @@
 // serialise (measured: 155 us against 19 us for a 100 MB full sum).
 //
 // These replace the eight kernel variants per op of the reference's device
-// path (hpt-cudakernels/src/reduce/reduce_template.cuh:8-198) and the CPU
+// path (hpt-cudakernels/src/reduce/reduce_template.hpp:8-198) and the CPU
 // kernels hpt/src/backends/cpu/kernels/reduce.rs:153-791.
 #pragma once
 
 #include "reduce_entry.hpp"
-#include "reduce_ops.cuh"
+#include "reduce_ops.hpp"
 
 namespace hpt {
 

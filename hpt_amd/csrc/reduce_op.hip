@@ -1,7 +1,7 @@
 // One reduction op for all thirteen dtypes. Compiled once per op with
 // -DHPT_REDUCE_ENTRY=<n> (see reduce_entry.hpp for the numbering).
 #include "reduce_entry.hpp"
-#include "reduce_kernels.cuh"
+#include "reduce_kernels.hpp"
 
 #ifndef HPT_REDUCE_ENTRY
 #error "compile with -DHPT_REDUCE_ENTRY=<op number>"

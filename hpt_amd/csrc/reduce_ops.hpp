@@ -9,7 +9,7 @@
 // rounded once when the result is stored.
 #pragma once
 
-#include "device_utils.cuh"
+#include "device_utils.hpp"
 
 namespace hpt {
 

@@ -16,12 +16,12 @@
 //       vectors of VEC consecutive columns. Both sides move whole 128-byte
 //       lines; the transpose is only a renaming of registers: no LDS.
 //
-// Arithmetic is that of norm_kernels.cuh (the CPU reference's
+// Arithmetic is that of norm_kernels.hpp (the CPU reference's
 // hpt/src/backends/cpu/kernels/softmax.rs:81-201 column form and
 // hpt/src/backends/cpu/tensor_internal/normalization.rs:126-201).
 #pragma once
 
-#include "norm_kernels.cuh"
+#include "norm_kernels.hpp"
 
 namespace hpt {
 
