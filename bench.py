@@ -27,6 +27,9 @@ restated Hpt CPU path has the op (contiguous f32 rows: softmax, log_softmax, lay
 it is timed on this box's host cores and reported beside it as `cpu_GBps`.
 `cpu_baseline` is the headline's: the CPU restatement of Hpt's layernorm (oracle/, test
 infrastructure).
+
+Two side modes print a table instead of the JSON line: `--sweep f32,f16` (achieved TB/s of seven ops
+over [N, C] shapes from C = 3 to C = 2^20) and `--host-time` (host time per call of the selected ops).
 """
 from __future__ import annotations
 
@@ -481,6 +484,54 @@ def cpu_baseline(x, g, b, gpu_out, budget_s=15.0):
             "rows_per_s": round(8192 / med, 1), "port_max_abs_err_vs_f64_oracle": port_err}
 
 
+def shape_sweep(ev, dtypes):
+    """Achieved algorithmic TB/s over 2-D tensors [N, C] of 32 Mi elements, C from 3 to 2^20, for the seven
+    ops of the path (looking for cliffs between the planner's regions). Prints a markdown table per dtype."""
+    import hpt_amd as hpt
+    P = Prepared()
+    total = 32 << 20
+    for dname in dtypes:
+        npdt = {"f32": np.float32, "f16": np.float16}[dname]
+        print(f"| `[N, C]`, {dname} | sum(1) | sum(0) | argmax(1) | argmax(0) | softmax(1) | softmax(0) | layernorm |")
+        print("|---|---|---|---|---|---|---|---|")
+        for cols in (3, 8, 33, 100, 257, 1000, 1024, 4097, 10000, 65536, 1 << 20):
+            rows = max(1, total // cols)
+            base = np.random.default_rng(0).standard_normal((rows, cols)).astype(npdt)
+            ts = [hpt.Tensor.from_numpy(base).to_hip(0) for _ in range(3)]
+            nb = base.nbytes
+            g, b = hpt.Tensor.ones([cols], ts[0].dtype, 0), hpt.Tensor.zeros([cols], ts[0].dtype, 0)
+            cells = []
+            for mk, algo in ((lambda: P.reduce(ts, "sum", [1]), nb), (lambda: P.reduce(ts, "sum", [0]), nb),
+                             (lambda: P.reduce(ts, "argmax", 1, arg=True), nb), (lambda: P.reduce(ts, "argmax", 0, arg=True), nb),
+                             (lambda: P.norm(ts, "softmax", axis=1), 2 * nb), (lambda: P.norm(ts, "softmax", axis=0), 2 * nb),
+                             (lambda: P.norm(ts, "layernorm", n_norm=1, gamma=g, beta=b), 2 * nb)):
+                run, outs = mk()
+                med = float(np.median(time_groups(ev, Case("", "", dname, rows, algo, run, 3), groups=5, per=8, warmup=4)))
+                cells.append(f"{algo / (med * 1e-6) / 1e12:.1f}")
+                del outs
+            print(f"| N = {rows}, C = {cols} | " + " | ".join(cells) + " |", flush=True)
+            P.keep.clear()
+            del ts
+
+
+def host_time(cases, calls=2000):
+    """Host time per call (the call returns when its launches are queued) of each case, in microseconds:
+    `calls` calls back to back without waiting for the device, then one wait."""
+    import hpt_amd as hpt
+    for c in cases:
+        for i in range(20):
+            c.run(i)
+        hpt.synchronize(0)
+        t0 = time.perf_counter()
+        for i in range(calls):
+            c.run(i)
+        t1 = time.perf_counter()
+        hpt.synchronize(0)
+        t2 = time.perf_counter()
+        print(f"  {c.cfg:<58} {c.name:<16} host {1e6 * (t1 - t0) / calls:7.2f} us/call   "
+              f"with the device's work {1e6 * (t2 - t0) / calls:7.2f} us/call", flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -493,6 +544,10 @@ def main():
                     help="after the timed region, run one plain device-to-device copy of the headline input "
                          "(134217728 bytes read + as many written): the known-size dispatch that hardware "
                          "counter runs (FETCH_SIZE / WRITE_SIZE) are scaled by")
+    ap.add_argument("--sweep", default="", help="comma list of f32,f16: instead of the benchmark, print the table of "
+                    "achieved TB/s over [N, C] shapes of 32 Mi elements (C = 3 ... 2^20) and exit")
+    ap.add_argument("--host-time", action="store_true",
+                    help="instead of the benchmark, print the host time per call of the ops selected by --configs and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU form (every op but a full "
@@ -505,9 +560,15 @@ def main():
         build.build()
     assert hpt.device_count() >= 1, "no HIP device visible"
     ev = HipEvents()
+    if args.sweep:
+        shape_sweep(ev, args.sweep.split(","))
+        return
 
     configs = set(args.configs.split(",")) if args.configs else None
     cases, prepared, (x, g, b, head_out) = build_cases(args.ops, configs)
+    if args.host_time:
+        host_time(cases)
+        return
     head = cases[0]
     wall, dev_ms = time_case(ev, head, args.steps, args.warmup)
     ms_per_step = wall * 1e3 / args.steps
