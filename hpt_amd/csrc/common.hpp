@@ -191,6 +191,7 @@ struct EwPlan {
     int sstride = 1;  // 2: (copy) the innermost input stride is 2: full vectors in, every second element kept
     // Transpose: dim `tdim` has input stride 1; the innermost dim is strided in the input
     int tdim = -1;
+    bool tile_lds = false;  // Transpose: both dims hold a whole (16 vec)^2 tile: staged through LDS
 };
 
 EwPlan plan_elementwise(const void* out_data, const int64_t* shape, int ndim, int nin, const void* const* in_data,

@@ -162,6 +162,7 @@ struct TransposeArgs {
     int nother;
     int osize[kMaxDims];
     int64_t oin[kMaxDims], oout[kMaxDims];  // strides of the other dims in input / output
+    int ntA;            // (LDS form) tiles along A
 };
 
 template <class U>
@@ -212,6 +213,73 @@ __global__ void __launch_bounds__(256) ew_transpose_kernel(const TransposeArgs a
             for (int i = 0; i < VEC; ++i) o.v[i] = v[s][i].v[k];
             store_pack_stream<U, VEC>(out + (int64_t)k * a.oB + s * TA, o);
         }
+}
+
+// The same copy for views with at least a whole tile in both dims, through LDS: a workgroup moves a
+// (16 VEC along B) x (16 VEC along A) tile. Loading, 16 lanes run along B (256 contiguous bytes of
+// the input per A position, four A positions per instruction); a lane transposes its VEC x VEC block
+// in registers and parks the VEC result vectors in LDS, one per B position; storing, 16 lanes run
+// along A (256 contiguous bytes of the output per B position, four B positions per instruction).
+// With the register transpose alone a lane's share of B and of A is fixed, 128 bytes each way, and
+// eight 128-byte pieces per instruction is the slowest of the store patterns.
+// LDS holds [16 VEC rows (B)][16 chunks of 16 bytes (A)]; chunk c of row b sits at c ^ (b / VEC): the
+// 16 lanes of a quarter wavefront then hit 16 different 16-byte bank groups both when they write
+// (same chunk, rows VEC apart) and when they read (same row, chunks 0..15).
+template <class U>
+__global__ void __launch_bounds__(256) ew_transpose_lds_kernel(const TransposeArgs a) {
+    constexpr int VEC = 16 / sizeof(U);
+    constexpr int TB = 16 * VEC, TA = 16 * VEC;
+    __shared__ __align__(16) unsigned char tile[TB * 256];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    int64_t ioff = 0, ooff = 0;
+    {
+        uint32_t q = blockIdx.z;
+        for (int i = a.nother - 1; i >= 0; --i) {
+            const uint32_t s = (uint32_t)a.osize[i];
+            const uint32_t q2 = q / s;
+            const uint32_t idx = q - q2 * s;
+            q = q2;
+            ioff += (int64_t)idx * a.oin[i];
+            ooff += (int64_t)idx * a.oout[i];
+        }
+    }
+    // Tiles are numbered along A first: workgroups that run at the same time then write neighbouring
+    // 256-byte pieces of the same output rows (f16 [4096, 8192].permute(1, 0): 26.7 us; numbered along B
+    // first, which gives the READS that locality instead, 28.7 us).
+    const int tb = blockIdx.x / a.ntA, ta = blockIdx.x - tb * a.ntA;
+    const int B0 = tb * TB, A0 = ta * TA;
+    {
+        const int jb = lane & 15, ac = w * 4 + (lane >> 4);
+        const int b = B0 + jb * VEC, a0 = A0 + ac * VEC;
+        if (b < a.nB && a0 < a.nA) {  // (both sizes are multiples of VEC: a chunk is inside or outside as a whole)
+            const U* in = (const U*)a.in + ioff + (int64_t)a0 * a.sA + b;
+            Pack<U, VEC> v[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) v[i] = load_pack_stream<U, VEC>(in + (int64_t)i * a.sA);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                Pack<U, VEC> o;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) o.v[i] = v[i].v[k];
+                *(Pack<U, VEC>*)(tile + (jb * VEC + k) * 256 + ((ac ^ jb) << 4)) = o;
+            }
+        }
+    }
+    __syncthreads();
+    {
+        const int ca = lane & 15, rl = w * 4 + (lane >> 4);
+        const int a0 = A0 + ca * VEC;
+        U* out = (U*)a.out + ooff + a0;
+#pragma unroll
+        for (int it = 0; it < VEC; ++it) {
+            const int row = it * 16 + rl;
+            const int b = B0 + row;
+            if (b < a.nB && a0 < a.nA) {
+                const Pack<U, VEC> o = *(const Pack<U, VEC>*)(tile + row * 256 + (((ca ^ (row / VEC)) & 15) << 4));
+                store_pack_stream<U, VEC>(out + (int64_t)b * a.oB, o);
+            }
+        }
+    }
 }
 
 // ---- dtype casts ----------------------------------------------------------------------
@@ -344,6 +412,15 @@ template <class U> void launch_transpose(const EwPlan& p, void* out, const void*
         t.oout[t.nother] = ostride[i];
         ++t.nother;
         others *= p.size[i];
+    }
+    if (p.tile_lds) {
+        constexpr int T = 16 * VEC;
+        t.ntA = (t.nA + T - 1) / T;
+        const int64_t tiles = (int64_t)t.ntA * ((t.nB + T - 1) / T);
+        if (tiles > 0x7fffffff) fail(HPT_ERR_SHAPE, "strided copy: too many tiles for the transposing kernel");
+        dim3 grid((unsigned)tiles, 1, (unsigned)others);
+        ew_transpose_lds_kernel<U><<<grid, dim3(256), 0, st>>>(t);
+        return;
     }
     constexpr int TILE = 8 * VEC;
     dim3 grid((unsigned)((t.nB + 4 * TILE - 1) / (4 * TILE)), (unsigned)((t.nA + 2 * TILE - 1) / (2 * TILE)), (unsigned)others);

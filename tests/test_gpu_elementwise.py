@@ -35,6 +35,10 @@ COPY_CASES = [
     ("2-D transpose, ragged tiles", [200, 136], (("permute", (1, 0)),), "transpose"),
     ("3-D rotate", [24, 40, 72], (("permute", (2, 0, 1)),), "transpose"),
     ("batched transpose", [3, 80, 48], (("permute", (0, 2, 1)),), "transpose"),
+    # whole (16 vectors)^2 tiles in both dims for every element size, with ragged last tiles: staged through LDS
+    ("2-D transpose through LDS, ragged tiles", [400, 304], (("permute", (1, 0)),), "transpose"),
+    ("batched transpose through LDS", [3, 272, 400], (("permute", (0, 2, 1)),), "transpose"),
+    ("3-D rotate through LDS", [272, 5, 288], (("permute", (2, 1, 0)),), "transpose"),
     ("4-D middle swap keeps inner rows", [4, 6, 10, 64], (("permute", (0, 2, 1, 3)),), "inner"),
     ("row slice", [50, 128], (("slice", ((3, 41, 1), (0, 128, 1))),), "inner"),
     ("column slice (unaligned rows)", [50, 128], (("slice", ((0, 50, 1), (5, 77, 1))),), "inner"),
@@ -77,12 +81,12 @@ def test_contiguous_bf16_random_layouts_and_empty(hpt, dev):
 
 
 def test_contiguous_large_transpose_and_errors(hpt, dev):
-    """f16 [4096, 2048] transposed: 16 MiB through the register-tile kernel; f64 [1024, 1536]."""
+    """f16 [4096, 2048] transposed: 16 MiB through the LDS-staged tile kernel; f64 [1024, 1536]; i8."""
     rng = np.random.default_rng(302)
     for npdt, shape in ((np.float16, [4096, 2048]), (np.float64, [1024, 1536]), (np.int8, [2048, 4096])):
         base = rand(rng, shape, npdt)
         t = hpt.Tensor.from_numpy(base).to_hip(dev).permute([1, 0])
-        assert hpt.contiguous_plan(t).startswith("transpose")
+        assert hpt.contiguous_plan(t).startswith("transpose") and hpt.contiguous_plan(t).endswith("lds")
         same_bits(t.contiguous().numpy(), ew.contiguous(base.T), f"large transpose {np.dtype(npdt).name}")
     from hpt_amd import _ffi
     import ctypes as C
