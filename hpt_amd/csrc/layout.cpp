@@ -597,7 +597,8 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 for (int i = 0; i < p.kept_in.n; ++i)
                     if (((p.kept_in.stride[i] - p.kept_out.stride[i]) * (int64_t)elem_size) % 16 != 0) same = false;
                 const int64_t nvs = (p.cols + 2 * (max_vec - 1)) / max_vec;
-                // (two-byte layernorm keeps two vectors per thread: beyond 512 threads per row it only loses)
+                // (two-byte layernorm keeps two vectors per thread, so its rows stay in registers up to 1024
+                // vectors, 512 threads; f16 [8190, 4097] 1.9 -> 2.2 TB/s, [5461, 6145] 1.9 -> 2.8 against streaming)
                 if (same && n_norm_dims <= 0 && elem_size == 2 && nvs > 4096 && nvs <= 8192) {
                     // two-byte softmax rows of 32769 ... 65521 elements (a vocabulary of 50257): the raw row
                     // in registers (see below), f16 [4096, 50257] log_softmax 3.1 -> 4.0 TB/s. The
@@ -635,7 +636,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     p.nchunk = 16;
                     return p;
                 }
-                if (same && nvs > ((n_norm_dims > 0 && elem_size == 2) ? 512 : 2048)) {
+                if (same && nvs > ((n_norm_dims > 0 && elem_size == 2) ? 1024 : 2048)) {
                     p.kind = NormKind::RowStream;
                     p.vec = max_vec;
                     p.shift = 1;

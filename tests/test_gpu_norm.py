@@ -362,6 +362,10 @@ WIDE_ROW_CASES = [
     ("f16 rows of 65537: registers and LDS, shifted", np.float16, [130, 65537]),
     ("bf16 rows of 131001: the longest shifted two-byte row on chip", "bf16", [133, 131001]),
     ("f16 rows of 131003: streamed", np.float16, [131, 131003]),
+    # two-byte layernorm rows of 513 ... 1024 shifted vectors: 512 threads, two vectors each, rows walked
+    ("f16 rows of 4097: layernorm from registers, 512 threads", np.float16, [2100, 4097]),
+    ("bf16 rows of 8185: the longest such row", "bf16", [1500, 8185]),
+    ("f16 rows of 6148 (rows start on 8-byte boundaries)", np.float16, [1300, 6148]),
 ]
 
 
