@@ -748,6 +748,43 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 if (n_norm_dims <= 0 && v > 1 && elem_size >= 4 && p.tpr >= 512 && nv <= (p.tpr / 2) * 5) p.tpr /= 2;
                 int64_t nc = (nv + p.tpr - 1) / p.tpr;
                 p.nchunk = std::max(1, pow2_ceil(nc));
+                // Threads per row and vectors per thread are powers of two so far, which leaves a quarter
+                // to a third of the lanes idle on rows of 3, 5, 6 or 7 times a power of two - the hidden
+                // sizes 768, 1536, 2560, 3072, 5120, 6144, 12288. Aligned rows of whole vectors may take 3
+                // (any type) or 5, 6, 7 (4- and 8-byte softmax; layernorm up to 6) vectors per thread: the
+                // fewest slots win; among equals, rows of up to 256 threads (layernorm: 512) with the fewest
+                // vectors per thread, else the fewest threads. Measured, TB/s: f32 softmax [21845, 1536]
+                // 256 x 2 4.7 -> 128 x 3 6.0, [5461, 6144] 512 x 4 4.8 -> 256 x 6 5.8, [2730, 12288] 4.3 -> 5.2;
+                // f32 layernorm [13107, 2560] 256 x 4 4.5 -> 128 x 5 5.5, [6553, 5120] 4.7 -> 5.6 (256 x 5),
+                // [10922, 3072] 4.9 -> 5.7 (256 x 3); f16 softmax [21845, 3072] 256 x 2 4.5 -> 128 x 3 5.9,
+                // [13107, 5120] 4.7 -> 5.8 (256 x 3); f16 layernorm [87381, 768] 4.1 -> 5.0 (32 x 3), [43690, 1536]
+                // 3.9 -> 4.9 (64 x 3). (Two-byte rows of five vectors or more per thread lose: layernorm spills.)
+                // (gamma / beta in LDS: three or four vectors per thread, 256 threads or more)
+                if (v == max_vec && v > 1 && p.sstride == 1 && !p.shift && !p.tile_rows) {
+                    const int maxc = elem_size == 2 ? (ln_half ? 3 : 4) : (n_norm_dims > 0 ? 6 : 8);
+                    const int pref_tpr = n_norm_dims > 0 ? 512 : 256;
+                    int64_t best = (int64_t)p.tpr * p.nchunk;
+                    int bt = 0, bc = 0;
+                    for (int t = p.gb_lds ? 256 : 16; t <= 1024; t <<= 1) {
+                        const int64_t c = std::max<int64_t>((nv + t - 1) / t, p.gb_lds ? 3 : 1);
+                        if (c > maxc) continue;
+                        const int64_t slots = t * c;
+                        bool take = slots < best;
+                        if (!take && bt && slots == best) {
+                            // equal: inside the preferred width the wider row (fewer vectors per thread) wins
+                            take = t <= pref_tpr;
+                        }
+                        if (take) {
+                            best = slots;
+                            bt = t;
+                            bc = (int)c;
+                        }
+                    }
+                    if (bt) {
+                        p.tpr = bt;
+                        p.nchunk = bc;
+                    }
+                }
                 int block = std::max(256, p.tpr);
                 p.rpb = block / p.tpr;
                 // Layernorm workgroups walk the rows; how many of them is best depends on how many a compute unit

@@ -22,6 +22,17 @@ inline int ilog2(int v) {
 
 template <class T, int VEC, int SS = 1, bool SHIFT = false, bool PF = false>
 void launch_row_reg(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block, hipStream_t st) {
+    // (3, 5, 6 and 7 vectors per thread: rows of whole vectors whose length is 3, 5, 6 or 7 times a power of
+    // two - 768, 1536, 2560, 3072, 3584, 5120, 6144 ... - without idle lanes; aligned full-vector rows only)
+    if constexpr (VEC > 1 && SS == 1 && !SHIFT) {
+        switch (p.nchunk) {
+            case 3: row_reg_kernel<KIND, T, VEC, 3, SS, SHIFT, PF><<<grid, block, 0, st>>>(a); return;
+            case 5: row_reg_kernel<KIND, T, VEC, 5, SS, SHIFT, PF><<<grid, block, 0, st>>>(a); return;
+            case 6: row_reg_kernel<KIND, T, VEC, 6, SS, SHIFT, PF><<<grid, block, 0, st>>>(a); return;
+            case 7: row_reg_kernel<KIND, T, VEC, 7, SS, SHIFT, PF><<<grid, block, 0, st>>>(a); return;
+            default: break;
+        }
+    }
     switch (p.nchunk) {
         case 1: row_reg_kernel<KIND, T, VEC, 1, SS, SHIFT, PF><<<grid, block, 0, st>>>(a); break;
         case 2: row_reg_kernel<KIND, T, VEC, 2, SS, SHIFT, PF><<<grid, block, 0, st>>>(a); break;
@@ -320,13 +331,15 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
             }
         }
         if constexpr (FULL > 1 && sizeof(T) == 2 && norm_is_layer(KIND)) {
-            if (p.gb_lds && p.vec == FULL && p.sstride == 1 && !p.shift && p.nchunk == 4) {
+            if (p.gb_lds && p.vec == FULL && p.sstride == 1 && !p.shift && (p.nchunk == 4 || p.nchunk == 3)) {
                 const size_t smem = 2 * (size_t)p.cols * sizeof(T);
                 if (p.tpr >= 512 && KIND != NORM_ADD_LAYERNORM) {
                     if (grid.x > 512u) grid.x = 512u;
-                    row_reg_kernel<KIND, T, FULL, 4, 1, false, true, true><<<grid, block, smem, st>>>(a);
+                    if (p.nchunk == 3) row_reg_kernel<KIND, T, FULL, 3, 1, false, true, true><<<grid, block, smem, st>>>(a);
+                    else row_reg_kernel<KIND, T, FULL, 4, 1, false, true, true><<<grid, block, smem, st>>>(a);
                 } else {
-                    row_reg_kernel<KIND, T, FULL, 4, 1, false, false, true><<<grid, block, smem, st>>>(a);
+                    if (p.nchunk == 3) row_reg_kernel<KIND, T, FULL, 3, 1, false, false, true><<<grid, block, smem, st>>>(a);
+                    else row_reg_kernel<KIND, T, FULL, 4, 1, false, false, true><<<grid, block, smem, st>>>(a);
                 }
                 return;
             }

@@ -34,6 +34,9 @@ CAUSAL_CASES = [
     ("negative offset: first rows have no key", [24, 24], (), 0.5, -3),
     ("long rows (streaming kernel would not be used, registers)", [5, 4096], (), 1.0, 0),
     ("rows beyond registers: 40000 keys", [3, 40000], (), 0.5, 39990),
+    ("1536 keys: three vectors per thread", [2, 300, 1536], (), 0.5, 1236),
+    ("2560 keys: five vectors per thread", [1, 200, 2560], (), 1.0, 2360),
+    ("6144 keys: six vectors per thread", [1, 96, 6144], (), 1.0, 6048),
     ("sliced view", [4, 33, 70], (("slice", ((0, 4, 1), (1, 33, 1), (3, 67, 1))),), 2.0, 5),
     ("step-2 keys", [2, 32, 128], (("slice", ((0, 2, 1), (0, 32, 1), (0, 128, 2))),), 1.0, 0),
     ("permuted: keys not contiguous", [48, 2, 40], (("permute", (1, 2, 0)),), 0.5, 4),

@@ -362,6 +362,20 @@ WIDE_ROW_CASES = [
     ("f16 rows of 65537: registers and LDS, shifted", np.float16, [130, 65537]),
     ("bf16 rows of 131001: the longest shifted two-byte row on chip", "bf16", [133, 131001]),
     ("f16 rows of 131003: streamed", np.float16, [131, 131003]),
+    # rows of 3, 5, 6 or 7 times a power of two: that many vectors per thread, no idle lanes
+    ("f32 rows of 768: 64 threads x 3 vectors", np.float32, [5003, 768]),
+    ("f32 rows of 1280: 64 x 5", np.float32, [4100, 1280]),
+    ("f32 rows of 1536: 128 x 3", np.float32, [2300, 1536]),
+    ("f32 rows of 2560: 128 x 5", np.float32, [2100, 2560]),
+    ("f32 rows of 3584: softmax 128 x 7", np.float32, [2051, 3584]),
+    ("f32 rows of 6144: softmax 256 x 6, layernorm 512 x 3 with prefetch", np.float32, [1100, 6144]),
+    ("f32 rows of 12288: 512 x 6 with prefetch", np.float32, [700, 12288]),
+    ("f64 rows of 1536: 256 x 3", np.float64, [1500, 1536]),
+    ("f16 rows of 768: 32 x 3", np.float16, [9001, 768]),
+    ("f16 rows of 3072: 128 x 3", np.float16, [2101, 3072]),
+    ("bf16 rows of 2560: 128 x 3, the last vectors of each thread empty", "bf16", [2300, 2560]),
+    ("f16 rows of 5120: softmax 256 x 3", np.float16, [1300, 5120]),
+    ("bf16 rows of 12288: softmax 512 x 3", "bf16", [600, 12288]),
     # two-byte layernorm rows of 513 ... 1024 shifted vectors: 512 threads, two vectors each, rows walked
     ("f16 rows of 4097: layernorm from registers, 512 threads", np.float16, [2100, 4097]),
     ("bf16 rows of 8185: the longest such row", "bf16", [1500, 8185]),
