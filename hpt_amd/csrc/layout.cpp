@@ -214,7 +214,7 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
                 p.tpr = 256;
                 p.rpb = 1;
             }
-            int64_t want = (512 + p.K - 1) / p.K;
+            int64_t want = std::max<int64_t>(1, 512 / p.K);  // (never just over two rounds of the compute units)
             int64_t can = nv / (256 * (p.K >= 64 ? 8 : 16));
             int64_t split = std::min<int64_t>(std::min(want, can), 4096);
             if (split > 1) {
@@ -584,7 +584,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             const int64_t R = p.kept_in.size[nk - 1];
             const int64_t batch = nk > 1 ? p.kept_in.size[0] : 1;
             const int64_t groups = (R + 64 * v - 1) / (64 * v) * batch;
-            int64_t S = std::max<int64_t>(1, std::min<int64_t>((512 + groups - 1) / groups, p.cols / 128));
+            int64_t S = std::max<int64_t>(1, std::min<int64_t>(512 / groups, p.cols / 128));
             p.tsplit = (int)std::min<int64_t>(S, 64);
             p.tpr = 4;  // wavefronts per workgroup of the statistics pass
             p.scratch_bytes = (size_t)p.rows * p.tsplit * 16 + (size_t)p.rows * 3 * 8;
@@ -785,8 +785,12 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 // [13107, 5120] 4.7 -> 5.8 (256 x 3); f16 layernorm [87381, 768] 4.1 -> 5.0 (32 x 3), [43690, 1536]
                 // 3.9 -> 4.9 (64 x 3). (Two-byte rows of five vectors or more per thread lose: layernorm spills.)
                 // (gamma / beta in LDS: three or four vectors per thread, 256 threads or more)
-                if (v == max_vec && v > 1 && p.sstride == 1 && !p.shift && !p.tile_rows) {
-                    const int maxc = elem_size == 2 ? (ln_half ? 3 : 4) : (n_norm_dims > 0 ? 6 : 8);
+                // (Rows of odd length, covered by aligned vectors: softmax alike - f16 [116306, 577] 3.6 -> 4.1,
+                // [44739, 1500] 4.2 -> 4.9, f32 [8190, 4097] 4.4 -> 5.3, [16000, 2051] 4.3 -> 5.5; layernorm, which
+                // carries the masks and the unaligned gamma / beta besides, only up to what it had: more spills.)
+                if (v == max_vec && v > 1 && p.sstride == 1 && !p.tile_rows) {
+                    const int maxc = n_norm_dims > 0 && p.shift ? (elem_size == 2 ? 2 : 4)
+                                                                : elem_size == 2 ? (ln_half ? 3 : 4) : (n_norm_dims > 0 ? 6 : 8);
                     const int pref_tpr = n_norm_dims > 0 ? 512 : 256;
                     int64_t best = (int64_t)p.tpr * p.nchunk;
                     int bt = 0, bc = 0;
@@ -955,7 +959,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 }
             }
             const int64_t groups = (L + 64 * v - 1) / (64 * v) * batch;
-            int64_t S = std::max<int64_t>(1, std::min<int64_t>((512 + groups - 1) / groups, p.cols / 32));
+            int64_t S = std::max<int64_t>(1, std::min<int64_t>(512 / groups, p.cols / 32));
             p.tsplit = (int)std::min<int64_t>(S, 64);
             p.tpr = 4;  // wavefronts per workgroup of the statistics pass
             p.scratch_bytes = (size_t)p.rows * p.tsplit * 16 + (size_t)p.rows * 3 * 8;

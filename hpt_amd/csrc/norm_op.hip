@@ -23,8 +23,8 @@ inline int ilog2(int v) {
 template <class T, int VEC, int SS = 1, bool SHIFT = false, bool PF = false>
 void launch_row_reg(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block, hipStream_t st) {
     // (3, 5, 6 and 7 vectors per thread: rows of whole vectors whose length is 3, 5, 6 or 7 times a power of
-    // two - 768, 1536, 2560, 3072, 3584, 5120, 6144 ... - without idle lanes; aligned full-vector rows only)
-    if constexpr (VEC > 1 && SS == 1 && !SHIFT) {
+    // two - 768, 1536, 2560, 3072, 3584, 5120, 6144 ... - without idle lanes; full-vector rows only)
+    if constexpr (VEC > 1 && SS == 1) {
         switch (p.nchunk) {
             case 3: row_reg_kernel<KIND, T, VEC, 3, SS, SHIFT, PF><<<grid, block, 0, st>>>(a); return;
             case 5: row_reg_kernel<KIND, T, VEC, 5, SS, SHIFT, PF><<<grid, block, 0, st>>>(a); return;

@@ -376,6 +376,11 @@ WIDE_ROW_CASES = [
     ("bf16 rows of 2560: 128 x 3, the last vectors of each thread empty", "bf16", [2300, 2560]),
     ("f16 rows of 5120: softmax 256 x 3", np.float16, [1300, 5120]),
     ("bf16 rows of 12288: softmax 512 x 3", "bf16", [600, 12288]),
+    # odd lengths with 3 or 5 vectors per thread (softmax; layernorm keeps powers of two there)
+    ("f16 rows of 577: shifted, 32 x 3", np.float16, [9000, 577]),
+    ("bf16 rows of 1500 (8-byte row starts): shifted, 64 x 3", "bf16", [4400, 1500]),
+    ("f32 rows of 2051: shifted, 128 x 5", np.float32, [2300, 2051]),
+    ("f32 rows of 3001: shifted, 256 x 3", np.float32, [2100, 3001]),
     # two-byte layernorm rows of 513 ... 1024 shifted vectors: 512 threads, two vectors each, rows walked
     ("f16 rows of 4097: layernorm from registers, 512 threads", np.float16, [2100, 4097]),
     ("bf16 rows of 8185: the longest such row", "bf16", [1500, 8185]),
