@@ -706,10 +706,11 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             // Two-byte types hold eight elements per vector: with gamma and beta beside the row, sixteen
             // elements per thread is what fits 128 registers, i.e. two vectors (four of a stride-2 row).
             bool ln_half = n_norm_dims > 0 && v > 1 && elem_size == 2;
-            // Long two-byte layernorm rows (4096 < cols <= 16384): gamma / beta go to LDS (at most 64 KiB)
-            // and the row takes four vectors per thread like any other. Measured, f16 (TB/s): [6553, 5120]
-            // 3.5 -> 4.6, [4096, 8192] 4.7 -> 5.0, [2730, 12288] 3.2 -> 4.6, [2048, 16384] 3.8 -> 4.6.
-            if (ln_half && p.sstride == 1 && !p.shift && nv * v > 4096 && nv * v <= 16384) {
+            // Two-byte layernorm rows of 1024 ... 16384 elements: gamma / beta go to LDS (at most 64 KiB)
+            // and the row takes three or four vectors per thread like any other. Measured, f16 (TB/s): [6553, 5120]
+            // 3.5 -> 4.6, [4096, 8192] 4.7 -> 5.0, [2730, 12288] 3.2 -> 4.6, [2048, 16384] 3.8 -> 4.6; [65536, 1024]
+            // 5.0 -> 5.4, [32768, 2048] 4.6 -> 5.3.
+            if (ln_half && p.sstride == 1 && !p.shift && nv * v >= 1024 && nv * v <= 16384) {
                 p.gb_lds = 1;
                 ln_half = false;
             }
@@ -792,9 +793,10 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     const int maxc = n_norm_dims > 0 && p.shift ? (elem_size == 2 ? 2 : 4)
                                                                 : elem_size == 2 ? (ln_half ? 3 : 4) : (n_norm_dims > 0 ? 6 : 8);
                     const int pref_tpr = n_norm_dims > 0 ? 512 : 256;
-                    int64_t best = (int64_t)p.tpr * p.nchunk;
+                    // (gamma / beta in LDS: the form exists for three and four vectors per thread only)
+                    int64_t best = p.gb_lds ? INT64_MAX : (int64_t)p.tpr * p.nchunk;
                     int bt = 0, bc = 0;
-                    for (int t = p.gb_lds ? 256 : 16; t <= 1024; t <<= 1) {
+                    for (int t = p.gb_lds ? 32 : 16; t <= 1024; t <<= 1) {
                         const int64_t c = std::max<int64_t>((nv + t - 1) / t, p.gb_lds ? 3 : 1);
                         if (c > maxc) continue;
                         const int64_t slots = t * c;
