@@ -18,7 +18,7 @@ own duration come from profiles/headline.json (written when the rocprofv3 summar
 profiles/ are regenerated), and the plan the library reports for the headline call is printed
 beside the plan recorded there, so a planner change that makes the profile stale shows.
 
-`ops` lists every op of the five benchmark configurations (and the groups c6-c8), each timed
+`ops` lists every op of the five benchmark configurations (and the groups c6-c9), each timed
 the same way whatever --steps says: 10 warm-up launches, then 13 groups of 8 back-to-back
 launches, every group bracketed by a pair of HIP events; `us_per_launch` is the median over the
 groups of (group time / 8) - 104 timed launches. (Bracketing every single launch instead adds
@@ -439,6 +439,34 @@ def cases_c8(P):
     return cases
 
 
+def cases_c9(P):
+    """Transformer hidden sizes that are 3 or 5 times a power of two (768, 1536, 2560, 3072, 5120), ~128 MiB
+    each: layernorm and softmax over the hidden dim, sum over the tokens."""
+    import hpt_amd as hpt
+    rng = np.random.default_rng(9)
+    cases = []
+    for dname, npdt, rows, cols in (("f16", np.float16, 21845, 3072), ("f16", np.float16, 13107, 5120),
+                                    ("f32", np.float32, 21845, 1536), ("f32", np.float32, 13107, 2560),
+                                    ("f32", np.float32, 43690, 768)):
+        base = rng.standard_normal((rows, cols), dtype=np.float32).astype(npdt)
+        ts = [hpt.Tensor.from_numpy(np.roll(base, k, 0)).to_hip(0) for k in range(4)]
+        nb = base.nbytes
+        g, b = hpt.Tensor.ones([cols], ts[0].dtype, 0), hpt.Tensor.zeros([cols], ts[0].dtype, 0)
+        cfg = f"{dname} [{rows},{cols}] (hidden size {cols})"
+        run, outs = P.norm(ts, "layernorm", n_norm=1, gamma=g, beta=b)
+        P.keep.append(outs)
+        cases.append(Case("layernorm", cfg, dname, rows, 2 * nb + 2 * cols * base.itemsize, run, 4, plan=P.last_plan))
+        run, outs = P.norm(ts, "softmax", axis=1)
+        P.keep.append(outs)
+        cases.append(Case("softmax(axis=1)", cfg, dname, rows, 2 * nb, run, 4, plan=P.last_plan))
+        if cols in (768, 5120):
+            run, outs = P.reduce(ts, "sum", [0])
+            P.keep.append(outs)
+            cases.append(Case("sum(axis=0)", cfg, dname, cols, nb + cols * base.itemsize, run, 4, plan=P.last_plan))
+        del ts
+    return cases
+
+
 def build_cases(which: str, configs=None):
     """Synthetic inputs of the benchmark configurations, uploaded once; outputs preallocated.
     The headline (C2 layernorm) is always first; `configs` limits the others (e.g. {"c3"})."""
@@ -446,7 +474,7 @@ def build_cases(which: str, configs=None):
     cases, head = cases_c2(P, which == "headline")
     if which != "headline":
         for name, fn in (("c1", cases_c1), ("c3", cases_c3), ("c4", cases_c4), ("c5", cases_c5), ("c6", cases_c6),
-                         ("c7", cases_c7), ("c8", cases_c8)):
+                         ("c7", cases_c7), ("c8", cases_c8), ("c9", cases_c9)):
             if configs is None or name in configs:
                 cases += fn(P)
     return cases, P, head
@@ -539,7 +567,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--ops", choices=["all", "headline"], default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--configs", default="", help="comma list of c1,c3,c4,c5,c6,c7,c8 to measure besides the headline (c6 = the steps either side: contiguous / in-place affine / full; c7 = the fused forms; c8 = shapes off the reference's list)")
+    ap.add_argument("--configs", default="", help="comma list of c1,c3,c4,c5,c6,c7,c8,c9 to measure besides the headline (c6 = the steps either side: contiguous / in-place affine / full; c7 = the fused forms; c8 = shapes off the reference's list; c9 = hidden sizes of 3 or 5 times a power of two)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region, run one plain device-to-device copy of the headline input "
                          "(134217728 bytes read + as many written): the known-size dispatch that hardware "
