@@ -156,9 +156,10 @@ struct NormPlan {
 };
 
 // axis >= 0: softmax-style single axis; n_norm_dims > 0: trailing dims (layernorm).
+// with_residual: the plan is for layernorm(x + residual), whose rows are held twice.
 NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t* shape,
                         const int64_t* strides, int ndim, int64_t axis, int n_norm_dims,
-                        size_t elem_size);
+                        size_t elem_size, bool with_residual = false);
 
 std::string describe(const NormPlan& p);
 

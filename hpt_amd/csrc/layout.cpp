@@ -479,7 +479,7 @@ std::string describe(const ReducePlan& p) {
 
 NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t* shape,
                         const int64_t* strides, int ndim, int64_t axis, int n_norm_dims,
-                        size_t elem_size) {
+                        size_t elem_size, bool with_residual) {
     NormPlan p;
     int64_t total = 1;
     for (int i = 0; i < ndim; ++i) total *= shape[i];
@@ -800,7 +800,10 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 // carries the masks and the unaligned gamma / beta besides, only up to what it had: more spills.)
                 if (v == max_vec && v > 1 && p.sstride == 1 && !p.tile_rows) {
                     const int maxc = n_norm_dims > 0 && p.shift ? (elem_size == 2 ? 2 : 4)
-                                                                : elem_size == 2 ? (ln_half ? 3 : 4) : (n_norm_dims > 0 ? 6 : 8);
+                                                                : elem_size == 2 ? (ln_half ? 3 : 4)
+                                                                : (n_norm_dims > 0 ? (with_residual ? 4 : 6) : 8);
+                    // (layernorm(x + residual) holds the residual's vectors beside the row's: with five or six
+                    // per thread it spills - f32 [2730, 12288] 3.1 TB/s)
                     const int pref_tpr = n_norm_dims > 0 ? 512 : 256;
                     // (gamma / beta in LDS: the form exists for three and four vectors per thread only)
                     int64_t best = p.gb_lds ? INT64_MAX : (int64_t)p.tpr * p.nchunk;
