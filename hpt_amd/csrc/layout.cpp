@@ -837,7 +837,9 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 // 45.1 / 46.2 / 47.1, [65536, 512] 45.0 / 46.4 / 47.4; [16384, 2048] 52.9 / 47.5 / 46.3, [8192, 2048]
                 // 29.1 / 26.2 / 25.2, [8192, 1536] 26.9 / 23.1 / 20.3. Two-byte rows prefetch their next row and stay at 1024.
                 if (n_norm_dims > 0 && elem_size == 4 && v > 1 && p.tpr <= 256) {
-                    if (p.nchunk >= 4) p.max_blocks = 768;
+                    // (Few rows: with 1024 every workgroup of [1024, 4096] has one row instead of one or two -
+                    // 9.7 -> 8.3 us; [1536, 4096] 13.1 -> 11.6, [3072, 4096] 20.9 -> 20.5, from 4096 rows on no difference.)
+                    if (p.nchunk >= 4) p.max_blocks = (p.rows + p.rpb - 1) / p.rpb > 3072 ? 768 : 1024;
                     else if (p.nchunk == 2) p.max_blocks = 1536;
                 }
             } else {

@@ -135,21 +135,6 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     extern __shared__ __align__(16) unsigned char gb_raw[];
     T* lds_gamma = reinterpret_cast<T*>(gb_raw);
     T* lds_beta = lds_gamma + (GBL ? (size_t)nv * UV : 0);
-    if constexpr (GBL) {
-        for (int i = threadIdx.x; i < nv; i += blockDim.x) {
-            Pack<T, UV> g, b;
-#pragma unroll
-            for (int j = 0; j < UV; ++j) {
-                g.v[j] = Elem<T>::narrow((CT)1);
-                b.v[j] = Elem<T>::narrow((CT)0);
-            }
-            if (a.gamma) g = load_pack<T, UV>((const T*)a.gamma + (int64_t)i * UV);
-            if (a.beta) b = load_pack<T, UV>((const T*)a.beta + (int64_t)i * UV);
-            store_pack<T, UV>(lds_gamma + (size_t)i * UV, g);
-            store_pack<T, UV>(lds_beta + (size_t)i * UV, b);
-        }
-        __syncthreads();
-    }
     Pack<T, UV> gam[GBL ? 1 : NCHUNK], bet[GBL ? 1 : NCHUNK];
     if constexpr (!kSoft && !GBL) {
 #pragma unroll
@@ -236,6 +221,22 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
         }
     };
     if constexpr (kPrefetch) issue_loads((int64_t)blockIdx.x * a.rpb);
+    // (gamma / beta are staged while the first row's loads are in flight)
+    if constexpr (GBL) {
+        for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+            Pack<T, UV> g, b;
+#pragma unroll
+            for (int j = 0; j < UV; ++j) {
+                g.v[j] = Elem<T>::narrow((CT)1);
+                b.v[j] = Elem<T>::narrow((CT)0);
+            }
+            if (a.gamma) g = load_pack<T, UV>((const T*)a.gamma + (int64_t)i * UV);
+            if (a.beta) b = load_pack<T, UV>((const T*)a.beta + (int64_t)i * UV);
+            store_pack<T, UV>(lds_gamma + (size_t)i * UV, g);
+            store_pack<T, UV>(lds_beta + (size_t)i * UV, b);
+        }
+        __syncthreads();
+    }
     for (int64_t row0 = (int64_t)blockIdx.x * a.rpb; row0 < a.rows; row0 += row_step) {
         if constexpr (!kPrefetch) issue_loads(row0);
         const int64_t row = row0 + ty;
