@@ -715,11 +715,12 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             // Two-byte types hold eight elements per vector: with gamma and beta beside the row, sixteen
             // elements per thread is what fits 128 registers, i.e. two vectors (four of a stride-2 row).
             bool ln_half = n_norm_dims > 0 && v > 1 && elem_size == 2;
-            // Two-byte layernorm rows of 1024 ... 16384 elements: gamma / beta go to LDS (at most 64 KiB)
+            // Two-byte layernorm rows of 640 ... 16384 elements: gamma / beta go to LDS (at most 64 KiB)
             // and the row takes three or four vectors per thread like any other. Measured, f16 (TB/s): [6553, 5120]
             // 3.5 -> 4.6, [4096, 8192] 4.7 -> 5.0, [2730, 12288] 3.2 -> 4.6, [2048, 16384] 3.8 -> 4.6; [65536, 1024]
-            // 5.0 -> 5.4, [32768, 2048] 4.6 -> 5.3.
-            if (ln_half && p.sstride == 1 && !p.shift && nv * v >= 1024 && nv * v <= 16384) {
+            // 5.0 -> 5.4, [32768, 2048] 4.6 -> 5.3, [74898, 896] 4.5 -> 5.2, [104857, 640] 4.5 -> 4.9 (shorter rows lose:
+            // [131072, 512] 4.9 -> 4.5).
+            if (ln_half && p.sstride == 1 && !p.shift && nv * v >= 640 && nv * v <= 16384) {
                 p.gb_lds = 1;
                 ln_half = false;
             }
