@@ -795,18 +795,19 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 // [10922, 3072] 4.9 -> 5.7 (256 x 3); f16 softmax [21845, 3072] 256 x 2 4.5 -> 128 x 3 5.9,
                 // [13107, 5120] 4.7 -> 5.8 (256 x 3); f16 layernorm [87381, 768] 4.1 -> 5.0 (32 x 3), [43690, 1536]
                 // 3.9 -> 4.9 (64 x 3). (Two-byte rows of five vectors or more per thread lose: layernorm spills.)
-                // (gamma / beta in LDS: three or four vectors per thread, 256 threads or more)
+                // (gamma / beta in LDS: three, four or five vectors per thread - f16 [58254, 1152] 4.4 -> 4.8,
+                // [26214, 2560] 4.6 -> 5.0 with five)
                 // (Rows of odd length, covered by aligned vectors: softmax alike - f16 [116306, 577] 3.6 -> 4.1,
                 // [44739, 1500] 4.2 -> 4.9, f32 [8190, 4097] 4.4 -> 5.3, [16000, 2051] 4.3 -> 5.5; layernorm, which
                 // carries the masks and the unaligned gamma / beta besides, only up to what it had: more spills.)
                 if (v == max_vec && v > 1 && p.sstride == 1 && !p.tile_rows) {
                     const int maxc = n_norm_dims > 0 && p.shift ? (elem_size == 2 ? 2 : 4)
-                                                                : elem_size == 2 ? (ln_half ? 3 : 4)
+                                                                : elem_size == 2 ? (ln_half ? 3 : (p.gb_lds ? 5 : 4))
                                                                 : (n_norm_dims > 0 ? (with_residual ? 4 : 6) : 8);
                     // (layernorm(x + residual) holds the residual's vectors beside the row's: with five or six
                     // per thread it spills - f32 [2730, 12288] 3.1 TB/s)
                     const int pref_tpr = n_norm_dims > 0 ? 512 : 256;
-                    // (gamma / beta in LDS: the form exists for three and four vectors per thread only)
+                    // (gamma / beta in LDS: the form exists for three to five vectors per thread only)
                     int64_t best = p.gb_lds ? INT64_MAX : (int64_t)p.tpr * p.nchunk;
                     int bt = 0, bc = 0;
                     for (int t = p.gb_lds ? 32 : 16; t <= 1024; t <<= 1) {

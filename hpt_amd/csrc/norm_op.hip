@@ -331,14 +331,16 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
             }
         }
         if constexpr (FULL > 1 && sizeof(T) == 2 && norm_is_layer(KIND)) {
-            if (p.gb_lds && p.vec == FULL && p.sstride == 1 && !p.shift && (p.nchunk == 4 || p.nchunk == 3)) {
+            if (p.gb_lds && p.vec == FULL && p.sstride == 1 && !p.shift && p.nchunk >= 3 && p.nchunk <= 5) {
                 const size_t smem = 2 * (size_t)p.cols * sizeof(T);
                 if (p.tpr >= 512 && KIND != NORM_ADD_LAYERNORM) {
                     if (grid.x > 512u) grid.x = 512u;
                     if (p.nchunk == 3) row_reg_kernel<KIND, T, FULL, 3, 1, false, true, true><<<grid, block, smem, st>>>(a);
+                    else if (p.nchunk == 5) row_reg_kernel<KIND, T, FULL, 5, 1, false, true, true><<<grid, block, smem, st>>>(a);
                     else row_reg_kernel<KIND, T, FULL, 4, 1, false, true, true><<<grid, block, smem, st>>>(a);
                 } else {
                     if (p.nchunk == 3) row_reg_kernel<KIND, T, FULL, 3, 1, false, false, true><<<grid, block, smem, st>>>(a);
+                    else if (p.nchunk == 5) row_reg_kernel<KIND, T, FULL, 5, 1, false, false, true><<<grid, block, smem, st>>>(a);
                     else row_reg_kernel<KIND, T, FULL, 4, 1, false, false, true><<<grid, block, smem, st>>>(a);
                 }
                 return;

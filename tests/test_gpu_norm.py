@@ -374,7 +374,9 @@ WIDE_ROW_CASES = [
     ("f16 rows of 768: 32 x 3", np.float16, [9001, 768]),
     ("f16 rows of 3072: 128 x 3", np.float16, [2101, 3072]),
     ("bf16 rows of 2560: 128 x 3, the last vectors of each thread empty", "bf16", [2300, 2560]),
-    ("f16 rows of 5120: softmax 256 x 3", np.float16, [1300, 5120]),
+    ("f16 rows of 5120: softmax 256 x 3, layernorm 128 x 5 with gamma / beta in LDS", np.float16, [1300, 5120]),
+    ("bf16 rows of 1152: layernorm 32 x 5 with gamma / beta in LDS", "bf16", [9001, 1152]),
+    ("f16 rows of 10240: layernorm 256 x 5 with gamma / beta in LDS", np.float16, [1100, 10240]),
     ("bf16 rows of 12288: softmax 512 x 3", "bf16", [600, 12288]),
     # odd lengths with 3 or 5 vectors per thread (softmax; layernorm keeps powers of two there)
     ("f16 rows of 577: shifted, 32 x 3", np.float16, [9000, 577]),
