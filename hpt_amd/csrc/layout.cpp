@@ -809,20 +809,27 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     const int pref_tpr = n_norm_dims > 0 ? 512 : 256;
                     // (gamma / beta in LDS: the form exists for three to five vectors per thread only)
                     int64_t best = p.gb_lds ? INT64_MAX : (int64_t)p.tpr * p.nchunk;
-                    int bt = 0, bc = 0;
+                    int bt = p.gb_lds ? 0 : p.tpr, bc = p.nchunk;
+                    bool base_stands = !p.gb_lds;  // the shape chosen above is still the best one
                     for (int t = p.gb_lds ? 32 : 16; t <= 1024; t <<= 1) {
                         const int64_t c = std::max<int64_t>((nv + t - 1) / t, p.gb_lds ? 3 : 1);
                         if (c > maxc) continue;
                         const int64_t slots = t * c;
                         bool take = slots < best;
-                        if (!take && bt && slots == best) {
-                            // equal: inside the preferred width the wider row (fewer vectors per thread) wins
-                            take = t <= pref_tpr;
+                        if (!take && bt && slots == best && t != bt) {
+                            // equal: a row inside the preferred width beats one outside it; inside, the wider row
+                            // (fewer vectors per thread) wins, outside, the narrower one (f32 softmax [4096, 8192]
+                            // 512 x 4 5.3 -> 256 x 8 5.7 TB/s, [2048, 16384] 1024 x 4 4.8 -> 512 x 8 5.2). The shape
+                            // chosen above only gives way when it lies outside the preferred width.
+                            const bool in_t = t <= pref_tpr, in_b = bt <= pref_tpr;
+                            take = in_t != in_b ? in_t : (in_t ? t > bt : t < bt);
+                            if (base_stands && in_b) take = false;
                         }
                         if (take) {
                             best = slots;
                             bt = t;
                             bc = (int)c;
+                            base_stands = false;
                         }
                     }
                     if (bt) {
