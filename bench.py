@@ -409,7 +409,7 @@ def cases_c8(P):
     red(ts, nb, "f32 [8190,4097]", "sum", [0], "sum(axis=0)", 4097)
     del ts
     ts, nb = up([2048, 16384])
-    nrm(ts, nb, "f32 [2048,16384] (rows of 1024 threads)", "log_softmax", 1, "log_softmax(axis=1)", 2048)
+    nrm(ts, nb, "f32 [2048,16384] (long rows walked with prefetch)", "log_softmax", 1, "log_softmax(axis=1)", 2048)
     del ts
     ts, nb = up([8, 21, 512, 512])
     nrm(ts, nb, "f32 [8,21,512,512] (softmax over channels)", "softmax", 1, "softmax(axis=1)", 8 * 512 * 512)
