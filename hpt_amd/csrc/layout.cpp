@@ -59,14 +59,14 @@ int reduce_out_dtype(int op, int in) {
 
 static int64_t iabs(int64_t v) { return v < 0 ? -v : v; }
 
-static int pow2_floor(int64_t v) {
-    int p = 1;
-    while ((int64_t)p * 2 <= v) p *= 2;
+static int64_t pow2_floor(int64_t v) {
+    int64_t p = 1;
+    while (p <= v / 2) p *= 2;
     return p;
 }
-static int pow2_ceil(int64_t v) {
-    int p = 1;
-    while (p < v) p *= 2;
+static int64_t pow2_ceil(int64_t v) {
+    int64_t p = 1;
+    while (p < v && p < ((int64_t)1 << 62)) p *= 2;
     return p;
 }
 
@@ -783,7 +783,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 // 4.1 -> 4.9, [4000, 10000] 4.7 -> 5.1; f16 [8192, 8200] loses (4.7 -> 3.0: eight widened vectors spill).
                 if (n_norm_dims <= 0 && v > 1 && elem_size >= 4 && p.tpr >= 512 && nv <= (p.tpr / 2) * 5) p.tpr /= 2;
                 int64_t nc = (nv + p.tpr - 1) / p.tpr;
-                p.nchunk = std::max(1, pow2_ceil(nc));
+                p.nchunk = (int)std::max<int64_t>(1, pow2_ceil(nc));
                 // Threads per row and vectors per thread are powers of two so far, which leaves a quarter
                 // to a third of the lanes idle on rows of 3, 5, 6 or 7 times a power of two - the hidden
                 // sizes 768, 1536, 2560, 3072, 5120, 6144, 12288. Aligned rows of whole vectors may take 3
