@@ -18,7 +18,7 @@ own duration come from profiles/headline.json (written when the rocprofv3 summar
 profiles/ are regenerated), and the plan the library reports for the headline call is printed
 beside the plan recorded there, so a planner change that makes the profile stale shows.
 
-`ops` lists every op of the five benchmark configurations (and the groups c6-c9), each timed
+`ops` lists every op of the five benchmark configurations (and the groups c6-c10), each timed
 the same way whatever --steps says: 10 warm-up launches, then 13 groups of 8 back-to-back
 launches, every group bracketed by a pair of HIP events; `us_per_launch` is the median over the
 groups of (group time / 8) - 104 timed launches. (Bracketing every single launch instead adds
@@ -467,6 +467,24 @@ def cases_c9(P):
     return cases
 
 
+def cases_c10(P):
+    """Logits over a vocabulary, ~0.5 GiB per tensor pair: softmax / log_softmax over rows of 30522 (odd:
+    row starts off the 16-byte grid), 128256 and 151936 elements, which stay on chip in registers + LDS."""
+    import hpt_amd as hpt
+    rng = np.random.default_rng(10)
+    cases = []
+    for dname, npdt, rows, cols, op in (("f32", np.float32, 4096, 30522, "softmax"), ("f32", np.float32, 1024, 128256, "log_softmax"),
+                                        ("f16", np.float16, 2048, 151936, "log_softmax")):
+        base = rng.standard_normal((rows, cols), dtype=np.float32).astype(npdt)
+        ts = [hpt.Tensor.from_numpy(np.roll(base, k, 0)).to_hip(0) for k in range(2)]
+        run, outs = P.norm(ts, op, axis=1)
+        P.keep.append(outs)
+        cases.append(Case(f"{op}(axis=1)", f"{dname} [{rows},{cols}] (vocabulary of {cols})", dname, rows, 2 * base.nbytes, run, 2,
+                          plan=P.last_plan))
+        del ts
+    return cases
+
+
 def build_cases(which: str, configs=None):
     """Synthetic inputs of the benchmark configurations, uploaded once; outputs preallocated.
     The headline (C2 layernorm) is always first; `configs` limits the others (e.g. {"c3"})."""
@@ -474,7 +492,7 @@ def build_cases(which: str, configs=None):
     cases, head = cases_c2(P, which == "headline")
     if which != "headline":
         for name, fn in (("c1", cases_c1), ("c3", cases_c3), ("c4", cases_c4), ("c5", cases_c5), ("c6", cases_c6),
-                         ("c7", cases_c7), ("c8", cases_c8), ("c9", cases_c9)):
+                         ("c7", cases_c7), ("c8", cases_c8), ("c9", cases_c9), ("c10", cases_c10)):
             if configs is None or name in configs:
                 cases += fn(P)
     return cases, P, head
@@ -567,7 +585,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--ops", choices=["all", "headline"], default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--configs", default="", help="comma list of c1,c3,c4,c5,c6,c7,c8,c9 to measure besides the headline (c6 = the steps either side: contiguous / in-place affine / full; c7 = the fused forms; c8 = shapes off the reference's list; c9 = hidden sizes of 3 or 5 times a power of two)")
+    ap.add_argument("--configs", default="", help="comma list of c1,c3,c4,c5,c6,c7,c8,c9,c10 to measure besides the headline (c6 = the steps either side: contiguous / in-place affine / full; c7 = the fused forms; c8 = shapes off the reference's list; c9 = hidden sizes of 3 or 5 times a power of two; c10 = logits over a vocabulary)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region, run one plain device-to-device copy of the headline input "
                          "(134217728 bytes read + as many written): the known-size dispatch that hardware "

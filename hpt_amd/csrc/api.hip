@@ -476,7 +476,7 @@ static NormCall prepare_norm(const hpt_view* in, const void* out_data, int64_t a
     }
     NormCall c;
     c.plan = plan_normalize(in->data, out_data, in->shape, in->strides, in->ndim, axis, n_norm_dims,
-                            dtype_size(norm_out_dtype(in->dtype)), float_only && n_norm_dims > 0);
+                            dtype_size(norm_out_dtype(in->dtype)), float_only);
     if (!is_float_dtype(in->dtype)) restrict_to_row_stream(c.plan);
     NormArgs& a = c.args;
     memset(&a, 0, sizeof a);

@@ -146,8 +146,8 @@ struct NormPlan {
     int flat_t = 0;     // ColSplit, > 0: a narrow inner dim; the slab is walked as a flat array by this many threads
     int slab_tile = 0;  // Col softmax over the middle axis of mid-sized contiguous [cols, L] slabs with a narrow L: one workgroup per slab through LDS (the value: lanes per column)
     int group_tile = 0; // Col softmax over a short middle axis of small contiguous [cols, L] groups: this many groups per workgroup through LDS
-    int lds_rows = 0;   // RowReg softmax of 4-byte types, 32769 ... 65536 elements per row: half the row in registers, half in LDS
-    int raw_rows = 0;   // RowReg softmax of 2-byte types, 32769 ... 131072 elements per row: only the raw row stays in registers
+    int lds_rows = 0;   // RowReg softmax of 2- and 4-byte types: long rows held in the registers and the LDS of tpr = 256 or 512 threads (nchunk: vectors per thread in both together)
+    int raw_rows = 0;   // RowReg softmax of 2-byte types, 98305 ... 131072 elements per row: only the raw row stays in registers
     int gb_lds = 0;     // RowReg layernorm of 2-byte types: gamma / beta in LDS, four vectors of the row per thread
     int tile_rows = 0;  // RowReg, > 0: short back-to-back rows; the plain kinds stage this many rows per workgroup in LDS
     int shift = 0;      // RowStream: rows start off 16-byte boundaries; aligned vectors, masked at both ends
@@ -156,10 +156,11 @@ struct NormPlan {
 };
 
 // axis >= 0: softmax-style single axis; n_norm_dims > 0: trailing dims (layernorm).
-// with_residual: the plan is for layernorm(x + residual), whose rows are held twice.
+// fused: the plan is for a fused kind: layernorm(x + residual), whose rows are held twice, or the
+// causal softmax, which the plain softmax's register + LDS kernels do not implement.
 NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t* shape,
                         const int64_t* strides, int ndim, int64_t axis, int n_norm_dims,
-                        size_t elem_size, bool with_residual = false);
+                        size_t elem_size, bool fused = false);
 
 std::string describe(const NormPlan& p);
 

@@ -477,9 +477,32 @@ std::string describe(const ReducePlan& p) {
 
 // ---- normalisation ---------------------------------------------------------
 
+// Softmax rows held in registers and LDS (row_lds_kernel): the smallest of its three launch shapes whose
+// slots hold the `nvec` vectors of a row's vector grid; false when none does. 24 + 8 vectors of a four-byte
+// type (16 + 8 of a two-byte type) per thread, 256 or 512 threads; twice that per thread, 512 threads.
+static bool lds_row_shape(NormPlan& p, int64_t nvec, size_t elem_size) {
+    const int per = elem_size == 4 ? 32 : 24;
+    if (nvec <= 256 * per) {
+        p.tpr = 256;
+        p.nchunk = per;
+    } else if (nvec <= 512 * per) {
+        p.tpr = 512;
+        p.nchunk = per;
+    } else if (nvec <= 512 * 2 * per) {
+        p.tpr = 512;
+        p.nchunk = 2 * per;
+    } else {
+        return false;
+    }
+    p.kind = NormKind::RowReg;
+    p.lds_rows = 1;
+    p.rpb = 1;
+    return true;
+}
+
 NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t* shape,
                         const int64_t* strides, int ndim, int64_t axis, int n_norm_dims,
-                        size_t elem_size, bool with_residual) {
+                        size_t elem_size, bool fused) {
     NormPlan p;
     int64_t total = 1;
     for (int i = 0; i < ndim; ++i) total *= shape[i];
@@ -633,41 +656,15 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 const int64_t nvs = (p.cols + 2 * (max_vec - 1)) / max_vec;
                 // (two-byte layernorm keeps two vectors per thread, so its rows stay in registers up to 1024
                 // vectors, 512 threads; f16 [8190, 4097] 1.9 -> 2.2 TB/s, [5461, 6145] 1.9 -> 2.8 against streaming)
-                if (same && n_norm_dims <= 0 && elem_size == 2 && nvs > 4096 && nvs <= 8192) {
-                    // two-byte softmax rows of 32769 ... 65521 elements (a vocabulary of 50257): the raw row
-                    // in registers (see below), f16 [4096, 50257] log_softmax 3.1 -> 4.0 TB/s. The
-                    // sixteen-vector form spills with the masks of the shifted walk and only matches streaming.
-                    p.kind = NormKind::RowReg;
-                    p.raw_rows = 1;
+                // Softmax rows beyond the register kernel's 2048 shifted vectors stay on chip in registers and
+                // LDS (row_lds_kernel, whose vector grid starts on the 128-byte line that holds the row's first
+                // element) up to 131038 four-byte or 196538 two-byte elements; they streamed before (two reads).
+                // Measured (TB/s): f32 [4096, 30522] 3.5 -> , [2048, 50257] 4.45 -> 4.8, [1024, 100277] 3.7 -> 4.3;
+                // f16 [8192, 32001] 4.0 -> , [4096, 50257] 4.35 -> 5.2, [2048, 98001] 4.2 -> 4.9.
+                if (same && n_norm_dims <= 0 && nvs > 2048 && (elem_size == 2 || elem_size == 4) &&
+                    lds_row_shape(p, (p.cols + 128 / (int64_t)elem_size + max_vec - 2) / max_vec, elem_size)) {
                     p.vec = max_vec;
                     p.shift = 1;
-                    p.tpr = 1024;
-                    p.rpb = 1;
-                    p.nchunk = 8;
-                    return p;
-                }
-                if (same && n_norm_dims <= 0 && elem_size == 2 && nvs > 8192 && p.cols <= 131072 - 70) {
-                    // two-byte softmax rows of 65522 ... 131002 elements: registers and LDS (see below; the
-                    // kernel's vector grid starts up to 63 elements before the row)
-                    p.kind = NormKind::RowReg;
-                    p.lds_rows = 1;
-                    p.vec = max_vec;
-                    p.shift = 1;
-                    p.tpr = 1024;
-                    p.rpb = 1;
-                    p.nchunk = 16;
-                    return p;
-                }
-                if (same && n_norm_dims <= 0 && elem_size == 4 && nvs > 8192 && p.cols <= 65536 - 34) {
-                    // four-byte softmax rows of 32769 ... 65502 elements: registers and LDS (see below; the
-                    // kernel's vector grid starts up to 31 elements before the row)
-                    p.kind = NormKind::RowReg;
-                    p.lds_rows = 1;
-                    p.vec = max_vec;
-                    p.shift = 1;
-                    p.tpr = 1024;
-                    p.rpb = 1;
-                    p.nchunk = 16;
                     return p;
                 }
                 if (same && nvs > ((n_norm_dims > 0 && elem_size == 2) ? 1024 : 2048)) {
@@ -724,33 +721,32 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 p.gb_lds = 1;
                 ln_half = false;
             }
-            // Two-byte softmax rows of 32769 ... 131072 elements: the raw row in registers (sixteen vectors
-            // per thread at most), one read instead of the streaming kernel's two.
-            // (f32 rows of sixteen vectors per thread measured slower this way than streaming: 2.6 against 3.3 TB/s)
-            const bool raw_rows = n_norm_dims <= 0 && elem_size == 2 && v == max_vec && p.sstride == 1 && !p.shift &&
-                                  nv > 4096 && nv <= 16384;
             const int64_t per = ln_half ? 2 * p.sstride : 4;
             const int64_t reg_limit = ln_half ? 1024 * per : (n_norm_dims > 0 && v > 1) ? 4096 : 8192;
-            if (raw_rows) {
-                p.kind = NormKind::RowReg;
-                p.raw_rows = 1;
-                p.tpr = 1024;
-                p.rpb = 1;
-                p.nchunk = nv > 8192 ? 16 : 8;
-                return p;
-            }
-            // Four-byte softmax rows of 32769 ... 65536 elements: eight vectors per thread in registers and
-            // up to eight more in LDS, one read instead of the streaming kernel's two. (Layernorm in that kernel,
-            // with gamma / beta from L2 in the last sweep, spilled 60 to 130 registers and ran at 1.6-3.3 TB/s:
-            // such rows stream, at 3.0-3.4.) (Twelve and eight, for
-            // two-byte rows up to 163840 elements, has twenty loads in flight per thread and spills 40 registers.)
-            if (n_norm_dims <= 0 && elem_size == 4 && v == max_vec && p.sstride == 1 && !p.shift && nv > 8192 && nv <= 16384) {
-                p.kind = NormKind::RowReg;
-                p.lds_rows = 1;
-                p.tpr = 1024;
-                p.rpb = 1;
-                p.nchunk = 16;
-                return p;
+            // Softmax rows beyond eight vectors per thread of a four-byte type (four of a two-byte type) stay on
+            // chip in registers and LDS, one read instead of the streaming kernel's two: row_lds_kernel, up to
+            // 131072 four-byte or 196608 two-byte elements. Two-byte rows of 98305 ... 131072 elements keep the
+            // raw row in the registers of 1024 threads (sixteen vectors each), which measured faster there.
+            // (Layernorm in such a kernel, with gamma / beta from L2 in the last sweep, spilled 60 to 130
+            // registers and ran at 1.6-3.3 TB/s: such rows stream, at 3.0-3.4.)
+            // Measured (TB/s; before: 1024 threads with 8 + 8 vectors staged through registers, the raw-row
+            // kernel, or streaming): f32 [640, 50304] 4.35 -> 5.05, [2048, 50304] 5.05 -> 5.35, [2048, 40960]
+            // 4.9 -> 5.35, [1024, 128256] 3.75 -> 4.7; f16 [4096, 50304] 4.75 -> 5.55, [4096, 65536] 5.0 -> 5.6,
+            // [2048, 98304] 4.45 -> 5.1, [2048, 151936] 4.25 -> 4.55.
+            if (n_norm_dims <= 0 && v == max_vec && p.sstride == 1 && !p.shift) {
+                const bool raw16 = elem_size == 2 && nv > 12288 && nv <= 16384;
+                if (raw16) {
+                    p.kind = NormKind::RowReg;
+                    p.raw_rows = 1;
+                    p.tpr = 1024;
+                    p.rpb = 1;
+                    p.nchunk = 16;
+                    return p;
+                }
+                // (the causal softmax has no such kernel: its rows stay with the register kernel while they fit)
+                if ((elem_size == 4 ? nv > 8192 : elem_size == 2 && nv > 4096) && !(fused && nv <= reg_limit) &&
+                    lds_row_shape(p, nv, elem_size))
+                    return p;
             }
             if (nv <= reg_limit) {
                 p.kind = NormKind::RowReg;
@@ -803,7 +799,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 if (v == max_vec && v > 1 && p.sstride == 1 && !p.tile_rows) {
                     const int maxc = n_norm_dims > 0 && p.shift ? (elem_size == 2 ? 2 : 4)
                                                                 : elem_size == 2 ? (ln_half ? 3 : (p.gb_lds ? 5 : 4))
-                                                                : (n_norm_dims > 0 ? (with_residual ? 4 : 6) : 8);
+                                                                : (n_norm_dims > 0 ? (fused ? 4 : 6) : 8);
                     // (layernorm(x + residual) holds the residual's vectors beside the row's: with five or six
                     // per thread it spills - f32 [2730, 12288] 3.1 TB/s)
                     const int pref_tpr = n_norm_dims > 0 ? 512 : 256;
@@ -836,6 +832,13 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                         p.tpr = bt;
                         p.nchunk = bc;
                     }
+                    // Softmax rows beyond 2048 vectors that still leave a sixteenth of those slots idle (threads
+                    // come in powers of two): row_lds_kernel's 256 threads take slots in steps of 256 vectors.
+                    // Measured (TB/s): f32 [4096, 16388] 4.8 -> 5.15; f16 [8192, 16392] 4.2 -> 5.45. (Full rows
+                    // gain nothing: f32 [4096, 32768] 5.55 -> 5.55, f16 [8192, 32768] 5.75 -> 5.35.)
+                    if (n_norm_dims <= 0 && !fused && !p.shift && nv > (elem_size == 2 ? 1024 : 2048) && (elem_size == 2 || elem_size == 4) &&
+                        (int64_t)p.tpr * p.nchunk - nv >= nv / 16 && lds_row_shape(p, nv, elem_size))
+                        return p;
                 }
                 int block = std::max(256, p.tpr);
                 p.rpb = block / p.tpr;
@@ -1040,7 +1043,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg) ? "-unaligned" : (p.raw_rows ? "-raw-shift" : (p.lds_rows ? "-lds-shift" : "-shift"))) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.group_tile ? "-group-tile" : (p.slab_tile ? "-slab" : "")), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg) ? "-unaligned" : (p.lds_rows ? "-lds-shift" : "-shift")) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.group_tile ? "-group-tile" : (p.slab_tile ? "-slab" : "")), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     if (p.kind == NormKind::RowReg) s += "max_blocks=" + std::to_string(p.max_blocks) + " ";  // (layernorm walks its rows)

@@ -382,18 +382,13 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
 }
 
 // ---- long rows of 2-byte elements: the raw row in registers ---------------------------------
-// softmax / log_softmax over rows of 32769 ... 131072 f16 / bf16 elements (a vocabulary). The row
-// kernel above keeps the widened row (f32) between its sweeps, which is 64 registers per thread at
-// eight vectors and does not fit at sixteen. Here only the RAW row stays (4 registers per vector:
-// 64 at sixteen vectors per thread, 1024 threads per row) and every sweep widens again: max, then
-// the sum of exponentials, then the result, the exponential taken twice. One HBM read and one
-// write where the streaming kernel reads twice.
-// PF (eight vectors per thread): the next row's loads are issued before the current row's sweeps;
-// there is one workgroup per compute unit, so nothing else hides a row's load -> sweeps -> store chain.
-// SHIFT: rows that start off 16-byte boundaries (a vocabulary of 50257): a row is covered by the
-// aligned vectors that contain it, as in row_reg_kernel; positions outside the row count as -inf and
-// the two end vectors are stored element by element. Input and output rows share their misalignment.
-template <int KIND, class T, int NCHUNK, bool PF = false, bool SHIFT = false>
+// softmax / log_softmax over aligned rows of 98305 ... 131072 f16 / bf16 elements (a vocabulary of
+// 128256). The row kernel above keeps the widened row (f32) between its sweeps, which is 64 registers
+// per thread at eight vectors and does not fit at sixteen. Here only the RAW row stays (4 registers
+// per vector: 64 at sixteen vectors per thread, 1024 threads per row) and every sweep widens again:
+// max, then the sum of exponentials, then the result, the exponential taken twice. One HBM read and
+// one write where the streaming kernel reads twice.
+template <int KIND, class T, int NCHUNK>
 __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
     static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX, "a softmax kernel");
     constexpr int VEC = 16 / sizeof(T);
@@ -401,53 +396,26 @@ __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
     using CT = typename Elem<T>::Wide;
     __shared__ CT smem[16];
     const int tx = threadIdx.x;
-    const int cols = (int)a.cols;
-    auto shift_of = [](const T* p) -> int { return SHIFT ? (int)(((uintptr_t)p / sizeof(T)) % VEC) : 0; };
-    // vectors that cover a row which starts sh elements after a 16-byte boundary
-    auto vectors = [&](int sh) -> int { return SHIFT ? (cols + sh + VEC - 1) / VEC : cols / VEC; };
-    Pack<T, VEC> raw[NCHUNK], nxt[PF ? NCHUNK : 1];
+    const int nv = (int)a.cols / VEC;
+    Pack<T, VEC> raw[NCHUNK];
     // (2-byte types: keep the compiler from holding the widened copies of one sweep for the next)
     auto forget = [](Pack<T, VEC>& v) {
         if constexpr (sizeof(T) == 2) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&v)));
     };
-    auto fetch = [&](Pack<T, VEC>* dst, int64_t row) {
-        if (row >= a.rows) return;
+    for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
         const T* in_row = (const T*)a.in + offset_of(a.kept_in, row);
-        const int sh = shift_of(in_row);
-        const int nv = vectors(sh);
+        T* out_row = (T*)a.out + row * a.cols;
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int iv = c * 1024 + tx;
-            if (iv < nv) dst[c] = load_pack_stream<T, VEC>(in_row - sh + (int64_t)iv * VEC);
+            if (iv < nv) raw[c] = load_pack_stream<T, VEC>(in_row + (int64_t)iv * VEC);
         }
-    };
-    if constexpr (PF) fetch(raw, blockIdx.x);
-    for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
-        T* out_row = (T*)a.out + row * a.cols;
-        const int sh = shift_of(out_row);
-        const int nv = vectors(sh);
-        if constexpr (PF) fetch(nxt, row + gridDim.x);
-        else fetch(raw, row);
-        if constexpr (SHIFT) {
-            // the row's two end vectors: positions outside the row become -inf once, here, and the
-            // sweeps below need no masks
-#pragma unroll
-            for (int c = 0; c < NCHUNK; ++c) {
-                const int iv = c * 1024 + tx;
-                if (iv == 0 || iv == nv - 1) {
-#pragma unroll
-                    for (int j = 0; j < VEC; ++j)
-                        if ((unsigned)(iv * VEC + j - sh) >= (unsigned)cols) raw[c].v[j] = Elem<T>::narrow(neg_inf<CT>());
-                }
-            }
-        }
-        auto elem = [&](const Pack<T, VEC>& v, int, int j) -> CT { return Elem<T>::widen(v.v[j]); };
         CT m = neg_inf<CT>();
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c)
             if (c * 1024 + tx < nv)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, elem(raw[c], c * 1024 + tx, j));
+                for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, Elem<T>::widen(raw[c].v[j]));
         m = row_all_reduce<MaxC<CT>>(m, 1024, 0, smem);
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) forget(raw[c]);
@@ -456,7 +424,7 @@ __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
         for (int c = 0; c < NCHUNK; ++c)
             if (c * 1024 + tx < nv)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) s += exp_ct<T>(elem(raw[c], c * 1024 + tx, j) - m);
+                for (int j = 0; j < VEC; ++j) s += exp_ct<T>(Elem<T>::widen(raw[c].v[j]) - m);
         s = row_all_reduce<SumC<CT>>(s, 1024, 0, smem);
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) forget(raw[c]);
@@ -471,43 +439,45 @@ __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
                     const CT d = Elem<T>::widen(raw[c].v[j]) - m;
                     o.v[j] = Elem<T>::narrow(kLog ? d - k : exp_ct<T>(d) * k);
                 }
-                const int e0 = iv * VEC - sh;
-                if (!SHIFT || (e0 >= 0 && e0 + VEC <= cols)) {
-                    store_pack_stream<T, VEC>(out_row + e0, o);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < VEC; ++j)
-                        if ((unsigned)(e0 + j) < (unsigned)cols) out_row[e0 + j] = o.v[j];
-                }
+                store_pack_stream<T, VEC>(out_row + (int64_t)iv * VEC, o);
             }
-        }
-        if constexpr (PF) {
-#pragma unroll
-            for (int c = 0; c < NCHUNK; ++c) raw[c] = nxt[c];
         }
     }
 }
 
-// ---- the longest rows that stay on chip: the row in registers AND LDS -------------------------
-// softmax / log_softmax over f32 rows of 32769 ... 65536 elements (logits of a 50257 / 50304 / 65536
-// vocabulary in f32) and two-byte rows of odd length from 65522 to 131002 elements.
-// NREG vectors per thread live in registers, up to NLDS more in LDS (NLDS * 16 KiB of the compute
-// unit's 160; every thread reads back only the slots it wrote, so the LDS part needs no barrier: it
-// is a second register file). One HBM read and one write where the streaming kernel reads twice.
+// ---- long rows that stay on chip: the row in registers AND LDS -----------------------------------
+// softmax / log_softmax over rows too long for the register kernel's eight vectors per thread: f32 rows
+// of 32769 ... 131072 elements and two-byte rows of 32769 ... 196608 (logits over a vocabulary: 50257,
+// 50304, 65536, 100277, 128256, 151936), and rows of odd length (row starts off the 16-byte grid) from
+// 2049 vectors on, which the register kernel does not take.
+// NREG vectors per thread live in registers, up to NLDS more in LDS (every thread reads back only the
+// slots it filled, so the LDS part needs no barrier: it is a second register file). One HBM read and
+// one write where the streaming kernel reads twice. The LDS part arrives by LDS-direct loads
+// (global_load_lds_dwordx4: a wavefront's 64 lanes fill 1 KiB of LDS from the wavefront's base on), so
+// no register is held for it while it is on its way and NREG can take what the register file has.
+// Shapes: NT = 256 or 512 threads with 24 + 8 vectors of a four-byte type (16 + 8 of a two-byte type)
+// and 128 registers each, so that two (512) or four (256) workgroups share a compute unit and one's
+// arithmetic overlaps the other's loads and stores; NT = 512 with 48 + 16 (32 + 16) vectors and 256
+// registers each for the longest rows, one workgroup per compute unit.
 // Four-byte types: the summing sweep overwrites the held row with exp(x - max) (softmax) or x - max
 // (log_softmax), so the exponential is taken once per element either way. Two-byte types keep the
 // raw row (rounding the intermediate to 16 bits would cost accuracy) and take the exponential twice.
-// SHIFT: as in row_raw_kernel.
-template <int KIND, class T, int NREG, int NLDS, bool SHIFT = false>
-__global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
+// SHIFT: rows that start off 16-byte boundaries (a vocabulary of 50257): a row is covered by aligned
+// vectors that contain it; positions outside the row count as -inf and the two end vectors are stored
+// element by element. Input and output rows share their misalignment.
+template <int KIND, class T, int NREG, int NLDS, bool SHIFT, int NT, int MINW>
+__global__ void __launch_bounds__(NT, MINW) row_lds_kernel(const NormArgs a) {
     static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX, "a softmax kernel");
-    static_assert(NLDS * 16 <= 144, "LDS of a compute unit");
+    static_assert(NLDS * NT * 16 <= 144 * 1024, "LDS of a compute unit");
     constexpr int VEC = 16 / sizeof(T);
     constexpr bool kKeep = sizeof(T) >= 4;  // the held row may be overwritten with intermediates
     constexpr bool kLog = KIND == NORM_LOGSOFTMAX;
+    // the walks over the LDS part stay loops (LDS takes a run-time index; unrolled, their reads are
+    // hoisted over the register part's work and push it out of the register file)
+    constexpr int kLdsUnroll = 2;
     using CT = typename Elem<T>::Wide;
     __shared__ CT smem[16];
-    __shared__ __align__(16) unsigned char lds_raw[NLDS * 1024 * 16];
+    __shared__ __align__(16) unsigned char lds_raw[NLDS * NT * 16];
     Pack<T, VEC>* lds = reinterpret_cast<Pack<T, VEC>*>(lds_raw);
     __shared__ Pack<T, VEC> ends[SHIFT ? 2 : 1];
     const int tx = threadIdx.x;
@@ -537,50 +507,59 @@ __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
         // (a vector that lies wholly before the row is not loaded: only a vector that holds an element of
         // the row is sure to stay on that element's page)
         auto touches = [&](int iv) { return !SHIFT || (iv + 1) * VEC > sh; };
+        // an address is the chunk's start (the same for every lane: a scalar) plus the lane's 32-bit offset;
+        // forty-odd 64-bit addresses per lane, computed ahead of the row loop, would not fit beside the row
+        auto chunk_of = [](auto* p, int c) { return p + (int64_t)c * (NT * VEC); };
+        const unsigned lane_off = (unsigned)tx * VEC;
         Pack<T, VEC> reg[NREG];
         {
-            Pack<T, VEC> tmp[NLDS];
-#pragma unroll
+#pragma unroll kLdsUnroll
             for (int c = 0; c < NLDS; ++c) {
-                const int iv = (NREG + c) * 1024 + tx;
-                if (iv < nv && touches(iv)) tmp[c] = load_pack_stream<T, VEC>(in_row - sh + (int64_t)iv * VEC);
+                const int iv = (NREG + c) * NT + tx;
+                if (iv < nv && touches(iv))
+                    __builtin_amdgcn_global_load_lds(
+                        (const __attribute__((address_space(1))) void*)(chunk_of(in_row - sh, NREG + c) + lane_off),
+                        (__attribute__((address_space(3))) void*)(lds + c * NT + (tx & ~63)), 16, 0, 0);
             }
 #pragma unroll
             for (int c = 0; c < NREG; ++c) {
-                const int iv = c * 1024 + tx;
-                if (iv < nv && touches(iv)) reg[c] = load_pack_stream<T, VEC>(in_row - sh + (int64_t)iv * VEC);
+                const int iv = c * NT + tx;
+                if (iv < nv && touches(iv)) reg[c] = load_pack_stream<T, VEC>(chunk_of(in_row - sh, c) + lane_off);
             }
-#pragma unroll
-            for (int c = 0; c < NLDS; ++c) {
-                const int iv = (NREG + c) * 1024 + tx;
-                if (iv < nv) {
-                    mask_ends(tmp[c], iv);
-                    lds[c * 1024 + tx] = tmp[c];
+            if constexpr (SHIFT) {
+#pragma unroll kLdsUnroll
+                for (int c = 0; c < NLDS; ++c) {
+                    const int iv = (NREG + c) * NT + tx;
+                    if (iv < nv && (iv * VEC < sh || iv == nv - 1)) {
+                        Pack<T, VEC> v = lds[c * NT + tx];
+                        mask_ends(v, iv);
+                        lds[c * NT + tx] = v;
+                    }
                 }
             }
         }
 #pragma unroll
-        for (int c = 0; c < NREG; ++c) mask_ends(reg[c], c * 1024 + tx);
+        for (int c = 0; c < NREG; ++c) mask_ends(reg[c], c * NT + tx);
         CT m = neg_inf<CT>();
 #pragma unroll
         for (int c = 0; c < NREG; ++c)
-            if (c * 1024 + tx < nv)
+            if (c * NT + tx < nv)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, Elem<T>::widen(reg[c].v[j]));
-#pragma unroll
+#pragma unroll kLdsUnroll
         for (int c = 0; c < NLDS; ++c)
-            if ((NREG + c) * 1024 + tx < nv) {
-                const Pack<T, VEC> v = lds[c * 1024 + tx];
+            if ((NREG + c) * NT + tx < nv) {
+                const Pack<T, VEC> v = lds[c * NT + tx];
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, Elem<T>::widen(v.v[j]));
             }
-        m = row_all_reduce<MaxC<CT>>(m, 1024, 0, smem);
+        m = row_all_reduce<MaxC<CT>>(m, NT, 0, smem);
 #pragma unroll
         for (int c = 0; c < NREG; ++c) forget(reg[c]);
         CT s = 0;
 #pragma unroll
         for (int c = 0; c < NREG; ++c)
-            if (c * 1024 + tx < nv)
+            if (c * NT + tx < nv)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
                     const CT d = Elem<T>::widen(reg[c].v[j]) - m;
@@ -588,10 +567,10 @@ __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
                     s += e;
                     if constexpr (kKeep) reg[c].v[j] = Elem<T>::narrow(kLog ? d : e);
                 }
-#pragma unroll
+#pragma unroll kLdsUnroll
         for (int c = 0; c < NLDS; ++c)
-            if ((NREG + c) * 1024 + tx < nv) {
-                Pack<T, VEC> v = lds[c * 1024 + tx];
+            if ((NREG + c) * NT + tx < nv) {
+                Pack<T, VEC> v = lds[c * NT + tx];
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
                     const CT d = Elem<T>::widen(v.v[j]) - m;
@@ -599,9 +578,9 @@ __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
                     s += e;
                     if constexpr (kKeep) v.v[j] = Elem<T>::narrow(kLog ? d : e);
                 }
-                if constexpr (kKeep) lds[c * 1024 + tx] = v;
+                if constexpr (kKeep) lds[c * NT + tx] = v;
             }
-        s = row_all_reduce<SumC<CT>>(s, 1024, 0, smem);
+        s = row_all_reduce<SumC<CT>>(s, NT, 0, smem);
 #pragma unroll
         for (int c = 0; c < NREG; ++c) forget(reg[c]);
         const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
@@ -614,15 +593,16 @@ __global__ void __launch_bounds__(1024) row_lds_kernel(const NormArgs a) {
                 else o.v[j] = Elem<T>::narrow(kLog ? (x - m) - k : exp_ct<T>(x - m) * k);
             }
             const int e0 = iv * VEC - sh;
-            if (!SHIFT || (e0 >= 0 && e0 + VEC <= cols)) store_pack_stream<T, VEC>(out_row + e0, o);
+            T* dst = chunk_of(out_row - sh, (iv - tx) / NT) + lane_off;
+            if (!SHIFT || (e0 >= 0 && e0 + VEC <= cols)) store_pack_stream<T, VEC>(dst, o);
             else if (e0 + VEC > 0) ends[e0 < 0 ? 0 : 1] = o;  // the row's two end vectors leave element by element below
         };
 #pragma unroll
         for (int c = 0; c < NREG; ++c)
-            if (c * 1024 + tx < nv) finish(reg[c], c * 1024 + tx);
-#pragma unroll
+            if (c * NT + tx < nv) finish(reg[c], c * NT + tx);
+#pragma unroll kLdsUnroll
         for (int c = 0; c < NLDS; ++c)
-            if ((NREG + c) * 1024 + tx < nv) finish(lds[c * 1024 + tx], (NREG + c) * 1024 + tx);
+            if ((NREG + c) * NT + tx < nv) finish(lds[c * NT + tx], (NREG + c) * NT + tx);
         if constexpr (SHIFT) {
             __syncthreads();
             if (tx < 2 * VEC) {

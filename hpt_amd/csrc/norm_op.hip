@@ -268,40 +268,48 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         return;
     }
     if (p.kind == NormKind::RowReg && p.lds_rows) {
-        // the longest rows that stay on chip: registers + LDS; the fused kinds stream
+        // long rows that stay on chip: registers + LDS; the fused kinds stream
         if constexpr (FULL > 1 && sizeof(T) <= 4 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX)) {
-            if (p.nchunk == 16) {
-                if (p.shift) row_lds_kernel<KIND, T, 8, 8, true><<<grid, dim3(1024), 0, st>>>(a);
-                else row_lds_kernel<KIND, T, 8, 8, false><<<grid, dim3(1024), 0, st>>>(a);
+            // 24 + 8 vectors of a four-byte type (16 + 8 of a two-byte type) per thread and 128 registers:
+            // 256 or 512 threads; 48 + 16 (32 + 16) and 256 registers: 512 threads
+            constexpr int kRegs = sizeof(T) == 4 ? 24 : 16;
+            if (p.nchunk == kRegs + 8 && p.tpr == 256) {
+                if (p.shift) row_lds_kernel<KIND, T, kRegs, 8, true, 256, 4><<<grid, dim3(256), 0, st>>>(a);
+                else row_lds_kernel<KIND, T, kRegs, 8, false, 256, 4><<<grid, dim3(256), 0, st>>>(a);
                 return;
             }
+            if (p.nchunk == kRegs + 8 && p.tpr == 512) {
+                if (p.shift) row_lds_kernel<KIND, T, kRegs, 8, true, 512, 4><<<grid, dim3(512), 0, st>>>(a);
+                else row_lds_kernel<KIND, T, kRegs, 8, false, 512, 4><<<grid, dim3(512), 0, st>>>(a);
+                return;
+            }
+            if (p.nchunk == 2 * kRegs + 16 && p.tpr == 512) {
+                if (p.shift) row_lds_kernel<KIND, T, 2 * kRegs, 16, true, 512, 1><<<grid, dim3(512), 0, st>>>(a);
+                else row_lds_kernel<KIND, T, 2 * kRegs, 16, false, 512, 1><<<grid, dim3(512), 0, st>>>(a);
+                return;
+            }
+            fail(HPT_ERR_KERNEL, "row_lds: no kernel for %d threads x %d vectors", p.tpr, p.nchunk);
         }
         if constexpr (FULL > 1) {
-            if (p.shift) row_stream_kernel<KIND, T, FULL, true><<<grid, block, 0, st>>>(a);
-            else row_stream_kernel<KIND, T, FULL><<<grid, block, 0, st>>>(a);
+            // (the fused kinds stream such rows, a full workgroup per row)
+            a.tpr = 1024;
+            a.tpr_log2 = 10;
+            if (p.shift) row_stream_kernel<KIND, T, FULL, true><<<grid, dim3(1024), 0, st>>>(a);
+            else row_stream_kernel<KIND, T, FULL><<<grid, dim3(1024), 0, st>>>(a);
         }
         return;
     }
     if (p.kind == NormKind::RowReg && p.raw_rows) {
-        // long two-byte softmax rows: the raw row in registers; the fused kinds stream (sixteen vectors
-        // per thread) or take the ordinary register kernel (eight)
+        // two-byte softmax rows of 98305 ... 131072 elements: the raw row in registers, sixteen vectors per
+        // thread; the fused kinds stream
         if constexpr (sizeof(T) == 2 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX)) {
             if (grid.x > 512u) grid.x = 512u;
-            if (p.shift) {
-                row_raw_kernel<KIND, T, 8, true, true><<<grid, dim3(1024), 0, st>>>(a);
-            } else {
-                if (p.nchunk == 16) row_raw_kernel<KIND, T, 16><<<grid, dim3(1024), 0, st>>>(a);
-                else row_raw_kernel<KIND, T, 8, true><<<grid, dim3(1024), 0, st>>>(a);
-            }
-            return;
-        } else if (p.shift) {  // the fused kinds stream shifted rows this long
-            if constexpr (FULL > 1) row_stream_kernel<KIND, T, FULL, true><<<grid, block, 0, st>>>(a);
-            return;
-        } else if (p.nchunk > 8) {
+            row_raw_kernel<KIND, T, 16><<<grid, dim3(1024), 0, st>>>(a);
+        } else {
             if (p.vec == FULL) row_stream_kernel<KIND, T, FULL><<<grid, block, 0, st>>>(a);
             else row_stream_kernel<KIND, T, 1><<<grid, block, 0, st>>>(a);
-            return;
         }
+        return;
     }
     if (p.kind == NormKind::RowReg) {
         // Layernorm workgroups walk the rows (gamma / beta stay in registers);

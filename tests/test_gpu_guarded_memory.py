@@ -186,6 +186,12 @@ DIRECTED = [
     ((3, 65540), F32, (), ("softmax",), [1]),
     ((2, 1048576), F32, (), ("softmax", "layernorm", "sum"), [1]),
     ((35, 131072), F16, (), ("softmax",), [1]),
+    ((5, 30522), F32, (), ("softmax", "log_softmax"), [1]),
+    ((3, 128256), F32, (), ("softmax",), [1]),
+    ((3, 100277), F32, (), ("log_softmax",), [1]),
+    ((3, 151936), F16, (), ("softmax",), [1]),
+    ((5, 32001), F16, (), ("softmax", "log_softmax"), [1]),
+    ((5, 16392), F16, (), ("softmax",), [1]),
     # 3, 5, 6, 7 vectors per thread; gamma / beta through LDS for the two-byte types
     ((67, 768), F16, (), ("layernorm", "softmax"), [1]),
     ((67, 5120), F16, (), ("layernorm", "softmax"), [1]),

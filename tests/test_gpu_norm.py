@@ -361,7 +361,32 @@ WIDE_ROW_CASES = [
     ("bf16 rows of 65521: the longest shifted raw row", "bf16", [517, 65521]),
     ("f16 rows of 65537: registers and LDS, shifted", np.float16, [130, 65537]),
     ("bf16 rows of 131001: the longest shifted two-byte row on chip", "bf16", [133, 131001]),
-    ("f16 rows of 131003: streamed", np.float16, [131, 131003]),
+    ("f16 rows of 131003: registers and LDS-direct loads, shifted", np.float16, [131, 131003]),
+    # longer rows on chip: 512 threads with 48 (f32) / 32 (two-byte) vectors in registers and 16 in LDS,
+    # which arrive by LDS-direct loads
+    ("f32 rows of 128256: registers and LDS-direct loads", np.float32, [270, 128256]),
+    ("f32 rows of 65540: one vector beyond the sixteen-vector kernel", np.float32, [133, 65540]),
+    ("f32 rows of 131072: every slot in use", np.float32, [70, 131072]),
+    ("f32 rows of 98308: the first LDS slots only", np.float32, [131, 98308]),
+    ("f32 rows of 100277: shifted", np.float32, [261, 100277]),
+    ("f32 rows of 131041: the longest shifted f32 row on chip", np.float32, [67, 131041]),
+    ("f16 rows of 151936: registers and LDS-direct loads", np.float16, [263, 151936]),
+    ("bf16 rows of 196608: every slot in use", "bf16", [70, 196608]),
+    ("bf16 rows of 131080: one vector beyond the raw-row kernel", "bf16", [131, 131080]),
+    ("f16 rows of 150001: shifted", np.float16, [259, 150001]),
+    ("bf16 rows of 196545: the longest shifted two-byte row on chip", "bf16", [66, 196545]),
+    ("f16 rows of 196610: streamed", np.float16, [35, 196610]),
+    # the same kernel with 256 threads: odd lengths beyond 2048 vectors, and aligned rows that would leave
+    # a sixteenth of a power-of-two row's slots idle
+    ("f32 rows of 30522: shifted, 256 threads", np.float32, [1300, 30522]),
+    ("f32 rows of 8197: the shortest such row", np.float32, [2100, 8197]),
+    ("f32 rows of 32733: the longest shifted row of 256 threads", np.float32, [530, 32733]),
+    ("f32 rows of 32737: shifted, 512 threads", np.float32, [530, 32737]),
+    ("f32 rows of 16388: 256 threads", np.float32, [1100, 16388]),
+    ("f16 rows of 32001: shifted, 256 threads", np.float16, [1100, 32001]),
+    ("bf16 rows of 16392: 256 threads", "bf16", [1500, 16392]),
+    ("f16 rows of 50304: 512 threads, 16 + 8 vectors", np.float16, [600, 50304]),
+    ("bf16 rows of 98304: every slot of 512 threads in use", "bf16", [270, 98304]),
     # rows of 3, 5, 6 or 7 times a power of two: that many vectors per thread, no idle lanes
     ("f32 rows of 768: 64 threads x 3 vectors", np.float32, [5003, 768]),
     ("f32 rows of 1280: 64 x 5", np.float32, [4100, 1280]),
@@ -629,8 +654,9 @@ def test_special_values_on_the_large_shape_kernels(hpt, orc, dev):
     """+inf and NaN entries on the kernels only large shapes reach: a row / column with +inf or NaN
     comes out NaN where the oracle says so, everything else matches."""
     rng = np.random.default_rng(213)
-    for shape, axis, plan in (((60001, 33), 1, "rowreg+tile"), ((1100, 8200), 1, "rowreg rows"), ((500001, 5), 0, "col-split-flat"),
-                              ((4, 21, 128, 128), 1, "col-reg"), ((300, 70000), 1, "rowstream"), ((2100, 4097), 1, "rowreg-shift")):
+    for shape, axis, plan in (((60001, 33), 1, "rowreg+tile"), ((1100, 8192), 1, "rowreg rows"), ((1100, 8200), 1, "rowreg-lds rows"), ((500001, 5), 0, "col-split-flat"),
+                              ((4, 21, 128, 128), 1, "col-reg"), ((300, 70000), 1, "rowreg-lds rows"), ((300, 70001), 1, "rowreg-lds-shift"),
+                              ((130, 140000), 1, "rowstream"), ((2100, 4097), 1, "rowreg-shift")):
         x = (rng.standard_normal(shape) * 2).astype(np.float32)
         flat = x.reshape(-1)
         flat[rng.integers(0, flat.size, 40)] = np.inf
