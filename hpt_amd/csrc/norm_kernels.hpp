@@ -479,7 +479,6 @@ __global__ void __launch_bounds__(NT, MINW) row_lds_kernel(const NormArgs a) {
     __shared__ CT smem[16];
     __shared__ __align__(16) unsigned char lds_raw[NLDS * NT * 16];
     Pack<T, VEC>* lds = reinterpret_cast<Pack<T, VEC>*>(lds_raw);
-    __shared__ Pack<T, VEC> ends[SHIFT ? 2 : 1];
     const int tx = threadIdx.x;
     const int cols = (int)a.cols;
     // SHIFT: the vector grid starts on the 128-byte line that holds the row's first element, so a
@@ -594,8 +593,13 @@ __global__ void __launch_bounds__(NT, MINW) row_lds_kernel(const NormArgs a) {
             }
             const int e0 = iv * VEC - sh;
             T* dst = chunk_of(out_row - sh, (iv - tx) / NT) + lane_off;
-            if (!SHIFT || (e0 >= 0 && e0 + VEC <= cols)) store_pack_stream<T, VEC>(dst, o);
-            else if (e0 + VEC > 0) ends[e0 < 0 ? 0 : 1] = o;  // the row's two end vectors leave element by element below
+            if (!SHIFT || (e0 >= 0 && e0 + VEC <= cols)) {
+                store_pack_stream<T, VEC>(dst, o);
+            } else {  // the row's two end vectors leave element by element
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    if ((unsigned)(e0 + j) < (unsigned)cols) out_row[e0 + j] = o.v[j];
+            }
         };
 #pragma unroll
         for (int c = 0; c < NREG; ++c)
@@ -603,16 +607,6 @@ __global__ void __launch_bounds__(NT, MINW) row_lds_kernel(const NormArgs a) {
 #pragma unroll kLdsUnroll
         for (int c = 0; c < NLDS; ++c)
             if ((NREG + c) * NT + tx < nv) finish(lds[c * NT + tx], (NREG + c) * NT + tx);
-        if constexpr (SHIFT) {
-            __syncthreads();
-            if (tx < 2 * VEC) {
-                const int which = tx / VEC, j = tx % VEC;
-                const int e = (which == 0 ? sh / VEC : nv - 1) * VEC - sh + j;
-                const bool partial = which == 0 ? sh % VEC != 0 : nv * VEC - sh > cols;
-                if (partial && (unsigned)e < (unsigned)cols) out_row[e] = ends[which].v[j];
-            }
-            __syncthreads();  // before the next row's end vectors
-        }
     }
 }
 
