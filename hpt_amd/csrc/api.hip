@@ -406,8 +406,11 @@ static ReduceCall prepare_reduce(int entry_id, const hpt_view* in, const int64_t
     ReduceCall c;
     c.entry = &reduce_entry_for(entry_id);
     c.out_dtype = entry_id < HPT_REDUCE_OP_COUNT ? reduce_out_dtype(entry_id, in->dtype) : HPT_I64;
+    // an exponential per element (two-byte results take the hardware exp2: cheap), or squares in f64
+    const bool heavy = (entry_id == HPT_LOGSUMEXP && dtype_size(c.out_dtype) > 2) ||
+                       ((entry_id == HPT_SUM_SQUARE || entry_id == HPT_REDUCEL2) && in->dtype == HPT_F32);
     c.plan = plan_reduce(in->data, in->shape, in->strides, in->ndim, norm, naxes,
-                         dtype_size(in->dtype), c.entry->acc_size[in->dtype]);
+                         dtype_size(in->dtype), c.entry->acc_size[in->dtype], heavy);
     return c;
 }
 

@@ -110,9 +110,11 @@ struct ReducePlan {
 
 // Build the plan for reducing `axes` (already normalised) of a view.
 // `elem_size` and `data` decide whether 128-bit loads are legal; `acc_size` is
-// the size of one accumulator (bounds the LDS a column kernel may use).
+// the size of one accumulator (bounds the LDS a column kernel may use). `heavy`: the op spends many
+// instructions per element (an exponential, f64 arithmetic on f32 data), which wants more wavefronts
+// per compute unit than a plain sum.
 ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* strides, int ndim,
-                       const int64_t* axes, int naxes, size_t elem_size, size_t acc_size);
+                       const int64_t* axes, int naxes, size_t elem_size, size_t acc_size, bool heavy = false);
 
 std::string describe(const ReducePlan& p);
 

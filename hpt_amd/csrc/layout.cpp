@@ -106,7 +106,7 @@ constexpr int64_t kBlocksToFill = 2048;
 constexpr int64_t kComputeUnits = 256;  // MI355X
 
 ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* strides, int ndim,
-                       const int64_t* axes, int naxes, size_t elem_size, size_t acc_size) {
+                       const int64_t* axes, int naxes, size_t elem_size, size_t acc_size, bool heavy) {
     ReducePlan p;
     bool is_red[kMaxRank] = {};
     for (int i = 0; i < naxes; ++i) is_red[axes[i]] = true;
@@ -396,8 +396,12 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
                     // no second launch at all. f16 [4096, 8192][:, ::2] over axis 0, 48 workgroup
                     // slices -> 16 of four thread rows: 17.9 -> 14.6 us; f32 [512, 65536] over axis 0,
                     // 3 slices -> one launch of four thread rows: 4.9 -> 6.1 TB/s.
+                    // (An op that spends a dozen instructions per element - an exponential, f64 squares of f32
+                    // data - needs a second wavefront per SIMD to run beside the loads: eight thread rows. f32
+                    // [8192, 4096] over axis 0, us with 4 / 8 thread rows x 16 splits: sum 25.1 / 25.4,
+                    // sum_square 27.7 / 25.8, logsumexp 34.7 / 28.4.)
                     const int64_t parts = std::min<int64_t>(pow2_ceil(rp), pow2_floor(can));
-                    const int64_t by = std::min<int64_t>(parts, 4);
+                    const int64_t by = std::min<int64_t>(parts, heavy ? 8 : 4);
                     p.split = (int)std::max<int64_t>(1, std::min<int64_t>(parts / by, cap));
                     p.by = (int)by * base_by;
                 }
