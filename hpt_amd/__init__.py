@@ -7,6 +7,6 @@ from ._ffi import (DeviceError, DTypeError, HptError, KernelError, MemoryError_,
 from .tensor import (ALL, ANY, BIN_ADD, BIN_DIV, BIN_MUL, BIN_SUB, DTYPES, LOGSUMEXP, MAX, MEAN, MIN, NANPROD, NANSUM, PROD, REDUCEL1,
                      REDUCEL2, REDUCEL3, SUM, SUM_SQUARE, DType, Tensor, bf16, bf16_bits_to_f32,
                      bool_, device_count, f16, f32, f32_to_bf16_bits, f64, i8, i16, i32, i64,
-                     contiguous_plan, normalize_plan, reduce_plan, synchronize, u8, u16, u32, u64)
+                     binary_plan, contiguous_plan, normalize_plan, reduce_plan, synchronize, u8, u16, u32, u64)
 
 __all__ = [n for n in dir() if not n.startswith("_")]

@@ -94,6 +94,7 @@ SIGNATURES = {
                                           C.POINTER(View), C.POINTER(View), C.c_double, C.POINTER(View)]),
     "hpt_hip_contiguous": (C.c_int32, [C.c_int32, C.c_void_p, C.POINTER(View), C.POINTER(View)]),
     "hpt_hip_contiguous_plan": (C.c_int32, [C.POINTER(View), C.POINTER(View), C.c_char_p, C.c_size_t]),
+    "hpt_hip_binary_plan": (C.c_int32, [C.POINTER(View), C.POINTER(View), C.POINTER(View), C.c_char_p, C.c_size_t]),
     "hpt_hip_cast": (C.c_int32, [C.c_int32, C.c_void_p, C.POINTER(View), C.POINTER(View)]),
     "hpt_hip_fill": (C.c_int32, [C.c_int32, C.c_void_p, C.POINTER(View), C.c_void_p]),
     "hpt_hip_binary": (C.c_int32, [C.c_int32, C.c_void_p, C.c_int32, C.POINTER(View), C.POINTER(View),

@@ -905,29 +905,40 @@ int32_t hpt_hip_fill(int32_t dev, void* stream, hpt_view* out, const void* value
     });
 }
 
+// Argument checks of a binary op and the plan its kernels run.
+static EwPlan prepare_binary(const hpt_view* lhs, const hpt_view* rhs, const hpt_view* out) {
+    check_view(lhs, "binary lhs", true);
+    check_view(rhs, "binary rhs", true);
+    if (lhs->dtype != rhs->dtype)
+        fail(HPT_ERR_DTYPE, "binary: operands must share one dtype, got %s and %s", dtype_name(lhs->dtype),
+             dtype_name(rhs->dtype));
+    check_out(out, lhs->dtype, view_size(lhs), "binary output");
+    check_same_shape(lhs, out, "binary lhs / out");
+    check_same_shape(rhs, out, "binary rhs / out");
+    // The output may be one of the operands (in place) but must not overlap one otherwise:
+    // every element is read before it is written only when the two walk the same addresses.
+    check_alias(lhs, out, true, "binary", "lhs");
+    check_alias(rhs, out, true, "binary", "rhs");
+    const void* datas[2] = {lhs->data, rhs->data};
+    const int64_t* strides[2] = {lhs->strides, rhs->strides};
+    return plan_elementwise(out->data, out->shape, out->ndim, 2, datas, strides, dtype_size(out->dtype), true);
+}
+
 int32_t hpt_hip_binary(int32_t dev, void* stream, int32_t op, const hpt_view* lhs, const hpt_view* rhs,
                        hpt_view* out) {
     return guarded([&] {
-        check_view(lhs, "binary lhs", true);
-        check_view(rhs, "binary rhs", true);
-        if (lhs->dtype != rhs->dtype)
-            fail(HPT_ERR_DTYPE, "binary: operands must share one dtype, got %s and %s", dtype_name(lhs->dtype),
-                 dtype_name(rhs->dtype));
-        check_out(out, lhs->dtype, view_size(lhs), "binary output");
-        check_same_shape(lhs, out, "binary lhs / out");
-        check_same_shape(rhs, out, "binary rhs / out");
-        // The output may be one of the operands (in place) but must not overlap one otherwise:
-        // every element is read before it is written only when the two walk the same addresses.
-        const size_t es = dtype_size(out->dtype);
-        check_alias(lhs, out, true, "binary", "lhs");
-        check_alias(rhs, out, true, "binary", "rhs");
-        const void* datas[2] = {lhs->data, rhs->data};
-        const int64_t* strides[2] = {lhs->strides, rhs->strides};
-        const EwPlan p = plan_elementwise(out->data, out->shape, out->ndim, 2, datas, strides, es, false);
+        const EwPlan p = prepare_binary(lhs, rhs, out);
         if (p.kind == EwKind::Empty) return;
         use_device(dev);
         launch_binary(op, out->dtype, p, out->data, lhs->data, rhs->data, (hipStream_t)stream);
         check_launch("binary");
+    });
+}
+
+int32_t hpt_hip_binary_plan(const hpt_view* lhs, const hpt_view* rhs, const hpt_view* out, char* buf, size_t buflen) {
+    return guarded([&] {
+        if (!buf || !buflen) fail(HPT_ERR_PARAM, "binary_plan: no buffer");
+        snprintf(buf, buflen, "%s", describe(prepare_binary(lhs, rhs, out)).c_str());
     });
 }
 

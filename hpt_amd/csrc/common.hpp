@@ -179,7 +179,7 @@ void restrict_to_row_stream(NormPlan& p);
 enum class EwKind {
     Empty,
     Inner,      // lanes walk the innermost coalesced dim (vectors where every operand allows them)
-    Transpose   // copy only: some other dim is the contiguous one in the input: register-tile transpose
+    Transpose   // some other dim is the contiguous one in the input (a binary op: in one or both): tiles transposed in registers / LDS
 };
 
 // The output is contiguous over `size[0..n)`; `stride[k][i]` is operand k's stride (in
@@ -196,6 +196,7 @@ struct EwPlan {
     // Transpose: dim `tdim` has input stride 1; the innermost dim is strided in the input
     int tdim = -1;
     bool tile_lds = false;  // Transpose: both dims hold a whole (16 vec)^2 tile: staged through LDS
+    int tmask = 0;          // Transpose: bit k set = operand k is the one contiguous along `tdim` (a binary op may have one such operand or two)
 };
 
 EwPlan plan_elementwise(const void* out_data, const int64_t* shape, int ndim, int nin, const void* const* in_data,

@@ -282,6 +282,108 @@ __global__ void __launch_bounds__(256) ew_transpose_lds_kernel(const TransposeAr
     }
 }
 
+// ---- binary op with operands whose contiguous dim is not the innermost one -------------------
+// a + b.t(), a.t() * b.t() into a contiguous result: the same tiles as ew_transpose_lds_kernel. The
+// operands of MASK (bit k = operand k) are contiguous along B and come through LDS, transposed; an
+// operand outside MASK lies like the result (contiguous along A, or broadcast along it) and is read
+// by the lane that writes the result, at the very position when the result overwrites it in place.
+// (The lanes-along-the-innermost-dim kernel gathers such an operand element by element: f32
+// [8192, 4096] x.t() + y.t() 283 us.)
+struct TransposeBinArgs {
+    const void* in[2];
+    void* out;
+    int64_t sA[2];  // operand strides along A, the result's innermost dim (outside MASK: 1 or 0)
+    int64_t sB[2];  // operand strides along B (in MASK: 1)
+    int64_t oB;     // result stride along B
+    int nA, nB, ntA;
+    int nother;
+    int osize[kMaxDims];
+    int64_t oin[2][kMaxDims], oout[kMaxDims];  // strides of the other dims
+};
+
+template <int OP, class T, int MASK>
+__global__ void __launch_bounds__(256) ew_binary_transpose_kernel(const TransposeBinArgs a) {
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr int TB = 16 * VEC, TA = 16 * VEC;
+    constexpr int NTILE = (MASK & 1) + (MASK >> 1 & 1);
+    static_assert(NTILE >= 1 && NTILE * TB * 256 <= 64 * 1024, "LDS");
+    __shared__ __align__(16) unsigned char tile[NTILE][TB * 256];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    int64_t ioff[2] = {0, 0}, ooff = 0;
+    {
+        uint32_t q = blockIdx.z;
+        for (int i = a.nother - 1; i >= 0; --i) {
+            const uint32_t s = (uint32_t)a.osize[i];
+            const uint32_t q2 = q / s;
+            const uint32_t idx = q - q2 * s;
+            q = q2;
+            ioff[0] += (int64_t)idx * a.oin[0][i];
+            ioff[1] += (int64_t)idx * a.oin[1][i];
+            ooff += (int64_t)idx * a.oout[i];
+        }
+    }
+    const int tb = blockIdx.x / a.ntA, ta = blockIdx.x - tb * a.ntA;
+    const int B0 = tb * TB, A0 = ta * TA;
+    {
+        const int jb = lane & 15, ac = w * 4 + (lane >> 4);
+        const int b = B0 + jb * VEC, a0 = A0 + ac * VEC;
+        if (b < a.nB && a0 < a.nA) {
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                if (!(MASK >> k & 1)) continue;
+                constexpr int kFirst = MASK & 1 ? 0 : 1;
+                unsigned char* tl = tile[k == kFirst ? 0 : NTILE - 1];
+                const T* in = (const T*)a.in[k] + ioff[k] + (int64_t)a0 * a.sA[k] + b;
+                Pack<T, VEC> v[VEC];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) v[i] = load_pack_stream<T, VEC>(in + (int64_t)i * a.sA[k]);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    Pack<T, VEC> o;
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) o.v[i] = v[i].v[j];
+                    *(Pack<T, VEC>*)(tl + (jb * VEC + j) * 256 + ((ac ^ jb) << 4)) = o;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    {
+        const int ca = lane & 15, rl = w * 4 + (lane >> 4);
+        const int a0 = A0 + ca * VEC;
+        T* out = (T*)a.out + ooff + a0;
+#pragma unroll
+        for (int it = 0; it < VEC; ++it) {
+            const int row = it * 16 + rl;
+            const int b = B0 + row;
+            if (b < a.nB && a0 < a.nA) {
+                Pack<T, VEC> x[2];
+#pragma unroll
+                for (int k = 0; k < 2; ++k) {
+                    if (MASK >> k & 1) {
+                        constexpr int kFirst = MASK & 1 ? 0 : 1;
+                        const unsigned char* tl = tile[k == kFirst ? 0 : NTILE - 1];
+                        x[k] = *(const Pack<T, VEC>*)(tl + row * 256 + (((ca ^ (row / VEC)) & 15) << 4));
+                    } else {
+                        const T* in = (const T*)a.in[k] + ioff[k] + (int64_t)b * a.sB[k];
+                        if (a.sA[k] == 1) {
+                            x[k] = load_pack_stream<T, VEC>(in + a0);
+                        } else {  // broadcast along A
+                            const T e = *in;
+#pragma unroll
+                            for (int j = 0; j < VEC; ++j) x[k].v[j] = e;
+                        }
+                    }
+                }
+                Pack<T, VEC> o;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) o.v[j] = BinOp<OP, T>::apply(x[0].v[j], x[1].v[j]);
+                store_pack_stream<T, VEC>(out + (int64_t)b * a.oB, o);
+            }
+        }
+    }
+}
+
 // ---- dtype casts ----------------------------------------------------------------------
 // Scalar<T>::cast as astype uses it (hpt/src/backends/cuda/tensor_impls.rs:129-140): integers go
 // to a float type through Rust's `as` (round to nearest even; f16 / bf16 through f32, as the
@@ -433,11 +535,61 @@ template <class U> void launch_copy_sized(const EwPlan& p, void* out, const void
     else launch_inner<EW_COPY, U, 1>(p, out, in, nullptr, st);
 }
 
+template <int OP, class T>
+void launch_binary_transpose(const EwPlan& p, void* out, const void* a, const void* b, hipStream_t st) {
+    if constexpr (sizeof(T) >= 2) {
+        constexpr int VEC = 16 / sizeof(T);
+        TransposeBinArgs t{};
+        const int last = p.n - 1;
+        t.in[0] = a;
+        t.in[1] = b;
+        t.out = out;
+        t.nA = (int)p.size[last];
+        t.nB = (int)p.size[p.tdim];
+        int64_t ostride[kMaxDims];
+        int64_t acc = 1;
+        for (int i = last; i >= 0; --i) {
+            ostride[i] = acc;
+            acc *= p.size[i];
+        }
+        t.oB = ostride[p.tdim];
+        for (int k = 0; k < 2; ++k) {
+            t.sA[k] = p.stride[k][last];
+            t.sB[k] = p.stride[k][p.tdim];
+        }
+        int64_t others = 1;
+        for (int i = 0; i < p.n; ++i) {
+            if (i == p.tdim || i == last) continue;
+            t.osize[t.nother] = (int)p.size[i];
+            t.oin[0][t.nother] = p.stride[0][i];
+            t.oin[1][t.nother] = p.stride[1][i];
+            t.oout[t.nother] = ostride[i];
+            ++t.nother;
+            others *= p.size[i];
+        }
+        constexpr int TILE = 16 * VEC;
+        t.ntA = (t.nA + TILE - 1) / TILE;
+        const int64_t tiles = (int64_t)t.ntA * ((t.nB + TILE - 1) / TILE);
+        if (tiles > 0x7fffffff) fail(HPT_ERR_SHAPE, "binary: too many tiles for the transposing kernel");
+        const dim3 grid((unsigned)tiles, 1, (unsigned)others);
+        switch (p.tmask) {
+            case 1: ew_binary_transpose_kernel<OP, T, 1><<<grid, dim3(256), 0, st>>>(t); return;
+            case 2: ew_binary_transpose_kernel<OP, T, 2><<<grid, dim3(256), 0, st>>>(t); return;
+            case 3: ew_binary_transpose_kernel<OP, T, 3><<<grid, dim3(256), 0, st>>>(t); return;
+            default: break;
+        }
+    }
+    fail(HPT_ERR_KERNEL, "binary: no transposing kernel for this plan");
+}
+
 template <int OP> void launch_binary_op(int dtype, const EwPlan& p, void* out, const void* a, const void* b, hipStream_t st) {
     switch (dtype) {
 #define HPT_CASE(DT)                                                                 \
     case DT:                                                                         \
-        launch_inner<OP, typename DType<DT>::type, 2>(p, out, a, b, st);             \
+        if (p.kind == EwKind::Transpose)                                             \
+            launch_binary_transpose<OP, typename DType<DT>::type>(p, out, a, b, st); \
+        else                                                                         \
+            launch_inner<OP, typename DType<DT>::type, 2>(p, out, a, b, st);         \
         return;
         HPT_CASE(HPT_I8) HPT_CASE(HPT_I16) HPT_CASE(HPT_I32) HPT_CASE(HPT_I64) HPT_CASE(HPT_U8) HPT_CASE(HPT_U16)
         HPT_CASE(HPT_U32) HPT_CASE(HPT_U64) HPT_CASE(HPT_F16) HPT_CASE(HPT_BF16) HPT_CASE(HPT_F32) HPT_CASE(HPT_F64)

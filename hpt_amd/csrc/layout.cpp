@@ -1143,7 +1143,44 @@ EwPlan plan_elementwise(const void* out_data, const int64_t* shape, int ndim, in
                 p.kind = EwKind::Transpose;
                 p.vec = full;
                 p.tdim = t;
+                p.tmask = 1;
                 p.tile_lds = p.size[last] >= 16 * full && p.size[t] >= 16 * full;
+            }
+        }
+    }
+    // binary op with an operand (or both) whose contiguous dim is not the innermost one (a + b.t()): whole
+    // tiles of those operands are transposed through LDS; an operand in the output's own layout (or
+    // broadcast along the innermost dim) is read as the result is written
+    if (allow_transpose && nin == 2 && full > 1 && full <= 8 && p.n <= 6) {
+        int mask = 0;
+        for (int k = 0; k < 2; ++k)
+            if (p.stride[k][last] != 1 && p.stride[k][last] != 0) mask |= 1 << k;
+        int t = -1;
+        for (int i = 0; i < last && mask; ++i) {
+            bool all = true;
+            for (int k = 0; k < 2; ++k)
+                if ((mask >> k & 1) && p.stride[k][i] != 1) all = false;
+            if (all) t = i;
+        }
+        if (t >= 0) {
+            bool ok = aligned(out_data) && p.size[last] % full == 0 && p.size[t] % full == 0 && p.size[last] >= 16 * full &&
+                      p.size[t] >= 16 * full && p.size[last] <= (1 << 30) && p.size[t] <= (1 << 30);
+            for (int k = 0; k < 2 && ok; ++k) {
+                const bool transposed = mask >> k & 1;
+                if (!transposed && p.stride[k][last] == 0) continue;  // single elements, splat
+                if (!aligned(in_data[k])) ok = false;
+                for (int i = 0; i < p.n; ++i)
+                    if (i != (transposed ? t : last) && p.stride[k][i] % full != 0) ok = false;
+            }
+            int64_t others = 1;
+            for (int i = 0; i < p.n; ++i)
+                if (i != t && i != last) others *= p.size[i];
+            if (ok && others <= 65535) {
+                p.kind = EwKind::Transpose;
+                p.vec = full;
+                p.tdim = t;
+                p.tmask = mask;
+                p.tile_lds = true;
             }
         }
     }
@@ -1166,7 +1203,8 @@ std::string describe(const EwPlan& p) {
     }
     s += "]";
     if (p.kind == EwKind::Transpose) {
-        snprintf(buf, sizeof buf, " tdim=%d%s", p.tdim, p.tile_lds ? " lds" : "");
+        snprintf(buf, sizeof buf, " tdim=%d%s%s", p.tdim, p.nin == 2 ? (p.tmask == 3 ? " both" : p.tmask == 1 ? " lhs" : " rhs") : "",
+                 p.tile_lds ? " lds" : "");
         s += buf;
     }
     return s;

@@ -756,6 +756,18 @@ def contiguous_plan(t: Tensor) -> str:
     return buf.value.decode()
 
 
+def binary_plan(lhs: Tensor, rhs: Tensor) -> str:
+    """The kernel `lhs.add(rhs)` (any of the four operators) would use, for operands already expanded to one
+    shape (no device needed; the output is assumed 16-byte aligned)."""
+    va, k1 = lhs._c_view()
+    vb, k2 = rhs._c_view()
+    out, k3 = make_view(4096, lhs.shape, _contiguous_strides(lhs.shape), lhs.dtype.code)
+    buf = C.create_string_buffer(512)
+    check(_ffi.lib().hpt_hip_binary_plan(C.byref(va), C.byref(vb), C.byref(out), buf, 512))
+    del k1, k2, k3
+    return buf.value.decode()
+
+
 def normalize_plan(t: Tensor, axis: int = 0, n_norm_dims: int = 0) -> str:
     v, k = t._c_view()
     buf = C.create_string_buffer(512)

@@ -298,9 +298,13 @@ typedef enum hpt_binary_op { HPT_BIN_ADD = 0, HPT_BIN_SUB = 1, HPT_BIN_MUL = 2, 
  * `add_` / `mul_` that layernorm's single-affine branches call
  * (hpt/src/backends/cpu/tensor_internal/normalization.rs:187-192). Integers wrap; bool
  * add is OR and mul is AND (sub / div undefined); div is for float dtypes (Hpt's
- * integer division changes the dtype). f16 / bf16 compute in f32 and round once. */
+ * integer division changes the dtype). f16 / bf16 compute in f32 and round once.
+ * An operand whose contiguous dim is not the innermost one (`b.t()`) is transposed
+ * tile by tile inside the kernel; no operand is copied first. */
 int32_t hpt_hip_binary(int32_t dev, void* stream, int32_t op, const hpt_view* lhs, const hpt_view* rhs,
                        hpt_view* out);
+/* Describes the kernel hpt_hip_binary would pick (tests, tuning). */
+int32_t hpt_hip_binary_plan(const hpt_view* lhs, const hpt_view* rhs, const hpt_view* out, char* buf, size_t buflen);
 
 #ifdef __cplusplus
 }

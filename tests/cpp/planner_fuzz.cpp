@@ -78,6 +78,7 @@ static View random_view(size_t elem, int64_t budget, bool allow_zero, bool allow
 }
 
 static int failures = 0;
+static long seen_transposed_binary = 0, seen_lds_rows = 0;
 #define CHECK(cond, ...)                       \
     do {                                       \
         if (!(cond)) {                         \
@@ -184,6 +185,7 @@ static void fuzz_normalize() {
             CHECK(slots >= cols * p.sstride || p.shift, "%s plan=%s", show(v).c_str(), d.c_str());
         }
         if (p.kind == NormKind::RowReg && p.lds_rows) {
+            ++seen_lds_rows;
             // the register + LDS kernel's vector grid may start up to a 128-byte line before the row
             const int64_t line = 128 / (int64_t)elem;
             const int64_t grid = (cols + (p.shift ? line - 1 : 0) + p.vec - 1) / p.vec;
@@ -220,13 +222,24 @@ static void fuzz_elementwise() {
             }
         }
         b.base = 0x7d0000000000ull + (uintptr_t)uni(0, 64) * elem;
+        if (uni(0, 2) == 0 && ndim >= 2) {  // the second operand contiguous along another dim than the last
+            const int t = (int)uni(0, ndim - 2);
+            int64_t run = a.shape[t];
+            b.strides[t] = 1;
+            for (int i = ndim - 1; i >= 0; --i) {
+                if (i == t) continue;
+                b.strides[i] = run;
+                run *= a.shape[i];
+            }
+            if (uni(0, 1)) b.base -= b.base % 16;
+        }
     }
     const void* in_data[2] = {(const void*)a.base, (const void*)b.base};
     const int64_t* in_strides[2] = {a.strides.data(), b.strides.data()};
     const uintptr_t out = 0x7c0000000000ull + (uintptr_t)uni(0, 1 << 20) * 256;
     try {
         EwPlan p = plan_elementwise((const void*)out, a.shape.data(), ndim, nin, in_data, in_strides, elem,
-                                    nin == 1 && uni(0, 3) != 0);
+                                    nin >= 1 && uni(0, 3) != 0);
         const std::string d = describe(p);
         const int64_t total = a.total();
         if (p.kind == EwKind::Empty) {
@@ -238,9 +251,18 @@ static void fuzz_elementwise() {
         CHECK(p.total == total && t == total, "%s plan=%s", show(a).c_str(), d.c_str());
         CHECK(p.n >= 1 && p.n <= kMaxDims && p.nin == nin, "%s plan=%s", show(a).c_str(), d.c_str());
         CHECK(pow2(p.vec) && (size_t)p.vec * elem <= 16, "%s plan=%s", show(a).c_str(), d.c_str());
-        if (p.kind == EwKind::Transpose)
-            CHECK(p.tdim >= 0 && p.tdim < p.n - 1 && p.stride[0][p.tdim] == 1, "%s plan=%s", show(a).c_str(),
+        if (p.kind == EwKind::Transpose) {
+            seen_transposed_binary += nin == 2;
+            CHECK(p.tdim >= 0 && p.tdim < p.n - 1 && p.tmask >= 1 && p.tmask < (1 << nin), "%s plan=%s", show(a).c_str(),
                   d.c_str());
+            for (int k = 0; k < nin; ++k) {
+                // an operand is contiguous along the transposed dim, or along the innermost one (or broadcast there)
+                const int64_t s_last = p.stride[k][p.n - 1];
+                CHECK((p.tmask >> k & 1) ? p.stride[k][p.tdim] == 1 : (s_last == 1 || s_last == 0), "%s plan=%s",
+                      show(a).c_str(), d.c_str());
+            }
+            CHECK(p.size[p.n - 1] % p.vec == 0 && p.size[p.tdim] % p.vec == 0, "%s plan=%s", show(a).c_str(), d.c_str());
+        }
         if (p.kind == EwKind::Inner && p.vec > 1)
             CHECK(p.size[p.n - 1] % p.vec == 0, "%s plan=%s", show(a).c_str(), d.c_str());
     } catch (const Error&) {
@@ -256,6 +278,7 @@ int main(int argc, char** argv) {
         fuzz_elementwise();
         if (failures > 20) break;
     }
-    std::printf("planner_fuzz: %ld iterations, %d failures\n", iters, failures);
+    std::printf("planner_fuzz: %ld iterations, %d failures (%ld transposing binary plans, %ld register + LDS row plans)\n", iters,
+                failures, seen_transposed_binary, seen_lds_rows);
     return failures ? 1 : 0;
 }

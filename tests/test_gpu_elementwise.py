@@ -25,6 +25,7 @@ def rand(rng, shape, npdt):
 
 def same_bits(got, want, msg):
     assert got.shape == want.shape and got.dtype == want.dtype, msg
+    got, want = np.ascontiguousarray(got), np.ascontiguousarray(want)
     assert np.array_equal(got.view(np.uint8) if got.size else got, want.view(np.uint8) if want.size else want), msg
 
 
@@ -190,6 +191,90 @@ def test_binary_strided_operands_inplace_and_bf16(hpt, dev):
         ta.add(hpt.Tensor.from_numpy(np.zeros([48, 80], np.float64)).to_hip(dev))
     with pytest.raises(hpt.ShapeError):
         ta.add(hpt.Tensor.from_numpy(np.zeros([48, 81], np.float32)).to_hip(dev))
+
+
+TRANSPOSED_OPERAND_CASES = [
+    # (dtype, shape of the result, which operands are permuted views, the permutation)
+    ("f32 a + b.t()", np.float32, [264, 136], "rhs", (1, 0)),
+    ("f32 a.t() - b", np.float32, [264, 136], "lhs", (1, 0)),
+    ("f32 a.t() * b.t()", np.float32, [200, 328], "both", (1, 0)),
+    ("f16 both, tiles of 128", np.float16, [264, 392], "both", (1, 0)),
+    ("f16 rhs", np.float16, [520, 136], "rhs", (1, 0)),
+    ("f64", np.float64, [72, 104], "both", (1, 0)),
+    ("i32 wraps", np.int32, [136, 200], "rhs", (1, 0)),
+    ("u16", np.uint16, [264, 136], "lhs", (1, 0)),
+    ("i64", np.int64, [40, 72], "both", (1, 0)),
+    ("f32 3-D, batch outermost", np.float32, [5, 136, 72], "rhs", (0, 2, 1)),
+    ("f32 3-D, the batch dim between", np.float32, [72, 3, 136], "both", (2, 1, 0)),
+    ("f16 4-D", np.float16, [2, 3, 136, 264], "lhs", (0, 1, 3, 2)),
+]
+
+
+@pytest.mark.parametrize("case", TRANSPOSED_OPERAND_CASES, ids=[c[0] for c in TRANSPOSED_OPERAND_CASES])
+def test_binary_with_transposed_operands(hpt, dev, case):
+    """An operand whose contiguous dim is not the innermost one (a + b.t()) is transposed tile by tile
+    through LDS inside the binary kernel; the other operand may lie like the result, be transposed too,
+    or be broadcast; the result may overwrite an operand that lies like it."""
+    name, npdt, shape, which, perm = case
+    rng = np.random.default_rng(330)
+    inv = list(np.argsort(perm))
+    pshape = [shape[i] for i in inv]  # parent shape whose permutation by `perm` is `shape`
+
+    def operand(transposed):
+        if transposed:
+            base = rand(rng, pshape, npdt)
+            return base.transpose(perm), hpt.Tensor.from_numpy(base).to_hip(dev).permute(list(perm))
+        base = rand(rng, shape, npdt)
+        return base, hpt.Tensor.from_numpy(base).to_hip(dev)
+
+    a, ta = operand(which in ("lhs", "both"))
+    b, tb = operand(which in ("rhs", "both"))
+    if np.dtype(npdt).kind == "f":
+        b = np.where(np.abs(b) < 0.25, npdt(1.0), b)
+        tb = hpt.Tensor.from_numpy(np.ascontiguousarray(b.transpose(inv) if which in ("rhs", "both") else b)).to_hip(dev)
+        if which in ("rhs", "both"):
+            tb = tb.permute(list(perm))
+    plan = hpt.binary_plan(ta, tb)
+    assert plan.startswith("transpose") and plan.endswith(f"{which} lds"), plan
+    for opname, op in OPS:
+        if op == ew.DIV and np.dtype(npdt).kind != "f":
+            continue
+        same_bits(getattr(ta, opname)(tb).numpy(), ew.binary(op, a, b), f"{opname} {name}")
+    # broadcast partners of a transposed operand: a row, a column, a scalar
+    if which != "both" and len(shape) == 2:
+        t_op, n_np = (ta, a) if which == "lhs" else (tb, b)
+        for bshape in ([shape[1]], [shape[0], 1], [1]):
+            o = rand(rng, bshape, npdt)
+            to = hpt.Tensor.from_numpy(o).to_hip(dev)
+            assert hpt.binary_plan(t_op, to.expand(shape)).startswith("transpose"), hpt.binary_plan(t_op, to.expand(shape))
+            same_bits(t_op.mul(to).numpy(), ew.binary(ew.MUL, n_np, o), f"mul by a broadcast {bshape} {name}")
+            same_bits(to.sub(t_op).numpy(), ew.binary(ew.SUB, o, n_np), f"broadcast {bshape} minus {name}")
+    # in place over the operand that lies like the result
+    if which == "rhs":
+        res = hpt.Tensor.from_numpy(np.ascontiguousarray(a)).to_hip(dev)
+        assert res.add_(tb, res) is res
+        same_bits(res.numpy(), ew.binary(ew.ADD, a, b), f"add_ in place {name}")
+
+
+def test_binary_transposed_operands_large_and_refusals(hpt, dev):
+    rng = np.random.default_rng(331)
+    a = rand(rng, [2048, 3072], np.float32)
+    b = rand(rng, [3072, 2048], np.float32)
+    ta, tb = hpt.Tensor.from_numpy(a).to_hip(dev), hpt.Tensor.from_numpy(b).to_hip(dev)
+    same_bits(ta.add(tb.permute([1, 0])).numpy(), a + b.T, "f32 [2048, 3072] a + b.t()")
+    same_bits(ta.permute([1, 0]).mul(tb).numpy(), a.T * b, "f32 [3072, 2048] a.t() * b")
+    # one-byte types, short dims and unaligned views keep the gathering kernel
+    u = hpt.Tensor.from_numpy(rand(rng, [512, 256], np.uint8)).to_hip(dev)
+    assert hpt.binary_plan(u.permute([1, 0]), u.permute([1, 0])).startswith("inner")
+    s = hpt.Tensor.from_numpy(rand(rng, [48, 80], np.float32)).to_hip(dev)
+    assert hpt.binary_plan(s, hpt.Tensor.from_numpy(rand(rng, [80, 48], np.float32)).to_hip(dev).permute([1, 0])).startswith("inner")
+    odd = ta[:, 1:2049]  # rows start off the 16-byte grid
+    assert hpt.binary_plan(odd, tb.permute([1, 0])[:, :2048]).startswith("inner")
+    same_bits(odd.add(tb.permute([1, 0])[:, :2048]).numpy(), a[:, 1:2049] + b.T[:, :2048], "unaligned partner")
+    # an output that overlaps the transposed operand without being it is refused
+    sq = hpt.Tensor.from_numpy(rand(rng, [256, 256], np.float32)).to_hip(dev)
+    with pytest.raises(hpt.ParamError):
+        sq.permute([1, 0]).add_(sq, sq)
 
 
 def test_layernorm_equals_normalise_then_affine_steps(hpt, orc, dev):
