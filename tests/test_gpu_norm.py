@@ -709,3 +709,45 @@ def test_half_rows_of_millions_of_elements_against_the_f64_truth(hpt, orc, dev):
         got = tof(t.softmax(3).numpy())
         want = tof(orc.softmax(a, 3, acc=orc.ACC_F32, dtype=odt))
         assert_close(got, want, HALF_RTOL, max(half_atol(want, bits), 6e-8), f"softmax(3), {bits} bits")
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_long_rows_of_random_length_and_alignment(hpt, orc, dev, seed):
+    """softmax / log_softmax over rows of 2049 ... 50000 vectors whose length, row pitch and first element
+    are drawn at random: windows [r0:, c0:c1] of a parent matrix, so rows start anywhere on the 16-byte
+    grid or off it, input and output rows are misaligned alike or not, and every plan of such rows is
+    reached: registers + LDS (aligned and shifted, 256 and 512 threads), the raw-row kernel, the
+    streaming kernel (aligned, shifted, element-wise)."""
+    rng = np.random.default_rng(4200 + seed)
+    seen = set()
+    for it in range(14):
+        kind = ("f32", "f16", "bf16")[int(rng.integers(0, 3))]
+        vec = 4 if kind == "f32" else 8
+        cols = int(rng.integers(2049 * vec, 50000 * vec // (2 if kind == "f32" else 3)))
+        if rng.integers(0, 3) == 0:
+            cols -= cols % vec                      # whole vectors
+        rows = int(rng.integers(129, 150))     # (fewer rows are shared among workgroups: another plan)
+        lead, tail = (int(rng.integers(0, 2 * vec)) if rng.integers(0, 2) else 0 for _ in range(2))
+        if rng.integers(0, 3) == 0:
+            tail += -(lead + cols + tail) % vec    # a pitch of whole vectors: every row misaligned alike
+        x = (rng.standard_normal((rows + 1, lead + cols + tail)) * 2).astype(np.float32)
+        if kind == "bf16":
+            a, dt, odt, bits, tof = hpt.f32_to_bf16_bits(x), hpt.bf16, orc.BF16, 8, hpt.bf16_bits_to_f32
+        elif kind == "f16":
+            a, dt, odt, bits, tof = x.astype(np.float16), None, None, 11, (lambda v: v.astype(np.float32))
+        else:
+            a, dt, odt, bits, tof = x, None, None, 0, (lambda v: v)
+        t = hpt.Tensor.from_numpy(a, dt).to_hip(dev)[1:, lead:lead + cols]
+        view = a[1:, lead:lead + cols]
+        plan = hpt.normalize_plan(t, 1).split(" ")[0]
+        seen.add(plan)
+        what = f"seed={seed} case={it} {kind} rows={rows} cols={cols} lead={lead} pitch={a.shape[1]} plan={plan}"
+        acc = orc.ACC_F32 if bits else orc.ACC_F64
+        for log in (False, True):
+            got = tof((t.log_softmax(1) if log else t.softmax(1)).numpy())
+            want = tof(orc.softmax(view, 1, log=log, acc=acc, dtype=odt))
+            if bits:
+                assert_close(got, want, HALF_RTOL, max(half_atol(want[np.isfinite(want)], bits), 6e-8), f"log={log} {what}")
+            else:
+                assert_close(got, want, F32_RTOL, 2 * F32_ATOL if log else F32_ATOL, f"log={log} {what}")
+    assert any(p.startswith("rowreg-lds") for p in seen), seen
