@@ -484,17 +484,21 @@ std::string describe(const ReducePlan& p) {
 // Softmax rows held in registers and LDS (row_lds_kernel): the smallest of its three launch shapes whose
 // slots hold the `nvec` vectors of a row's vector grid; false when none does. 24 + 8 vectors of a four-byte
 // type (16 + 8 of a two-byte type) per thread, 256 or 512 threads; twice that per thread, 512 threads.
-static bool lds_row_shape(NormPlan& p, int64_t nvec, size_t elem_size) {
-    const int per = elem_size == 4 ? 32 : 24;
+// Shifted four-byte rows keep four vectors fewer in registers (20 + 8, 44 + 16): the masks of the row ends
+// beside 24 or 48 vectors spilled 30 registers, and the spills' traffic showed in the HBM counters (f32
+// [640, 50257]: 1.22 times the algorithmic bytes; the aligned [640, 50304]: 1.00).
+static bool lds_row_shape(NormPlan& p, int64_t nvec, size_t elem_size, bool shift) {
+    const int per = elem_size == 4 ? (shift ? 28 : 32) : 24;
+    const int big = elem_size == 4 ? (shift ? 60 : 64) : 48;
     if (nvec <= 256 * per) {
         p.tpr = 256;
         p.nchunk = per;
     } else if (nvec <= 512 * per) {
         p.tpr = 512;
         p.nchunk = per;
-    } else if (nvec <= 512 * 2 * per) {
+    } else if (nvec <= 512 * big) {
         p.tpr = 512;
-        p.nchunk = 2 * per;
+        p.nchunk = big;
     } else {
         return false;
     }
@@ -662,11 +666,11 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 // vectors, 512 threads; f16 [8190, 4097] 1.9 -> 2.2 TB/s, [5461, 6145] 1.9 -> 2.8 against streaming)
                 // Softmax rows beyond the register kernel's 2048 shifted vectors stay on chip in registers and
                 // LDS (row_lds_kernel, whose vector grid starts on the 128-byte line that holds the row's first
-                // element) up to 131038 four-byte or 196538 two-byte elements; they streamed before (two reads).
-                // Measured (TB/s): f32 [4096, 30522] 3.5 -> , [2048, 50257] 4.45 -> 4.8, [1024, 100277] 3.7 -> 4.3;
-                // f16 [8192, 32001] 4.0 -> , [4096, 50257] 4.35 -> 5.2, [2048, 98001] 4.2 -> 4.9.
+                // element) up to 122846 four-byte or 196545 two-byte elements; they streamed before (two reads).
+                // Measured (TB/s): f32 [4096, 30522] 3.5 -> 5.55, [2048, 50257] 4.45 -> 5.3, [1024, 100277] 3.7 -> 4.55;
+                // f16 [8192, 32001] 4.0 -> 5.55, [4096, 50257] 4.35 -> 5.2, [2048, 98001] 4.2 -> 4.9.
                 if (same && n_norm_dims <= 0 && nvs > 2048 && (elem_size == 2 || elem_size == 4) &&
-                    lds_row_shape(p, (p.cols + 128 / (int64_t)elem_size + max_vec - 2) / max_vec, elem_size)) {
+                    lds_row_shape(p, (p.cols + 128 / (int64_t)elem_size + max_vec - 2) / max_vec, elem_size, true)) {
                     p.vec = max_vec;
                     p.shift = 1;
                     return p;
@@ -749,7 +753,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 }
                 // (the causal softmax has no such kernel: its rows stay with the register kernel while they fit)
                 if ((elem_size == 4 ? nv > 8192 : elem_size == 2 && nv > 4096) && !(fused && nv <= reg_limit) &&
-                    lds_row_shape(p, nv, elem_size))
+                    lds_row_shape(p, nv, elem_size, false))
                     return p;
             }
             if (nv <= reg_limit) {
@@ -841,7 +845,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     // Measured (TB/s): f32 [4096, 16388] 4.8 -> 5.15; f16 [8192, 16392] 4.2 -> 5.45. (Full rows
                     // gain nothing: f32 [4096, 32768] 5.55 -> 5.55, f16 [8192, 32768] 5.75 -> 5.35.)
                     if (n_norm_dims <= 0 && !fused && !p.shift && nv > (elem_size == 2 ? 1024 : 2048) && (elem_size == 2 || elem_size == 4) &&
-                        (int64_t)p.tpr * p.nchunk - nv >= nv / 16 && lds_row_shape(p, nv, elem_size))
+                        (int64_t)p.tpr * p.nchunk - nv >= nv / 16 && lds_row_shape(p, nv, elem_size, false))
                         return p;
                 }
                 int block = std::max(256, p.tpr);

@@ -458,7 +458,8 @@ __global__ void __launch_bounds__(1024) row_raw_kernel(const NormArgs a) {
 // Shapes: NT = 256 or 512 threads with 24 + 8 vectors of a four-byte type (16 + 8 of a two-byte type)
 // and 128 registers each, so that two (512) or four (256) workgroups share a compute unit and one's
 // arithmetic overlaps the other's loads and stores; NT = 512 with 48 + 16 (32 + 16) vectors and 256
-// registers each for the longest rows, one workgroup per compute unit.
+// registers each for the longest rows, one workgroup per compute unit. (Shifted four-byte rows: 20 + 8
+// and 44 + 16, which leaves the row-end masks their registers.)
 // Four-byte types: the summing sweep overwrites the held row with exp(x - max) (softmax) or x - max
 // (log_softmax), so the exponential is taken once per element either way. Two-byte types keep the
 // raw row (rounding the intermediate to 16 bits would cost accuracy) and take the exponential twice.

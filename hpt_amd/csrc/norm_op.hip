@@ -271,22 +271,37 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         // long rows that stay on chip: registers + LDS; the fused kinds stream
         if constexpr (FULL > 1 && sizeof(T) <= 4 && (KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX)) {
             // 24 + 8 vectors of a four-byte type (16 + 8 of a two-byte type) per thread and 128 registers:
-            // 256 or 512 threads; 48 + 16 (32 + 16) and 256 registers: 512 threads
+            // 256 or 512 threads; 48 + 16 (32 + 16) and 256 registers: 512 threads. Shifted four-byte rows:
+            // 20 + 8 and 44 + 16.
             constexpr int kRegs = sizeof(T) == 4 ? 24 : 16;
-            if (p.nchunk == kRegs + 8 && p.tpr == 256) {
-                if (p.shift) row_lds_kernel<KIND, T, kRegs, 8, true, 256, 4><<<grid, dim3(256), 0, st>>>(a);
-                else row_lds_kernel<KIND, T, kRegs, 8, false, 256, 4><<<grid, dim3(256), 0, st>>>(a);
-                return;
-            }
-            if (p.nchunk == kRegs + 8 && p.tpr == 512) {
-                if (p.shift) row_lds_kernel<KIND, T, kRegs, 8, true, 512, 4><<<grid, dim3(512), 0, st>>>(a);
-                else row_lds_kernel<KIND, T, kRegs, 8, false, 512, 4><<<grid, dim3(512), 0, st>>>(a);
-                return;
-            }
-            if (p.nchunk == 2 * kRegs + 16 && p.tpr == 512) {
-                if (p.shift) row_lds_kernel<KIND, T, 2 * kRegs, 16, true, 512, 1><<<grid, dim3(512), 0, st>>>(a);
-                else row_lds_kernel<KIND, T, 2 * kRegs, 16, false, 512, 1><<<grid, dim3(512), 0, st>>>(a);
-                return;
+            constexpr int kRegsShift = sizeof(T) == 4 ? 20 : 16;
+            constexpr int kBigShift = sizeof(T) == 4 ? 44 : 32;
+            if (!p.shift) {
+                if (p.nchunk == kRegs + 8 && p.tpr == 256) {
+                    row_lds_kernel<KIND, T, kRegs, 8, false, 256, 4><<<grid, dim3(256), 0, st>>>(a);
+                    return;
+                }
+                if (p.nchunk == kRegs + 8 && p.tpr == 512) {
+                    row_lds_kernel<KIND, T, kRegs, 8, false, 512, 4><<<grid, dim3(512), 0, st>>>(a);
+                    return;
+                }
+                if (p.nchunk == 2 * kRegs + 16 && p.tpr == 512) {
+                    row_lds_kernel<KIND, T, 2 * kRegs, 16, false, 512, 1><<<grid, dim3(512), 0, st>>>(a);
+                    return;
+                }
+            } else {
+                if (p.nchunk == kRegsShift + 8 && p.tpr == 256) {
+                    row_lds_kernel<KIND, T, kRegsShift, 8, true, 256, 4><<<grid, dim3(256), 0, st>>>(a);
+                    return;
+                }
+                if (p.nchunk == kRegsShift + 8 && p.tpr == 512) {
+                    row_lds_kernel<KIND, T, kRegsShift, 8, true, 512, 4><<<grid, dim3(512), 0, st>>>(a);
+                    return;
+                }
+                if (p.nchunk == kBigShift + 16 && p.tpr == 512) {
+                    row_lds_kernel<KIND, T, kBigShift, 16, true, 512, 1><<<grid, dim3(512), 0, st>>>(a);
+                    return;
+                }
             }
             fail(HPT_ERR_KERNEL, "row_lds: no kernel for %d threads x %d vectors", p.tpr, p.nchunk);
         }

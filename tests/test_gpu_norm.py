@@ -369,7 +369,7 @@ WIDE_ROW_CASES = [
     ("f32 rows of 131072: every slot in use", np.float32, [70, 131072]),
     ("f32 rows of 98308: the first LDS slots only", np.float32, [131, 98308]),
     ("f32 rows of 100277: shifted", np.float32, [261, 100277]),
-    ("f32 rows of 131041: the longest shifted f32 row on chip", np.float32, [67, 131041]),
+    ("f32 rows of 122849: the longest shifted f32 row on chip", np.float32, [67, 122849]),
     ("f16 rows of 151936: registers and LDS-direct loads", np.float16, [263, 151936]),
     ("bf16 rows of 196608: every slot in use", "bf16", [70, 196608]),
     ("bf16 rows of 131080: one vector beyond the raw-row kernel", "bf16", [131, 131080]),
@@ -378,10 +378,10 @@ WIDE_ROW_CASES = [
     ("f16 rows of 196610: streamed", np.float16, [35, 196610]),
     # the same kernel with 256 threads: odd lengths beyond 2048 vectors, and aligned rows that would leave
     # a sixteenth of a power-of-two row's slots idle
-    ("f32 rows of 30522: shifted, 256 threads", np.float32, [1300, 30522]),
+    ("f32 rows of 30522: shifted, 512 threads", np.float32, [1300, 30522]),
     ("f32 rows of 8197: the shortest such row", np.float32, [2100, 8197]),
-    ("f32 rows of 32733: the longest shifted row of 256 threads", np.float32, [530, 32733]),
-    ("f32 rows of 32737: shifted, 512 threads", np.float32, [530, 32737]),
+    ("f32 rows of 28641: the longest shifted row of 256 threads", np.float32, [530, 28641]),
+    ("f32 rows of 28645: shifted, 512 threads", np.float32, [530, 28645]),
     ("f32 rows of 16388: 256 threads", np.float32, [1100, 16388]),
     ("f16 rows of 32001: shifted, 256 threads", np.float16, [1100, 32001]),
     ("bf16 rows of 16392: 256 threads", "bf16", [1500, 16392]),
