@@ -10,23 +10,26 @@ the timed region starts; successive steps rotate over several input/output buffe
 that the working set is far larger than the 256 MB Infinity Cache and every step streams
 from HBM.
 
-Prints ONE JSON line. `value` is algorithmic GB/s (every logical input element read once +
-every output element written once + gamma/beta once, per step) over the wall-clock time of
-exactly K steps. `roofline.achieved` uses the same bytes over the kernel's average duration
-measured with HIP events on the launch stream; `roofline.kernel`, `traffic` and the profiler's
-own duration come from profiles/headline.json (written when the rocprofv3 summaries under
-profiles/ are regenerated), and the plan the library reports for the headline call is printed
-beside the plan recorded there, so a planner change that makes the profile stale shows.
+Prints ONE short JSON line (under 4 KB) on stdout. `value` is algorithmic GB/s (every logical input element
+read once + every output element written once + gamma/beta once, per step) over the wall-clock time of
+exactly K steps. `roofline.achieved` uses the same bytes over the kernel's average duration measured
+with HIP events on the launch stream; `roofline.kernel`, `traffic` and the profiler's own duration come
+from profiles/headline.json (written when the rocprofv3 summaries under profiles/ are regenerated), and
+`profile_matches_plan` says whether the plan the library reports for the headline call is the plan
+recorded there. `configs_pct_of_hbm_peak` carries one figure per op of the five benchmark
+configurations, `reference_shapes_pct_of_hbm_peak` one per shape / axis set of the reference's own
+published benchmarks.
 
-`ops` lists every op of the five benchmark configurations (and the groups c6-c10), each timed
-the same way whatever --steps says: 10 warm-up launches, then 13 groups of 8 back-to-back
-launches, every group bracketed by a pair of HIP events; `us_per_launch` is the median over the
-groups of (group time / 8) - 104 timed launches. (Bracketing every single launch instead adds
-about 3 us of event handling per launch, which is a sixth of a 17 us reduction.) Where the
-restated Hpt CPU path has the op (contiguous f32 rows: softmax, log_softmax, layernorm, sum, max)
-it is timed on this box's host cores and reported beside it as `cpu_GBps`.
-`cpu_baseline` is the headline's: the CPU restatement of Hpt's layernorm (oracle/, test
-infrastructure).
+The full per-op table (every op of the five configurations, of the reference's published shapes and of
+the groups c6-c10) goes to stderr and, as JSON, to the file `--ops-file` names (bench_ops.json). Every
+op is timed the same way whatever --steps says: 10 warm-up launches, then 13 groups of 8 back-to-back
+launches, every group bracketed by a pair of HIP events; `us_per_launch` is the median over the groups
+of (group time / 8) - 104 timed launches. (Bracketing every single launch instead adds about 3 us of
+event handling per launch, which is a sixth of a 17 us reduction.) Where the restated Hpt CPU path has
+the op (contiguous f32 rows: softmax, log_softmax, layernorm, sum, max) it is timed on this box's host
+cores and reported beside it as `cpu_GBps`; the half-precision ops of C4 / C5 also report their distance
+to the oracle's per-op-rounded restatement of the CPU result on a sample of rows (informational).
+`cpu_baseline` is the headline's: the CPU restatement of Hpt's layernorm (oracle/, test infrastructure).
 
 Two side modes print a table instead of the JSON line: `--sweep f32,f16` (achieved TB/s of seven ops
 over [N, C] shapes from C = 3 to C = 2^20) and `--host-time` (host time per call of the selected ops).
@@ -95,11 +98,16 @@ def gen_c2(seed=1):
 class Case:
     """One op on one configuration: `run(i)` enqueues one step on buffer set i % nbuf."""
 
-    def __init__(self, name, cfg, dtype, rows, algo_bytes, run, nbuf, check=None, plan=None, cpu=None):
+    def __init__(self, name, cfg, dtype, rows, algo_bytes, run, nbuf, check=None, plan=None, cpu=None, key=None,
+                 native=None):
         self.name, self.cfg, self.dtype, self.rows = name, cfg, dtype, rows
         self.bytes, self.run, self.nbuf, self.check = algo_bytes, run, nbuf, check
         self.plan = plan  # what the library's planner says it launches for this call
         self.cpu = cpu    # () -> seconds per pass of the restated Hpt CPU path on the same input, or None
+        self.key = key    # short name under which the op's % of peak goes into the one-line summary, or None
+        # () -> {"max_rel", "p99_rel", "sample"}: distance of the device result to the literal CPU semantics
+        # (every operation rounded to the half type) on a sample of rows; informational
+        self.native = native
 
 
 def time_case(ev: HipEvents, case: Case, steps: int, warmup: int):
@@ -151,17 +159,37 @@ def cpu_seconds(fn, budget_s=1.5, min_passes=3, max_passes=200):
 
 def cpu_rows(op, x):
     """The restated Hpt CPU path for a row op on the contiguous f32 matrix `x`: a callable that runs one
-    pass on this box's physical cores (rows split as Hpt's thread pool splits them)."""
+    pass on this box's physical cores (rows split as Hpt's thread pool splits them). Successive passes
+    rotate over copies of `x` that together exceed 512 MB, so that no pass is served from the host's
+    last-level caches (the device side rotates its buffers for the same reason)."""
     def call():
         from oracle import oracle as orc
         cores = orc.physical_cores()
+        copies = [x] + [x.copy() for _ in range(min(7, (512 << 20) // max(1, x.nbytes)))]
+        turn = [0]
+
+        def nxt():
+            turn[0] += 1
+            return copies[turn[0] % len(copies)]
         if op in ("softmax", "log_softmax"):
             out = np.empty_like(x)
-            return lambda: orc.mt_softmax_f32(x, op == "log_softmax", cores, out)
+            return lambda: orc.mt_softmax_f32(nxt(), op == "log_softmax", cores, out)
         out = np.empty(x.shape[0], np.float32)
         code = orc.SUM if op == "sum" else orc.MAX
-        return lambda: orc.mt_reduce_rows_f32(x, code, cores, out)
+        return lambda: orc.mt_reduce_rows_f32(nxt(), code, cores, out)
     return call
+
+
+def native_distance(got, native, sample):
+    """Distance between a device result and the oracle's ACC_NATIVE restatement (every operation rounded
+    to the half type, as Hpt's CPU kernels compute on f16 / bf16): max and 99th percentile of
+    |got - native| / max(|native|, 2^-10 * the row's largest |native|). Informational: the device
+    accumulates in f32 and rounds once, so it is the more accurate side."""
+    g, n = got.astype(np.float64), native.astype(np.float64)
+    floor = np.abs(n).max(axis=-1, keepdims=True) * 2.0 ** -10
+    ok = np.isfinite(n) & np.isfinite(g)
+    rel = (np.abs(g - n) / np.maximum(np.abs(n), np.maximum(floor, 1e-30)))[ok]
+    return {"max_rel": float(f"{rel.max():.3g}"), "p99_rel": float(f"{np.percentile(rel, 99):.3g}"), "sample": sample}
 
 
 class Prepared:
@@ -219,11 +247,12 @@ def cases_c2(P, headline_only):
     tg, tb = hpt.Tensor.from_numpy(g).to_hip(0), hpt.Tensor.from_numpy(b).to_hip(0)
     ln_bytes = 2 * x.nbytes + g.nbytes + b.nbytes
     run, ln_outs = P.norm(xs, "layernorm", n_norm=1, gamma=tg, beta=tb)
-    cases = [Case("layernorm", "C2 f32 [8192,4096] gamma,beta eps=1e-5", "f32", 8192, ln_bytes, run, nbuf, plan=P.last_plan)]
+    cases = [Case("layernorm", "C2 f32 [8192,4096] gamma,beta eps=1e-5", "f32", 8192, ln_bytes, run, nbuf, plan=P.last_plan,
+                  key="C2.layernorm")]
     if not headline_only:
         run, _ = P.norm(xs, "log_softmax", axis=1)
         cases.append(Case("log_softmax", "C2 f32 [8192,4096] axis=1", "f32", 8192, 2 * x.nbytes, run, nbuf, plan=P.last_plan,
-                          cpu=cpu_rows("log_softmax", x)))
+                          cpu=cpu_rows("log_softmax", x), key="C2.log_softmax"))
     return cases, (x, g, b, ln_outs[0])
 
 
@@ -236,7 +265,7 @@ def cases_c1(P):
     cases = []
     run, _ = P.norm(c1s, "softmax", axis=1)
     cases.append(Case("softmax", "C1 f32 [1024,1024] axis=1", "f32", 1024, 2 * c1.nbytes, run, 64, plan=P.last_plan,
-                      cpu=cpu_rows("softmax", c1)))
+                      cpu=cpu_rows("softmax", c1), key="C1.softmax"))
     run, _ = P.reduce(c1s, "sum", [1])
     cases.append(Case("sum(axis=1)", "C1 f32 [1024,1024]", "f32", 1024, c1.nbytes + 4096, run, 64, plan=P.last_plan,
                       cpu=cpu_rows("sum", c1)))
@@ -257,18 +286,19 @@ def cases_c3(P):
     c3is = [hpt.Tensor.from_numpy(np.roll(c3i, k, 0)).to_hip(0) for k in range(6)]
     nb = c3.nbytes
     cases = []
-    for name, op, axes, rows, outb in (("sum([2,3])", "sum", [2, 3], 8192, 8192 * 4),
-                                       ("mean([2,3])", "mean", [2, 3], 8192, 8192 * 4),
-                                       ("max(axis=1)", "max", [1], 200704, 200704 * 4),
-                                       ("sum(all)", "sum", [0, 1, 2, 3], 1, 4)):
+    for name, op, axes, rows, outb, key in (("sum([2,3])", "sum", [2, 3], 8192, 8192 * 4, "C3.sum23"),
+                                            ("mean([2,3])", "mean", [2, 3], 8192, 8192 * 4, None),
+                                            ("max(axis=1)", "max", [1], 200704, 200704 * 4, "C3.max1"),
+                                            ("sum(all)", "sum", [0, 1, 2, 3], 1, 4, "C3.sum_all")):
         run, _ = P.reduce(c3s, op, axes)
         # sum / mean over [2, 3] are row reductions of the contiguous [8192, 3136] matrix on the CPU path too
         cpu = cpu_rows("sum", c3.reshape(8192, 3136)) if axes == [2, 3] else None
-        cases.append(Case(name, "C3 f32 [64,128,56,56]", "f32", rows, nb + outb, run, 6, plan=P.last_plan, cpu=cpu))
+        cases.append(Case(name, "C3 f32 [64,128,56,56]", "f32", rows, nb + outb, run, 6, plan=P.last_plan, cpu=cpu, key=key))
     run, _ = P.reduce(c3is, "sum", [1])
     cases.append(Case("sum(axis=1)", "C3 i32 [64,128,56,56]", "i32", 200704, nb + 200704 * 4, run, 6, plan=P.last_plan))
     run, _ = P.reduce(c3is, "argmax", 1, arg=True)
-    cases.append(Case("argmax(axis=1)", "C3 i32 [64,128,56,56]", "i32", 200704, nb + 200704 * 8, run, 6, plan=P.last_plan))
+    cases.append(Case("argmax(axis=1)", "C3 i32 [64,128,56,56]", "i32", 200704, nb + 200704 * 8, run, 6, plan=P.last_plan,
+                      key="C3.i32_argmax1"))
     return cases
 
 
@@ -283,9 +313,17 @@ def cases_c4(P):
     del c4
     c4s = [hpt.Tensor.from_numpy(c4b, hpt.bf16).to_hip(0),
            hpt.Tensor.from_numpy(np.roll(c4b, 2048, 0), hpt.bf16).to_hip(0)]
-    run, _ = P.norm(c4s, "softmax", axis=1)
+    run, outs = P.norm(c4s, "softmax", axis=1)
+    P.keep.append(outs)
+    sample = c4b[1792:2048].copy()  # queries 1792..2047 of head 0: 1793..2048 live keys each
+
+    def native():
+        from oracle import oracle as orc
+        want = orc.bf16_to_f32(orc.softmax(sample, 1, acc=orc.ACC_NATIVE, dtype=orc.BF16))
+        got = hpt.bf16_bits_to_f32(outs[0][1792:2048].to_cpu().numpy())
+        return native_distance(got, want, "rows 1792..2047")
     return [Case("softmax", "C4 bf16 [65536,2048] causal mask as data, axis=1", "bf16", 65536,
-                 2 * c4b.nbytes, run, 2, plan=P.last_plan)]
+                 2 * c4b.nbytes, run, 2, plan=P.last_plan, key="C4.softmax", native=native)]
 
 
 def cases_c5(P):
@@ -301,18 +339,39 @@ def cases_c5(P):
     c5t = [t.permute([1, 0]) for t in c5s]
     c5h = [t[:, ::2] for t in c5s]
     cases = []
-    run, _ = P.norm(c5t, "layernorm", n_norm=1, gamma=tg5, beta=tb5)
-    cases.append(Case("layernorm", "C5a f16 [4096,8192].permute(1,0) -> [8192,4096]", "f16", 8192, 2 * n5 + 16384, run, 6, plan=P.last_plan))
-    run, _ = P.norm(c5t, "softmax", axis=1)
-    cases.append(Case("softmax", "C5a f16 [4096,8192].permute(1,0) axis=1", "f16", 8192, 2 * n5, run, 6, plan=P.last_plan))
-    run, _ = P.reduce(c5t, "sum", [0])
-    cases.append(Case("sum(axis=0)", "C5a f16 [4096,8192].permute(1,0)", "f16", 4096, n5 + 8192, run, 6, plan=P.last_plan))
-    run, _ = P.norm(c5h, "layernorm", n_norm=1, gamma=tg5, beta=tb5)
-    cases.append(Case("layernorm", "C5b f16 [4096,8192][:, ::2] -> [4096,4096]", "f16", 4096, n5 + 16384, run, 6, plan=P.last_plan))
-    run, _ = P.norm(c5h, "softmax", axis=1)
-    cases.append(Case("softmax", "C5b f16 [4096,8192][:, ::2] axis=1", "f16", 4096, n5, run, 6, plan=P.last_plan))
-    run, _ = P.reduce(c5h, "sum", [0])
-    cases.append(Case("sum(axis=0)", "C5b f16 [4096,8192][:, ::2]", "f16", 4096, n5 // 2 + 8192, run, 6, plan=P.last_plan))
+    R = slice(1024, 1152)  # the sample of logical rows the informational per-op-rounded distance is taken on
+
+    def nat(kind, view_np, outs, rows=R, axis=None):
+        """-> () -> distance of the device result (buffer 0) to the oracle's per-op-rounded f16 restatement."""
+        def call():
+            from oracle import oracle as orc
+            if kind == "sum":
+                want = orc.reduce(orc.SUM, view_np, [0], acc=orc.ACC_NATIVE)
+                return native_distance(outs[0].numpy()[None, :], want[None, :], "all 4096 outputs")
+            v = view_np[rows]
+            want = (orc.layernorm(v, 1, g5, b5, 1e-5, acc=orc.ACC_NATIVE) if kind == "layernorm"
+                    else orc.softmax(v, 1, acc=orc.ACC_NATIVE))
+            return native_distance(outs[0][rows].to_cpu().numpy(), want, f"logical rows {rows.start}..{rows.stop - 1}")
+        return call
+
+    run, outs = P.norm(c5t, "layernorm", n_norm=1, gamma=tg5, beta=tb5)
+    cases.append(Case("layernorm", "C5a f16 [4096,8192].permute(1,0) -> [8192,4096]", "f16", 8192, 2 * n5 + 16384, run, 6,
+                      plan=P.last_plan, key="C5a.layernorm", native=nat("layernorm", c5.T, outs)))
+    run, outs = P.norm(c5t, "softmax", axis=1)
+    cases.append(Case("softmax", "C5a f16 [4096,8192].permute(1,0) axis=1", "f16", 8192, 2 * n5, run, 6, plan=P.last_plan,
+                      native=nat("softmax", c5.T, outs)))
+    run, outs = P.reduce(c5t, "sum", [0])
+    cases.append(Case("sum(axis=0)", "C5a f16 [4096,8192].permute(1,0)", "f16", 4096, n5 + 8192, run, 6, plan=P.last_plan,
+                      key="C5a.sum0", native=nat("sum", c5.T, outs)))
+    run, outs = P.norm(c5h, "layernorm", n_norm=1, gamma=tg5, beta=tb5)
+    cases.append(Case("layernorm", "C5b f16 [4096,8192][:, ::2] -> [4096,4096]", "f16", 4096, n5 + 16384, run, 6,
+                      plan=P.last_plan, key="C5b.layernorm", native=nat("layernorm", c5[:, ::2], outs)))
+    run, outs = P.norm(c5h, "softmax", axis=1)
+    cases.append(Case("softmax", "C5b f16 [4096,8192][:, ::2] axis=1", "f16", 4096, n5, run, 6, plan=P.last_plan,
+                      native=nat("softmax", c5[:, ::2], outs)))
+    run, outs = P.reduce(c5h, "sum", [0])
+    cases.append(Case("sum(axis=0)", "C5b f16 [4096,8192][:, ::2]", "f16", 4096, n5 // 2 + 8192, run, 6, plan=P.last_plan,
+                      key="C5b.sum0", native=nat("sum", c5[:, ::2], outs)))
     return cases
 
 
@@ -485,13 +544,41 @@ def cases_c10(P):
     return cases
 
 
+def cases_ref(P):
+    """The shapes the reference publishes its own numbers for (docs/benchmarks/reduce.md:62-78, harness
+    hpt-bench/benches/benchmarks/reduction/reduction_benches.rs:26-93: f32 `sum` of [1024,1024,80] over the seven
+    axis sets; docs/benchmarks/normalization.md:3-123, harness hpt-bench/benches/benchmarks/softmax/softmax.rs:8-61:
+    f32 softmax of 256^3 and 512^3 over axes 0, 1, 2)."""
+    import hpt_amd as hpt
+    rng = np.random.default_rng(11)
+    cases = []
+    base = rng.standard_normal((1024, 1024, 80), dtype=np.float32)
+    ts = [hpt.Tensor.from_numpy(base).to_hip(0), hpt.Tensor.from_numpy(np.roll(base, 1, 0)).to_hip(0)]
+    for axes in ([0], [1], [2], [0, 1], [0, 2], [1, 2], [0, 1, 2]):
+        outs_n = int(np.prod([d for i, d in enumerate(base.shape) if i not in axes]))
+        run, _ = P.reduce(ts, "sum", axes)
+        label = "sum(" + ",".join(map(str, axes)) + ")"
+        cases.append(Case(label, "ref f32 [1024,1024,80]", "f32", outs_n, base.nbytes + 4 * outs_n, run, 2, plan=P.last_plan,
+                          key="ref." + label))
+    del ts, base
+    for n, nbuf in ((256, 6), (512, 2)):
+        base = rng.standard_normal((n, n, n), dtype=np.float32)
+        ts = [hpt.Tensor.from_numpy(np.roll(base, k, 0)).to_hip(0) for k in range(nbuf)]
+        for axis in (0, 1, 2):
+            run, _ = P.norm(ts, "softmax", axis=axis)
+            cases.append(Case(f"softmax({axis})", f"ref f32 [{n},{n},{n}]", "f32", n * n, 2 * base.nbytes, run, nbuf,
+                              plan=P.last_plan, key=f"ref.softmax{n}({axis})"))
+        del ts, base
+    return cases
+
+
 def build_cases(which: str, configs=None):
     """Synthetic inputs of the benchmark configurations, uploaded once; outputs preallocated.
     The headline (C2 layernorm) is always first; `configs` limits the others (e.g. {"c3"})."""
     P = Prepared()
     cases, head = cases_c2(P, which == "headline")
     if which != "headline":
-        for name, fn in (("c1", cases_c1), ("c3", cases_c3), ("c4", cases_c4), ("c5", cases_c5), ("c6", cases_c6),
+        for name, fn in (("c1", cases_c1), ("ref", cases_ref), ("c3", cases_c3), ("c4", cases_c4), ("c5", cases_c5), ("c6", cases_c6),
                          ("c7", cases_c7), ("c8", cases_c8), ("c9", cases_c9), ("c10", cases_c10)):
             if configs is None or name in configs:
                 cases += fn(P)
@@ -513,7 +600,7 @@ def cpu_baseline(x, g, b, gpu_out, budget_s=15.0):
         rows = slice(0, 512)
         truth = orc.layernorm(x[rows], 1, g, b, 1e-5, acc=orc.ACC_F64).astype(np.float64)
         err = np.abs(gpu_out[rows].astype(np.float64) - truth)
-        assert (err <= 2e-6 + 1e-5 * np.abs(truth)).all(), \
+        assert (err <= 1e-6 + 1e-5 * np.abs(truth)).all(), \
             f"GPU layernorm differs from the f64 oracle (max err {err.max():g})"
         port_err = float(np.abs(out[rows].astype(np.float64) - truth).max())
     times = []
@@ -578,6 +665,67 @@ def host_time(cases, calls=2000):
               f"with the device's work {1e6 * (t2 - t0) / calls:7.2f} us/call", flush=True)
 
 
+MAX_LINE_BYTES = 4096      # the one JSON line on stdout stays under this; everything else goes to OPS_FILE and stderr
+MAX_SUMMARY_OPS = 12       # per-op figures carried by the line: the ops of the five benchmark configurations
+OPS_FILE = "bench_ops.json"
+# the ops whose "% of peak" the line carries (the headline, C2 layernorm, is the line's own `value`)
+SUMMARY_KEYS = ("C1.softmax", "C2.log_softmax", "C3.sum23", "C3.max1", "C3.sum_all", "C3.i32_argmax1", "C4.softmax",
+                "C5a.layernorm", "C5a.sum0", "C5b.layernorm", "C5b.sum0")
+
+
+def op_record(case_fields: dict, per_launch_us) -> dict:
+    """The per-op record of the side file from a case's constants and its 13 group timings."""
+    med = float(np.median(per_launch_us))
+    nbytes = case_fields["algorithmic_bytes"]
+    gbps = nbytes / (med * 1e-6) / 1e9
+    rec = dict(case_fields)
+    rec.update({"us_per_launch": round(med, 2), "us_min": round(min(per_launch_us), 2), "us_max": round(max(per_launch_us), 2),
+                "launches_timed": GROUPS * PER_GROUP, "GBps": round(gbps, 1), "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBS, 1),
+                "rows_per_s": round(case_fields["rows"] / (med * 1e-6), 1)})
+    return rec
+
+
+def summary_line(steps, warmup, wall_s, dev_ms, head_bytes, head_rows, nbuf, roofline_extra, cpu, ops) -> dict:
+    """The ONE JSON object bench.py prints on stdout: the headline's throughput, its roofline and CPU baseline,
+    the % of peak of at most MAX_SUMMARY_OPS ops of the benchmark configurations, and the % of peak on the shapes of
+    the reference's own published matrix. Pure: the CPU test suite calls it with canned numbers and checks its length."""
+    value = head_bytes * steps / wall_s / 1e9
+    kernel_us = dev_ms * 1e3 / steps
+    achieved = head_bytes / (kernel_us * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": None, "kernel_us": round(kernel_us, 2)}
+    roofline.update(roofline_extra or {})
+    by_key = {o["key"]: o for o in ops if o.get("key")}
+    configs = {k: by_key[k]["pct_of_hbm_peak"] for k in SUMMARY_KEYS if k in by_key}
+    assert len(configs) <= MAX_SUMMARY_OPS
+    # the reference's own published matrix (f32 sum of [1024,1024,80] over seven axis sets, softmax of 256^3 / 512^3)
+    ref = {o["key"][4:]: o["pct_of_hbm_peak"] for o in ops if (o.get("key") or "").startswith("ref.")}
+    if cpu is not None:
+        cpu = {k: cpu[k] for k in ("value", "unit", "cores", "kind", "sample", "rows_per_s") if k in cpu}
+    return {
+        "metric": "achieved HBM GB/s (% of MI355X peak) + rows/s for softmax/layernorm/reduce",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(wall_s * 1e3 / steps, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "LayerNorm over the last axis, f32 [8192,4096] ~N(0,1)+row offset U(-5,5), "
+                               "gamma~N(1,0.1), beta~N(0,0.1), eps=1e-5 (the configuration the metric is quoted on)",
+                   "rows": head_rows, "cols": 4096, "algorithmic_bytes_per_step": head_bytes, "buffers_rotated": nbuf},
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1),
+        "rows_per_s": round(head_rows * steps / wall_s, 1),
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "configs_pct_of_hbm_peak": configs,
+        "reference_shapes_pct_of_hbm_peak": ref,
+        "ops_measured": len(ops), "ops_file": OPS_FILE if ops else None,
+    }
+
+
+def encode_line(line: dict) -> str:
+    text = json.dumps(line, separators=(",", ":"))
+    assert len(text.encode()) < MAX_LINE_BYTES, f"the summary line grew to {len(text.encode())} bytes"
+    return text
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -585,7 +733,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--ops", choices=["all", "headline"], default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--configs", default="", help="comma list of c1,c3,c4,c5,c6,c7,c8,c9,c10 to measure besides the headline (c6 = the steps either side: contiguous / in-place affine / full; c7 = the fused forms; c8 = shapes off the reference's list; c9 = hidden sizes of 3 or 5 times a power of two; c10 = logits over a vocabulary)")
+    ap.add_argument("--configs", default="", help="comma list of c1,ref,c3,c4,c5,c6,c7,c8,c9,c10 to measure besides the headline (ref = the shapes the reference publishes numbers for; c6 = the steps either side: contiguous / in-place affine / full; c7 = the fused forms; c8 = shapes off the reference's list; c9 = hidden sizes of 3 or 5 times a power of two; c10 = logits over a vocabulary)")
+    ap.add_argument("--ops-file", default=OPS_FILE, help="where the full per-op table goes (JSON; the stdout line stays short)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region, run one plain device-to-device copy of the headline input "
                          "(134217728 bytes read + as many written): the known-size dispatch that hardware "
@@ -617,28 +766,20 @@ def main():
         return
     head = cases[0]
     wall, dev_ms = time_case(ev, head, args.steps, args.warmup)
-    ms_per_step = wall * 1e3 / args.steps
-    value = head.bytes * args.steps / wall / 1e9
-    kernel_us = dev_ms * 1e3 / args.steps
-    achieved = head.bytes / (dev_ms / args.steps * 1e-3) / 1e9
 
     ops = []
     for c in cases:
-        per = time_groups(ev, c)
-        med = float(np.median(per))
-        o = {"config": c.cfg, "op": c.name, "dtype": c.dtype, "algorithmic_bytes": c.bytes,
-             "us_per_launch": round(med, 2), "us_min": round(min(per), 2), "us_max": round(max(per), 2),
-             "launches_timed": GROUPS * PER_GROUP,
-             "GBps": round(c.bytes / (med * 1e-6) / 1e9, 1),
-             "pct_of_hbm_peak": round(100 * c.bytes / (med * 1e-6) / 1e9 / HBM_PEAK_GBS, 1),
-             "rows_per_s": round(c.rows / (med * 1e-6), 1), "plan": c.plan}
-        if c.cpu is not None and not args.no_cpu:
-            from oracle import oracle as orc
-            sec, passes = cpu_seconds(c.cpu())
-            o["cpu_GBps"] = round(c.bytes / sec / 1e9, 2)
-            o["cpu_ms_per_pass"] = round(sec * 1e3, 3)
-            o["cpu_cores"] = orc.physical_cores()
-            o["cpu_kind"] = "port"
+        o = op_record({"key": c.key, "config": c.cfg, "op": c.name, "dtype": c.dtype, "algorithmic_bytes": c.bytes,
+                       "rows": c.rows, "plan": c.plan}, time_groups(ev, c))
+        if not args.no_cpu:
+            if c.cpu is not None:
+                from oracle import oracle as orc
+                sec, passes = cpu_seconds(c.cpu())
+                o.update({"cpu_GBps": round(c.bytes / sec / 1e9, 2), "cpu_ms_per_pass": round(sec * 1e3, 3),
+                          "cpu_cores": orc.physical_cores(), "cpu_kind": "port",
+                          "cpu_note": "inputs rotated over > 512 MB of copies: not served from the host's caches"})
+            if c.native is not None:
+                o["distance_to_per_op_rounded_cpu_result"] = c.native()
         ops.append(o)
 
     if args.copy_calibration:
@@ -655,41 +796,33 @@ def main():
 
     # The dominant kernel, its HBM traffic and the profiler's own duration come from the committed profile
     # summary; the plan the library reports NOW is set beside the plan recorded THERE.
-    plan_now = head.plan
-    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": None,
-                "kernel_us": round(kernel_us, 2), "plan": plan_now}
+    extra = {"plan": head.plan}
     if HEADLINE_PROFILE.exists():
         prof = json.loads(HEADLINE_PROFILE.read_text())
-        same = prof.get("plan") == plan_now
-        roofline.update({"kernel": prof.get("kernel"), "profile_plan": prof.get("plan"), "profile_matches_plan": same,
-                         "profiler_kernel_us": prof.get("profiler_avg_us"),
-                         # a stale profile says nothing about the kernel that ran: no traffic figure then
-                         "traffic": prof.get("traffic_bytes") if same else None})
+        same = prof.get("plan") == head.plan
+        extra.update({"kernel": prof.get("kernel"), "profile_matches_plan": same,
+                      "profiler_kernel_us": prof.get("profiler_avg_us"),
+                      # a stale profile says nothing about the kernel that ran: no traffic figure then
+                      "traffic": prof.get("traffic_bytes") if same else None})
         if not same:
+            extra["profile_plan"] = prof.get("plan")
             print(f"bench.py: profiles/headline.json was recorded for plan '{prof.get('plan')}', the library now plans "
-                  f"'{plan_now}': regenerate the profile", file=sys.stderr)
+                  f"'{head.plan}': regenerate the profile", file=sys.stderr)
 
-    line = {
-        "metric": "achieved HBM GB/s (% of MI355X peak) + rows/s for softmax/layernorm/reduce",
-        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "LayerNorm over the last axis, f32 [8192,4096] ~N(0,1)+row offset U(-5,5), "
-                               "gamma~N(1,0.1), beta~N(0,0.1), eps=1e-5 (the configuration the metric is quoted on)",
-                   "rows": 8192, "cols": 4096, "algorithmic_bytes_per_step": head.bytes,
-                   "buffers_rotated": head.nbuf},
-        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1),
-        "rows_per_s": round(8192 * args.steps / wall, 1),
-        "roofline": roofline,
-        "cpu_baseline": cpu,
-        "ops": ops,
-    }
+    line = summary_line(args.steps, args.warmup, wall, dev_ms, head.bytes, head.rows, head.nbuf, extra, cpu, ops)
     for o in ops:
-        cpu = f"  cpu {o['cpu_GBps']:.1f} GB/s on {o['cpu_cores']} cores" if "cpu_GBps" in o else ""
+        cpu_s = f"  cpu {o['cpu_GBps']:.1f} GB/s on {o['cpu_cores']} cores" if "cpu_GBps" in o else ""
+        d = o.get("distance_to_per_op_rounded_cpu_result")
+        nat = f"  per-op-rounded CPU result: max rel {d['max_rel']:.2g}, p99 {d['p99_rel']:.2g}" if d else ""
         print(f"  {o['config']:<58} {o['op']:<16} {o['us_per_launch']:>9.2f} us  {o['GBps']:>8.1f} GB/s "
-              f"{o['pct_of_hbm_peak']:>5.1f}%  {o['rows_per_s']:.3g} rows/s{cpu}", file=sys.stderr)
-    print(json.dumps(line))
+              f"{o['pct_of_hbm_peak']:>5.1f}%  {o['rows_per_s']:.3g} rows/s{cpu_s}{nat}", file=sys.stderr)
+    # the full per-op table and the untrimmed CPU baseline: a side file next to the working directory's other output
+    try:
+        Path(args.ops_file).write_text(json.dumps({"line": line, "cpu_baseline": cpu, "ops": ops}, indent=1))
+    except OSError as e:
+        print(f"bench.py: could not write {args.ops_file}: {e}", file=sys.stderr)
+    sys.stderr.flush()
+    print(encode_line(line), flush=True)
 
 
 if __name__ == "__main__":

@@ -89,7 +89,6 @@ def build(force: bool = False, jobs: int | None = None, verbose: bool = True) ->
         if r.returncode != 0:
             raise RuntimeError("link failed:\n" + r.stderr)
     build_host_test(force)
-    build_access_patterns(force)
     return LIB
 
 
@@ -110,23 +109,6 @@ def build_host_test(force: bool = False) -> Path:
     if r.returncode != 0:
         raise RuntimeError("host test build failed:\n" + r.stderr)
     return HOST_TEST_BIN
-
-
-PATTERNS_SRC = ROOT.parent / "tests" / "cpp" / "transposed_access_patterns.hip"
-PATTERNS_BIN = ROOT / "lib" / "transposed_access_patterns"
-
-
-def build_access_patterns(force: bool = False) -> Path:
-    """The standalone measurement program of the load / store arrangements a transposed register tile can
-    take (the ceilings the transposed plans are designed around)."""
-    if not force and PATTERNS_BIN.exists() and PATTERNS_BIN.stat().st_mtime > PATTERNS_SRC.stat().st_mtime:
-        return PATTERNS_BIN
-    cmd = [HIPCC, "-std=c++17", "-O3", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           "-Wno-unused-command-line-argument", str(PATTERNS_SRC), "-o", str(PATTERNS_BIN)]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("access pattern program build failed:\n" + r.stderr)
-    return PATTERNS_BIN
 
 
 if __name__ == "__main__":

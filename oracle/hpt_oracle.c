@@ -18,6 +18,7 @@
  *                            hpt-types/src/scalars/impls.rs:28-75
  *   orc_reduce (floats)      cpu/kernels/reduce.rs:608-791,                       doc KATs hpt-traits/src/ops/reduce.rs:58-350; vs
  *                            hpt-types/src/vectors/utils.rs:83-105                numpy float64 sums; lane-structure invariants
+ *   orc_reduce, ACC_EXACT    (no counterpart: the exactly summed f64 truth)        math.fsum: ill-conditioned sums (1e100 + 1 - 1e100), 1.3 M terms
  *   orc_argreduce            cpu/kernels/argreduce_kernels.rs:2-71                numpy argmax/argmin (first extremum), tie cases
  *   orc_softmax              cpu/kernels/softmax.rs:81-362,                       torch.softmax/log_softmax (float64) as the
  *                            cpu/kernels/normalization/logsoftmax.rs:81-364       reference's tests do; rows sum to 1; shift invariance
@@ -397,7 +398,7 @@ int orc_reduce_out_dtype(int op, int dt) {
 /* the type arithmetic is rounded to, for a value type `vt` under an accumulate mode */
 static int acc_dtype(int vt, int mode) {
     if (!dt_is_float(vt)) return vt;
-    if (mode == ORC_ACC_F64) return ORC_F64;
+    if (mode == ORC_ACC_F64 || mode == ORC_ACC_EXACT) return ORC_F64;
     if (mode == ORC_ACC_F32) return vt == ORC_F64 ? ORC_F64 : ORC_F32;
     return vt;
 }
@@ -538,6 +539,65 @@ static uint64_t i_comb(const rctx* c, uint64_t a, uint64_t b) {
     }
 }
 
+/* Exact summation of doubles (Shewchuk's expansions, the algorithm of Python's math.fsum): `p` holds
+ * non-overlapping partials in increasing magnitude whose exact sum is the exact sum of everything added;
+ * two-sum (hi = x + y, lo = y - (hi - x) with |x| >= |y|) moves each new term through them without error.
+ * Non-finite terms are added apart, as IEEE would (inf + -inf = NaN). */
+typedef struct {
+    int n;
+    double p[80];
+    double special;
+    int has_special;
+} exact_sum;
+
+static void exact_reset(exact_sum* e) {
+    e->n = 0;
+    e->special = 0.0;
+    e->has_special = 0;
+}
+static void exact_add(exact_sum* e, double x) {
+    if (!isfinite(x)) {
+        e->special += x;
+        e->has_special = 1;
+        return;
+    }
+    int i = 0;
+    for (int j = 0; j < e->n; ++j) {
+        double y = e->p[j];
+        if (fabs(x) < fabs(y)) {
+            const double t = x;
+            x = y;
+            y = t;
+        }
+        const double hi = x + y;
+        const double lo = y - (hi - x);
+        if (lo != 0.0) e->p[i++] = lo;
+        x = hi;
+    }
+    e->p[i++] = x;
+    e->n = i;
+}
+static double exact_result(const exact_sum* e) {
+    if (e->has_special) return e->special;
+    int n = e->n;
+    double hi = 0.0, lo = 0.0;
+    if (n > 0) {
+        hi = e->p[--n];
+        while (n > 0) { /* add the partials from the largest down until one does not fit exactly */
+            const double x = hi, y = e->p[--n];
+            hi = x + y;
+            lo = y - (hi - x);
+            if (lo != 0.0) break;
+        }
+        /* half-way case: the rest of the partials decides the rounding direction */
+        if (n > 0 && ((lo < 0.0 && e->p[n - 1] < 0.0) || (lo > 0.0 && e->p[n - 1] > 0.0))) {
+            const double y = lo * 2.0, x = hi + y;
+            if (y == x - hi) hi = x;
+        }
+    }
+    return hi;
+}
+
 static int split_axes(const orc_view* in, const int64_t* axes, int naxes, odo* kept, odo* red) {
     int64_t norm[ORC_MAX_RANK];
     if (orc_process_axes(axes, naxes, in->ndim, norm, NULL, 0)) return 1;
@@ -574,7 +634,13 @@ int orc_reduce(int op, const orc_view* in, const int64_t* axes, int naxes, void*
     /* the innermost reduced axis, when dense, is walked with `lanes` accumulators
      * folded in lane order (hpt-types/src/vectors/utils.rs:83-105) */
     const int lane_mode = lanes > 1 && red.n > 0 && red.stride[red.n - 1] == 1 && !c.is_int &&
-                          !float_op && acc_mode != ORC_ACC_F64;
+                          !float_op && acc_mode != ORC_ACC_F64 && acc_mode != ORC_ACC_EXACT;
+    /* ORC_ACC_EXACT: the additive ops keep the running sum as a list of non-overlapping f64 partials
+     * (exact_sum below), so the result is the f64 nearest the exact sum of the terms whatever their
+     * number or order: the truth does not drift the way a running f64 sum does */
+    const int additive = op == ORC_SUM || op == ORC_MEAN || op == ORC_NANSUM || op == ORC_REDUCEL1 ||
+                         op == ORC_REDUCEL2 || op == ORC_REDUCEL3 || op == ORC_SUM_SQUARE || op == ORC_LOGSUMEXP;
+    const int exact = acc_mode == ORC_ACC_EXACT && additive && !c.is_int;
     const int64_t inner = red.n ? red.size[red.n - 1] : 1;
 
     int64_t koff = 0;
@@ -618,6 +684,17 @@ int orc_reduce(int op, const orc_view* in, const int64_t* axes, int naxes, void*
                     if (outer.n == 0) break;
                     roff += odo_next(&outer, &done);
                 }
+            } else if (R > 0 && exact) {
+                int64_t roff = 0;
+                int done = 0;
+                exact_sum es;
+                exact_reset(&es);
+                odo_reset(&red);
+                while (!done) {
+                    exact_add(&es, f_pre(&c, load_f(in->data, in->dtype, koff + roff)));
+                    roff += odo_next(&red, &done);
+                }
+                acc = exact_result(&es);
             } else if (R > 0) {
                 int64_t roff = 0;
                 int done = 0;

@@ -37,8 +37,13 @@ enum {
  *           the result is rounded to the output type once (what the north star
  *           calls "accumulated in f32"); other types as NATIVE.
  *   F64   : floating types accumulate in f64 and round once at the end
- *           (the "truth" the f32 tolerance is measured against).           */
-enum { ORC_ACC_NATIVE = 0, ORC_ACC_F32 = 1, ORC_ACC_F64 = 2 };
+ *           (the "truth" the f32 tolerance is measured against).
+ *   EXACT : as F64, and the additive reductions (sum, mean, nansum, reducel1/2/3,
+ *           sum_square, logsumexp) add their terms without error (expansion
+ *           arithmetic, as Python's math.fsum) and round the exact sum once: the
+ *           truth for sums of millions of f64 terms, where a running f64 sum
+ *           itself drifts. Reductions only.                                  */
+enum { ORC_ACC_NATIVE = 0, ORC_ACC_F32 = 1, ORC_ACC_F64 = 2, ORC_ACC_EXACT = 3 };
 
 typedef struct orc_view {
     const void* data;        /* already-offset element pointer */

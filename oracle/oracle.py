@@ -20,7 +20,7 @@ LIB_PATH = HERE / "libhpt_oracle.so"
 
 BOOL, I8, I16, I32, I64, U8, U16, U32, U64, F16, BF16, F32, F64 = range(13)
 SUM, PROD, MAX, MIN, MEAN, NANSUM, NANPROD, REDUCEL1, REDUCEL2, REDUCEL3, SUM_SQUARE, LOGSUMEXP, ALL, ANY = range(14)
-ACC_NATIVE, ACC_F32, ACC_F64 = 0, 1, 2
+ACC_NATIVE, ACC_F32, ACC_F64, ACC_EXACT = 0, 1, 2, 3
 
 _NP2DT = {np.dtype(np.bool_): BOOL, np.dtype(np.int8): I8, np.dtype(np.int16): I16,
           np.dtype(np.int32): I32, np.dtype(np.int64): I64, np.dtype(np.uint8): U8,

@@ -129,7 +129,7 @@ def test_add_layernorm(hpt, orc, dev, case):
                          f"add_layernorm f16 {name}")
         else:
             want = orc.layernorm(np.ascontiguousarray(summed), nn, g, b, 1e-5, acc=orc.ACC_F64)
-            assert_close(got, want, F32_RTOL, 2e-6, f"add_layernorm {npdt.__name__} {name}")
+            assert_close(got, want, F32_RTOL, F32_ATOL, f"add_layernorm {npdt.__name__} {name}")
             # unfused on the device: (x + r) then layernorm
             u = t.add(tr).layernorm(ns, tg, tb, 1e-5).numpy()
             assert_close(got, u, 2e-6, 2e-7, f"fused vs unfused on device {name}")
@@ -140,7 +140,7 @@ def test_add_layernorm(hpt, orc, dev, case):
         if npdt == np.float16:
             assert_close(got2.astype(np.float32), want2.astype(np.float32), HALF_RTOL, half_atol(want2, 11), "no affine")
         else:
-            assert_close(got2, want2, F32_RTOL, 2e-6, f"add_layernorm no affine {name}")
+            assert_close(got2, want2, F32_RTOL, F32_ATOL, f"add_layernorm no affine {name}")
 
 
 def test_fused_argument_errors(hpt, dev):

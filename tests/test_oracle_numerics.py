@@ -305,3 +305,34 @@ def test_timed_restatement_equals_oracle(orc):
     want = np.exp(xs.astype(np.float64))
     assert (np.abs(got - want) <= 3e-7 * want + 1e-45).all()
     assert orc.physical_cores() >= 1
+
+
+def test_compensated_f64_mode_against_fsum(orc):
+    """ACC_EXACT (the truth for long f64 sums) equals math.fsum where a running f64 sum does not:
+    ill-conditioned sums whose large terms cancel, and a million random terms; views and several axes go
+    through the same path; mean / sum_square / reducel1 are built on it."""
+    import math
+    x = np.array([1e100, 1.0, -1e100, 1e-5, 3.0, -1e80, 1e80] * 1000)
+    assert orc.reduce(orc.SUM, x, [0], acc=orc.ACC_EXACT)[0] == math.fsum(x)
+    assert orc.reduce(orc.SUM, x, [0], acc=orc.ACC_F64)[0] != math.fsum(x)   # the plain mode loses the small terms
+    rng = np.random.default_rng(5)
+    y = rng.standard_normal(1_300_000) * 3
+    assert orc.reduce(orc.SUM, y, [0], acc=orc.ACC_EXACT)[0] == math.fsum(y)
+    assert abs(orc.reduce(orc.SUM, y, [0], acc=orc.ACC_F64)[0] - math.fsum(y)) > 1e-12
+    m = orc.reduce(orc.MEAN, y, [0], acc=orc.ACC_EXACT)[0]
+    assert m == math.fsum(y) / y.size
+    assert orc.reduce(orc.SUM_SQUARE, y, [0], acc=orc.ACC_EXACT)[0] == math.fsum(v * v for v in y)
+    assert orc.reduce(orc.REDUCEL1, y, [0], acc=orc.ACC_EXACT)[0] == math.fsum(abs(v) for v in y)
+    z = rng.standard_normal((7, 300, 11)) * np.array([1e12, 1.0, 1e-9] * 100)[None, :, None]
+    v = z.transpose(2, 0, 1)[::2, :, 5:]
+    got = orc.reduce(orc.SUM, v, [1, 2], acc=orc.ACC_EXACT)
+    want = [math.fsum(v[i].ravel()) for i in range(v.shape[0])]
+    assert np.array_equal(got, want)
+    # f32 input: the exact sum rounded once to f32
+    w = (rng.standard_normal(200_000) * 3).astype(np.float32)
+    assert orc.reduce(orc.SUM, w, [0], acc=orc.ACC_EXACT)[0] == np.float32(math.fsum(w.astype(np.float64)))
+    # infinities and NaN pass through as in the plain mode
+    assert orc.reduce(orc.SUM, np.array([1.0, np.inf, 2.0]), [0], acc=orc.ACC_EXACT)[0] == np.inf
+    assert np.isnan(orc.reduce(orc.SUM, np.array([1.0, np.inf, -np.inf]), [0], acc=orc.ACC_EXACT)[0])
+    assert np.isnan(orc.reduce(orc.SUM, np.array([1.0, np.nan, 2.0]), [0], acc=orc.ACC_EXACT)[0])
+    assert orc.reduce(orc.NANSUM, np.array([1.0, np.nan, 2.0]), [0], acc=orc.ACC_EXACT)[0] == 3.0
