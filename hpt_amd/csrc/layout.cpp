@@ -932,10 +932,18 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 // f16 [4097, 12, 96, 5] over axis 2, 0.4 -> 1.3 TB/s)
                 for (int ev = max_vec; ev >= ((elem_size == 2 && p.cols > 16 && L >= 64) ? 4 : 1); ev /= 2) {
                     const int64_t regs = std::max<int64_t>(1, ev * (int64_t)elem_size / 4);
-                    const int64_t nc_max = std::min<int64_t>(64, 64 / regs);
+                    int64_t nc_max = std::min<int64_t>(64, 64 / regs);
                     const size_t vb = (size_t)ev * elem_size;
                     // thread rows that share an inner position when the axis is longer than one thread holds
-                    const int64_t ty = pow2_ceil((p.cols + nc_max - 1) / nc_max);
+                    int64_t ty = pow2_ceil((p.cols + nc_max - 1) / nc_max);
+                    // A four-byte axis of 257 ... 512 elements fits sixteen thread rows only as 8-byte pieces, i.e.
+                    // 128-byte segments of each inner row per workgroup, fetched by sixteen workgroups on eight XCDs at
+                    // different moments. With 128 registers of raw values per thread instead of 64 the pieces are whole
+                    // vectors and the segments 256 bytes (f32 [512, 512, 512] over axis 0 or 1: 4.8 TB/s before).
+                    if (ty > 16 && elem_size == 4 && ev == 4 && p.cols <= 512 && L % 64 == 0) {
+                        nc_max = 32;
+                        ty = 16;
+                    }
                     // enough threads to fill the chip: inner positions x thread rows
                     if (!(ty <= 16 && p.rows / ev * ty >= 8 * 1024)) continue;
                     // (a long axis of two-byte elements that only fits with sixteen thread rows of 4-byte pieces: the

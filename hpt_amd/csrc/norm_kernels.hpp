@@ -254,6 +254,25 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int iv = c * tpr + tx;
+            if constexpr (kCausal && !SHIFT) {
+                // A chunk (the tpr vectors the row's lanes hold side by side) lies wholly below the diagonal, wholly
+                // above it, or across it. Only the one across it needs a test per element; the masked half of the
+                // logits costs no arithmetic at all. (With the tests on every element the two-byte kernel was bound
+                // by its instructions, not by memory: bf16 [32, 2048, 2048] with nothing masked took 104 us where the
+                // plain softmax of the same bytes takes 85.)
+                const int c_lo = c * tpr * UV;
+                if (!valid || c_lo >= limit) {
+#pragma unroll
+                    for (int j = 0; j < UV; ++j) x[c][j] = fill;
+                    continue;
+                }
+                if (c_lo + tpr * UV <= limit) {
+#pragma unroll
+                    for (int j = 0; j < UV; ++j)
+                        x[c][j] = Elem<T>::widen(Elem<T>::narrow(Elem<T>::widen(raw[c].v[j * SS]) * scale_t));
+                    continue;
+                }
+            }
 #pragma unroll
             for (int j = 0; j < UV; ++j) {
                 const bool have = valid && inside(iv, j);

@@ -112,9 +112,10 @@ template <class T, int VEC> void launch_col_split(const NormPlan& p, const NormA
 }
 
 // A short strided axis held in registers (softmax kinds).
-template <class T, int EV> void launch_col_reg(const NormPlan& p, const NormArgs& a, hipStream_t st) {
+// WIDE: twice the vectors per thread (128 registers of raw values instead of 64).
+template <class T, int EV, bool WIDE = false> void launch_col_reg(const NormPlan& p, const NormArgs& a, hipStream_t st) {
     constexpr int REGS = (EV * (int)sizeof(T) + 3) / 4;
-    constexpr int NC = 64 / REGS > 64 ? 64 : 64 / REGS;
+    constexpr int NC = (64 / REGS > 64 ? 64 : 64 / REGS) * (WIDE ? 2 : 1);
     ColRegArgs c{};
     const int nk = p.kept_in.n;
     c.in = a.in;
@@ -243,7 +244,14 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
             switch (p.vec) {
                 case 1: launch_col_reg<T, 1>(p, a, st); break;
                 case 2: if constexpr (FULL >= 2) launch_col_reg<T, 2>(p, a, st); break;
-                case 4: if constexpr (FULL >= 4) launch_col_reg<T, 4>(p, a, st); break;
+                case 4:
+                    if constexpr (FULL == 4) {
+                        if (p.nchunk == 32) launch_col_reg<T, 4, true>(p, a, st);
+                        else launch_col_reg<T, 4>(p, a, st);
+                    } else if constexpr (FULL > 4) {
+                        launch_col_reg<T, 4>(p, a, st);
+                    }
+                    break;
                 case 8: if constexpr (FULL >= 8) launch_col_reg<T, 8>(p, a, st); break;
                 default: fail(HPT_ERR_KERNEL, "col-reg: unsupported vector width %d", p.vec);
             }

@@ -169,6 +169,11 @@ struct RowArgs {
     int64_t ichunk;  // inner vectors per split
     double count;    // elements reduced per output (mean)
     int tpr, tpr_log2, rpb, split_q, split_i, init_out;
+    // > 0: workgroup x takes row block (x % 8) * xcd_chunk + x / 8 (gridDim.x = 8 * xcd_chunk). Workgroups are
+    // dealt round-robin to the chip's eight XCDs, each with an L2 of its own: numbered this way, the row blocks
+    // that run on one XCD at a time are neighbours, and when neighbouring rows' runs share cache lines (runs of
+    // 320 bytes laid back to back) a line is fetched from memory once instead of once per XCD that needs it.
+    int xcd_chunk;
 };
 
 // Vector iv of a run of `rin` contiguous elements at p. UA (runs that are not whole, aligned
@@ -206,7 +211,8 @@ __global__ void __launch_bounds__(1024) row_reduce_kernel(const RowArgs a) {
     const int tpr = a.tpr;
     const int tx = threadIdx.x & (tpr - 1);
     const int ty = threadIdx.x >> a.tpr_log2;
-    const int64_t row = (int64_t)blockIdx.x * a.rpb + ty;
+    const int64_t rb = a.xcd_chunk > 0 ? (int64_t)(blockIdx.x & 7) * a.xcd_chunk + (blockIdx.x >> 3) : (int64_t)blockIdx.x;
+    const int64_t row = rb * a.rpb + ty;
     const bool valid = row < a.K;
     Acc acc = Op::identity();
 
@@ -1017,6 +1023,14 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.split_q = p.split_q;
             a.split_i = p.split_i;
             a.init_out = init_out;
+            // neighbouring outputs whose runs lie within a few lines of each other: number the row blocks per XCD
+            if (p.kept.n >= 1 && grid.x >= 64) {
+                const int64_t ks = p.kept.stride[p.kept.n - 1] < 0 ? -p.kept.stride[p.kept.n - 1] : p.kept.stride[p.kept.n - 1];
+                if (ks * (int64_t)sizeof(T) * p.rpb < 4096) {
+                    a.xcd_chunk = (int)((grid.x + 7) / 8);
+                    grid.x = (unsigned)a.xcd_chunk * 8;
+                }
+            }
             if (vec && p.unaligned) row_reduce_kernel<Op, FULL, true><<<grid, block, 0, st>>>(a);
             else if (vec) row_reduce_kernel<Op, FULL><<<grid, block, 0, st>>>(a);
             else row_reduce_kernel<Op, 1><<<grid, block, 0, st>>>(a);
