@@ -71,6 +71,7 @@ SIGNATURES = {
     "hpt_hip_memcpy_d2h_sync": (C.c_int32, [C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t]),
     "hpt_hip_memcpy_d2d_sync": (C.c_int32, [C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t]),
     "hpt_hip_stream_synchronize": (C.c_int32, [C.c_int32, C.c_void_p]),
+    "hpt_hip_device_synchronize": (C.c_int32, [C.c_int32]),
     "hpt_hip_process_axes": (C.c_int32, [C.POINTER(C.c_int64), C.c_int32, C.c_int32, C.POINTER(C.c_int64)]),
     "hpt_hip_reduce_shape": (C.c_int32, [C.POINTER(C.c_int64), C.c_int32, C.POINTER(C.c_int64), C.c_int32,
                                          C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int32)]),

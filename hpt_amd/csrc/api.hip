@@ -212,14 +212,20 @@ static void* scratch_reserve(int dev, StreamScratch& s, size_t bytes) {
     return s.base;
 }
 
-// Give every scratch buffer of `dev` back to its allocator. The caller has made the device idle.
+// Give every scratch buffer of `dev` back to its allocator. The table and every buffer of the device are
+// locked BEFORE the device is waited for and stay locked until the buffers are back: a call on another thread
+// that needs scratch either got its buffer earlier (its kernels are then queued, and waited for here) or
+// blocks until this is over and allocates afresh. (Locks are taken table -> buffer -> allocator everywhere.)
 static void scratch_release_all(int dev) {
     std::lock_guard<std::mutex> gt(g_scratch_table_mu);
+    std::vector<std::unique_lock<std::mutex>> held;
+    for (auto& kv : g_scratch)
+        if (kv.first.first == dev) held.emplace_back(kv.second->mu);
+    hip_check(hipDeviceSynchronize(), HPT_ERR_KERNEL, "hipDeviceSynchronize");
     DeviceAllocator& a = allocator_of(dev);
     for (auto& kv : g_scratch) {
         if (kv.first.first != dev) continue;
         StreamScratch& s = *kv.second;
-        std::lock_guard<std::mutex> gs(s.mu);
         std::lock_guard<std::mutex> ga(a.mu);
         if (s.base) s.retired.emplace_back(s.base, s.bytes);
         for (auto& r : s.retired) {
@@ -561,6 +567,7 @@ int32_t hpt_hip_free(int32_t dev, void* p, size_t bytes, size_t align) {
 int32_t hpt_hip_forget(int32_t dev, void* p) {
     return guarded([&] {
         if (!p) return;
+        use_device(dev);  // (validates `dev`, as hpt_hip_free does)
         DeviceAllocator& a = allocator_of(dev);
         std::lock_guard<std::mutex> g(a.mu);
         (void)a.forget(p);  // a pointer the allocator does not know is left alone, as in the reference
@@ -580,8 +587,7 @@ int32_t hpt_hip_cache_resize(int32_t dev, size_t entries) {
 int32_t hpt_hip_cache_clear(int32_t dev) {
     return guarded([&] {
         use_device(dev);
-        // the scratch buffers go back first; work that uses them may still be queued
-        hip_check(hipDeviceSynchronize(), HPT_ERR_KERNEL, "hipDeviceSynchronize");
+        // the scratch buffers go back first (work that uses them may still be queued: waited for inside)
         scratch_release_all(dev);
         DeviceAllocator& a = allocator_of(dev);
         std::lock_guard<std::mutex> g(a.mu);
@@ -631,6 +637,13 @@ int32_t hpt_hip_stream_synchronize(int32_t dev, void* stream) {
     return guarded([&] {
         use_device(dev);
         hip_check(hipStreamSynchronize((hipStream_t)stream), HPT_ERR_KERNEL, "hipStreamSynchronize");
+    });
+}
+
+int32_t hpt_hip_device_synchronize(int32_t dev) {
+    return guarded([&] {
+        use_device(dev);
+        hip_check(hipDeviceSynchronize(), HPT_ERR_KERNEL, "hipDeviceSynchronize");
     });
 }
 

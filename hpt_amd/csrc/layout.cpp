@@ -856,6 +856,12 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 // with six. Measured, us (768 / 1024 / 1536 workgroups): [8192, 4096] 45.7 / 47.6 / 47.5, [32768, 1024]
                 // 45.1 / 46.2 / 47.1, [65536, 512] 45.0 / 46.4 / 47.4; [16384, 2048] 52.9 / 47.5 / 46.3, [8192, 2048]
                 // 29.1 / 26.2 / 25.2, [8192, 1536] 26.9 / 23.1 / 20.3. Two-byte rows prefetch their next row and stay at 1024.
+                // Two-byte rows with gamma / beta in LDS, up to four vectors per thread: three times as many workgroups
+                // as a compute unit holds at once, so that one that ends early is replaced (with 1024 a workgroup walks
+                // 10 or 11 row pairs and the last step runs two thirds empty). Measured, us (1024 / 1536 / 3072 / all rows):
+                // f16 [21845, 3072] 52.1 / 50.5 / 48.6 / 51.0, [16384, 4096] 50.7 / 54.3 / 48.6 / 51.3, [65536, 1024]
+                // 49.0 / 49.9 / 47.3 / 46.4; rows of five vectors per thread do best with 1024 ([13107, 5120] 53.2 / 61.9 / 59.2 / 64.2).
+                if (n_norm_dims > 0 && p.gb_lds && p.nchunk <= 4 && p.tpr < 512) p.max_blocks = 3072;
                 if (n_norm_dims > 0 && elem_size == 4 && v > 1 && p.tpr <= 256) {
                     // (Few rows: with 1024 every workgroup of [1024, 4096] has one row instead of one or two -
                     // 9.7 -> 8.3 us; [1536, 4096] 13.1 -> 11.6, [3072, 4096] 20.9 -> 20.5, from 4096 rows on no difference.)

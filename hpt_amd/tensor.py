@@ -102,9 +102,19 @@ class _StreamTracked:
         self.pending.add(_stream_key(stream))
 
     def wait(self) -> None:
+        """Wait for every stream that has touched this memory. A stream its owner has destroyed in the
+        meantime cannot be waited for by handle: the whole device is waited for instead (a destroyed
+        stream's work has either finished or is covered by that)."""
         while self.pending:
             k = self.pending.pop()
-            check(_ffi.lib().hpt_hip_stream_synchronize(self.device, C.c_void_p(k) if k else None))
+            try:
+                check(_ffi.lib().hpt_hip_stream_synchronize(self.device, C.c_void_p(k) if k else None))
+            except Exception:
+                check(_ffi.lib().hpt_hip_device_synchronize(self.device))
+
+    def forget_streams(self) -> None:
+        """The caller has waited for (or destroyed) the streams this memory was used on."""
+        self.pending.clear()
 
 
 class _DeviceStorage(_StreamTracked):
@@ -118,13 +128,18 @@ class _DeviceStorage(_StreamTracked):
         self._init_streams()
 
     def __del__(self):
+        if not self.ptr:
+            return
         try:
-            if self.ptr:
-                self.wait()  # kernels still queued on a caller's stream may use the block
-                _ffi.lib().hpt_hip_free(self.device, C.c_void_p(self.ptr), self.nbytes, ALIGN)
-                self.ptr = 0
+            self.wait()  # kernels still queued on a caller's stream may use the block
+        except Exception:
+            pass  # (interpreter shutdown, or the device is gone: nothing more can be waited for)
+        try:
+            # the block always goes back to the allocator, whatever the wait did
+            _ffi.lib().hpt_hip_free(self.device, C.c_void_p(self.ptr), self.nbytes, ALIGN)
         except Exception:
             pass
+        self.ptr = 0
 
 
 class _RawStorage(_StreamTracked):

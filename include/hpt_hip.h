@@ -143,6 +143,11 @@ int32_t hpt_hip_memcpy_d2h_sync(int32_t dev, void* dst, const void* src, size_t 
 int32_t hpt_hip_memcpy_d2d_sync(int32_t dev, void* dst, const void* src, size_t bytes);
 /* Block until everything queued on `stream` has finished. */
 int32_t hpt_hip_stream_synchronize(int32_t dev, void* stream);
+/* Block until everything queued on the device, on any stream, has finished. The reference's device
+ * backend has one stream per device and synchronous copies (hpt/src/backends/cuda/tensor_impls.rs:142-169),
+ * so it never needs this; here streams belong to the caller, and an owner of memory that was used on
+ * a stream which no longer exists has only the whole device to wait for before the block is freed. */
+int32_t hpt_hip_device_synchronize(int32_t dev);
 
 /* ---- host-side shape logic ---------------------------------------------- */
 

@@ -120,3 +120,44 @@ def test_c5_non_contiguous_f16(hpt, orc, dev):
         s0 = f(tv.sum([0]).numpy())
         want = f(orc.reduce(orc.SUM, av, [0], acc=orc.ACC_F32))
         assert_close(s0, want, HALF_RTOL, half_atol(want, 11), name + " sum(axis=0)")
+
+
+def test_reference_published_sum_shape(hpt, orc, dev):
+    """f32 [1024, 1024, 80] summed over the seven axis sets the reference publishes timings for
+    (docs/benchmarks/reduce.md:62-78): every output against numpy's float64 sum of the same elements."""
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((1024, 1024, 80), dtype=np.float32)
+    t = hpt.Tensor.from_numpy(x).to_hip(dev)
+    xd = x.astype(np.float64)
+    for axes in ([0], [1], [2], [0, 1], [0, 2], [1, 2], [0, 1, 2]):
+        got = t.sum(axes).numpy()
+        want = xd.sum(tuple(axes))
+        assert_close(got.reshape(want.shape) if want.shape else got.reshape(()), want, F32_RTOL, F32_ATOL, f"sum over {axes}")
+    # the exactly summed oracle on one output row of each kind (numpy's pairwise f64 sum is the other witness)
+    assert_close(t.sum([0, 2]).numpy()[:8], orc.reduce(orc.SUM, x[:, :8, :], [0, 2], acc=orc.ACC_EXACT), F32_RTOL, F32_ATOL, "sum(0,2) exact")
+    del xd
+
+
+@pytest.mark.parametrize("n", [256, 512])
+def test_reference_published_softmax_shapes(hpt, orc, dev, n):
+    """f32 softmax of n^3 over each axis (docs/benchmarks/normalization.md:55-123): a sample of positions against the
+    f64 oracle, and over the whole output every softmax vector sums to one and keeps the order of its inputs."""
+    rng = np.random.default_rng(12 + n)
+    x = rng.standard_normal((n, n, n), dtype=np.float32) * 2
+    t = hpt.Tensor.from_numpy(x).to_hip(dev)
+    for axis in (0, 1, 2):
+        y = t.softmax(axis).numpy()
+        assert_close(y.sum(axis, dtype=np.float64), np.ones((n, n)), 2e-6, 0, f"softmax({axis}) sums to one")
+        sl = [slice(None)] * 3
+        for d in range(3):
+            if d != axis:
+                sl[d] = slice(n // 2 - 3, n // 2 + 5) if d == (axis + 1) % 3 else slice(0, n, max(1, n // 16))
+        sl = tuple(sl)
+        assert_close(y[sl], orc.softmax(np.ascontiguousarray(x[sl]), axis, acc=orc.ACC_F64), F32_RTOL, F32_ATOL, f"softmax({axis}) sample")
+        # monotone: the largest input of a vector has the largest output
+        assert np.array_equal(y.argmax(axis), x.argmax(axis)) or np.allclose(
+            np.take_along_axis(y, np.expand_dims(x.argmax(axis), axis), axis), y.max(axis, keepdims=True))
+        ly = t.log_softmax(axis).numpy()
+        assert_close(ly[sl], orc.softmax(np.ascontiguousarray(x[sl]), axis, log=True, acc=orc.ACC_F64), F32_RTOL, F32_ATOL,
+                     f"log_softmax({axis}) sample")
+        del y, ly

@@ -53,8 +53,8 @@ def test_reduce_static_matches_reduce_twice_in_a_row(hpt, dev, name, op, dt, sha
         assert g.tobytes() == w.tobytes(), f"{name} {shape}: static scratch result differs from hpt_hip_reduce"
         # and the oracle, so that both being wrong the same way does not pass
         if op == "SUM" and dt == np.float32:
-            ref = orc.reduce(orc.SUM, x, ax, acc=orc.ACC_F64)
-            np.testing.assert_allclose(g, ref.reshape(g.shape), rtol=1e-5, atol=1e-6 * max(1.0, float(np.abs(x).sum()) ** 0.5))
+            ref = orc.reduce(orc.SUM, x, ax, acc=orc.ACC_EXACT)
+            np.testing.assert_allclose(g, ref.reshape(g.shape), rtol=1e-5, atol=1e-6)
         if op == "SUM" and dt == np.uint8:
             assert np.array_equal(g, x.sum(0, dtype=np.uint8))
         del t, want, out, got
