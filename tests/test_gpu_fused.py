@@ -155,3 +155,50 @@ def test_fused_argument_errors(hpt, dev):
         hpt.Tensor.from_numpy(np.zeros(8, np.float32)).to_hip(dev).softmax_causal()
     with pytest.raises(hpt.DTypeError):
         hpt.Tensor.from_numpy(np.zeros((4, 8), np.int32)).to_hip(dev).softmax_causal()
+
+
+CHUNK_CASES = [
+    # every row length from 1 to K: each chunk of a row (the vectors its lanes hold side by side) is met wholly
+    # below the diagonal, wholly above it and cut by it, at every position of the cut
+    ("f32 2048 keys, one wavefront per row", np.float32, [2, 2048, 2048], 1.0, 0),
+    ("f32 2048 keys, diagonal shifted by one", np.float32, [1, 2048, 2048], 0.5, 1),
+    ("f32 2048 keys, first row without keys", np.float32, [1, 2048, 2048], 0.5, -1),
+    ("f32 256 keys, several rows per wavefront", np.float32, [3, 512, 256], 0.25, -100),
+    ("f32 1000 keys (not a power of two), more queries than keys", np.float32, [2, 1500, 1000], 1.0, 0),
+    ("f16 2048 keys", np.float16, [2, 2048, 2048], 0.125, 0),
+    ("bf16 2048 keys", "bf16", [2, 2048, 2048], 0.125, 0),
+    ("bf16 4096 keys, two wavefronts per row", "bf16", [1, 1024, 4096], 0.125, 3072),
+    ("f16 320 keys, several rows per wavefront", np.float16, [4, 320, 320], 1.0, 0),
+]
+
+
+@pytest.mark.parametrize("log", [False, True])
+@pytest.mark.parametrize("case", CHUNK_CASES, ids=[c[0] for c in CHUNK_CASES])
+def test_softmax_causal_every_row_length(hpt, orc, dev, case, log):
+    name, npdt, shape, scale, offset = case
+    rng = np.random.default_rng(402)
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    if npdt == "bf16":
+        base, dt, bits, tof, bf, acc = hpt.f32_to_bf16_bits(x), hpt.bf16, 8, hpt.bf16_bits_to_f32, True, orc.ACC_F32
+    elif npdt == np.float16:
+        base, dt, bits, tof, bf, acc = x.astype(np.float16), None, 11, (lambda v: v.astype(np.float32)), False, orc.ACC_F32
+    else:
+        base, dt, bits, tof, bf, acc = x, None, 0, (lambda v: v), False, orc.ACC_F64
+    t = hpt.Tensor.from_numpy(base, dt).to_hip(dev)
+    got = tof(t.softmax_causal(scale, offset, log=log).numpy())
+    xs, want = causal_reference(orc, base, scale, offset, log, bf16=bf, acc=acc)
+    want = tof(want)
+    xs = tof(xs) if bf or bits else xs
+    dead = np.all(np.isneginf(xs), axis=-1)
+    assert np.all(np.isnan(got[dead])), f"{name}: rows without keys must be NaN"
+    if bits:
+        atol = max(half_atol(want[~dead][np.isfinite(want[~dead])], bits), 6e-8 if npdt == np.float16 else 0.0)
+        assert_close(got[~dead], want[~dead], HALF_RTOL, atol, f"{name} log={log}")
+    else:
+        assert_close(got[~dead], want[~dead], F32_RTOL, F32_ATOL, f"{name} log={log}")
+    q = np.arange(shape[-2])[:, None]
+    k = np.arange(shape[-1])[None, :]
+    m = np.broadcast_to(k > q + offset, shape) & ~dead[..., None]
+    assert np.all(np.isneginf(got[m]) if log else got[m] == 0), f"{name}: masked keys must come out exactly 0 / -inf"
+    if not log:
+        assert_close(got[~dead].astype(np.float64).sum(-1), np.ones(int((~dead).sum())), 2 ** -bits if bits else 2e-6, 0, f"{name}: rows sum to one")

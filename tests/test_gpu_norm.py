@@ -751,3 +751,33 @@ def test_long_rows_of_random_length_and_alignment(hpt, orc, dev, seed):
             else:
                 assert_close(got, want, F32_RTOL, 2 * F32_ATOL if log else F32_ATOL, f"log={log} {what}")
     assert any(p.startswith("rowreg-lds") for p in seen), seen
+
+
+WIDE_AXIS_CASES = [
+    # four-byte axes of 257 ... 512 elements with a wide inner dim: 128 registers of raw values per thread
+    ([2, 512, 2048], 1), ([3, 257, 1024], 1), ([384, 8192], 0), ([1, 300, 4096], 1), ([5, 512, 64, 32], 1),
+]
+
+
+@pytest.mark.parametrize("case", WIDE_AXIS_CASES, ids=[str(c[0]) for c in WIDE_AXIS_CASES])
+def test_softmax_over_a_strided_axis_of_up_to_512_in_registers(hpt, orc, dev, case):
+    shape, axis = case
+    rng = np.random.default_rng(611)
+    x = (rng.standard_normal(shape) * 4).astype(np.float32)
+    x[..., 0] += 30  # one inner position with a dominating band: the maximum matters
+    t = hpt.Tensor.from_numpy(x).to_hip(dev)
+    plan = hpt.normalize_plan(t, axis)
+    assert plan.startswith("col-reg") and "nchunk=32" in plan, plan
+    for log in (False, True):
+        got = (t.log_softmax(axis) if log else t.softmax(axis)).numpy()
+        assert_close(got, orc.softmax(x, axis, log=log, acc=orc.ACC_F64), F32_RTOL, F32_ATOL, f"{shape} axis={axis} log={log}")
+    # -inf entries and a position whose whole axis is -inf (NaN, as the reference's x - max gives)
+    x[..., 5] = -np.inf
+    idx = [slice(None)] * len(shape)
+    idx[axis] = slice(0, shape[axis] // 2)
+    x[tuple(idx)][..., 7] = -np.inf
+    t = hpt.Tensor.from_numpy(x).to_hip(dev)
+    got = t.softmax(axis).numpy()
+    want = orc.softmax(x, axis, acc=orc.ACC_F64)
+    assert_close(got, want, F32_RTOL, F32_ATOL, f"{shape} axis={axis} with -inf")
+    assert np.isnan(got[..., 5]).all()

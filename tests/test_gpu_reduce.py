@@ -543,3 +543,28 @@ def test_empty_and_degenerate(hpt, orc, dev):
         one.sum([3])
     with pytest.raises(hpt.ParamError, match="Axis 1 is duplicated"):
         one.sum([1, 1])
+
+
+XCD_ROW_CASES = [
+    # neighbouring outputs whose runs lie back to back (general row kernel, row blocks numbered per XCD):
+    # output counts that are and are not multiples of eight, with and without a split of the reduced range
+    ([37, 67, 80], [0, 2]), ([64, 1000, 20], [0, 2]), ([9, 130, 7, 12], [0, 3]), ([4096, 70, 24], [0, 2]),
+    ([3, 200, 5, 16], [0, 2]), ([1024, 65, 80], [0, 2]), ([16, 513, 33], [0, 2]),
+]
+
+
+@pytest.mark.parametrize("case", XCD_ROW_CASES, ids=[f"{c[0]} over {c[1]}" for c in XCD_ROW_CASES])
+def test_neighbouring_outputs_with_runs_back_to_back(hpt, orc, dev, case):
+    shape, axes = case
+    rng = np.random.default_rng(77)
+    xi = rng.integers(-1000, 1001, shape).astype(np.int32)
+    ti = hpt.Tensor.from_numpy(xi).to_hip(dev)
+    assert np.array_equal(ti.sum(axes).numpy(), xi.sum(tuple(axes), dtype=np.int32)), "i32 sum"
+    assert np.array_equal(ti.max(axes).numpy(), xi.max(tuple(axes))), "i32 max"
+    x = rng.standard_normal(shape).astype(np.float32)
+    t = hpt.Tensor.from_numpy(x).to_hip(dev)
+    assert_close(t.sum(axes).numpy(), orc.reduce(orc.SUM, x, axes, acc=orc.ACC_EXACT), F32_RTOL, F32_ATOL, "f32 sum")
+    assert_close(t.mean(axes).numpy(), orc.reduce(orc.MEAN, x, axes, acc=orc.ACC_EXACT), F32_RTOL, F32_ATOL, "f32 mean")
+    h = x.astype(np.float16)
+    th = hpt.Tensor.from_numpy(h).to_hip(dev)
+    assert np.array_equal(th.max(axes).numpy(), h.max(tuple(axes))), "f16 max"
