@@ -496,6 +496,12 @@ static bool lds_row_shape(NormPlan& p, int64_t nvec, size_t elem_size, bool shif
     } else if (nvec <= 512 * per) {
         p.tpr = 512;
         p.nchunk = per;
+    } else if (nvec <= 1024 * per) {
+        // one workgroup fills the compute unit either way; sixteen wavefronts of 128 registers keep more loads and
+        // stores in flight than eight of 256 (f32 [1024, 128256] log_softmax 217 -> 208 us, f16 [2048, 151936] 262 -> 249,
+        // f32 [1024, 100277] 183 -> 171, [2048, 69632] 237 -> 224)
+        p.tpr = 1024;
+        p.nchunk = per;
     } else if (nvec <= 512 * big) {
         p.tpr = 512;
         p.nchunk = big;

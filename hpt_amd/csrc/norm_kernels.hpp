@@ -530,6 +530,11 @@ __global__ void __launch_bounds__(NT, MINW) row_lds_kernel(const NormArgs a) {
         // forty-odd 64-bit addresses per lane, computed ahead of the row loop, would not fit beside the row
         auto chunk_of = [](auto* p, int c) { return p + (int64_t)c * (NT * VEC); };
         const unsigned lane_off = (unsigned)tx * VEC;
+        // The LDS part arrives by LDS-direct loads, which the LOAD counter tracks, not the LDS one. Whether the compiler
+        // waits for them before an ordinary LDS read of the same slot depends on what it can prove about the two
+        // addresses (a working build that issued the loads from inside a lambda lost that wait, and the sweeps read slots
+        // that had not arrived). The wait is therefore written out, before the first LDS read of a row.
+        auto wait_for_lds_part = [] { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
         Pack<T, VEC> reg[NREG];
         {
 #pragma unroll kLdsUnroll
@@ -546,6 +551,7 @@ __global__ void __launch_bounds__(NT, MINW) row_lds_kernel(const NormArgs a) {
                 if (iv < nv && touches(iv)) reg[c] = load_pack_stream<T, VEC>(chunk_of(in_row - sh, c) + lane_off);
             }
             if constexpr (SHIFT) {
+                wait_for_lds_part();
 #pragma unroll kLdsUnroll
                 for (int c = 0; c < NLDS; ++c) {
                     const int iv = (NREG + c) * NT + tx;
@@ -565,6 +571,7 @@ __global__ void __launch_bounds__(NT, MINW) row_lds_kernel(const NormArgs a) {
             if (c * NT + tx < nv)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) m = MaxC<CT>::comb(m, Elem<T>::widen(reg[c].v[j]));
+        if constexpr (!SHIFT) wait_for_lds_part();
 #pragma unroll kLdsUnroll
         for (int c = 0; c < NLDS; ++c)
             if ((NREG + c) * NT + tx < nv) {

@@ -293,6 +293,10 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
                     row_lds_kernel<KIND, T, kRegs, 8, false, 512, 4><<<grid, dim3(512), 0, st>>>(a);
                     return;
                 }
+                if (p.nchunk == kRegs + 8 && p.tpr == 1024) {
+                    row_lds_kernel<KIND, T, kRegs, 8, false, 1024, 1><<<grid, dim3(1024), 0, st>>>(a);
+                    return;
+                }
                 if (p.nchunk == 2 * kRegs + 16 && p.tpr == 512) {
                     row_lds_kernel<KIND, T, 2 * kRegs, 16, false, 512, 1><<<grid, dim3(512), 0, st>>>(a);
                     return;
@@ -304,6 +308,10 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
                 }
                 if (p.nchunk == kRegsShift + 8 && p.tpr == 512) {
                     row_lds_kernel<KIND, T, kRegsShift, 8, true, 512, 4><<<grid, dim3(512), 0, st>>>(a);
+                    return;
+                }
+                if (p.nchunk == kRegsShift + 8 && p.tpr == 1024) {
+                    row_lds_kernel<KIND, T, kRegsShift, 8, true, 1024, 1><<<grid, dim3(1024), 0, st>>>(a);
                     return;
                 }
                 if (p.nchunk == kBigShift + 16 && p.tpr == 512) {

@@ -102,17 +102,17 @@ def test_plans_for_shapes_off_the_benchmark_list(hpt):
         # (shape, dtype, axis, n_norm_dims, plan prefix)
         ([1016800, 33], None, 1, 0, "rowreg+tile"), ([1016800, 33], None, 0, 1, "rowreg+tile"),
         ([262144, 128], None, 1, 0, "rowreg rows"),                 # whole vectors, 512 bytes: registers
-        ([8190, 4097], None, 1, 0, "rowreg-shift"), ([1043, 50257], None, 1, 0, "rowreg-lds-shift"), ([1043, 70001], None, 1, 0, "rowreg-lds-shift rows=1043 cols=70001 vec=4 tpr=512 rpb=1 nchunk=60"), ([1043, 122849], None, 1, 0, "rowreg-lds-shift"), ([1043, 122850], None, 1, 0, "rowstream-shift"),
+        ([8190, 4097], None, 1, 0, "rowreg-shift"), ([1043, 50257], None, 1, 0, "rowreg-lds-shift"), ([1043, 70001], None, 1, 0, "rowreg-lds-shift rows=1043 cols=70001 vec=4 tpr=1024 rpb=1 nchunk=28"), ([1043, 122849], None, 1, 0, "rowreg-lds-shift"), ([1043, 122850], None, 1, 0, "rowstream-shift"),
         ([3355, 10000], None, 1, 0, "rowreg rows=3355 cols=10000 vec=4 tpr=512 rpb=1 nchunk=5"), ([3355, 12000], None, 1, 0, "rowreg rows=3355 cols=12000 vec=4 tpr=512 rpb=1 nchunk=6"),
-        ([512, 65536], None, 1, 0, "rowreg-lds rows=512 cols=65536 vec=4 tpr=512 rpb=1 nchunk=32"), ([512, 65540], None, 1, 0, "rowreg-lds rows=512 cols=65540 vec=4 tpr=512 rpb=1 nchunk=64"),
-        ([512, 131072], None, 1, 0, "rowreg-lds rows=512 cols=131072 vec=4 tpr=512"), ([512, 131076], None, 1, 0, "rowstream"), ([512, 65540], None, 0, 1, "rowstream"),
+        ([512, 65536], None, 1, 0, "rowreg-lds rows=512 cols=65536 vec=4 tpr=512 rpb=1 nchunk=32"), ([512, 65540], None, 1, 0, "rowreg-lds rows=512 cols=65540 vec=4 tpr=1024 rpb=1 nchunk=32"),
+        ([512, 131072], None, 1, 0, "rowreg-lds rows=512 cols=131072 vec=4 tpr=1024 rpb=1 nchunk=32"), ([512, 131076], None, 1, 0, "rowstream"), ([512, 65540], None, 0, 1, "rowstream"),
         # rows that leave a sixteenth of a power-of-two row's slots idle, and odd lengths beyond 2048 vectors: 256 threads
         ([4096, 16388], None, 1, 0, "rowreg-lds rows=4096 cols=16388 vec=4 tpr=256 rpb=1 nchunk=32"), ([4096, 32768], None, 1, 0, "rowreg rows=4096 cols=32768 vec=4 tpr=1024 rpb=1 nchunk=8"),
         ([4096, 30522], None, 1, 0, "rowreg-lds-shift rows=4096 cols=30522 vec=4 tpr=512 rpb=1 nchunk=28"), ([8192, 32001], hpt.f16, 1, 0, "rowreg-lds-shift rows=8192 cols=32001 vec=8 tpr=256 rpb=1 nchunk=24"),
         ([8192, 16392], hpt.f16, 1, 0, "rowreg-lds rows=8192 cols=16392 vec=8 tpr=256 rpb=1 nchunk=24"), ([4096, 50304], hpt.f16, 1, 0, "rowreg-lds rows=4096 cols=50304 vec=8 tpr=512 rpb=1 nchunk=24"),
         ([4096, 8197], None, 1, 0, "rowreg-lds-shift rows=4096 cols=8197 vec=4 tpr=256"), ([4096, 8189], None, 1, 0, "rowreg-shift"),
-        ([512, 131072], hpt.f16, 1, 0, "rowreg-raw"), ([512, 151936], hpt.f16, 1, 0, "rowreg-lds rows=512 cols=151936 vec=8 tpr=512 rpb=1 nchunk=48"),
-        ([512, 196608], hpt.bf16, 1, 0, "rowreg-lds"), ([512, 196616], hpt.bf16, 1, 0, "rowstream"), ([512, 150001], hpt.f16, 1, 0, "rowreg-lds-shift rows=512 cols=150001 vec=8 tpr=512 rpb=1 nchunk=48"),
+        ([512, 131072], hpt.f16, 1, 0, "rowreg-raw"), ([512, 151936], hpt.f16, 1, 0, "rowreg-lds rows=512 cols=151936 vec=8 tpr=1024 rpb=1 nchunk=24"),
+        ([512, 196608], hpt.bf16, 1, 0, "rowreg-lds"), ([512, 196616], hpt.bf16, 1, 0, "rowstream"), ([512, 150001], hpt.f16, 1, 0, "rowreg-lds-shift rows=512 cols=150001 vec=8 tpr=1024 rpb=1 nchunk=24"),
         ([512, 196545], hpt.f16, 1, 0, "rowreg-lds-shift"), ([512, 196546], hpt.f16, 1, 0, "rowstream-shift"), ([32, 1048576], None, 1, 0, "rowsplit"),
         # rows of 3, 5, 6, 7 times a power of two: that many vectors per thread
         ([4096, 768], hpt.f16, 0, 1, "rowreg-ldsgb rows=4096 cols=768 vec=8 tpr=32 rpb=8 nchunk=3"), ([4096, 384], hpt.f16, 0, 1, "rowreg rows=4096 cols=384 vec=8 tpr=16 rpb=16 nchunk=3"), ([4096, 1536], None, 1, 0, "rowreg rows=4096 cols=1536 vec=4 tpr=128 rpb=2 nchunk=3"),
