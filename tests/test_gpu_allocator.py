@@ -118,3 +118,74 @@ def test_round_trip_and_tensor_lifetime(hpt, dev):
     del v
     gc.collect()
     assert stats(hpt, dev)[0] == live0
+
+
+def test_storage_is_freed_after_its_stream_is_gone(hpt, dev):
+    """A tensor used on a caller's stream that the caller destroys before the tensor dies: the per-stream wait
+    can fail, the whole device is waited for instead, and the block still goes back to the allocator."""
+    import gc
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipStreamCreate.argtypes = [C.POINTER(C.c_void_p)]
+    hip.hipStreamDestroy.argtypes = [C.c_void_p]
+    hip.hipStreamSynchronize.argtypes = [C.c_void_p]
+    gc.collect()
+    live0 = stats(hpt, dev)[0]
+    s = C.c_void_p()
+    assert hip.hipStreamCreate(C.byref(s)) == 0
+    x = np.random.default_rng(3).standard_normal((64, 4096)).astype(np.float32)
+    t = hpt.Tensor.from_numpy(x).to_hip(dev)
+    y = t.softmax(1, stream=s)
+    z = t.sum([0, 1], stream=s)     # a split reduction: per-stream scratch as well
+    assert hip.hipStreamSynchronize(s) == 0
+    got = y.numpy()
+    assert abs(float(got.sum()) - 64.0) < 1e-3
+    assert hip.hipStreamDestroy(s) == 0
+    assert stats(hpt, dev)[0] >= live0 + 3
+    del t, y, z
+    gc.collect()
+    assert stats(hpt, dev)[0] == live0, "blocks used on a destroyed stream were not returned"
+
+
+def test_device_synchronize_and_device_checks(hpt, dev):
+    l = hpt.lib()
+    assert l.hpt_hip_device_synchronize(dev) == 0
+    n = hpt.device_count()
+    for bad in (-1, n, n + 7):
+        assert l.hpt_hip_device_synchronize(bad) != 0
+        assert b"does not exist" in l.hpt_hip_last_error()
+        # forget validates the device like free does (a foreign pointer is otherwise left alone)
+        assert l.hpt_hip_forget(bad, C.c_void_p(0x1000)) != 0
+    assert l.hpt_hip_forget(dev, C.c_void_p(0x1000)) == 0
+
+
+def test_cache_clear_while_other_threads_reduce(hpt, orc, dev):
+    """cache_clear hands the scratch buffers back while other host threads keep running split reductions (which use
+    them): every result stays right, and nothing is handed out twice."""
+    import threading
+    rng = np.random.default_rng(5)
+    xs = [rng.integers(-1000, 1001, (3, 1 << 18)).astype(np.int32) for _ in range(3)]
+    want = [x.sum(dtype=np.int32) for x in xs]
+    errors, stop = [], threading.Event()
+
+    def worker(k):
+        try:
+            t = hpt.Tensor.from_numpy(xs[k]).to_hip(dev)
+            while not stop.is_set():
+                got = t.sum([0, 1]).numpy()
+                if int(got[0]) != int(want[k]):
+                    errors.append((k, int(got[0]), int(want[k])))
+                    return
+        except Exception as e:  # noqa: BLE001
+            errors.append((k, repr(e)))
+
+    th = [threading.Thread(target=worker, args=(k,)) for k in range(3)]
+    for t in th:
+        t.start()
+    try:
+        for _ in range(40):
+            assert hpt.lib().hpt_hip_cache_clear(dev) == 0
+    finally:
+        stop.set()
+        for t in th:
+            t.join()
+    assert not errors, errors[:3]
