@@ -169,6 +169,17 @@ CHUNK_CASES = [
     ("bf16 2048 keys", "bf16", [2, 2048, 2048], 0.125, 0),
     ("bf16 4096 keys, two wavefronts per row", "bf16", [1, 1024, 4096], 0.125, 3072),
     ("f16 320 keys, several rows per wavefront", np.float16, [4, 320, 320], 1.0, 0),
+    # rows dealt out by live length (one wavefront per full row): every class boundary, offsets either way,
+    # more queries than keys, a query count that no class divides
+    ("f32 1024 keys, 1024 queries", np.float32, [3, 1024, 1024], 1.0, 0),
+    ("f32 1024 keys, offset -5", np.float32, [2, 1024, 1024], 0.5, -5),
+    ("f32 1024 keys, offset 300", np.float32, [2, 1024, 1024], 0.5, 300),
+    ("f32 768 keys (three vectors per thread), 1000 queries", np.float32, [2, 1000, 768], 1.0, -232),
+    ("bf16 2048 keys, offset -100", "bf16", [2, 2048, 2048], 0.125, -100),
+    ("bf16 2048 keys, offset 700", "bf16", [2, 2048, 2048], 0.125, 700),
+    ("f16 2048 keys, 512 queries at the end (offset K - Q)", np.float16, [3, 512, 2048], 0.25, 1536),
+    ("f16 2048 keys, 2101 queries", np.float16, [1, 2101, 2048], 1.0, 0),
+    ("bf16 2048 keys, nothing kept in most rows", "bf16", [2, 2048, 2048], 1.0, -1900),
 ]
 
 
