@@ -1000,7 +1000,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 int64_t g = L, b = max_vec;
                 while (b) { int64_t t = g % b; g = b; b = t; }
                 const int64_t lp = L / g;  // threads per period
-                int64_t tmax = std::min<int64_t>(1024, (64 << 10) / (max_vec * (elem_size == 8 ? 16 : 8)));
+                int64_t tmax = std::min<int64_t>(1024, (64 << 10) / (max_vec * (elem_size >= 4 ? 16 : 8)));
                 // (each batch slab must be worth at least two periods of the walk: small slabs, of which there
                 // are many, take fewer threads each)
                 tmax = std::min(tmax, p.cols * L / (2 * max_vec));

@@ -70,6 +70,10 @@ template <class T> struct StatType { using type = float; };
 template <> struct StatType<float> { using type = double; };
 template <> struct StatType<double> { using type = double; };
 
+// (The kernels that sum exponentials one lane at a time carry that sum in StatType too: a long chain
+// of f32 additions next to a total near 1, as when one element dominates its row, loses ~6e-8 per step,
+// which shows in log_softmax results close to zero.)
+
 // All-reduce over the `tpr` lanes that share a row: shuffles inside a wavefront,
 // LDS across the wavefronts of the row. Every thread of the workgroup must call it.
 template <class Op, class A>
@@ -828,8 +832,10 @@ __global__ void __launch_bounds__(256) norm_group_tile_kernel(const NormArgs a, 
         const int base = g * G + i;
         CT m = neg_inf<CT>();
         for (int c = 0; c < C; ++c) m = MaxC<CT>::comb(m, Elem<T>::widen(tile[pad(base + c * L)]));
-        CT s = 0;
-        for (int c = 0; c < C; ++c) s += exp_ct<T>(Elem<T>::widen(tile[pad(base + c * L)]) - m);
+        using ST = typename StatType<T>::type;
+        ST total = 0;
+        for (int c = 0; c < C; ++c) total += (ST)exp_ct<T>(Elem<T>::widen(tile[pad(base + c * L)]) - m);
+        const CT s = (CT)total;
         const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
         for (int c = 0; c < C; ++c) {
             T* q = tile + pad(base + c * L);
@@ -889,9 +895,10 @@ __global__ void __launch_bounds__(256) norm_slab_kernel(const NormArgs a, int L,
         CT m = neg_inf<CT>();
         for (int c = lane; c < C; c += tpc) m = MaxC<CT>::comb(m, Elem<T>::widen(p[c * L]));
         m = group_reduce<MaxC<CT>>(m, tpc);
-        CT s = 0;
-        for (int c = lane; c < C; c += tpc) s += exp_ct<T>(Elem<T>::widen(p[c * L]) - m);
-        s = group_reduce<SumC<CT>>(s, tpc);
+        using ST = typename StatType<T>::type;
+        ST total = 0;
+        for (int c = lane; c < C; c += tpc) total += (ST)exp_ct<T>(Elem<T>::widen(p[c * L]) - m);
+        const CT s = (CT)group_reduce<SumC<ST>>(total, tpc);
         const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
         for (int c = lane; c < C; c += tpc) {
             const CT d = Elem<T>::widen(p[c * L]) - m;

@@ -42,7 +42,7 @@ struct TransposedArgs {
 };
 
 // A partial row statistic over some of the columns.
-//   softmax  : (max, sum of exp(x - max)); merged with SoftStatOp.
+//   softmax  : (max, sum of exp(x - max)), the sum in StatType; merged with SoftStatOp.
 //   layernorm: (sum of (x - k), sum of (x - k)^2) with k the row's FIRST element,
 //              the same shift for every partial of the row, so that partials
 //              merge by plain addition and only the last step divides.
@@ -51,7 +51,8 @@ template <class CT> struct ShiftedSums {
 };
 template <int KIND, class T> struct RowPartial {
     using CT = typename Elem<T>::Wide;
-    using type = typename std::conditional<KIND == NORM_LAYERNORM, ShiftedSums<CT>, SoftStat<CT>>::type;
+    using ST = typename StatType<T>::type;  // the sum of exponentials of f32 rows is carried in f64
+    using type = typename std::conditional<KIND == NORM_LAYERNORM, ShiftedSums<CT>, SoftStat<CT, ST>>::type;
 };
 
 // Pass 1: partial row statistics. Lanes run along the rows (a wavefront reads 1 KiB
@@ -63,6 +64,7 @@ template <int KIND, class T, int VEC = 16 / sizeof(T)>
 __global__ void __launch_bounds__(1024) transposed_stats_kernel(const TransposedArgs a) {
     using CT = typename Elem<T>::Wide;
     using Part = typename RowPartial<KIND, T>::type;
+    using ST = typename StatType<T>::type;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int NW = blockDim.x >> 6;  // wavefronts per workgroup (1...16)
 
@@ -82,6 +84,7 @@ __global__ void __launch_bounds__(1024) transposed_stats_kernel(const Transposed
 
     // per row: softmax (m, s); layernorm s = sum (x - k), s2 = sum (x - k)^2, k = x[row][0]
     CT m[VEC], s[VEC], s2[VEC];
+    ST se[VEC];  // softmax: the sum of exponentials
     if constexpr (KIND == NORM_LAYERNORM) {
         Pack<T, VEC> f = load_pack<T, VEC>(base);
 #pragma unroll
@@ -94,6 +97,7 @@ __global__ void __launch_bounds__(1024) transposed_stats_kernel(const Transposed
     for (int k = 0; k < VEC; ++k) {
         s[k] = 0;
         s2[k] = 0;
+        se[k] = 0;
     }
     auto fold = [&](const Pack<T, VEC>* v, auto cnt_tag) {
         constexpr int CNT = decltype(cnt_tag)::value;
@@ -113,12 +117,12 @@ __global__ void __launch_bounds__(1024) transposed_stats_kernel(const Transposed
 #pragma unroll
                 for (int i = 0; i < CNT; ++i) bm = MaxC<CT>::comb(bm, Elem<T>::widen(v[i].v[k]));
                 if (bm > m[k]) {
-                    s[k] = s[k] == (CT)0 ? (CT)0 : s[k] * exp_ct<T>(m[k] - bm);
+                    se[k] = se[k] == (ST)0 ? (ST)0 : se[k] * (ST)exp_ct<T>(m[k] - bm);
                     m[k] = bm;
                 }
                 if (m[k] > neg_inf<CT>()) {
 #pragma unroll
-                    for (int i = 0; i < CNT; ++i) s[k] += exp_ct<T>(Elem<T>::widen(v[i].v[k]) - m[k]);
+                    for (int i = 0; i < CNT; ++i) se[k] += (ST)exp_ct<T>(Elem<T>::widen(v[i].v[k]) - m[k]);
                 }
             }
         }
@@ -153,7 +157,7 @@ __global__ void __launch_bounds__(1024) transposed_stats_kernel(const Transposed
             t.s2 = s2[k];
         } else {
             t.m = m[k];
-            t.s = s[k];
+            t.s = se[k];
         }
         sm[(w * VEC + k) * 64 + lane] = t;
     }
@@ -168,7 +172,7 @@ __global__ void __launch_bounds__(1024) transposed_stats_kernel(const Transposed
                 t.s1 += u.s1;
                 t.s2 += u.s2;
             } else {
-                t = SoftStatOp<T, CT>::comb(t, u);
+                t = SoftStatOp<T, CT, ST>::comb(t, u);
             }
         }
         dst[k] = t;
@@ -199,8 +203,8 @@ __global__ void __launch_bounds__(256) transposed_finalize_kernel(const Transpos
                 acc0 += (ST)t.s1;
                 acc1 += (ST)t.s2;
             } else {
-                SoftStat<CT> x{(CT)acc0, (CT)acc1};
-                x = SoftStatOp<T, CT>::comb(x, t);
+                SoftStat<CT, ST> x{(CT)acc0, acc1};
+                x = SoftStatOp<T, CT, ST>::comb(x, t);
                 acc0 = x.m;
                 acc1 = x.s;
             }
@@ -224,8 +228,8 @@ __global__ void __launch_bounds__(256) transposed_finalize_kernel(const Transpos
             acc0 += sm0[y][threadIdx.x];
             acc1 += sm1[y][threadIdx.x];
         } else {
-            SoftStat<CT> x{(CT)acc0, (CT)acc1}, t{(CT)sm0[y][threadIdx.x], (CT)sm1[y][threadIdx.x]};
-            x = SoftStatOp<T, CT>::comb(x, t);
+            SoftStat<CT, ST> x{(CT)acc0, acc1}, t{(CT)sm0[y][threadIdx.x], sm1[y][threadIdx.x]};
+            x = SoftStatOp<T, CT, ST>::comb(x, t);
             acc0 = x.m;
             acc1 = x.s;
         }
@@ -372,15 +376,14 @@ struct ColRegArgs {
     int ty_log2;    // log2 of the thread rows that share an inner position
 };
 
-// Make the compiler forget what it knows about a pack of 2-byte elements: between two sweeps over
-// the raw values it would otherwise keep the widened (f32) copies of the first sweep alive for the
-// second, at twice the registers of the values themselves. Widening again costs one conversion.
+// Make the compiler forget what it knows about a pack: between two sweeps over the raw values it
+// would otherwise keep what the first sweep derived from them (the widened f32 copies of 2-byte
+// elements, x - max) alive for the second, at up to twice the registers of the values themselves.
+// Deriving again costs an instruction.
 template <class T, int N> __device__ __forceinline__ void forget_pack(Pack<T, N>& v) {
-    if constexpr (sizeof(T) == 2) {
-        if constexpr (sizeof(T) * N == 16) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&v)));
-        else if constexpr (sizeof(T) * N == 8) asm volatile("" : "+v"(*reinterpret_cast<u32x2*>(&v)));
-        else if constexpr (sizeof(T) * N == 4) asm volatile("" : "+v"(*reinterpret_cast<uint32_t*>(&v)));
-    }
+    if constexpr (sizeof(T) * N == 16) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&v)));
+    else if constexpr (sizeof(T) * N == 8) asm volatile("" : "+v"(*reinterpret_cast<u32x2*>(&v)));
+    else if constexpr (sizeof(T) * N == 4) asm volatile("" : "+v"(*reinterpret_cast<uint32_t*>(&v)));
 }
 
 // UA: the inner dim is not whole, aligned vectors (an odd length, odd strides): unaligned vectors all the
@@ -390,6 +393,7 @@ template <int KIND, class T, int EV, int NC, bool UA = false>
 __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
     static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX, "a softmax kernel");
     using CT = typename Elem<T>::Wide;
+    using ST = typename StatType<T>::type;
     constexpr bool kLog = KIND == NORM_LOGSOFTMAX;
     __shared__ CT sm[256 * EV];
     const int TY = 1 << a.ty_log2;
@@ -421,21 +425,35 @@ __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
             if constexpr (UA) raw[i] = load_pack_unaligned<T, EV>(in + (int64_t)(ty + (i << a.ty_log2)) * a.sa);
             else raw[i] = load_pack_stream<T, EV>(in + (int64_t)(ty + (i << a.ty_log2)) * a.sa);
         }
-    // all-reduce over the thread rows of an inner position
+    // All-reduce over the thread rows of an inner position. With TX < 64 a wavefront holds 64 / TX of
+    // them, TX lanes apart: those meet in a shuffle butterfly, and only one partial row per wavefront
+    // goes through LDS (for sixteen thread rows, 4 LDS reads per value instead of 16). Every thread of
+    // an inner position ends with the same bits: the butterfly adds the same pairs in every lane.
+    const int rpw = TX < 64 ? 64 / TX : 1;  // thread rows per wavefront
+    const int nrow = TY / rpw;              // partial rows left after the butterfly
+    const int prow = ty / rpw;
     auto across = [&](CT(&v)[EV], auto op) {
         if (TY == 1) return;
+        if (TX <= 16)
 #pragma unroll
-        for (int k = 0; k < EV; ++k) sm[(ty * TX + tx) * EV + k] = v[k];
+            for (int k = 0; k < EV; ++k) v[k] = op(v[k], shfl_xor_any(v[k], 16));
+        if (TX <= 32)
+#pragma unroll
+            for (int k = 0; k < EV; ++k) v[k] = op(v[k], shfl_xor_any(v[k], 32));
+        if (nrow == 1) return;
+#pragma unroll
+        for (int k = 0; k < EV; ++k) sm[(prow * TX + tx) * EV + k] = v[k];
         __syncthreads();
 #pragma unroll
         for (int k = 0; k < EV; ++k) {
             CT r = sm[tx * EV + k];
-            for (int y = 1; y < TY; ++y) r = op(r, sm[(y * TX + tx) * EV + k]);
+            for (int y = 1; y < nrow; ++y) r = op(r, sm[(y * TX + tx) * EV + k]);
             v[k] = r;
         }
         __syncthreads();
     };
-    CT m[EV], s[EV], kk[EV];
+    CT m[EV], kk[EV], sf[EV];
+    ST s[EV];  // this thread's sum of exponentials, carried in the wider type
 #pragma unroll
     for (int k = 0; k < EV; ++k) {
         m[k] = neg_inf<CT>();
@@ -459,17 +477,24 @@ __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
 #pragma unroll
             for (int k = 0; k < EV; ++k) {
                 const CT e = exp_ct<T>(Elem<T>::widen(raw[i].v[k]) - m[k]);
-                s[k] += e;
+                s[k] += (ST)e;
                 if constexpr (kKeepExp) raw[i].v[k] = Elem<T>::narrow(e);
             }
-    across(s, [](CT x, CT y) { return x + y; });
+    // (the thread's total is rounded to the compute type once; the thread rows then add up along a tree)
+#pragma unroll
+    for (int k = 0; k < EV; ++k) sf[k] = (CT)s[k];
+    across(sf, [](CT x, CT y) { return x + y; });
 #pragma unroll
     for (int i = 0; i < NC; ++i) forget_pack(raw[i]);
+    // (likewise the channel indices and the `i < mine` masks of the load sweep: carried to the store sweep
+    // they cost a register per chunk; recomputing them is an instruction each)
+    int ty_st = ty, mine_st = mine;
+    asm volatile("" : "+v"(ty_st), "+v"(mine_st));
 #pragma unroll
-    for (int k = 0; k < EV; ++k) kk[k] = kLog ? log_ct<T>(s[k]) : (CT)1 / s[k];
+    for (int k = 0; k < EV; ++k) kk[k] = kLog ? log_ct<T>(sf[k]) : (CT)1 / sf[k];
 #pragma unroll
     for (int i = 0; i < NC; ++i)
-        if (i < mine) {
+        if (i < mine_st) {
             Pack<T, EV> o;
 #pragma unroll
             for (int k = 0; k < EV; ++k) {
@@ -480,7 +505,7 @@ __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
                     o.v[k] = Elem<T>::narrow(kLog ? d - kk[k] : exp_ct<T>(d) * kk[k]);
                 }
             }
-            T* dst = out + (int64_t)(ty + (i << a.ty_log2)) * a.L;
+            T* dst = out + (int64_t)(ty_st + (i << a.ty_log2)) * a.L;
             if constexpr (UA) {
                 if (skip == 0) {
                     store_pack_unaligned<T, EV>(dst, o);
@@ -509,7 +534,8 @@ template <int KIND, class T, int VEC, bool UA = false>
 __global__ void __launch_bounds__(1024) col_flat_stats_kernel(const TransposedArgs a, int threads) {
     static_assert(KIND != NORM_LAYERNORM, "a softmax pass");
     using CT = typename Elem<T>::Wide;
-    using Part = SoftStat<CT>;
+    using ST = typename StatType<T>::type;
+    using Part = SoftStat<CT, ST>;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     Part* sm = (Part*)smem_raw;
     const int t = threadIdx.x;
@@ -517,7 +543,8 @@ __global__ void __launch_bounds__(1024) col_flat_stats_kernel(const TransposedAr
     const int Lp = threads * VEC;
     const int p0 = t * VEC;
     const int64_t total = (int64_t)a.cols * L;
-    CT m[VEC], s[VEC];
+    CT m[VEC];
+    ST s[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; ++k) {
         m[k] = neg_inf<CT>();
@@ -531,12 +558,12 @@ __global__ void __launch_bounds__(1024) col_flat_stats_kernel(const TransposedAr
 #pragma unroll
             for (int i = 0; i < CNT; ++i) bm = MaxC<CT>::comb(bm, Elem<T>::widen(v[i].v[k]));
             if (bm > m[k]) {
-                s[k] = s[k] == (CT)0 ? (CT)0 : s[k] * exp_ct<T>(m[k] - bm);
+                s[k] = s[k] == (ST)0 ? (ST)0 : s[k] * (ST)exp_ct<T>(m[k] - bm);
                 m[k] = bm;
             }
             if (m[k] > neg_inf<CT>()) {
 #pragma unroll
-                for (int i = 0; i < CNT; ++i) s[k] += exp_ct<T>(Elem<T>::widen(v[i].v[k]) - m[k]);
+                for (int i = 0; i < CNT; ++i) s[k] += (ST)exp_ct<T>(Elem<T>::widen(v[i].v[k]) - m[k]);
             }
         }
     };
@@ -576,7 +603,7 @@ __global__ void __launch_bounds__(1024) col_flat_stats_kernel(const TransposedAr
     for (int h = top >> 1; h >= 1; h >>= 1) {
         const int n = h * L;
         for (int i = t; i < n; i += blockDim.x)
-            if (i + n < Lp) sm[i] = SoftStatOp<T, CT>::comb(sm[i], sm[i + n]);
+            if (i + n < Lp) sm[i] = SoftStatOp<T, CT, ST>::comb(sm[i], sm[i + n]);
         __syncthreads();
     }
     Part* dst = (Part*)a.stats + ((int64_t)blockIdx.z * a.S + blockIdx.x) * L;

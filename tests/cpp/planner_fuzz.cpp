@@ -189,7 +189,7 @@ static void fuzz_normalize() {
             // the register + LDS kernel's vector grid may start up to a 128-byte line before the row
             const int64_t line = 128 / (int64_t)elem;
             const int64_t grid = (cols + (p.shift ? line - 1 : 0) + p.vec - 1) / p.vec;
-            CHECK((p.tpr == 256 || p.tpr == 512) && p.rpb == 1 && grid <= (int64_t)p.tpr * p.nchunk && (size_t)p.vec * elem == 16,
+            CHECK((p.tpr == 256 || p.tpr == 512 || p.tpr == 1024) && p.rpb == 1 && grid <= (int64_t)p.tpr * p.nchunk && (size_t)p.vec * elem == 16,
                   "%s plan=%s", show(v).c_str(), d.c_str());
         }
         NormPlan g = p;

@@ -781,3 +781,36 @@ def test_softmax_over_a_strided_axis_of_up_to_512_in_registers(hpt, orc, dev, ca
     want = orc.softmax(x, axis, acc=orc.ACC_F64)
     assert_close(got, want, F32_RTOL, F32_ATOL, f"{shape} axis={axis} with -inf")
     assert np.isnan(got[..., 5]).all()
+
+
+DOMINANT_CASES = [
+    # (shape, axis, transposed view, first word of the plan)
+    ([4096, 4096], 1, False, "rowreg"), ([8192, 1000], 1, False, "rowreg"), ([1000000, 8], 1, False, "rowreg+tile"),
+    ([64, 65536], 1, False, "rowsplit"), ([8, 400000], 1, False, "rowsplit"),
+    ([17310, 256, 2], 1, False, "col-group-tile"), ([100000, 16, 2], 1, False, "col-group-tile"),
+    ([2048, 2048, 2], 1, False, "col-slab"), ([512, 1000, 3], 1, False, "col-slab"),
+    ([8, 512, 4096], 1, False, "col-reg"), ([4, 128, 3136], 1, False, "col-reg"), ([64, 64, 3000], 1, False, "col-reg"),
+    ([200000, 3], 0, False, "col-split"), ([100000, 33], 0, False, "col-split-flat"), ([32768, 1024], 0, False, "col-split-flat"),
+    ([4096, 4096], 1, True, "transposed-tile"),
+]
+
+
+@pytest.mark.parametrize("case", DOMINANT_CASES, ids=[f"{c[3]}-{'x'.join(map(str, c[0]))}" for c in DOMINANT_CASES])
+def test_log_softmax_with_a_dominating_first_element(hpt, orc, dev, case):
+    """The FIRST element along the axis dominates (+14): the sum of exponentials is 1 + many tiny terms, so a
+    running f32 sum sits just above 1 for the whole walk and loses up to 6e-8 per addition, and the entry at the
+    maximum, -ln(sum), is close to zero where only the absolute tolerance helps. One case per kernel family."""
+    shape, axis, transposed, family = case
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(shape).astype(np.float32)
+    idx = [slice(None)] * len(shape)
+    idx[axis] = 0
+    x[tuple(idx)] += 14
+    if transposed:
+        t = hpt.Tensor.from_numpy(np.ascontiguousarray(x.T)).to_hip(dev).permute([1, 0])
+    else:
+        t = hpt.Tensor.from_numpy(x).to_hip(dev)
+    assert hpt.normalize_plan(t, axis).split(" ")[0] == family, hpt.normalize_plan(t, axis)
+    for log in (True, False):
+        got = (t.log_softmax(axis) if log else t.softmax(axis)).numpy()
+        assert_close(got, orc.softmax(x, axis, log=log, acc=orc.ACC_F64), F32_RTOL, F32_ATOL, f"{shape} axis={axis} log={log}")
