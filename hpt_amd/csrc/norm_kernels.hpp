@@ -324,14 +324,16 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                 for (int j = 0; j < UV; ++j)
                     x[c][j] = kLog ? x[c][j] - k : x[c][j] * k;
         } else {
-            CT s = 0;
+            // (the lane's own sum is taken in the wide type too: a lane may hold the whole of a short row,
+            // and a row whose spread is small against its offset loses digits of the mean that matter)
+            ST s = 0;
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
-                for (int j = 0; j < UV; ++j) s += x[c][j];
+                for (int j = 0; j < UV; ++j) s += (ST)x[c][j];
             // mean = sum / cols, as a reciprocal multiply plus one correction step
             // (exact quotient for the cases that matter, e.g. constant rows)
-            const ST sum = row_all_reduce<SumC<ST>>((ST)s, tpr, ty, ssmem);
+            const ST sum = row_all_reduce<SumC<ST>>(s, tpr, ty, ssmem);
             const ST m0 = sum * (ST)a.inv_cols;
             const ST mean = fma_ct(fma_ct(-m0, (ST)a.cols, sum), (ST)a.inv_cols, m0);
             const CT mean_hi = (CT)mean;

@@ -914,7 +914,26 @@ __global__ void __launch_bounds__(1024) transposed_tile_kernel(const TileArgs a)
         }
     } else {
         ST sum[VEC];
-        {
+        if constexpr (sizeof(ST) > sizeof(CT)) {
+            // (f32 rows: the lane's own sum in the wide type too, or a row whose spread is small against its
+            // offset loses digits of the mean that matter: offset 1000, spread 1 came out 9e-6 off)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) sum[k] = 0;
+#pragma unroll
+            for (int h = 0; h < H; ++h) {
+                ST th[VEC];
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) th[k] = 0;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i)
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) th[k] += (ST)Elem<T>::widen(v[h * VEC + i].v[k]);
+                if (col_ok[h]) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) sum[k] += th[k];
+                }
+            }
+        } else {
             CT t[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; ++k) t[k] = 0;

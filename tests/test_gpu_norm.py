@@ -814,3 +814,35 @@ def test_log_softmax_with_a_dominating_first_element(hpt, orc, dev, case):
     for log in (True, False):
         got = (t.log_softmax(axis) if log else t.softmax(axis)).numpy()
         assert_close(got, orc.softmax(x, axis, log=log, acc=orc.ACC_F64), F32_RTOL, F32_ATOL, f"{shape} axis={axis} log={log}")
+
+
+OFFSET_CASES = [
+    # (shape, view, first word of the plan)
+    ([8192, 4096], None, "rowreg"), ([200001, 3], "drop", "rowreg"), ([1000000, 8], None, "rowreg+tile"), ([100000, 33], None, "rowreg+tile"),
+    ([4096, 4096], "T", "transposed-tile"), ([64, 65536], None, "rowsplit"), ([640, 50304], None, "rowstream"),
+    ([512, 4097], None, "rowreg-shift"), ([1024, 12288], None, "rowreg"),
+]
+
+
+@pytest.mark.parametrize("case", OFFSET_CASES, ids=[f"{c[2]}-{'x'.join(map(str, c[0]))}" for c in OFFSET_CASES])
+def test_layernorm_of_rows_whose_offset_dwarfs_their_spread(hpt, orc, dev, case):
+    """Rows of 1000 + N(0, 1): the mean must be right to a few 1e-6 of the SPREAD, i.e. 1e-9 of its own size,
+    which needs the lanes' own sums in f64 as well as the sum across lanes. (Three-element rows also meet rows
+    whose elements nearly coincide, where 1 / sqrt(var + eps) multiplies the mean's error by up to 316.)"""
+    shape, view, family = case
+    rng = np.random.default_rng(2)
+    for off in (0.0, 1000.0):
+        x = (rng.standard_normal(shape) * (3 if shape[-1] == 3 else 1) + off).astype(np.float32)
+        if view == "T":
+            t = hpt.Tensor.from_numpy(np.ascontiguousarray(x.T)).to_hip(dev).permute([1, 0])
+            a = x
+        elif view == "drop":  # rows that start off a 16-byte boundary: one lane per row
+            t = hpt.Tensor.from_numpy(x).to_hip(dev)[1:, :]
+            a = np.ascontiguousarray(x[1:])
+        else:
+            t = hpt.Tensor.from_numpy(x).to_hip(dev)
+            a = x
+        n = shape[-1]
+        assert hpt.normalize_plan(t, 0, 1).split(" ")[0] == family, hpt.normalize_plan(t, 0, 1)
+        got = t.layernorm([n], None, None, 1e-5).numpy()
+        assert_close(got, orc.layernorm(a, 1, None, None, 1e-5, acc=orc.ACC_F64), F32_RTOL, F32_ATOL, f"{shape} offset {off}")
