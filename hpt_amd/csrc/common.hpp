@@ -150,7 +150,8 @@ struct NormPlan {
     int group_tile = 0; // Col softmax over a short middle axis of small contiguous [cols, L] groups: this many groups per workgroup through LDS
     int lds_rows = 0;   // RowReg softmax of 2- and 4-byte types: long rows held in the registers and the LDS of tpr = 256 or 512 threads (nchunk: vectors per thread in both together)
     int raw_rows = 0;   // RowReg softmax of 2-byte types, 98305 ... 131072 elements per row: only the raw row stays in registers
-    int gb_lds = 0;     // RowReg layernorm of 2-byte types: gamma / beta in LDS, four vectors of the row per thread
+    int gb_lds = 0;     // RowReg layernorm: 1 = gamma / beta in LDS (2-byte types, three or four vectors of the row per
+                        // thread), 2 = gamma / beta read from L2 for every row (rows too long for either)
     int tile_rows = 0;  // RowReg, > 0: short back-to-back rows; the plain kinds stage this many rows per workgroup in LDS
     int shift = 0;      // RowStream: rows start off 16-byte boundaries; aligned vectors, masked at both ends
     int tsplit = 1;     // Transposed: workgroups sharing the axis in the statistics pass

@@ -762,6 +762,27 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     lds_row_shape(p, nv, elem_size, false))
                     return p;
             }
+            // Layernorm rows beyond that (up to 32768 four-byte, 49152 two-byte or 16384 eight-byte elements) still fit
+            // the registers of 512 or 1024 threads when gamma / beta do not sit beside them: those are read again for
+            // every row, vector by vector in the last sweep, from L2. One read of the row instead of the streaming
+            // kernel's two. Measured (% of the HBM peak, streaming -> this): f32 [1771, 18944] 39 -> 60, [1310, 25600]
+            // 37 -> 57, [1024, 32768] 43 -> 62; f16 [1771, 18944] 27 -> 55, [1310, 25600] 28 -> 43, [1024, 32768] 33 -> 50.
+            // (Two-byte rows of seven or eight vectors per thread spill. Where the forms above exist they are as fast
+            // or faster: f32 [4096, 8192] 67.5 against 68, [2730, 12288] 68 against 65; f16 [4096, 8192] 59 against 53.)
+            if (n_norm_dims > 0 && v == max_vec && v > 1 && p.sstride == 1 && !p.shift && !p.gb_lds && nv > reg_limit) {
+                int t = 1024;
+                if (elem_size == 2 && nv <= 512 * 5) t = 512;  // f16 [1771, 18944]: 512 x 5 55 %, 1024 x 3 45 %
+                const int64_t c = (nv + t - 1) / t;
+                // (layernorm(x + residual) holds the residual's vectors beside the row's: fewer fit before it spills)
+                if (c <= (fused ? (elem_size == 2 ? 4 : 6) : (elem_size == 2 ? 6 : 8))) {
+                    p.kind = NormKind::RowReg;
+                    p.gb_lds = 2;
+                    p.tpr = t;
+                    p.nchunk = (int)c;
+                    p.rpb = 1;
+                    return p;
+                }
+            }
             if (nv <= reg_limit) {
                 p.kind = NormKind::RowReg;
                 // Short rows laid back to back: the plain kinds move whole 16 KiB tiles through LDS
@@ -805,14 +826,15 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 // [10922, 3072] 4.9 -> 5.7 (256 x 3); f16 softmax [21845, 3072] 256 x 2 4.5 -> 128 x 3 5.9,
                 // [13107, 5120] 4.7 -> 5.8 (256 x 3); f16 layernorm [87381, 768] 4.1 -> 5.0 (32 x 3), [43690, 1536]
                 // 3.9 -> 4.9 (64 x 3). (Two-byte rows of five vectors or more per thread lose: layernorm spills.)
-                // (gamma / beta in LDS: three, four or five vectors per thread - f16 [58254, 1152] 4.4 -> 4.8,
-                // [26214, 2560] 4.6 -> 5.0 with five)
+                // (gamma / beta in LDS: three or four vectors per thread. Five lose to three with twice the threads, idle
+                // lanes and all - f16, % of the HBM peak: [29127, 1152] 58 -> 66.5, [13107, 2560] 58 -> 64, [6553, 5120]
+                // 56 -> 62, [3640, 9216] 53 -> 58, [3276, 10240] 39 -> 61)
                 // (Rows of odd length, covered by aligned vectors: softmax alike - f16 [116306, 577] 3.6 -> 4.1,
                 // [44739, 1500] 4.2 -> 4.9, f32 [8190, 4097] 4.4 -> 5.3, [16000, 2051] 4.3 -> 5.5; layernorm, which
                 // carries the masks and the unaligned gamma / beta besides, only up to what it had: more spills.)
                 if (v == max_vec && v > 1 && p.sstride == 1 && !p.tile_rows) {
                     const int maxc = n_norm_dims > 0 && p.shift ? (elem_size == 2 ? 2 : 4)
-                                                                : elem_size == 2 ? (ln_half ? 3 : (p.gb_lds ? 5 : 4))
+                                                                : elem_size == 2 ? (ln_half ? 3 : 4)
                                                                 : (n_norm_dims > 0 ? (fused ? 4 : 6) : 8);
                     // (layernorm(x + residual) holds the residual's vectors beside the row's: with five or six
                     // per thread it spills - f32 [2730, 12288] 3.1 TB/s)
@@ -1071,7 +1093,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg) ? "-unaligned" : (p.lds_rows ? "-lds-shift" : "-shift")) : (p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.group_tile ? "-group-tile" : (p.slab_tile ? "-slab" : "")), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg) ? "-unaligned" : (p.lds_rows ? "-lds-shift" : "-shift")) : (p.gb_lds == 2 ? "-l2gb" : p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.group_tile ? "-group-tile" : (p.slab_tile ? "-slab" : "")), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     if (p.kind == NormKind::RowReg) s += "max_blocks=" + std::to_string(p.max_blocks) + " ";  // (layernorm walks its rows)

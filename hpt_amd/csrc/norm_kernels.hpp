@@ -109,12 +109,17 @@ __device__ __forceinline__ A row_all_reduce(A v, int tpr, int ty, A* smem) {
 // launch makes the row step of the walk a multiple of VEC.
 // PF: always issue the next row's loads before the current row's statistics (see kPrefetch below);
 // the launch then caps the grid so that workgroups do walk rows.
-// GBL (layernorm of 2-byte types, long rows): gamma / beta live in LDS instead of registers (loaded
+// GB = 2 (layernorm rows of more vectors per thread than leave room for gamma / beta beside them): gamma / beta are
+// read again for every row, vector by vector in the last sweep, from L2 (they are 2 x cols elements, which every
+// workgroup keeps reading). A workgroup then needs nothing from one row to the next.
+// GB = 1, "GBL" (layernorm of 2-byte types, long rows): gamma / beta live in LDS instead of registers (loaded
 // once per workgroup, read per row), which leaves room for four vectors of the row per thread where
 // the register form holds two: half as many threads per row, twice as many rows in flight.
-template <int KIND, class T, int VEC, int NCHUNK, int SS = 1, bool SHIFT = false, bool PF = false, bool GBL = false>
+template <int KIND, class T, int VEC, int NCHUNK, int SS = 1, bool SHIFT = false, bool PF = false, int GB = 0>
 __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
-    static_assert(!GBL || (norm_is_layer(KIND) && VEC > 1 && SS == 1 && !SHIFT), "GBL is an aligned layernorm form");
+    constexpr bool GBL = GB == 1;  // gamma / beta in LDS
+    constexpr bool GBG = GB == 2;  // gamma / beta from global memory, every row
+    static_assert(GB == 0 || (norm_is_layer(KIND) && VEC > 1 && SS == 1 && !SHIFT), "gamma / beta outside registers: an aligned layernorm form");
     static_assert(!SHIFT || (VEC > 1 && SS == 1), "SHIFT is a full-vector mode");
     constexpr int UV = VEC / SS;  // useful elements per vector
     using CT = typename Elem<T>::Wide;
@@ -139,8 +144,8 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     extern __shared__ __align__(16) unsigned char gb_raw[];
     T* lds_gamma = reinterpret_cast<T*>(gb_raw);
     T* lds_beta = lds_gamma + (GBL ? (size_t)nv * UV : 0);
-    Pack<T, UV> gam[GBL ? 1 : NCHUNK], bet[GBL ? 1 : NCHUNK];
-    if constexpr (!kSoft && !GBL) {
+    Pack<T, UV> gam[GB ? 1 : NCHUNK], bet[GB ? 1 : NCHUNK];
+    if constexpr (!kSoft && !GB) {
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int iv = c * tpr + tx;
@@ -184,7 +189,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     // Rows that take 512 or 1024 threads leave room for one or two workgroups per compute unit, so
     // nothing else hides a row's load -> reduce -> reduce -> store chain: there (PF) the prefetch
     // pays for every type (f32 [3355, 10000] softmax: 3.2 TB/s without).
-    constexpr bool kPrefetch = ((sizeof(T) == 2 && NCHUNK * UV <= ((kSoft || GBL) ? 32 : 16)) || PF) && !kRes;
+    constexpr bool kPrefetch = ((sizeof(T) == 2 && NCHUNK * UV <= ((kSoft || GB) ? 32 : 16)) || PF) && !kRes;
     const int64_t row_step = (int64_t)gridDim.x * a.rpb;
     Pack<T, VEC> raw[NCHUNK];
     Pack<T, UV> raw_res[kRes ? NCHUNK : 1];
@@ -352,7 +357,30 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
             }
             const ST var = row_all_reduce<SumC<ST>>((ST)q, tpr, ty, ssmem) * (ST)a.inv_cols;
             const CT rstd = rsqrt_ct((CT)var + (CT)a.eps);
-            if constexpr (GBL) {
+            if constexpr (GBG) {
+                // (the pointers are made opaque per row, or the loads would be hoisted out of the row loop and
+                // gamma / beta would sit in registers after all)
+                const T* gp = (const T*)a.gamma;
+                const T* bp = (const T*)a.beta;
+                asm volatile("" : "+s"(gp), "+s"(bp));
+#pragma unroll
+                for (int c = 0; c < NCHUNK; ++c) {
+                    const int iv = c * tpr + tx;
+                    if (iv < nv) {
+                        Pack<T, UV> g, b;
+#pragma unroll
+                        for (int j = 0; j < UV; ++j) {
+                            g.v[j] = Elem<T>::narrow((CT)1);
+                            b.v[j] = Elem<T>::narrow((CT)0);
+                        }
+                        if (gp) g = load_pack<T, UV>(gp + (size_t)iv * UV);
+                        if (bp) b = load_pack<T, UV>(bp + (size_t)iv * UV);
+#pragma unroll
+                        for (int j = 0; j < UV; ++j)
+                            x[c][j] = x[c][j] * rstd * Elem<T>::widen(g.v[j]) + Elem<T>::widen(b.v[j]);
+                    }
+                }
+            } else if constexpr (GBL) {
 #pragma unroll
                 for (int c = 0; c < NCHUNK; ++c) {
                     const int iv = c * tpr + tx;

@@ -369,18 +369,38 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
                 return;
             }
         }
+        if constexpr (FULL > 1 && norm_is_layer(KIND)) {
+            if (p.gb_lds == 2 && p.vec == FULL && p.sstride == 1 && !p.shift) {
+                // gamma / beta from L2 in the last sweep: one row per group of threads, nothing carried between rows
+                // (rows of 512 or 1024 threads: 512 workgroups walk the rows and prefetch)
+                const bool pf = p.tpr >= 512 && KIND != NORM_ADD_LAYERNORM;
+                if (pf && grid.x > 512u) grid.x = 512u;
+#define HPT_L2GB_CASE(N)                                                                                  \
+    case 2 * N: row_reg_kernel<KIND, T, FULL, N, 1, false, false, 2><<<grid, block, 0, st>>>(a); return; \
+    case 2 * N + 1: row_reg_kernel<KIND, T, FULL, N, 1, false, true, 2><<<grid, block, 0, st>>>(a); return;
+                if constexpr (sizeof(T) >= 4) {  // (two-byte rows of seven or eight vectors per thread spill: not planned)
+                    switch (p.nchunk * 2 + (pf ? 1 : 0)) {
+                        HPT_L2GB_CASE(7) HPT_L2GB_CASE(8)
+                        default: break;
+                    }
+                }
+                switch (p.nchunk * 2 + (pf ? 1 : 0)) {
+                    HPT_L2GB_CASE(3) HPT_L2GB_CASE(4) HPT_L2GB_CASE(5) HPT_L2GB_CASE(6)
+                    default: fail(HPT_ERR_KERNEL, "row_reg: unsupported chunk count %d with gamma / beta from L2", p.nchunk);
+                }
+#undef HPT_L2GB_CASE
+            }
+        }
         if constexpr (FULL > 1 && sizeof(T) == 2 && norm_is_layer(KIND)) {
-            if (p.gb_lds && p.vec == FULL && p.sstride == 1 && !p.shift && p.nchunk >= 3 && p.nchunk <= 5) {
+            if (p.gb_lds == 1 && p.vec == FULL && p.sstride == 1 && !p.shift && p.nchunk >= 3 && p.nchunk <= 4) {
                 const size_t smem = 2 * (size_t)p.cols * sizeof(T);
                 if (p.tpr >= 512 && KIND != NORM_ADD_LAYERNORM) {
                     if (grid.x > 512u) grid.x = 512u;
-                    if (p.nchunk == 3) row_reg_kernel<KIND, T, FULL, 3, 1, false, true, true><<<grid, block, smem, st>>>(a);
-                    else if (p.nchunk == 5) row_reg_kernel<KIND, T, FULL, 5, 1, false, true, true><<<grid, block, smem, st>>>(a);
-                    else row_reg_kernel<KIND, T, FULL, 4, 1, false, true, true><<<grid, block, smem, st>>>(a);
+                    if (p.nchunk == 3) row_reg_kernel<KIND, T, FULL, 3, 1, false, true, 1><<<grid, block, smem, st>>>(a);
+                    else row_reg_kernel<KIND, T, FULL, 4, 1, false, true, 1><<<grid, block, smem, st>>>(a);
                 } else {
-                    if (p.nchunk == 3) row_reg_kernel<KIND, T, FULL, 3, 1, false, false, true><<<grid, block, smem, st>>>(a);
-                    else if (p.nchunk == 5) row_reg_kernel<KIND, T, FULL, 5, 1, false, false, true><<<grid, block, smem, st>>>(a);
-                    else row_reg_kernel<KIND, T, FULL, 4, 1, false, false, true><<<grid, block, smem, st>>>(a);
+                    if (p.nchunk == 3) row_reg_kernel<KIND, T, FULL, 3, 1, false, false, 1><<<grid, block, smem, st>>>(a);
+                    else row_reg_kernel<KIND, T, FULL, 4, 1, false, false, 1><<<grid, block, smem, st>>>(a);
                 }
                 return;
             }

@@ -102,6 +102,8 @@ ADD_LN_CASES = [
     ("long rows: streaming", [3, 40000], (), 1),
     ("rows of 8192 (two-byte types keep gamma / beta in LDS)", [1300, 8192], (), 1),
     ("rows of 12288, more rows than workgroups", [1100, 12288], (), 1),
+    ("rows of 20480: in registers with gamma / beta from L2 (f64: streaming)", [600, 20480], (), 1),
+    ("rows of 10240 (f64: five vectors per thread, gamma / beta from L2)", [700, 10240], (), 1),
     ("sliced input", [20, 300], (("slice", ((2, 19, 1), (4, 260, 1))),), 1),
     ("step-2 input", [16, 512], (("slice", ((0, 16, 1), (0, 512, 2))),), 1),
     ("transposed input: demoted to the generic rows", [256, 4096], (("permute", (1, 0)),), 1),

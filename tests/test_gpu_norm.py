@@ -846,3 +846,40 @@ def test_layernorm_of_rows_whose_offset_dwarfs_their_spread(hpt, orc, dev, case)
         assert hpt.normalize_plan(t, 0, 1).split(" ")[0] == family, hpt.normalize_plan(t, 0, 1)
         got = t.layernorm([n], None, None, 1e-5).numpy()
         assert_close(got, orc.layernorm(a, 1, None, None, 1e-5, acc=orc.ACC_F64), F32_RTOL, F32_ATOL, f"{shape} offset {off}")
+
+
+L2GB_CASES = [
+    # (dtype, shape, plan words) - layernorm rows too long for gamma / beta beside them in registers or LDS
+    (np.float32, [300, 16388], "tpr=1024 rpb=1 nchunk=5 "), (np.float32, [600, 18944], "tpr=1024 rpb=1 nchunk=5 "), (np.float32, [520, 28672], "tpr=1024 rpb=1 nchunk=7 "),
+    (np.float32, [257, 32768], "tpr=1024 rpb=1 nchunk=8 "), (np.float16, [600, 18944], "tpr=512 rpb=1 nchunk=5 "), ("bf16", [300, 25600], "tpr=1024 rpb=1 nchunk=4 "),
+    (np.float16, [515, 49152], "tpr=1024 rpb=1 nchunk=6 "), (np.float64, [300, 8194], "tpr=1024 rpb=1 nchunk=5 "), (np.float64, [513, 16384], "tpr=1024 rpb=1 nchunk=8 "),
+    (np.float32, [1100, 20480], "tpr=1024 rpb=1 nchunk=5 "),  # more rows than workgroups: they walk the rows and prefetch
+]
+
+
+@pytest.mark.parametrize("case", L2GB_CASES, ids=[f"{getattr(c[0], '__name__', c[0])}-{'x'.join(map(str, c[1]))}" for c in L2GB_CASES])
+def test_layernorm_rows_with_gamma_beta_read_from_l2(hpt, orc, dev, case):
+    npdt, shape, words = case
+    rng = np.random.default_rng(811)
+    x = (rng.standard_normal(shape) * 2 + 1).astype(np.float32)
+    n = shape[-1]
+    g32 = rng.normal(1, 0.2, n).astype(np.float32)
+    b32 = rng.normal(0, 0.3, n).astype(np.float32)
+    if npdt == "bf16":
+        conv, dt, odt, bits, tof = hpt.f32_to_bf16_bits, hpt.bf16, orc.BF16, 8, hpt.bf16_bits_to_f32
+    else:
+        conv, dt, odt, bits, tof = (lambda v: v.astype(npdt)), None, None, 11, (lambda v: v)
+    base, g, b = conv(x), conv(g32), conv(b32)
+    t = hpt.Tensor.from_numpy(base, dt).to_hip(dev)
+    plan = hpt.normalize_plan(t, 0, 1)
+    assert plan.startswith("rowreg-l2gb ") and words in plan, plan
+    tg, tb = hpt.Tensor.from_numpy(g, dt).to_hip(dev), hpt.Tensor.from_numpy(b, dt).to_hip(dev)
+    half = npdt in ("bf16", np.float16)
+    for gg, bb, tgg, tbb in ((g, b, tg, tb), (None, None, None, None), (g, None, tg, None), (None, b, None, tb)):
+        got = t.layernorm([n], tgg, tbb, 1e-5).numpy()
+        want = orc.layernorm(base, 1, gg, bb, 1e-5, acc=orc.ACC_F64, dtype=odt)
+        if half:
+            w = tof(want).astype(np.float32)
+            assert_close(tof(got).astype(np.float32), w, HALF_RTOL, half_atol(w, bits), f"{npdt} {shape} g={gg is not None} b={bb is not None}")
+        else:
+            assert_close(got, want, F32_RTOL, F32_ATOL, f"{npdt} {shape} g={gg is not None} b={bb is not None}")

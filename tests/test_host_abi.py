@@ -118,7 +118,11 @@ def test_plans_for_shapes_off_the_benchmark_list(hpt):
         ([4096, 768], hpt.f16, 0, 1, "rowreg-ldsgb rows=4096 cols=768 vec=8 tpr=32 rpb=8 nchunk=3"), ([4096, 384], hpt.f16, 0, 1, "rowreg rows=4096 cols=384 vec=8 tpr=16 rpb=16 nchunk=3"), ([4096, 1536], None, 1, 0, "rowreg rows=4096 cols=1536 vec=4 tpr=128 rpb=2 nchunk=3"),
         ([4096, 2560], None, 0, 1, "rowreg rows=4096 cols=2560 vec=4 tpr=128 rpb=2 nchunk=5"), ([4096, 6144], None, 1, 0, "rowreg rows=4096 cols=6144 vec=4 tpr=256 rpb=1 nchunk=6"),
         ([4096, 6144], None, 0, 1, "rowreg rows=4096 cols=6144 vec=4 tpr=512 rpb=1 nchunk=3"), ([4096, 7168], None, 1, 0, "rowreg rows=4096 cols=7168 vec=4 tpr=256 rpb=1 nchunk=7"),
-        ([4096, 5120], hpt.f16, 0, 1, "rowreg-ldsgb rows=4096 cols=5120 vec=8 tpr=128 rpb=2 nchunk=5"), ([4096, 5120], hpt.f16, 1, 0, "rowreg rows=4096 cols=5120 vec=8 tpr=256 rpb=1 nchunk=3"),
+        ([4096, 5120], hpt.f16, 0, 1, "rowreg-ldsgb rows=4096 cols=5120 vec=8 tpr=256 rpb=1 nchunk=3"),
+        # layernorm rows too long for gamma / beta beside them: those come from L2 in the last sweep
+        ([1771, 18944], None, 0, 1, "rowreg-l2gb rows=1771 cols=18944 vec=4 tpr=1024 rpb=1 nchunk=5"), ([1024, 32768], None, 0, 1, "rowreg-l2gb rows=1024 cols=32768 vec=4 tpr=1024 rpb=1 nchunk=8"),
+        ([1024, 32772], None, 0, 1, "rowstream"), ([1771, 18944], hpt.f16, 0, 1, "rowreg-l2gb rows=1771 cols=18944 vec=8 tpr=512 rpb=1 nchunk=5"),
+        ([1024, 49152], hpt.bf16, 0, 1, "rowreg-l2gb rows=1024 cols=49152 vec=8 tpr=1024 rpb=1 nchunk=6"), ([1024, 49160], hpt.bf16, 0, 1, "rowstream"), ([4096, 5120], hpt.f16, 1, 0, "rowreg rows=4096 cols=5120 vec=8 tpr=256 rpb=1 nchunk=3"),
         ([32768, 1024], hpt.f16, 0, 1, "rowreg-ldsgb rows=32768 cols=1024 vec=8 tpr=32 rpb=8 nchunk=4"), ([32768, 512], hpt.f16, 0, 1, "rowreg rows=32768 cols=512 vec=8 tpr=32 rpb=8 nchunk=2"),
         ([32768, 1024], hpt.f32, 0, 1, "rowreg rows=32768 cols=1024 vec=4 tpr=64 rpb=4 nchunk=4"),
         # softmax over an axis that is not the last
