@@ -978,6 +978,14 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                         nc_max = 32;
                         ty = 16;
                     }
+                    // Likewise 129 ... 256 elements: eight thread rows of 128 registers read 512-byte segments where sixteen
+                    // of 64 read 256-byte ones. f32 [256, 256, 256] over axis 0 / 1, five processes each, us: 26.3-29.1 /
+                    // 23.6-28.9 (which end depends on where the allocator put the buffers) -> 25.2-25.7 / 25.2-26.9.
+                    // (65 ... 128 elements the same way, four thread rows, lose: C3 [64, 128, 56, 56] over the channels 41.3 -> 44.6 us)
+                    if (ty == 16 && nc_max == 16 && elem_size == 4 && ev == 4 && p.cols > 128 && L % 128 == 0) {
+                        nc_max = 32;
+                        ty = 8;
+                    }
                     // enough threads to fill the chip: inner positions x thread rows
                     if (!(ty <= 16 && p.rows / ev * ty >= 8 * 1024)) continue;
                     // (a long axis of two-byte elements that only fits with sixteen thread rows of 4-byte pieces: the

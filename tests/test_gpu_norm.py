@@ -756,6 +756,8 @@ def test_long_rows_of_random_length_and_alignment(hpt, orc, dev, seed):
 WIDE_AXIS_CASES = [
     # four-byte axes of 257 ... 512 elements with a wide inner dim: 128 registers of raw values per thread
     ([2, 512, 2048], 1), ([3, 257, 1024], 1), ([384, 8192], 0), ([1, 300, 4096], 1), ([5, 512, 64, 32], 1),
+    # 129 ... 256 elements: the same registers over eight thread rows
+    ([16, 200, 1024], 1), ([256, 8192], 0), ([2, 129, 4096], 1), ([64, 256, 16, 8], 1),
 ]
 
 
