@@ -872,6 +872,27 @@ __global__ void __launch_bounds__(256) finish_rows_kernel(const void* part_, voi
     if (threadIdx.x == 0) write_out<Op>(out, o, acc, init_out, count);
 }
 
+// finish_rows_thin_kernel: the same partials when every output has only a few (split <= 16: sum([0, 2, 3]) of
+// [64, 128, 56, 56] has 128 outputs of 4): a thread folds one output, in the order of the partials, and the whole
+// launch is one or two workgroups instead of one per output.
+template <class Op>
+__global__ void __launch_bounds__(256) finish_rows_thin_kernel(const void* part_, void* out, int64_t K, int split, int init_out,
+                                                               double count) {
+    using Acc = typename Op::Acc;
+    const Acc* part = (const Acc*)part_;
+    const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (o >= K) return;
+    Acc v[16];
+#pragma unroll
+    for (int s = 0; s < 16; ++s)
+        if (s < split) v[s] = part[o * split + s];
+    Acc acc = v[0];
+#pragma unroll
+    for (int s = 1; s < 16; ++s)
+        if (s < split) acc = Op::comb(acc, v[s]);
+    write_out<Op>(out, o, acc, init_out, count);
+}
+
 // finish_cols_kernel: many outputs (column splits; partial s of output o at
 // part[s * K + o]): 64 neighbouring outputs per workgroup, the partials of each dealt
 // over blockDim.y thread rows so that no thread walks a long chain of dependent
@@ -1035,7 +1056,10 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             else if (vec) row_reduce_kernel<Op, FULL><<<grid, block, 0, st>>>(a);
             else row_reduce_kernel<Op, 1><<<grid, block, 0, st>>>(a);
         }
-        if (p.split > 1)
+        if (p.split > 1 && p.split <= 16)
+            finish_rows_thin_kernel<Op><<<dim3((unsigned)((p.K + 255) / 256)), dim3(256), 0, st>>>(sc.partial, out, p.K, p.split,
+                                                                                                   init_out, count);
+        else if (p.split > 1)
             finish_rows_kernel<Op><<<dim3((unsigned)p.K), dim3(256), 0, st>>>(sc.partial, out, p.split, init_out,
                                                                               count);
         return;
