@@ -568,3 +568,43 @@ def test_neighbouring_outputs_with_runs_back_to_back(hpt, orc, dev, case):
     h = x.astype(np.float16)
     th = hpt.Tensor.from_numpy(h).to_hip(dev)
     assert np.array_equal(th.max(axes).numpy(), h.max(tuple(axes))), "f16 max"
+
+
+FEW_PARTIAL_CASES = [
+    # (shape, axes, words of the plan): few outputs of 2 ... 16 partials each, folded by one thread per output
+    ([64, 128, 784], [0, 2], "split=4(4x1)"), ([40, 300000], [1], "split=12(1x12)"), ([200, 100000], [1], "split=2(1x2)"),
+    ([130, 70001], [1], "split=3(1x3)"), ([96, 33, 4000], [1, 2], "split=5(1x5)"),
+]
+
+
+@pytest.mark.parametrize("case", FEW_PARTIAL_CASES, ids=[f"{'x'.join(map(str, c[0]))}-{c[2]}" for c in FEW_PARTIAL_CASES])
+def test_few_outputs_of_few_partials_each(hpt, orc, dev, case):
+    shape, axes, words = case
+    rng = np.random.default_rng(131)
+    base = rng.standard_normal(shape).astype(np.float32)
+    # ties for the arg-reductions across the split: the maximum sits in the first and in the last partial's range
+    idx_first = tuple(0 if i in axes else slice(None) for i in range(len(shape)))
+    idx_last = tuple(shape[i] - 1 if i in axes else slice(None) for i in range(len(shape)))
+    base[idx_first] = 9.0
+    base[idx_last] = 9.0
+    t, a = upload(hpt, base, dev=dev)
+    assert words in hpt.reduce_plan(t, hpt.SUM, axes), hpt.reduce_plan(t, hpt.SUM, axes)
+    assert_close(t.sum(axes).numpy(), orc.reduce(orc.SUM, a, axes, acc=orc.ACC_F64), F32_RTOL, F32_ATOL, f"sum {shape}")
+    assert_close(t.mean(axes).numpy(), orc.reduce(orc.MEAN, a, axes, acc=orc.ACC_F64), F32_RTOL, F32_ATOL, f"mean {shape}")
+    assert np.array_equal(t.max(axes).numpy(), a.max(tuple(axes)))
+    assert np.array_equal(t.min(axes).numpy(), a.min(tuple(axes)))
+    if len(axes) == 1:
+        assert np.array_equal(t.argmax(axes[0]).numpy(), orc.argreduce(True, a, axes[0]))   # lowest index wins
+        assert np.array_equal(t.argmin(axes[0]).numpy(), orc.argreduce(False, a, axes[0]))
+    ib = rng.integers(-1000, 1001, shape).astype(np.int32)
+    ti, ai = upload(hpt, ib, dev=dev)
+    assert np.array_equal(ti.sum(axes).numpy(), orc.reduce(orc.SUM, ai, axes))
+    hb = (rng.standard_normal(shape) * 0.5).astype(np.float16)
+    th, ah = upload(hpt, hb, dev=dev)
+    want = orc.reduce(orc.SUM, ah, axes, acc=orc.ACC_F32).astype(np.float32)
+    assert_close(th.sum(axes).numpy().astype(np.float32), want, HALF_RTOL, half_atol(want, 11), f"f16 sum {shape}")
+    # accumulate into the output, and the same bits from run to run
+    out = hpt.Tensor.from_numpy(np.ones(want.shape, np.float32)).to_hip(dev)
+    t.sum_(axes, False, False, out)
+    assert_close(out.numpy(), orc.reduce(orc.SUM, a, axes, acc=orc.ACC_F64) + 1, F32_RTOL, F32_ATOL, f"sum into out {shape}")
+    assert np.array_equal(t.sum(axes).numpy().view(np.uint32), t.sum(axes).numpy().view(np.uint32))
