@@ -675,9 +675,13 @@ __global__ void __launch_bounds__(NT, MINW) row_lds_kernel(const NormArgs a) {
 // A contiguous [rows, cols] matrix with short rows (cols <= 512): a workgroup brings a.rpb
 // consecutive rows (16 KiB; a multiple of VEC rows, so the tile starts on a 16-byte boundary
 // whatever cols is) into LDS with aligned 128-bit loads, groups of `tpr` lanes normalise the rows
-// in place (at most eight elements per lane, held in registers between the passes), and the tile
+// in place (EPL elements per lane, at most eight, held in registers between the passes), and the tile
 // leaves with aligned 128-bit stores. HBM sees whole lines only, in both directions.
-template <int KIND, class T, int VEC>
+// EPL is what a lane of THIS row length has (rows of 257 over 64 lanes: 5): sweeps unrolled to eight would run
+// three steps with every lane masked off - f32 [130561, 257] softmax 59.4 -> 48.0 us, [260111, 129] 54.6 -> 49.0,
+// f16 [130561, 257] 38.0 -> 34.5. (Stopping the unrolled sweeps at run time instead costs more than the idle steps:
+// f16 [170327, 197] 28.5 -> 36.7 us.)
+template <int KIND, class T, int VEC, int EPL = 8>
 __global__ void __launch_bounds__(256) norm_tile_kernel(const NormArgs a) {
     static_assert(KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX || KIND == NORM_LAYERNORM, "plain kinds only");
     using CT = typename Elem<T>::Wide;
@@ -685,7 +689,6 @@ __global__ void __launch_bounds__(256) norm_tile_kernel(const NormArgs a) {
     constexpr bool kSoft = !norm_is_layer(KIND);
     constexpr bool kLog = norm_is_log(KIND);
     constexpr int NV = 4;   // vectors per thread: 256 * 4 * 16 bytes = 16 KiB
-    constexpr int EPL = 8;  // elements per lane at most
     __shared__ __align__(16) unsigned char tile_raw[256 * NV * 16];
     T* tile = reinterpret_cast<T*>(tile_raw);
     const int t = threadIdx.x;

@@ -351,8 +351,20 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
                 a.tpr = 1;
                 while (a.tpr < 64 && a.tpr * 8 < p.cols) a.tpr <<= 1;
                 a.tpr_log2 = ilog2(a.tpr);
-                norm_tile_kernel<KIND, T, FULL>
-                    <<<dim3((unsigned)((p.rows + p.tile_rows - 1) / p.tile_rows)), dim3(256), 0, st>>>(a);
+                // (the lanes' sweeps are unrolled to exactly the elements a lane of this row length has: rows of 257 take
+                // 5 per lane of 64, and three more steps with every lane masked off cost a fifth of the launch)
+                const dim3 tgrid((unsigned)((p.rows + p.tile_rows - 1) / p.tile_rows));
+                switch ((int)((p.cols + a.tpr - 1) / a.tpr)) {
+                    case 1: norm_tile_kernel<KIND, T, FULL, 1><<<tgrid, dim3(256), 0, st>>>(a); break;
+                    case 2: norm_tile_kernel<KIND, T, FULL, 2><<<tgrid, dim3(256), 0, st>>>(a); break;
+                    case 3: norm_tile_kernel<KIND, T, FULL, 3><<<tgrid, dim3(256), 0, st>>>(a); break;
+                    case 4: norm_tile_kernel<KIND, T, FULL, 4><<<tgrid, dim3(256), 0, st>>>(a); break;
+                    case 5: norm_tile_kernel<KIND, T, FULL, 5><<<tgrid, dim3(256), 0, st>>>(a); break;
+                    case 6: norm_tile_kernel<KIND, T, FULL, 6><<<tgrid, dim3(256), 0, st>>>(a); break;
+                    case 7: norm_tile_kernel<KIND, T, FULL, 7><<<tgrid, dim3(256), 0, st>>>(a); break;
+                    case 8: norm_tile_kernel<KIND, T, FULL, 8><<<tgrid, dim3(256), 0, st>>>(a); break;
+                    default: fail(HPT_ERR_KERNEL, "norm_tile: %d elements per lane", (int)((p.cols + a.tpr - 1) / a.tpr));
+                }
                 return;
             }
         }

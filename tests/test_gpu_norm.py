@@ -885,3 +885,31 @@ def test_layernorm_rows_with_gamma_beta_read_from_l2(hpt, orc, dev, case):
             assert_close(tof(got).astype(np.float32), w, HALF_RTOL, half_atol(w, bits), f"{npdt} {shape} g={gg is not None} b={bb is not None}")
         else:
             assert_close(got, want, F32_RTOL, F32_ATOL, f"{npdt} {shape} g={gg is not None} b={bb is not None}")
+
+
+TILE_LENGTHS = [2, 3, 5, 7, 9, 15, 17, 24, 31, 33, 47, 63, 65, 97, 129, 161, 197, 225, 257, 321, 385, 449, 511]
+
+
+@pytest.mark.parametrize("npdt", [np.float32, np.float16], ids=["f32", "f16"])
+def test_short_rows_of_every_count_per_lane(hpt, orc, dev, npdt):
+    """The tile kernel is compiled once per number of elements a lane holds (1 ... 8) and picks the lanes per row from the
+    row length: row lengths on both sides of every boundary, softmax, log_softmax and layernorm."""
+    rng = np.random.default_rng(907)
+    half = npdt == np.float16
+    acc = orc.ACC_F32 if half else orc.ACC_F64
+    for n in TILE_LENGTHS:
+        rows = (4 << 20) // (n * np.dtype(npdt).itemsize) + 37   # (at least 4 MiB, or the rows stay with the register kernel)
+        x = (rng.standard_normal((rows, n)) * 2 + 0.5).astype(npdt)
+        t = hpt.Tensor.from_numpy(x).to_hip(dev)
+        assert "+tile" in hpt.normalize_plan(t, 1), (n, hpt.normalize_plan(t, 1))
+        g = rng.normal(1, 0.1, n).astype(npdt)
+        b = rng.normal(0, 0.1, n).astype(npdt)
+        tg, tb = hpt.Tensor.from_numpy(g).to_hip(dev), hpt.Tensor.from_numpy(b).to_hip(dev)
+        for what, got, want in (("softmax", t.softmax(1).numpy(), orc.softmax(x, 1, acc=acc)),
+                                ("log_softmax", t.log_softmax(1).numpy(), orc.softmax(x, 1, log=True, acc=acc)),
+                                ("layernorm", t.layernorm([n], tg, tb, 1e-5).numpy(), orc.layernorm(x, 1, g, b, 1e-5, acc=acc))):
+            if half:
+                w = want.astype(np.float32)
+                assert_close(got.astype(np.float32), w, HALF_RTOL, max(half_atol(w[np.isfinite(w)], 11), 6e-8), f"f16 {what} rows of {n}")
+            else:
+                assert_close(got, want, F32_RTOL, F32_ATOL, f"f32 {what} rows of {n}")
