@@ -1277,16 +1277,33 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const NormArgs a) {
                 for (int j = 0; j < VEC; ++j)
                     x[j] = ((x[j] - mean_hi) - mean_lo) * rstd * Elem<T>::widen(g.v[j]) + Elem<T>::widen(b.v[j]);
             } else {
+                // (the end vectors of a shifted row, or single elements: gamma / beta from indices clamped into the row,
+                // no branch around a load - with a test per element the compiler waits for every load in turn, and the
+                // wavefronts that hold a row's two ends kept the whole row waiting)
+                T g[VEC], b[VEC];
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
-                    CT y = ((x[j] - mean_hi) - mean_lo) * rstd;
-                    const int64_t col = iv * VEC + j - m;
-                    if (inside(iv, j)) {
-                        if (a.gamma) y *= Elem<T>::widen(((const T*)a.gamma)[col]);
-                        if (a.beta) y += Elem<T>::widen(((const T*)a.beta)[col]);
-                    }
-                    x[j] = y;
+                    g[j] = Elem<T>::narrow((CT)1);
+                    b[j] = Elem<T>::narrow((CT)0);
                 }
+                const int64_t c0 = iv * VEC - m;
+                if (a.gamma) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        const int64_t col = c0 + j;
+                        g[j] = ((const T*)a.gamma)[col < 0 ? 0 : (col < a.cols ? col : a.cols - 1)];
+                    }
+                }
+                if (a.beta) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        const int64_t col = c0 + j;
+                        b[j] = ((const T*)a.beta)[col < 0 ? 0 : (col < a.cols ? col : a.cols - 1)];
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    x[j] = ((x[j] - mean_hi) - mean_lo) * rstd * Elem<T>::widen(g[j]) + Elem<T>::widen(b[j]);
             }
             store(iv, x);
         };

@@ -384,6 +384,7 @@ template <class T, int N> __device__ __forceinline__ void forget_pack(Pack<T, N>
     if constexpr (sizeof(T) * N == 16) asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&v)));
     else if constexpr (sizeof(T) * N == 8) asm volatile("" : "+v"(*reinterpret_cast<u32x2*>(&v)));
     else if constexpr (sizeof(T) * N == 4) asm volatile("" : "+v"(*reinterpret_cast<uint32_t*>(&v)));
+    else if constexpr (sizeof(T) * N == 2) asm volatile("" : "+v"(*reinterpret_cast<uint16_t*>(&v)));
 }
 
 // UA: the inner dim is not whole, aligned vectors (an odd length, odd strides): unaligned vectors all the
@@ -425,6 +426,12 @@ __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
             if constexpr (UA) raw[i] = load_pack_unaligned<T, EV>(in + (int64_t)(ty + (i << a.ty_log2)) * a.sa);
             else raw[i] = load_pack_stream<T, EV>(in + (int64_t)(ty + (i << a.ty_log2)) * a.sa);
         }
+    // (Nothing may look inside a loaded value before every load is out: left alone, the compiler widens a 2-byte value
+    // right behind its load, inside the branch that guards it, and so waits for each of the 64 loads before it issues
+    // the next. Pairs of f16 are still taken apart there - a <2 x half> is split in the block of its load - and run
+    // one load at a time; bf16 pairs and every wider vector do not.)
+#pragma unroll
+    for (int i = 0; i < NC; ++i) forget_pack(raw[i]);
     // All-reduce over the thread rows of an inner position. With TX < 64 a wavefront holds 64 / TX of
     // them, TX lanes apart: those meet in a shuffle butterfly, and only one partial row per wavefront
     // goes through LDS (for sixteen thread rows, 4 LDS reads per value instead of 16). Every thread of
@@ -588,7 +595,9 @@ __global__ void __launch_bounds__(1024) col_flat_stats_kernel(const TransposedAr
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
                 const int64_t pos = whole * Lp + p0 + k;
-                v.v[k] = pos < total ? base[pos] : Elem<T>::narrow(neg_inf<CT>());
+                // (the index is clamped and the load unconditional: loads behind a test each wait for the one before)
+                const T e = base[pos < total ? pos : total - 1];
+                v.v[k] = pos < total ? e : Elem<T>::narrow(neg_inf<CT>());
             }
             fold(&v, std::integral_constant<int, 1>{});
         }
@@ -659,10 +668,16 @@ __global__ void __launch_bounds__(1024) col_flat_apply_kernel(const TransposedAr
         else store_pack_stream<T, VEC>(out + it * Lp + p0, o);
     }
     if (it == whole) {
+        T e[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {  // (clamped, unconditional loads: they go out together)
+            const int64_t pos = whole * Lp + p0 + k;
+            e[k] = in[pos < total ? pos : total - 1];
+        }
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
             const int64_t pos = whole * Lp + p0 + k;
-            if (pos < total) out[pos] = apply1(in[pos], k);
+            if (pos < total) out[pos] = apply1(e[k], k);
         }
     }
 }
