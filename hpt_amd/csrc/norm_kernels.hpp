@@ -758,8 +758,18 @@ __global__ void __launch_bounds__(256) norm_tile_kernel(const NormArgs a) {
         CT x[EPL];
 #pragma unroll
         for (int i = 0; i < EPL; ++i) {
+            // Read from an index clamped into the row, all lanes, then select. (Behind a test per element the 2-byte LDS
+            // reads went out one at a time, each waited for before the next; and a value that only the kept side of a
+            // select uses is moved back behind the test, so the reads are pinned first.)
             const int c = tx + i * tpr;
-            x[i] = c < R ? Elem<T>::widen(row[c]) : fill;
+            x[i] = Elem<T>::widen(row[c < R ? c : R - 1]);
+        }
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) asm volatile("" : "+v"(x[i]));
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+            const int c = tx + i * tpr;
+            x[i] = c < R ? x[i] : fill;
         }
         if constexpr (kSoft) {
             CT m = neg_inf<CT>();
