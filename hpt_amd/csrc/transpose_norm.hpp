@@ -419,19 +419,37 @@ __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
     T* out = (T*)a.out + b * a.cols * a.L + e0;
     // this thread's channels: ty, ty + TY, ...
     const int mine = valid ? (a.cols - ty + TY - 1) >> a.ty_log2 : 0;
-    Pack<T, EV> raw[NC];
+    // A pair of f16 is held as its 32 bits until a sweep takes it apart: a loaded <2 x half> is split in the block of
+    // its load, behind the test that guards it, and each of the 64 loads then waits for the one before.
+    constexpr bool kBits = std::is_same<T, f16_t>::value && EV == 2;
+    using Held = typename std::conditional<kBits, uint32_t, Pack<T, EV>>::type;
+    Held raw[NC];
+    auto get = [&](int i) -> Pack<T, EV> {
+        if constexpr (kBits) return __builtin_bit_cast(Pack<T, EV>, raw[i]);
+        else return raw[i];
+    };
+    auto forget = [&](int i) {
+        if constexpr (kBits) asm volatile("" : "+v"(raw[i]));
+        else forget_pack(raw[i]);
+    };
 #pragma unroll
     for (int i = 0; i < NC; ++i)
         if (i < mine) {
-            if constexpr (UA) raw[i] = load_pack_unaligned<T, EV>(in + (int64_t)(ty + (i << a.ty_log2)) * a.sa);
-            else raw[i] = load_pack_stream<T, EV>(in + (int64_t)(ty + (i << a.ty_log2)) * a.sa);
+            const T* src = in + (int64_t)(ty + (i << a.ty_log2)) * a.sa;
+            if constexpr (kBits) {
+                if constexpr (UA) __builtin_memcpy(&raw[i], src, 4);
+                else raw[i] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(src));
+            } else if constexpr (UA) {
+                raw[i] = load_pack_unaligned<T, EV>(src);
+            } else {
+                raw[i] = load_pack_stream<T, EV>(src);
+            }
         }
     // (Nothing may look inside a loaded value before every load is out: left alone, the compiler widens a 2-byte value
     // right behind its load, inside the branch that guards it, and so waits for each of the 64 loads before it issues
-    // the next. Pairs of f16 are still taken apart there - a <2 x half> is split in the block of its load - and run
-    // one load at a time; bf16 pairs and every wider vector do not.)
+    // the next.)
 #pragma unroll
-    for (int i = 0; i < NC; ++i) forget_pack(raw[i]);
+    for (int i = 0; i < NC; ++i) forget(i);
     // All-reduce over the thread rows of an inner position. With TX < 64 a wavefront holds 64 / TX of
     // them, TX lanes apart: those meet in a shuffle butterfly, and only one partial row per wavefront
     // goes through LDS (for sixteen thread rows, 4 LDS reads per value instead of 16). Every thread of
@@ -470,10 +488,10 @@ __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
     for (int i = 0; i < NC; ++i)
         if (i < mine)
 #pragma unroll
-            for (int k = 0; k < EV; ++k) m[k] = MaxC<CT>::comb(m[k], Elem<T>::widen(raw[i].v[k]));
+            for (int k = 0; k < EV; ++k) m[k] = MaxC<CT>::comb(m[k], Elem<T>::widen(get(i).v[k]));
     across(m, [](CT x, CT y) { return MaxC<CT>::comb(x, y); });
 #pragma unroll
-    for (int i = 0; i < NC; ++i) forget_pack(raw[i]);
+    for (int i = 0; i < NC; ++i) forget(i);
     // Types that are their own compute type (f32, f64) have nothing to widen: the softmax sweep overwrites
     // the raw value with its exponential, which is then taken once per element instead of twice (the
     // second exponential cost a quarter of the kernel's time on f32 [512, 512, 512] over axis 0 or 1).
@@ -483,16 +501,16 @@ __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
         if (i < mine)
 #pragma unroll
             for (int k = 0; k < EV; ++k) {
-                const CT e = exp_ct<T>(Elem<T>::widen(raw[i].v[k]) - m[k]);
+                const CT e = exp_ct<T>(Elem<T>::widen(get(i).v[k]) - m[k]);
                 s[k] += (ST)e;
-                if constexpr (kKeepExp) raw[i].v[k] = Elem<T>::narrow(e);
+                if constexpr (kKeepExp) raw[i].v[k] = Elem<T>::narrow(e);  // (f32 / f64 only: raw is the pack itself)
             }
     // (the thread's total is rounded to the compute type once; the thread rows then add up along a tree)
 #pragma unroll
     for (int k = 0; k < EV; ++k) sf[k] = (CT)s[k];
     across(sf, [](CT x, CT y) { return x + y; });
 #pragma unroll
-    for (int i = 0; i < NC; ++i) forget_pack(raw[i]);
+    for (int i = 0; i < NC; ++i) forget(i);
     // (likewise the channel indices and the `i < mine` masks of the load sweep: carried to the store sweep
     // they cost a register per chunk; recomputing them is an instruction each)
     int ty_st = ty, mine_st = mine;
@@ -506,9 +524,9 @@ __global__ void __launch_bounds__(256) col_reg_kernel(const ColRegArgs a) {
 #pragma unroll
             for (int k = 0; k < EV; ++k) {
                 if constexpr (kKeepExp) {
-                    o.v[k] = Elem<T>::narrow(Elem<T>::widen(raw[i].v[k]) * kk[k]);
+                    o.v[k] = Elem<T>::narrow(Elem<T>::widen(get(i).v[k]) * kk[k]);
                 } else {
-                    const CT d = Elem<T>::widen(raw[i].v[k]) - m[k];
+                    const CT d = Elem<T>::widen(get(i).v[k]) - m[k];
                     o.v[k] = Elem<T>::narrow(kLog ? d - kk[k] : exp_ct<T>(d) * kk[k]);
                 }
             }

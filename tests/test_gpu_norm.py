@@ -592,6 +592,10 @@ CHANNEL_CASES = [
     ("f32 [2, 21, 213, 211] axis 1", np.float32, [2, 21, 213, 211], 1),
     ("f64 [2, 9, 70001] axis 1", np.float64, [2, 9, 70001], 1),
     ("f16 [300, 70001] axis 0 (16 thread rows)", np.float16, [300, 70001], 0),
+    # a narrow inner dim of whole PAIRS of two-byte elements: 64 four-byte loads per thread
+    ("f16 [300, 300, 18] axis 1 (pairs, 8 thread rows)", np.float16, [300, 300, 18], 1),
+    ("bf16 [200, 512, 10] axis 1 (single two-byte elements, 8 thread rows)", "bf16", [200, 512, 10], 1),
+    ("f16 [500, 100, 14] axis 1 (single two-byte elements, 2 thread rows)", np.float16, [500, 100, 14], 1),
 ]
 
 
