@@ -935,11 +935,16 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
         }
         // Mid-sized slabs with a very narrow inner dim ([B, 1000, 3], [B, 2048, 5]): one workgroup per slab through LDS.
         // (From 16 bytes of inner dim on the register kernel, which serves axes up to 1024, is as fast or faster:
-        // f32 [2048, 1024, 8] 4.0 against 2.6 TB/s; beyond 1024 the alternative is the three-pass flat walk.)
+        // f32 [2048, 1024, 8] 4.0 against 2.6 TB/s; beyond 1024 the alternative is the three-pass flat walk.
+        // Four-byte inner dims of 5 ... 11 elements that are not whole vectors are the exception - the register kernel
+        // loads them one or two elements at a time: f32, % of the HBM peak, registers -> slab: [4000, 512, 5] 29.5 -> 45.7,
+        // [4000, 512, 7] 31.6 -> 46.8, [4000, 300, 10] 37.1 -> 45.3, [4000, 300, 11] 34.0 -> 43.9, [8000, 100, 6] 23.3 -> 33.1.
+        // Two-byte inner dims of 7 ... 20 elements go either way by a few points and stay; f64 gains nothing.)
         if (nk == 2 && max_vec > 1 && p.cols > 64 && sa == p.kept_in.size[1] && p.kept_in.stride[1] == 1 &&
             p.kept_out.stride[1] == 1 && p.kept_in.size[1] == p.out_axis_stride &&
             p.kept_in.stride[0] == p.cols * sa && p.kept_out.stride[0] == p.cols * sa &&
-            p.cols * sa * (int64_t)elem_size <= (64 << 10) && sa * (int64_t)elem_size <= (p.cols > 1024 ? 32 : 12) && p.kept_in.size[0] >= 256 &&
+            p.cols * sa * (int64_t)elem_size <= (64 << 10) && sa * (int64_t)elem_size <= ((p.cols > 1024 || (elem_size == 4 && sa % max_vec != 0)) ? (elem_size == 4 && sa % max_vec != 0 ? 48 : 32) : 12) &&
+            p.kept_in.size[0] >= 256 &&
             p.rows * p.cols * (int64_t)elem_size >= (4ll << 20) && ((uintptr_t)in_data % elem_size) == 0 &&
             ((uintptr_t)out_data % elem_size) == 0) {
             p.kind = NormKind::Col;

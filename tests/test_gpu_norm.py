@@ -617,6 +617,10 @@ SLAB_CASES = [
     ("f32 [1200, 500, 2] axis 1", np.float32, [1200, 500, 2], 1),
     ("f64 [300, 1100, 3] axis 1", np.float64, [300, 1100, 3], 1),
     ("f16 [2, 300, 2049, 7] axis 2 (odd slab size)", np.float16, [2, 300, 2049, 7], 2),
+    # four-byte inner dims up to 11 elements that are not whole vectors
+    ("f32 [600, 512, 7] axis 1", np.float32, [600, 512, 7], 1),
+    ("f32 [500, 300, 11] axis 1", np.float32, [500, 300, 11], 1),
+    ("f32 [8000, 100, 6] axis 1 (short axis)", np.float32, [8000, 100, 6], 1),
 ]
 
 
