@@ -1049,6 +1049,16 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                     return p;
                 }
             }
+            // Inner rows that are not whole, aligned vectors and too wide for the flat walk (an odd inner length of
+            // thousands): a lane still takes a vector's worth of neighbouring inner positions, unaligned, instead of one
+            // element (a wavefront then reads 1 KiB per axis position, not 128 or 256 bytes). Below a wavefront of vectors
+            // the single elements already cover the inner row in one step.
+            if (!vec_ok && max_vec > 1 && L >= 64 * max_vec && ((uintptr_t)in_data % elem_size) == 0 &&
+                ((uintptr_t)out_data % elem_size) == 0) {
+                v = max_vec;
+                p.vec = v;
+                p.shift = 1;
+            }
             const int64_t groups = (L + 64 * v - 1) / (64 * v) * batch;
             int64_t S = std::max<int64_t>(1, std::min<int64_t>(512 / groups, p.cols / 32));
             p.tsplit = (int)std::min<int64_t>(S, 64);
@@ -1106,7 +1116,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg) ? "-unaligned" : (p.lds_rows ? "-lds-shift" : "-shift")) : (p.gb_lds == 2 ? "-l2gb" : p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.group_tile ? "-group-tile" : (p.slab_tile ? "-slab" : "")), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg || p.kind == NormKind::ColSplit) ? "-unaligned" : (p.lds_rows ? "-lds-shift" : "-shift")) : (p.gb_lds == 2 ? "-l2gb" : p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.group_tile ? "-group-tile" : (p.slab_tile ? "-slab" : "")), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     if (p.kind == NormKind::RowReg) s += "max_blocks=" + std::to_string(p.max_blocks) + " ";  // (layernorm walks its rows)

@@ -99,8 +99,16 @@ template <class T, int VEC> void launch_col_split(const NormPlan& p, const NormA
     }
     const unsigned nw = (unsigned)p.tpr;
     const unsigned rg = (unsigned)((t.R + 64 * VEC - 1) / (64 * VEC));
-    transposed_stats_kernel<KIND, T, VEC>
-        <<<dim3(rg, (unsigned)t.S, batch), dim3(64 * nw), (size_t)nw * VEC * 64 * sizeof(Part), st>>>(t);
+    const bool ua = VEC > 1 && p.shift;  // inner rows off the vector grid: unaligned vectors
+    if (ua && t.R < VEC) fail(HPT_ERR_KERNEL, "col-split: an inner row of %d elements holds no vector of %d", t.R, VEC);
+    if constexpr (VEC > 1) {
+        if (ua)
+            transposed_stats_kernel<KIND, T, VEC, true>
+                <<<dim3(rg, (unsigned)t.S, batch), dim3(64 * nw), (size_t)nw * VEC * 64 * sizeof(Part), st>>>(t);
+    }
+    if (!ua)
+        transposed_stats_kernel<KIND, T, VEC>
+            <<<dim3(rg, (unsigned)t.S, batch), dim3(64 * nw), (size_t)nw * VEC * 64 * sizeof(Part), st>>>(t);
     transposed_finalize_kernel<KIND, T><<<dim3((unsigned)((t.R + 15) / 16), 1, batch), dim3(16, 16), 0, st>>>(t);
     // apply: enough axis chunks for ~2048 workgroups, at least 16 positions each
     int64_t want = (2048 + (int64_t)rg * batch - 1) / ((int64_t)rg * batch);
@@ -108,6 +116,12 @@ template <class T, int VEC> void launch_col_split(const NormPlan& p, const NormA
     chunks = std::min<int64_t>(chunks, 65535);
     const int chunk = (int)((t.cols + chunks - 1) / chunks);
     chunks = (t.cols + chunk - 1) / chunk;
+    if constexpr (VEC > 1) {
+        if (ua) {
+            col_apply_kernel<KIND, T, VEC, true><<<dim3(rg, (unsigned)chunks, batch), dim3(256), 0, st>>>(t, chunk);
+            return;
+        }
+    }
     col_apply_kernel<KIND, T, VEC><<<dim3(rg, (unsigned)chunks, batch), dim3(256), 0, st>>>(t, chunk);
 }
 

@@ -60,7 +60,10 @@ template <int KIND, class T> struct RowPartial {
 // cross-lane merge. Every wavefront takes its own columns; the wavefronts of a
 // workgroup meet in LDS and write one partial per row: partial y of row r goes to
 // stats[b][y][r], y = blockIdx.y.
-template <int KIND, class T, int VEC = 16 / sizeof(T)>
+// UA: the inner rows are not whole, aligned vectors (an odd inner length): the same vectors unaligned; the last
+// lane of an inner row takes its vector from the row's end backwards, so no load leaves the row, and computes the
+// rows it shares with the lane before a second time (the same bits, stored twice).
+template <int KIND, class T, int VEC = 16 / sizeof(T), bool UA = false>
 __global__ void __launch_bounds__(1024) transposed_stats_kernel(const TransposedArgs a) {
     using CT = typename Elem<T>::Wide;
     using Part = typename RowPartial<KIND, T>::type;
@@ -73,7 +76,7 @@ __global__ void __launch_bounds__(1024) transposed_stats_kernel(const Transposed
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // lanes past the last row keep going (they meet the others at the barrier below) on row 0
     const bool valid = (blockIdx.x * 64 + lane) * VEC < a.R;
-    const int r0 = valid ? (blockIdx.x * 64 + lane) * VEC : 0;
+    const int r0 = valid ? (UA ? min((int)(blockIdx.x * 64 + lane) * VEC, a.R - VEC) : (int)(blockIdx.x * 64 + lane) * VEC) : 0;
     // Columns are dealt out round-robin over all P = 4 S wavefronts that share these
     // rows: wavefront p takes columns p, p + P, ... Wavefronts running at the same time
     // then read neighbouring columns, which keeps a power-of-two column pitch from
@@ -133,14 +136,14 @@ __global__ void __launch_bounds__(1024) transposed_stats_kernel(const Transposed
     for (; c + 7 * P < a.cols; c += 8 * P) {  // eight columns in flight per lane
         Pack<T, VEC> v[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = load_pack<T, VEC>(p + i * stepb);
+        for (int i = 0; i < 8; ++i) v[i] = UA ? load_pack_unaligned<T, VEC>(p + i * stepb) : load_pack<T, VEC>(p + i * stepb);
         p += 8 * stepb;
         // keep the scheduler from sinking loads into the arithmetic: all eight stay in flight
         __builtin_amdgcn_sched_barrier(0);
         fold(v, std::integral_constant<int, 8>{});
     }
     for (; c < a.cols; c += P) {
-        Pack<T, VEC> v = load_pack<T, VEC>(p);
+        Pack<T, VEC> v = UA ? load_pack_unaligned<T, VEC>(p) : load_pack<T, VEC>(p);
         p += stepb;
         fold(&v, std::integral_constant<int, 1>{});
     }
@@ -322,16 +325,17 @@ __global__ void __launch_bounds__(256) transposed_apply_kernel(const TransposedA
 // "columns" the axis); the last pass keeps the layout: lanes along the inner dim, each thread
 // holds the VEC per-row numbers in registers and walks a slice of the axis with batches of
 // loads in flight. out is contiguous: [batch][cols][R].
-template <int KIND, class T, int VEC>
+template <int KIND, class T, int VEC, bool UA = false>
 __global__ void __launch_bounds__(256) col_apply_kernel(const TransposedArgs a, int chunk) {
     using CT = typename Elem<T>::Wide;
     constexpr bool kLog = KIND == NORM_LOGSOFTMAX;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    const int r0 = (blockIdx.x * 64 + tx) * VEC;
+    int r0 = (blockIdx.x * 64 + tx) * VEC;
     if (r0 >= a.R) return;
+    if constexpr (UA) r0 = min(r0, a.R - VEC);  // the row's last vector, from its end backwards
     const CT* pp = (const CT*)a.params + (int64_t)blockIdx.z * 3 * a.R + r0;
-    const Pack<CT, VEC> p0 = *reinterpret_cast<const Pack<CT, VEC>*>(pp);
-    const Pack<CT, VEC> p1 = *reinterpret_cast<const Pack<CT, VEC>*>(pp + a.R);
+    const Pack<CT, VEC> p0 = UA ? load_pack_unaligned<CT, VEC>(pp) : *reinterpret_cast<const Pack<CT, VEC>*>(pp);
+    const Pack<CT, VEC> p1 = UA ? load_pack_unaligned<CT, VEC>(pp + a.R) : *reinterpret_cast<const Pack<CT, VEC>*>(pp + a.R);
     const T* in = (const T*)a.in + (int64_t)blockIdx.z * a.bi + r0;
     T* out = (T*)a.out + (int64_t)blockIdx.z * a.cols * a.R + r0;
     const int c_end = min(a.cols, (int)(blockIdx.y + 1) * chunk);
@@ -342,18 +346,23 @@ __global__ void __launch_bounds__(256) col_apply_kernel(const TransposedArgs a, 
             const CT d = Elem<T>::widen(v.v[k]) - p0.v[k];
             o.v[k] = Elem<T>::narrow(kLog ? d - p1.v[k] : exp_ct<T>(d) * p1.v[k]);
         }
-        if constexpr (VEC > 1) store_pack_stream<T, VEC>(out + (int64_t)c * a.R, o);
+        if constexpr (UA) store_pack_unaligned<T, VEC>(out + (int64_t)c * a.R, o);
+        else if constexpr (VEC > 1) store_pack_stream<T, VEC>(out + (int64_t)c * a.R, o);
         else out[(int64_t)c * a.R] = o.v[0];
+    };
+    auto fetch = [&](int c) {
+        if constexpr (UA) return load_pack_unaligned<T, VEC>(in + (int64_t)c * a.sa);
+        else return load_pack<T, VEC>(in + (int64_t)c * a.sa);
     };
     int c = blockIdx.y * chunk + ty;
     for (; c + 12 < c_end; c += 16) {  // four positions in flight per thread (thread rows are 4 apart)
         Pack<T, VEC> v[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = load_pack<T, VEC>(in + (int64_t)(c + 4 * u) * a.sa);
+        for (int u = 0; u < 4; ++u) v[u] = fetch(c + 4 * u);
 #pragma unroll
         for (int u = 0; u < 4; ++u) apply(v[u], c + 4 * u);
     }
-    for (; c < c_end; c += 4) apply(load_pack<T, VEC>(in + (int64_t)c * a.sa), c);
+    for (; c < c_end; c += 4) apply(fetch(c), c);
 }
 
 // ---- a SHORT strided axis: the whole axis in registers ---------------------------------------

@@ -244,6 +244,36 @@ def test_transposed_tile_masked_and_constant_rows(hpt, dev):
     assert np.array_equal(out, np.broadcast_to(b, out.shape))
 
 
+UNALIGNED_SPLIT_CASES = [  # (dtype, shape, axis, slice of the inner dim or None)
+    ("f32", (1100, 4097), 0, None), ("f16", (1200, 4097), 0, None), ("bf16", (1030, 1025), 0, None), ("f64", (1025, 2049), 0, None),
+    ("f32", (3, 1100, 515), 1, None), ("f16", (2, 1500, 1029), 1, None), ("f32", (300, 259), 0, None), ("f16", (300, 519), 0, None),
+    ("f32", (1100, 4100), 0, (1, 4098)), ("f16", (1100, 2056), 0, (3, 2052)),
+]
+
+
+@pytest.mark.parametrize("dname,shape,axis,cut", UNALIGNED_SPLIT_CASES, ids=lambda v: str(v).replace(" ", ""))
+def test_softmax_over_an_outer_axis_with_an_odd_wide_inner_dim(hpt, orc, dev, dname, shape, axis, cut):
+    """Inner rows that are not whole aligned vectors and too wide for the flat walk: lanes take unaligned vectors, the last
+    lane of an inner row one that overlaps its neighbour's (both then write the same values)."""
+    rng = np.random.default_rng(977)
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    base = hpt.f32_to_bf16_bits(x) if dname == "bf16" else x.astype({"f16": np.float16, "f32": np.float32, "f64": np.float64}[dname])
+    ops = () if cut is None else (("slice", tuple((0, n, 1) for n in shape[:-1]) + ((cut[0], cut[1], 1),)),)
+    t, a = upload(hpt, base, ops, dtype=hpt.bf16 if dname == "bf16" else None, dev=dev)
+    assert hpt.normalize_plan(t, axis).startswith("col-split-unaligned rows"), hpt.normalize_plan(t, axis)
+    for log in (False, True):
+        res = t.log_softmax(axis) if log else t.softmax(axis)
+        if dname in ("f16", "bf16"):
+            tof = hpt.bf16_bits_to_f32 if dname == "bf16" else (lambda v: v.astype(np.float32))
+            got = tof(res.numpy())
+            want = tof(orc.softmax(a, axis, log=log, acc=orc.ACC_F32, dtype=orc.BF16 if dname == "bf16" else None))
+            assert_close(got, want, HALF_RTOL, max(half_atol(want, 8 if dname == "bf16" else 11), 6e-8), f"{dname} {shape} log={log}")
+        elif dname == "f32":
+            assert_close(res.numpy(), orc.softmax(a, axis, log=log, acc=orc.ACC_F64), F32_RTOL, F32_ATOL, f"f32 {shape} log={log}")
+        else:
+            assert_close(res.numpy(), orc.softmax(a, axis, log=log, acc=orc.ACC_F64), 1e-12, 1e-14, f"f64 {shape} log={log}")
+
+
 def test_softmax_over_axis_0_with_a_wide_inner_dim(hpt, orc, dev):
     """Inner dims wider than a workgroup's period (more than 1024 vectors) keep lanes along the inner dim:
     statistics over the axis dealt to wavefronts and workgroups, finalize, apply."""

@@ -128,6 +128,9 @@ def test_plans_for_shapes_off_the_benchmark_list(hpt):
         # softmax over an axis that is not the last
         ([8, 21, 512, 512], None, 1, 0, "col-reg"), ([64, 128, 56, 56], None, 1, 0, "col-reg"),
         ([11184810, 3], None, 0, 0, "col-split-flat"), ([32768, 1024], None, 0, 0, "col-split-flat"), ([4096, 8192], None, 0, 0, "col-split rows"),
+        # an odd inner dim of thousands: unaligned vectors; below a wavefront of vectors, single elements
+        ([8190, 4097], hpt.f16, 0, 0, "col-split-unaligned rows=4097 cols=8190 vec=8"), ([8190, 4097], None, 0, 0, "col-split-unaligned rows=4097 cols=8190 vec=4"),
+        ([2000, 70], None, 0, 0, "col-split rows=70 cols=2000 vec=1"),
     ]
     for shape, dt, axis, nn, want in norm:
         got = hpt.normalize_plan(view(shape, dt), axis, nn)
