@@ -492,7 +492,11 @@ def cases_c8(P):
     nrm(ts, nb, "f32 [131072,8,32] (small groups)", "softmax", 1, "softmax(axis=1)", 131072 * 32)
     del ts
     ts, nb = up([8192, 2048, 2])
-    nrm(ts, nb, "f32 [8192,2048,2] (slabs with a narrow inner dim)", "softmax", 1, "softmax(axis=1)", 8192 * 2)
+    nrm(ts, nb, "f32 [8192,2048,2] (slabs with an inner dim that divides the vector)", "softmax", 1, "softmax(axis=1)", 8192 * 2)
+    del ts
+    ts, nb = up([5592, 2000, 3])
+    nrm(ts, nb, "f32 [5592,2000,3] (slabs with a narrow inner dim)", "softmax", 1, "softmax(axis=1)", 5592 * 3)
+    del ts
     ts1, nb1 = up([33554403])
     red(ts1, nb1, "f32 [33554403] (odd length)", "sum", [0], "sum(all)", 1)
     return cases

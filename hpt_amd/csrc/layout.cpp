@@ -933,6 +933,22 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
                 return p;
             }
         }
+        // Slabs whose inner dim divides the vector (2 or 4 four-byte elements; 2, 4 or 8 two-byte ones; 2 of eight bytes):
+        // the slab is a ROW of cols * L elements for the register row kernel, which keeps one maximum and one sum per
+        // place in the vector - one read and one write, no round trip through LDS.
+        if (nk == 2 && max_vec > 1 && p.cols > 64 && sa > 1 && sa == p.kept_in.size[1] && max_vec % sa == 0 &&
+            p.kept_in.stride[1] == 1 && p.kept_out.stride[1] == 1 && p.kept_in.size[1] == p.out_axis_stride &&
+            p.kept_in.stride[0] == p.cols * sa && p.kept_out.stride[0] == p.cols * sa && (p.cols * sa) % max_vec == 0 &&
+            p.cols * sa * (int64_t)elem_size <= (64 << 10) && p.kept_in.size[0] >= 256 &&
+            p.rows * p.cols * (int64_t)elem_size >= (4ll << 20) && (((uintptr_t)in_data | (uintptr_t)out_data) & 15) == 0) {
+            const int64_t shp[2] = {p.kept_in.size[0], p.cols * sa}, str[2] = {p.cols * sa, 1};
+            NormPlan q = plan_normalize(in_data, out_data, shp, str, 2, 1, 0, elem_size, fused);
+            if (q.kind == NormKind::RowReg && q.vec == max_vec && q.sstride == 1 && !q.shift && !q.tile_rows && !q.gb_lds &&
+                !q.lds_rows && !q.raw_rows) {
+                q.interleave = (int)sa;
+                return q;
+            }
+        }
         // Mid-sized slabs with a very narrow inner dim ([B, 1000, 3], [B, 2048, 5]): one workgroup per slab through LDS.
         // (From 16 bytes of inner dim on the register kernel, which serves axes up to 1024, is as fast or faster:
         // f32 [2048, 1024, 8] 4.0 against 2.6 TB/s; beyond 1024 the alternative is the three-pass flat walk.
@@ -1116,7 +1132,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg || p.kind == NormKind::ColSplit) ? "-unaligned" : (p.lds_rows ? "-lds-shift" : "-shift")) : (p.gb_lds == 2 ? "-l2gb" : p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.group_tile ? "-group-tile" : (p.slab_tile ? "-slab" : "")), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg || p.kind == NormKind::ColSplit) ? "-unaligned" : (p.lds_rows ? "-lds-shift" : "-shift")) : (p.gb_lds == 2 ? "-l2gb" : p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.interleave > 1 ? "-interleaved" : p.group_tile ? "-group-tile" : (p.slab_tile ? "-slab" : "")), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     if (p.kind == NormKind::RowReg) s += "max_blocks=" + std::to_string(p.max_blocks) + " ";  // (layernorm walks its rows)

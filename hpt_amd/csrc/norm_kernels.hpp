@@ -91,6 +91,27 @@ __device__ __forceinline__ A row_all_reduce(A v, int tpr, int ty, A* smem) {
     return v;
 }
 
+// The same for N values at once (one exchange through LDS for all of them; smem holds 16 * N values).
+template <class Op, class A, int N>
+__device__ __forceinline__ void row_all_reduce_n(A (&v)[N], int tpr, int ty, A* smem) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) v[k] = group_reduce<Op>(v[k], tpr < 64 ? tpr : 64);
+    if (tpr > 64) {
+        const int wpr = tpr >> 6;
+        __syncthreads();
+        if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+            for (int k = 0; k < N; ++k) smem[(threadIdx.x >> 6) * N + k] = v[k];
+        }
+        __syncthreads();
+        // (lane w of every wavefront takes wavefront w's values and a butterfly over wpr lanes folds them: N reads and
+        // N * log2(wpr) shuffles per thread instead of N * wpr reads)
+        const int w = threadIdx.x & (wpr - 1);
+#pragma unroll
+        for (int k = 0; k < N; ++k) v[k] = group_reduce<Op>(smem[(ty * wpr + w) * N + k], wpr);
+    }
+}
+
 // ---- rows held in registers ---------------------------------------------------
 // grid.x workgroups walk the rows in steps of gridDim.x * rpb, so that gamma and
 // beta are fetched once per thread (they index by column, and a thread keeps its
@@ -115,8 +136,13 @@ __device__ __forceinline__ A row_all_reduce(A v, int tpr, int ty, A* smem) {
 // GB = 1, "GBL" (layernorm of 2-byte types, long rows): gamma / beta live in LDS instead of registers (loaded
 // once per workgroup, read per row), which leaves room for four vectors of the row per thread where
 // the register form holds two: half as many threads per row, twice as many rows in flight.
-template <int KIND, class T, int VEC, int NCHUNK, int SS = 1, bool SHIFT = false, bool PF = false, int GB = 0>
+// IL > 1 (softmax kinds, IL divides VEC): a "row" is a contiguous [cols / IL, IL] slab and the softmax runs over its
+// first dim - IL interleaved softmaxes, element e of the row belonging to number e % IL, which for whole aligned
+// vectors is the element's place in its vector. The statistics are IL values instead of one; loads and stores are
+// those of a plain row (softmax over the middle axis of a contiguous [B, C, 2] or [B, C, 4]).
+template <int KIND, class T, int VEC, int NCHUNK, int SS = 1, bool SHIFT = false, bool PF = false, int GB = 0, int IL = 1>
 __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
+    static_assert(IL == 1 || (!norm_is_layer(KIND) && !norm_is_causal(KIND) && SS == 1 && !SHIFT && VEC % IL == 0), "interleaved rows: a plain softmax of whole vectors");
     constexpr bool GBL = GB == 1;  // gamma / beta in LDS
     constexpr bool GBG = GB == 2;  // gamma / beta from global memory, every row
     static_assert(GB == 0 || (norm_is_layer(KIND) && VEC > 1 && SS == 1 && !SHIFT), "gamma / beta outside registers: an aligned layernorm form");
@@ -124,7 +150,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     constexpr int UV = VEC / SS;  // useful elements per vector
     using CT = typename Elem<T>::Wide;
     using ST = typename StatType<T>::type;
-    __shared__ __align__(8) unsigned char smem_stat[16 * sizeof(double)];
+    __shared__ __align__(8) unsigned char smem_stat[16 * IL * sizeof(double)];
     CT* smem = reinterpret_cast<CT*>(smem_stat);
     ST* ssmem = reinterpret_cast<ST*>(smem_stat);
     const int tpr = a.tpr;
@@ -296,13 +322,18 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
         if constexpr (kPrefetch) issue_loads(row0 + row_step);
 
         if constexpr (kSoft) {
-            CT m = neg_inf<CT>();
+            CT mv[IL];
+#pragma unroll
+            for (int k = 0; k < IL; ++k) mv[k] = neg_inf<CT>();
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
-                for (int j = 0; j < UV; ++j) m = MaxC<CT>::comb(m, x[c][j]);
-            m = row_all_reduce<MaxC<CT>>(m, tpr, ty, smem);
-            CT s = 0;
+                for (int j = 0; j < UV; ++j) mv[j % IL] = MaxC<CT>::comb(mv[j % IL], x[c][j]);
+            if constexpr (IL == 1) mv[0] = row_all_reduce<MaxC<CT>>(mv[0], tpr, ty, smem);
+            else row_all_reduce_n<MaxC<CT>>(mv, tpr, ty, smem);
+            CT sv[IL];
+#pragma unroll
+            for (int k = 0; k < IL; ++k) sv[k] = 0;
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c) {
                 // causal kinds: a chunk that lies wholly above the diagonal (the same for every lane
@@ -315,19 +346,22 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                 }
 #pragma unroll
                 for (int j = 0; j < UV; ++j) {
-                    CT d = x[c][j] - m;
+                    CT d = x[c][j] - mv[j % IL];
                     CT e = exp_ct<T>(d);
-                    s += e;
+                    sv[j % IL] += e;
                     x[c][j] = kLog ? d : e;
                 }
             }
-            s = row_all_reduce<SumC<CT>>(s, tpr, ty, smem);
-            const CT k = kLog ? log_ct<T>(s) : (CT)1 / s;
+            if constexpr (IL == 1) sv[0] = row_all_reduce<SumC<CT>>(sv[0], tpr, ty, smem);
+            else row_all_reduce_n<SumC<CT>>(sv, tpr, ty, smem);
+            CT kv[IL];
+#pragma unroll
+            for (int k = 0; k < IL; ++k) kv[k] = kLog ? log_ct<T>(sv[k]) : (CT)1 / sv[k];
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
                 for (int j = 0; j < UV; ++j)
-                    x[c][j] = kLog ? x[c][j] - k : x[c][j] * k;
+                    x[c][j] = kLog ? x[c][j] - kv[j % IL] : x[c][j] * kv[j % IL];
         } else {
             // (the lane's own sum is taken in the wide type too: a lane may hold the whole of a short row,
             // and a row whose spread is small against its offset loses digits of the mean that matter)

@@ -42,6 +42,25 @@ void launch_row_reg(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block,
     }
 }
 
+// Rows that are [cols / IL, IL] slabs, softmax over the first dim (whole aligned vectors, IL a divisor of the vector).
+template <class T, int VEC, int IL>
+void launch_row_reg_interleaved(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block, hipStream_t st) {
+    if constexpr ((KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX) && IL > 1 && VEC % IL == 0) {
+        switch (p.nchunk) {
+            case 1: row_reg_kernel<KIND, T, VEC, 1, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 2: row_reg_kernel<KIND, T, VEC, 2, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 3: row_reg_kernel<KIND, T, VEC, 3, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 4: row_reg_kernel<KIND, T, VEC, 4, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 5: row_reg_kernel<KIND, T, VEC, 5, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 6: row_reg_kernel<KIND, T, VEC, 6, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 7: row_reg_kernel<KIND, T, VEC, 7, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 8: row_reg_kernel<KIND, T, VEC, 8, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
+            default: break;
+        }
+    }
+    fail(HPT_ERR_KERNEL, "interleaved rows: no kernel for %d vectors per thread of %d interleaved softmaxes", p.nchunk, IL);
+}
+
 // Few, very long rows: several workgroups per row.
 template <class T, int VEC, bool UA> void launch_row_split(const NormPlan& p, const NormArgs& a, hipStream_t st) {
     RowSplitArgs r{};
@@ -355,6 +374,16 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
             else row_stream_kernel<KIND, T, 1><<<grid, block, 0, st>>>(a);
         }
         return;
+    }
+    if (p.kind == NormKind::RowReg && p.interleave > 1) {
+        if (p.vec != FULL || p.sstride != 1 || p.shift || p.tile_rows || p.gb_lds || FULL % p.interleave != 0 || p.cols % FULL != 0)
+            fail(HPT_ERR_KERNEL, "interleaved rows need whole aligned vectors");
+        switch (p.interleave) {
+            case 2: launch_row_reg_interleaved<T, FULL, 2>(p, a, grid, block, st); return;
+            case 4: launch_row_reg_interleaved<T, FULL, 4>(p, a, grid, block, st); return;
+            case 8: launch_row_reg_interleaved<T, FULL, 8>(p, a, grid, block, st); return;
+            default: fail(HPT_ERR_KERNEL, "interleaved rows: %d softmaxes per row", p.interleave);
+        }
     }
     if (p.kind == NormKind::RowReg) {
         // Layernorm workgroups walk the rows (gamma / beta stay in registers);

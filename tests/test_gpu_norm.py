@@ -244,6 +244,35 @@ def test_transposed_tile_masked_and_constant_rows(hpt, dev):
     assert np.array_equal(out, np.broadcast_to(b, out.shape))
 
 
+INTERLEAVED_CASES = [  # (dtype, shape, axis): softmax over the middle axis, the inner dim a divisor of the 16-byte vector
+    ("f32", (600, 2048, 2), 1), ("f32", (700, 1000, 4), 1), ("f32", (3000, 200, 4), 1), ("f32", (300, 4000, 4), 1), ("f32", (3, 300, 1000, 2), 2),
+    ("f32", (2000, 1001, 4), 1), ("f32", (2000, 330, 2), 1), ("f16", (900, 1000, 8), 1), ("f16", (800, 3000, 2), 1), ("f16", (4000, 300, 4), 1),
+    ("f16", (256, 4096, 8), 1), ("bf16", (700, 1500, 4), 1), ("bf16", (600, 700, 8), 1), ("f64", (600, 1000, 2), 1), ("f64", (256, 4096, 2), 1),
+]
+
+
+@pytest.mark.parametrize("dname,shape,axis", INTERLEAVED_CASES, ids=lambda v: str(v).replace(" ", ""))
+def test_softmax_over_the_middle_axis_with_an_inner_dim_that_divides_the_vector(hpt, orc, dev, dname, shape, axis):
+    """Contiguous [B, C, L] slabs with L | 16 bytes run as rows of C * L elements in registers, one (max, sum) per place in
+    the vector. The inner positions get offsets far apart, so a statistic taken over the wrong place shows at once."""
+    rng = np.random.default_rng(978)
+    x = (rng.standard_normal(shape) * 3).astype(np.float32) + (np.arange(shape[-1], dtype=np.float32) * 37.0 - 40.0)
+    base = hpt.f32_to_bf16_bits(x) if dname == "bf16" else x.astype({"f16": np.float16, "f32": np.float32, "f64": np.float64}[dname])
+    t, a = upload(hpt, base, dtype=hpt.bf16 if dname == "bf16" else None, dev=dev)
+    assert hpt.normalize_plan(t, axis).startswith("rowreg-interleaved rows"), hpt.normalize_plan(t, axis)
+    for log in (False, True):
+        res = t.log_softmax(axis) if log else t.softmax(axis)
+        if dname in ("f16", "bf16"):
+            tof = hpt.bf16_bits_to_f32 if dname == "bf16" else (lambda v: v.astype(np.float32))
+            got = tof(res.numpy())
+            want = tof(orc.softmax(a, axis, log=log, acc=orc.ACC_F32, dtype=orc.BF16 if dname == "bf16" else None))
+            assert_close(got, want, HALF_RTOL, max(half_atol(want, 8 if dname == "bf16" else 11), 6e-8), f"{dname} {shape} log={log}")
+        elif dname == "f32":
+            assert_close(res.numpy(), orc.softmax(a, axis, log=log, acc=orc.ACC_F64), F32_RTOL, F32_ATOL, f"f32 {shape} log={log}")
+        else:
+            assert_close(res.numpy(), orc.softmax(a, axis, log=log, acc=orc.ACC_F64), 1e-12, 1e-14, f"f64 {shape} log={log}")
+
+
 UNALIGNED_SPLIT_CASES = [  # (dtype, shape, axis, slice of the inner dim or None)
     ("f32", (1100, 4097), 0, None), ("f16", (1200, 4097), 0, None), ("bf16", (1030, 1025), 0, None), ("f64", (1025, 2049), 0, None),
     ("f32", (3, 1100, 515), 1, None), ("f16", (2, 1500, 1029), 1, None), ("f32", (300, 259), 0, None), ("f16", (300, 519), 0, None),
@@ -644,7 +673,7 @@ SLAB_CASES = [
     ("f16 [900, 1000, 3] axis 1", np.float16, [900, 1000, 3], 1),
     ("f32 [300, 1092, 5] axis 1 (slabs off 16-byte boundaries)", np.float32, [300, 1092, 5], 1),
     ("bf16 [260, 2047, 16] axis 1 (64 KiB slabs)", "bf16", [260, 2047, 16], 1),
-    ("f32 [1200, 500, 2] axis 1", np.float32, [1200, 500, 2], 1),
+    ("f32 [1200, 501, 2] axis 1 (slabs of half vectors)", np.float32, [1200, 501, 2], 1),
     ("f64 [300, 1100, 3] axis 1", np.float64, [300, 1100, 3], 1),
     ("f16 [2, 300, 2049, 7] axis 2 (odd slab size)", np.float16, [2, 300, 2049, 7], 2),
     # four-byte inner dims up to 11 elements that are not whole vectors
@@ -654,7 +683,16 @@ SLAB_CASES = [
 ]
 
 
-@pytest.mark.parametrize("case", CHANNEL_CASES + GROUP_CASES + SLAB_CASES, ids=[c[0] for c in CHANNEL_CASES + GROUP_CASES + SLAB_CASES])
+INTERLEAVED_SLAB_CASES = [  # an inner dim that divides the vector: the slab is a row in registers
+    ("f32 [1200, 500, 2] axis 1", np.float32, [1200, 500, 2], 1),
+    ("f16 [700, 900, 4] axis 1", np.float16, [700, 900, 4], 1),
+    ("bf16 [2, 300, 2048, 8] axis 2", "bf16", [2, 300, 2048, 8], 2),
+    ("f64 [300, 1100, 2] axis 1", np.float64, [300, 1100, 2], 1),
+]
+
+
+@pytest.mark.parametrize("case", CHANNEL_CASES + GROUP_CASES + SLAB_CASES + INTERLEAVED_SLAB_CASES,
+                         ids=[c[0] for c in CHANNEL_CASES + GROUP_CASES + SLAB_CASES + INTERLEAVED_SLAB_CASES])
 def test_softmax_over_a_short_strided_axis_in_registers(hpt, orc, dev, case):
     """softmax over the channels of [B, C, H, W], C <= 64: every thread keeps the whole axis of its
     inner positions in registers (one read, one write). Small [C, L] groups laid back to back go
@@ -674,7 +712,8 @@ def test_softmax_over_a_short_strided_axis_in_registers(hpt, orc, dev, case):
         cv, dt, odt, bits, tof, acc = (lambda v: v.astype(npdt)), None, None, 0, (lambda v: v), orc.ACC_F64
     a = cv(x)
     t = hpt.Tensor.from_numpy(a, dt).to_hip(dev)
-    want_plan = "col-group-tile" if case in GROUP_CASES else "col-slab" if case in SLAB_CASES else "col-reg"
+    want_plan = ("col-group-tile" if case in GROUP_CASES else "col-slab" if case in SLAB_CASES else
+                 "rowreg-interleaved" if case in INTERLEAVED_SLAB_CASES else "col-reg")
     assert hpt.normalize_plan(t, axis).startswith(want_plan), hpt.normalize_plan(t, axis)
     for log in (False, True):
         got = tof((t.log_softmax(axis) if log else t.softmax(axis)).numpy())
@@ -828,7 +867,7 @@ DOMINANT_CASES = [
     ([4096, 4096], 1, False, "rowreg"), ([8192, 1000], 1, False, "rowreg"), ([1000000, 8], 1, False, "rowreg+tile"),
     ([64, 65536], 1, False, "rowsplit"), ([8, 400000], 1, False, "rowsplit"),
     ([17310, 256, 2], 1, False, "col-group-tile"), ([100000, 16, 2], 1, False, "col-group-tile"),
-    ([2048, 2048, 2], 1, False, "col-slab"), ([512, 1000, 3], 1, False, "col-slab"),
+    ([2048, 2047, 2], 1, False, "col-slab"), ([512, 1000, 3], 1, False, "col-slab"), ([2048, 2048, 2], 1, False, "rowreg-interleaved"),
     ([8, 512, 4096], 1, False, "col-reg"), ([4, 128, 3136], 1, False, "col-reg"), ([64, 64, 3000], 1, False, "col-reg"),
     ([200000, 3], 0, False, "col-split"), ([100000, 33], 0, False, "col-split-flat"), ([32768, 1024], 0, False, "col-split-flat"),
     ([4096, 4096], 1, True, "transposed-tile"),
