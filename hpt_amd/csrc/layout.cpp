@@ -936,15 +936,20 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
         // Slabs whose inner dim divides the vector (2 or 4 four-byte elements; 2, 4 or 8 two-byte ones; 2 of eight bytes):
         // the slab is a ROW of cols * L elements for the register row kernel, which keeps one maximum and one sum per
         // place in the vector - one read and one write, no round trip through LDS.
-        if (nk == 2 && max_vec > 1 && p.cols > 64 && sa > 1 && sa == p.kept_in.size[1] && max_vec % sa == 0 &&
+        // An inner dim of two vectors (8 four-byte heads, 16 two-byte ones) likewise, where the axis is too long for the
+        // register columns (which are faster up to 1024: f32 [2048, 512, 16] 22.1 against 28.3 us; beyond, against the
+        // slab and the flat walk, f32 [1000, 2048, 8] 60.0 -> 31.1): a thread's vectors all hold the same places, and
+        // only threads two apart are folded together.
+        if (nk == 2 && max_vec > 1 && p.cols > 64 && sa > 1 && sa == p.kept_in.size[1] &&
+            (max_vec % sa == 0 || (sa == 2 * max_vec && p.cols > 1024)) &&
             p.kept_in.stride[1] == 1 && p.kept_out.stride[1] == 1 && p.kept_in.size[1] == p.out_axis_stride &&
             p.kept_in.stride[0] == p.cols * sa && p.kept_out.stride[0] == p.cols * sa && (p.cols * sa) % max_vec == 0 &&
-            p.cols * sa * (int64_t)elem_size <= (64 << 10) && p.kept_in.size[0] >= 256 &&
+            p.cols * sa * (int64_t)elem_size <= (128 << 10) && p.kept_in.size[0] >= 256 &&
             p.rows * p.cols * (int64_t)elem_size >= (4ll << 20) && (((uintptr_t)in_data | (uintptr_t)out_data) & 15) == 0) {
             const int64_t shp[2] = {p.kept_in.size[0], p.cols * sa}, str[2] = {p.cols * sa, 1};
             NormPlan q = plan_normalize(in_data, out_data, shp, str, 2, 1, 0, elem_size, fused);
             if (q.kind == NormKind::RowReg && q.vec == max_vec && q.sstride == 1 && !q.shift && !q.tile_rows && !q.gb_lds &&
-                !q.lds_rows && !q.raw_rows) {
+                !q.lds_rows && !q.raw_rows && q.tpr * max_vec >= sa) {
                 q.interleave = (int)sa;
                 return q;
             }

@@ -91,24 +91,47 @@ __device__ __forceinline__ A row_all_reduce(A v, int tpr, int ty, A* smem) {
     return v;
 }
 
-// The same for N values at once (one exchange through LDS for all of them; smem holds 16 * N values).
-template <class Op, class A, int N>
+// The same for N values at once (one exchange through LDS for all of them; smem holds 16 * G * N values).
+// G > 1: neighbouring lanes hold DIFFERENT statistics - lane l those of number l % G - and only lanes with the same
+// l % G are folded: the butterflies start at distance G.
+template <class Op, class A, int N, int G = 1>
 __device__ __forceinline__ void row_all_reduce_n(A (&v)[N], int tpr, int ty, A* smem) {
+    static_assert(G == 1 || G == 2 || G == 4, "up to four lanes side by side (the wavefronts' partials are folded by one wavefront's lanes)");
+    const int width = tpr < 64 ? tpr : 64;
 #pragma unroll
-    for (int k = 0; k < N; ++k) v[k] = group_reduce<Op>(v[k], tpr < 64 ? tpr : 64);
+    for (int k = 0; k < N; ++k) {
+        if constexpr (G == 1) {
+            v[k] = group_reduce<Op>(v[k], width);
+        } else {
+#pragma unroll
+            for (int d = G; d < 64; d <<= 1)
+                if (d < width) v[k] = Op::comb(v[k], shfl_xor_any(v[k], d));
+        }
+    }
     if (tpr > 64) {
         const int wpr = tpr >> 6;
+        const int lane = threadIdx.x & 63;
         __syncthreads();
-        if ((threadIdx.x & 63) == 0) {
+        if (lane < G) {
 #pragma unroll
-            for (int k = 0; k < N; ++k) smem[(threadIdx.x >> 6) * N + k] = v[k];
+            for (int k = 0; k < N; ++k) smem[((threadIdx.x >> 6) * G + lane) * N + k] = v[k];
         }
         __syncthreads();
-        // (lane w of every wavefront takes wavefront w's values and a butterfly over wpr lanes folds them: N reads and
+        // (lanes take one wavefront's values each and a butterfly over them folds the wavefronts: N reads and
         // N * log2(wpr) shuffles per thread instead of N * wpr reads)
-        const int w = threadIdx.x & (wpr - 1);
+        const int w = (lane / G) & (wpr - 1), g = lane % G;
 #pragma unroll
-        for (int k = 0; k < N; ++k) v[k] = group_reduce<Op>(smem[(ty * wpr + w) * N + k], wpr);
+        for (int k = 0; k < N; ++k) {
+            A r = smem[((ty * wpr + w) * G + g) * N + k];
+            if constexpr (G == 1) {
+                r = group_reduce<Op>(r, wpr);
+            } else {
+#pragma unroll
+                for (int d = G; d < 64; d <<= 1)
+                    if (d < G * wpr) r = Op::comb(r, shfl_xor_any(r, d));
+            }
+            v[k] = r;
+        }
     }
 }
 
@@ -136,13 +159,16 @@ __device__ __forceinline__ void row_all_reduce_n(A (&v)[N], int tpr, int ty, A* 
 // GB = 1, "GBL" (layernorm of 2-byte types, long rows): gamma / beta live in LDS instead of registers (loaded
 // once per workgroup, read per row), which leaves room for four vectors of the row per thread where
 // the register form holds two: half as many threads per row, twice as many rows in flight.
-// IL > 1 (softmax kinds, IL divides VEC): a "row" is a contiguous [cols / IL, IL] slab and the softmax runs over its
-// first dim - IL interleaved softmaxes, element e of the row belonging to number e % IL, which for whole aligned
-// vectors is the element's place in its vector. The statistics are IL values instead of one; loads and stores are
-// those of a plain row (softmax over the middle axis of a contiguous [B, C, 2] or [B, C, 4]).
+// IL > 1 (softmax kinds): a "row" is a contiguous [cols / IL, IL] slab and the softmax runs over its first dim - IL
+// interleaved softmaxes, element e of the row belonging to number e % IL. IL divides VEC: that is the element's place
+// in its vector, and a thread keeps IL (max, sum) pairs. IL = 2 vectors: a thread's vectors all hold the same VEC
+// numbers (threads per row are even), its neighbour the other VEC, and only threads two apart are folded together. Loads and stores are those of a plain row (softmax over the middle axis of a contiguous
+// [B, C, 2], [B, C, 4], [B, C, 8 heads]).
 template <int KIND, class T, int VEC, int NCHUNK, int SS = 1, bool SHIFT = false, bool PF = false, int GB = 0, int IL = 1>
 __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
-    static_assert(IL == 1 || (!norm_is_layer(KIND) && !norm_is_causal(KIND) && SS == 1 && !SHIFT && VEC % IL == 0), "interleaved rows: a plain softmax of whole vectors");
+    static_assert(IL == 1 || (!norm_is_layer(KIND) && !norm_is_causal(KIND) && SS == 1 && !SHIFT && (VEC % IL == 0 || IL % VEC == 0)), "interleaved rows: a plain softmax of whole vectors");
+    constexpr int NS = IL < VEC ? IL : VEC;      // statistics a thread keeps
+    constexpr int IG = IL > VEC ? IL / VEC : 1;  // neighbouring threads that hold different ones
     constexpr bool GBL = GB == 1;  // gamma / beta in LDS
     constexpr bool GBG = GB == 2;  // gamma / beta from global memory, every row
     static_assert(GB == 0 || (norm_is_layer(KIND) && VEC > 1 && SS == 1 && !SHIFT), "gamma / beta outside registers: an aligned layernorm form");
@@ -322,18 +348,18 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
         if constexpr (kPrefetch) issue_loads(row0 + row_step);
 
         if constexpr (kSoft) {
-            CT mv[IL];
+            CT mv[NS];
 #pragma unroll
-            for (int k = 0; k < IL; ++k) mv[k] = neg_inf<CT>();
+            for (int k = 0; k < NS; ++k) mv[k] = neg_inf<CT>();
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
-                for (int j = 0; j < UV; ++j) mv[j % IL] = MaxC<CT>::comb(mv[j % IL], x[c][j]);
+                for (int j = 0; j < UV; ++j) mv[j % NS] = MaxC<CT>::comb(mv[j % NS], x[c][j]);
             if constexpr (IL == 1) mv[0] = row_all_reduce<MaxC<CT>>(mv[0], tpr, ty, smem);
-            else row_all_reduce_n<MaxC<CT>>(mv, tpr, ty, smem);
-            CT sv[IL];
+            else row_all_reduce_n<MaxC<CT>, CT, NS, IG>(mv, tpr, ty, smem);
+            CT sv[NS];
 #pragma unroll
-            for (int k = 0; k < IL; ++k) sv[k] = 0;
+            for (int k = 0; k < NS; ++k) sv[k] = 0;
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c) {
                 // causal kinds: a chunk that lies wholly above the diagonal (the same for every lane
@@ -346,22 +372,22 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                 }
 #pragma unroll
                 for (int j = 0; j < UV; ++j) {
-                    CT d = x[c][j] - mv[j % IL];
+                    CT d = x[c][j] - mv[j % NS];
                     CT e = exp_ct<T>(d);
-                    sv[j % IL] += e;
+                    sv[j % NS] += e;
                     x[c][j] = kLog ? d : e;
                 }
             }
             if constexpr (IL == 1) sv[0] = row_all_reduce<SumC<CT>>(sv[0], tpr, ty, smem);
-            else row_all_reduce_n<SumC<CT>>(sv, tpr, ty, smem);
-            CT kv[IL];
+            else row_all_reduce_n<SumC<CT>, CT, NS, IG>(sv, tpr, ty, smem);
+            CT kv[NS];
 #pragma unroll
-            for (int k = 0; k < IL; ++k) kv[k] = kLog ? log_ct<T>(sv[k]) : (CT)1 / sv[k];
+            for (int k = 0; k < NS; ++k) kv[k] = kLog ? log_ct<T>(sv[k]) : (CT)1 / sv[k];
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
                 for (int j = 0; j < UV; ++j)
-                    x[c][j] = kLog ? x[c][j] - kv[j % IL] : x[c][j] * kv[j % IL];
+                    x[c][j] = kLog ? x[c][j] - kv[j % NS] : x[c][j] * kv[j % NS];
         } else {
             // (the lane's own sum is taken in the wide type too: a lane may hold the whole of a short row,
             // and a row whose spread is small against its offset loses digits of the mean that matter)

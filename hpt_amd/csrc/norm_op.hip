@@ -45,7 +45,7 @@ void launch_row_reg(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block,
 // Rows that are [cols / IL, IL] slabs, softmax over the first dim (whole aligned vectors, IL a divisor of the vector).
 template <class T, int VEC, int IL>
 void launch_row_reg_interleaved(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block, hipStream_t st) {
-    if constexpr ((KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX) && IL > 1 && VEC % IL == 0) {
+    if constexpr ((KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX) && IL > 1 && (VEC % IL == 0 || IL == 2 * VEC)) {
         switch (p.nchunk) {
             case 1: row_reg_kernel<KIND, T, VEC, 1, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
             case 2: row_reg_kernel<KIND, T, VEC, 2, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
@@ -376,12 +376,14 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         return;
     }
     if (p.kind == NormKind::RowReg && p.interleave > 1) {
-        if (p.vec != FULL || p.sstride != 1 || p.shift || p.tile_rows || p.gb_lds || FULL % p.interleave != 0 || p.cols % FULL != 0)
+        if (p.vec != FULL || p.sstride != 1 || p.shift || p.tile_rows || p.gb_lds || p.cols % FULL != 0 ||
+            (FULL % p.interleave != 0 && (p.interleave != 2 * FULL || p.tpr < 2)))
             fail(HPT_ERR_KERNEL, "interleaved rows need whole aligned vectors");
         switch (p.interleave) {
             case 2: launch_row_reg_interleaved<T, FULL, 2>(p, a, grid, block, st); return;
             case 4: launch_row_reg_interleaved<T, FULL, 4>(p, a, grid, block, st); return;
             case 8: launch_row_reg_interleaved<T, FULL, 8>(p, a, grid, block, st); return;
+            case 16: launch_row_reg_interleaved<T, FULL, 16>(p, a, grid, block, st); return;
             default: fail(HPT_ERR_KERNEL, "interleaved rows: %d softmaxes per row", p.interleave);
         }
     }

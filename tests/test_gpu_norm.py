@@ -248,6 +248,11 @@ INTERLEAVED_CASES = [  # (dtype, shape, axis): softmax over the middle axis, the
     ("f32", (600, 2048, 2), 1), ("f32", (700, 1000, 4), 1), ("f32", (3000, 200, 4), 1), ("f32", (300, 4000, 4), 1), ("f32", (3, 300, 1000, 2), 2),
     ("f32", (2000, 1001, 4), 1), ("f32", (2000, 330, 2), 1), ("f16", (900, 1000, 8), 1), ("f16", (800, 3000, 2), 1), ("f16", (4000, 300, 4), 1),
     ("f16", (256, 4096, 8), 1), ("bf16", (700, 1500, 4), 1), ("bf16", (600, 700, 8), 1), ("f64", (600, 1000, 2), 1), ("f64", (256, 4096, 2), 1),
+    # inner dims of two vectors along an axis beyond 1024: neighbouring threads hold different places
+    ("f32", (600, 1280, 8), 1), ("f32", (300, 2048, 8), 1), ("f32", (260, 4096, 8), 1), ("f16", (300, 1536, 16), 1), ("f16", (256, 2048, 16), 1),
+    ("bf16", (1000, 1500, 16), 1), ("f64", (600, 1040, 4), 1), ("f64", (300, 2048, 4), 1), ("f32", (2, 200, 1536, 8), 2),
+    # slabs of 128 KiB
+    ("f32", (256, 16384, 2), 1), ("f16", (256, 6144, 4), 1),
 ]
 
 
@@ -256,7 +261,7 @@ def test_softmax_over_the_middle_axis_with_an_inner_dim_that_divides_the_vector(
     """Contiguous [B, C, L] slabs with L | 16 bytes run as rows of C * L elements in registers, one (max, sum) per place in
     the vector. The inner positions get offsets far apart, so a statistic taken over the wrong place shows at once."""
     rng = np.random.default_rng(978)
-    x = (rng.standard_normal(shape) * 3).astype(np.float32) + (np.arange(shape[-1], dtype=np.float32) * 37.0 - 40.0)
+    x = (rng.standard_normal(shape) * 3).astype(np.float32) + ((np.arange(shape[-1], dtype=np.float32) * 37.0) % 250.0 - 40.0)
     base = hpt.f32_to_bf16_bits(x) if dname == "bf16" else x.astype({"f16": np.float16, "f32": np.float32, "f64": np.float64}[dname])
     t, a = upload(hpt, base, dtype=hpt.bf16 if dname == "bf16" else None, dev=dev)
     assert hpt.normalize_plan(t, axis).startswith("rowreg-interleaved rows"), hpt.normalize_plan(t, axis)
@@ -672,7 +677,7 @@ GROUP_CASES = [
 SLAB_CASES = [
     ("f16 [900, 1000, 3] axis 1", np.float16, [900, 1000, 3], 1),
     ("f32 [300, 1092, 5] axis 1 (slabs off 16-byte boundaries)", np.float32, [300, 1092, 5], 1),
-    ("bf16 [260, 2047, 16] axis 1 (64 KiB slabs)", "bf16", [260, 2047, 16], 1),
+    ("bf16 [260, 2730, 12] axis 1 (64 KiB slabs)", "bf16", [260, 2730, 12], 1),
     ("f32 [1200, 501, 2] axis 1 (slabs of half vectors)", np.float32, [1200, 501, 2], 1),
     ("f64 [300, 1100, 3] axis 1", np.float64, [300, 1100, 3], 1),
     ("f16 [2, 300, 2049, 7] axis 2 (odd slab size)", np.float16, [2, 300, 2049, 7], 2),
@@ -688,6 +693,7 @@ INTERLEAVED_SLAB_CASES = [  # an inner dim that divides the vector: the slab is 
     ("f16 [700, 900, 4] axis 1", np.float16, [700, 900, 4], 1),
     ("bf16 [2, 300, 2048, 8] axis 2", "bf16", [2, 300, 2048, 8], 2),
     ("f64 [300, 1100, 2] axis 1", np.float64, [300, 1100, 2], 1),
+    ("bf16 [260, 2047, 16] axis 1 (64 KiB slabs, two vectors side by side)", "bf16", [260, 2047, 16], 1),
 ]
 
 
