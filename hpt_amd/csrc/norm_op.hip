@@ -43,19 +43,25 @@ void launch_row_reg(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block,
 }
 
 // Rows that are [cols / IL, IL] slabs, softmax over the first dim (whole aligned vectors, IL a divisor of the vector).
-template <class T, int VEC, int IL>
+template <class T, int VEC, int IL, bool PF = false>
 void launch_row_reg_interleaved(const NormPlan& p, const NormArgs& a, dim3 grid, dim3 block, hipStream_t st) {
     if constexpr ((KIND == NORM_SOFTMAX || KIND == NORM_LOGSOFTMAX) && IL > 1 && (VEC % IL == 0 || IL == 2 * VEC)) {
         switch (p.nchunk) {
-            case 1: row_reg_kernel<KIND, T, VEC, 1, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
-            case 2: row_reg_kernel<KIND, T, VEC, 2, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
-            case 3: row_reg_kernel<KIND, T, VEC, 3, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
-            case 4: row_reg_kernel<KIND, T, VEC, 4, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
-            case 5: row_reg_kernel<KIND, T, VEC, 5, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
-            case 6: row_reg_kernel<KIND, T, VEC, 6, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
-            case 7: row_reg_kernel<KIND, T, VEC, 7, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
-            case 8: row_reg_kernel<KIND, T, VEC, 8, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 3: row_reg_kernel<KIND, T, VEC, 3, 1, false, PF, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 4: row_reg_kernel<KIND, T, VEC, 4, 1, false, PF, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 5: row_reg_kernel<KIND, T, VEC, 5, 1, false, PF, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 6: row_reg_kernel<KIND, T, VEC, 6, 1, false, PF, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 7: row_reg_kernel<KIND, T, VEC, 7, 1, false, PF, 0, IL><<<grid, block, 0, st>>>(a); return;
+            case 8: row_reg_kernel<KIND, T, VEC, 8, 1, false, PF, 0, IL><<<grid, block, 0, st>>>(a); return;
             default: break;
+        }
+        // (rows of 512 and 1024 threads hold at least three vectors per thread)
+        if constexpr (!PF) {
+            switch (p.nchunk) {
+                case 1: row_reg_kernel<KIND, T, VEC, 1, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
+                case 2: row_reg_kernel<KIND, T, VEC, 2, 1, false, false, 0, IL><<<grid, block, 0, st>>>(a); return;
+                default: break;
+            }
         }
     }
     fail(HPT_ERR_KERNEL, "interleaved rows: no kernel for %d vectors per thread of %d interleaved softmaxes", p.nchunk, IL);
@@ -379,6 +385,18 @@ template <class T> void launch_t(const NormPlan& p, NormArgs a, hipStream_t st) 
         if (p.vec != FULL || p.sstride != 1 || p.shift || p.tile_rows || p.gb_lds || p.cols % FULL != 0 ||
             (FULL % p.interleave != 0 && (p.interleave != 2 * FULL || p.tpr < 2)))
             fail(HPT_ERR_KERNEL, "interleaved rows need whole aligned vectors");
+        // (the longest slabs: 512 workgroups walk the rows and prefetch the next one - f32 [1000, 16384, 2] 59.7 -> 54.7 us,
+        // f16 [2000, 4096, 8] 98.3 -> 89.3; rows of 512 threads lose by it, f32 [2000, 1280, 8] 35.8 -> 41.5)
+        if (p.tpr == 1024 && p.nchunk >= 3) {
+            if (grid.x > 512u) grid.x = 512u;
+            switch (p.interleave) {
+                case 2: launch_row_reg_interleaved<T, FULL, 2, true>(p, a, grid, block, st); return;
+                case 4: launch_row_reg_interleaved<T, FULL, 4, true>(p, a, grid, block, st); return;
+                case 8: launch_row_reg_interleaved<T, FULL, 8, true>(p, a, grid, block, st); return;
+                case 16: launch_row_reg_interleaved<T, FULL, 16, true>(p, a, grid, block, st); return;
+                default: break;
+            }
+        }
         switch (p.interleave) {
             case 2: launch_row_reg_interleaved<T, FULL, 2>(p, a, grid, block, st); return;
             case 4: launch_row_reg_interleaved<T, FULL, 4>(p, a, grid, block, st); return;
