@@ -492,6 +492,7 @@ def cases_c8(P):
     nrm(ts, nb, "f32 [131072,8,32] (small groups)", "softmax", 1, "softmax(axis=1)", 131072 * 32)
     del ts
     ts, nb = up([8192, 2048, 2])
+    red(ts, nb, "f32 [8192,2048,2] (slabs with an inner dim that divides the vector)", "sum", [1], "sum(axis=1)", 8192 * 2)
     nrm(ts, nb, "f32 [8192,2048,2] (slabs with an inner dim that divides the vector)", "softmax", 1, "softmax(axis=1)", 8192 * 2)
     del ts
     ts, nb = up([5592, 2000, 3])

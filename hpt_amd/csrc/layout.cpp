@@ -234,6 +234,30 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
         // ---- Col: lanes walk the outputs -----------------------------------
         p.kind = ReduceKind::Col;
         const int nk = p.kept.n;
+        // A reduction over the MIDDLE axis of a contiguous [B, C, L] whose inner dim divides the 16-byte vector (L = 2
+        // or 4 four-byte elements; 2, 4 or 8 two-byte ones): the [C, L] slab is one ROW of C * L elements for the lean
+        // row kernel, an element's place in its vector names its output, and a thread keeps L accumulators. Lanes
+        // along L would idle, and the flat walk takes two launches.
+        {
+            const int64_t full = elem_size <= 16 ? (int64_t)(16 / elem_size) : 1;
+            if (nk == 2 && p.red.n == 1 && full > 1 && p.kept.stride[1] == 1 && p.kept.size[1] > 1 && p.kept.size[1] <= 8 && full % p.kept.size[1] == 0 &&
+                p.red.stride[0] == p.kept.size[1] && p.kept.stride[0] == p.R * p.kept.size[1] && p.R > 64 &&
+                (p.R * p.kept.size[1]) % full == 0 && p.R * p.kept.size[1] * (int64_t)elem_size <= (128 << 10) &&
+                p.kept.size[0] >= 256 && p.K * p.R * (int64_t)elem_size >= (4ll << 20) && ((uintptr_t)data & 15) == 0) {
+                const int64_t L = p.kept.size[1];
+                const int64_t shp[2] = {p.kept.size[0], p.R * L}, str[2] = {p.R * L, 1}, ax[1] = {1};
+                ReducePlan q = plan_reduce(data, shp, str, 2, ax, 1, elem_size, acc_size, heavy);
+                if (q.kind == ReduceKind::Row && q.lean && q.vec == full && !q.ragged && !q.unaligned && q.sstride == 1 &&
+                    q.split == 1 && !q.row_tile) {
+                    q.interleave = (int)L;
+                    q.K = p.K;
+                    q.R = p.R;
+                    q.kept = p.kept;
+                    q.red = p.red;
+                    return q;
+                }
+            }
+        }
         // Two kept dims of which the FIRST is the contiguous one (a reduction over the last axis of a
         // permuted view): the lanes must run along that one. List it last; the kernel then scatters
         // its (few) outputs instead of gathering its (many) inputs.
@@ -461,7 +485,7 @@ std::string describe(const ReducePlan& p) {
         case ReduceKind::Identity: return "identity";
         case ReduceKind::Row:
             snprintf(buf, sizeof buf, "row%s%s vec=%d tpr=%d rpb=%d rows=%lld cols=%lld split=%d(%dx%d) ",
-                     p.row_tile ? "-tile" : p.ragged ? "-ragged" : p.lean ? "" : "-general", p.sstride == 2 ? "-step2" : p.unaligned ? "-unaligned" : "", p.vec, p.tpr, p.rpb,
+                     p.row_tile ? "-tile" : p.ragged ? "-ragged" : p.lean ? "" : "-general", p.sstride == 2 ? "-step2" : p.unaligned ? "-unaligned" : p.interleave > 1 ? "-interleaved" : "", p.vec, p.tpr, p.rpb,
                      (long long)p.K, (long long)p.R, p.split, p.split_q, p.split_i);
             break;
         case ReduceKind::Col:

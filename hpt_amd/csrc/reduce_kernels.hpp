@@ -79,19 +79,26 @@ struct RowLeanArgs {
 // UA: short or strided-pitch rows off the grid: unaligned 128-bit loads from the row start on; the
 // last vector of a row is taken from the row's END backwards and the elements it shares with the
 // vector before are skipped, so no load leaves the row.
-template <class Op, int VEC, int SS = 1, bool RAG = false, bool UA = false>
+// IL > 1 (whole aligned vectors, IL divides VEC): a row is a contiguous [rin / IL, IL] slab reduced over its first
+// dim; element e of the row belongs to output e % IL of the row, which is its place in its vector, and to index
+// e / IL along the reduced dim. A thread keeps IL accumulators; output k of a row is out[row * IL + k].
+template <class Op, int VEC, int SS = 1, bool RAG = false, bool UA = false, int IL = 1>
 __global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
     static_assert(!UA || (VEC > 1 && SS == 1 && !RAG), "UA is a full-vector mode of its own");
+    static_assert(IL == 1 || (VEC % IL == 0 && SS == 1 && !RAG && !UA), "interleaved rows are whole aligned vectors");
     using T = typename Op::In;
     using Acc = typename Op::Acc;
     constexpr int UV = VEC / SS;
-    __shared__ Acc smem[16];
+    __shared__ Acc smem[16 * IL];
     const int tpr = a.tpr;
     const int tx = threadIdx.x & (tpr - 1);
     const int ty = threadIdx.x >> a.tpr_log2;
     const int row = blockIdx.x * a.rpb + ty;
     const bool valid = row < a.K;
-    Acc acc = Op::identity();
+    Acc accs[IL];
+#pragma unroll
+    for (int k = 0; k < IL; ++k) accs[k] = Op::identity();
+    Acc& acc = accs[0];
     if (valid) {
         const T* p = (const T*)a.in + (int64_t)row * a.row_stride;
         int nvec = a.rin_v, head = 0;
@@ -117,6 +124,9 @@ __global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
 #pragma unroll
                     for (int j = 0; j < VEC; ++j)
                         if (from + j >= e) fold_in<Op>(acc, v.v[j], from + j);
+                } else if constexpr (IL > 1) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) fold_in<Op>(accs[j % IL], v.v[j], i * (VEC / IL) + j / IL);
                 } else {
 #pragma unroll
                     for (int j = 0; j < UV; ++j) fold_in<Op>(acc, v.v[j * SS], head + i * UV + j);
@@ -140,17 +150,29 @@ __global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
                 for (int i = nvec * VEC + tx; i < a.rin - head; i += tpr) fold_in<Op>(acc, p[i], head + i);
         }
     }
-    acc = group_reduce<Op>(acc, tpr < 64 ? tpr : 64);
+#pragma unroll
+    for (int k = 0; k < IL; ++k) accs[k] = group_reduce<Op>(accs[k], tpr < 64 ? tpr : 64);
     if (tpr > 64) {
         const int wpr = tpr >> 6;  // wavefronts per row
-        if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = acc;
+        if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+            for (int k = 0; k < IL; ++k) smem[(threadIdx.x >> 6) * IL + k] = accs[k];
+        }
         __syncthreads();
         if (tx == 0)
-            for (int w = 1; w < wpr; ++w) acc = Op::comb(acc, smem[ty * wpr + w]);
+            for (int w = 1; w < wpr; ++w) {
+#pragma unroll
+                for (int k = 0; k < IL; ++k) accs[k] = Op::comb(accs[k], smem[(ty * wpr + w) * IL + k]);
+            }
     }
     if (tx == 0 && valid) {
-        if (a.split == 1) write_out<Op>(a.out, row, acc, a.init_out, a.count);
-        else ((Acc*)a.out)[(int64_t)row * a.split + blockIdx.y] = acc;
+        if constexpr (IL > 1) {
+#pragma unroll
+            for (int k = 0; k < IL; ++k) write_out<Op>(a.out, (int64_t)row * IL + k, accs[k], a.init_out, a.count);
+        } else {
+            if (a.split == 1) write_out<Op>(a.out, row, acc, a.init_out, a.count);
+            else ((Acc*)a.out)[(int64_t)row * a.split + blockIdx.y] = acc;
+        }
     }
 }
 
@@ -997,6 +1019,40 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             row_tile_kernel<Op, FULL><<<dim3((unsigned)((p.K + p.row_tile - 1) / p.row_tile)), dim3(256), 0, st>>>(a);
         }
         return;
+    }
+    if (p.kind == ReduceKind::Row && p.interleave > 1) {
+        // rows that are [R, interleave] slabs: the lean kernel over rows of R * interleave elements
+        if (!p.lean || !vec || p.split != 1 || p.sstride != 1 || p.ragged || p.unaligned || FULL % p.interleave != 0 ||
+            p.K % p.interleave != 0 || (p.R * p.interleave) % FULL != 0)
+            fail(HPT_ERR_KERNEL, "interleaved rows need whole aligned vectors and one workgroup per row");
+        const int64_t rows = p.K / p.interleave;
+        const dim3 grid((unsigned)((rows + p.rpb - 1) / p.rpb));
+        const dim3 block((unsigned)(p.tpr * p.rpb));
+        RowLeanArgs a{};
+        a.in = in;
+        a.out = out;
+        a.row_stride = p.R * p.interleave;
+        a.count = count;
+        a.K = (int)rows;
+        a.rin_v = (int)(p.R * p.interleave / FULL);
+        a.rin = (int)(p.R * p.interleave);
+        a.sr = 1;
+        a.ichunk = a.rin_v;
+        a.tpr = p.tpr;
+        a.tpr_log2 = ilog2(p.tpr);
+        a.rpb = p.rpb;
+        a.split = 1;
+        a.init_out = init_out;
+        if constexpr (FULL >= 2) {
+            if (p.interleave == 2) { row_lean_kernel<Op, FULL, 1, false, false, 2><<<grid, block, 0, st>>>(a); return; }
+        }
+        if constexpr (FULL >= 4) {
+            if (p.interleave == 4) { row_lean_kernel<Op, FULL, 1, false, false, 4><<<grid, block, 0, st>>>(a); return; }
+        }
+        if constexpr (FULL >= 8) {
+            if (p.interleave == 8) { row_lean_kernel<Op, FULL, 1, false, false, 8><<<grid, block, 0, st>>>(a); return; }
+        }
+        fail(HPT_ERR_KERNEL, "interleaved rows: %d outputs per row", p.interleave);
     }
     if (p.kind == ReduceKind::Row) {
         dim3 grid((unsigned)((p.K + p.rpb - 1) / p.rpb), (unsigned)p.split);

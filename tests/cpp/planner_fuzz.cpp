@@ -134,6 +134,13 @@ static void fuzz_reduce() {
         CHECK(p.kept.count() == K && p.red.count() == R, "%s plan=%s", show(v).c_str(), d.c_str());
         CHECK(pow2(p.vec) && (size_t)p.vec * elem <= 16, "%s plan=%s", show(v).c_str(), d.c_str());
         CHECK(p.split >= 1 && p.split_q >= 1 && p.split_i >= 1, "%s plan=%s", show(v).c_str(), d.c_str());
+        CHECK(p.interleave >= 1, "%s plan=%s", show(v).c_str(), d.c_str());
+        if (p.interleave > 1)  // rows that are [R, interleave] slabs: whole aligned vectors, one workgroup per row
+            CHECK(p.kind == ReduceKind::Row && p.lean && p.split == 1 && (size_t)p.vec * elem == 16 && p.vec % p.interleave == 0 &&
+                      p.interleave <= 8 && p.K % p.interleave == 0 && (p.R * p.interleave) % p.vec == 0 && !p.ragged && !p.unaligned &&
+                      p.sstride == 1 && !p.row_tile && p.kept.n == 2 && p.kept.size[1] == p.interleave && p.kept.stride[1] == 1 &&
+                      p.kept.stride[0] == p.R * p.interleave && v.base % 16 == 0,
+                  "%s plan=%s", show(v).c_str(), d.c_str());
         if (p.kind == ReduceKind::Row) {
             CHECK(pow2(p.tpr) && p.rpb >= 1 && (int64_t)p.tpr * p.rpb <= 1024, "%s plan=%s", show(v).c_str(),
                   d.c_str());

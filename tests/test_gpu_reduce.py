@@ -608,3 +608,50 @@ def test_few_outputs_of_few_partials_each(hpt, orc, dev, case):
     t.sum_(axes, False, False, out)
     assert_close(out.numpy(), orc.reduce(orc.SUM, a, axes, acc=orc.ACC_F64) + 1, F32_RTOL, F32_ATOL, f"sum into out {shape}")
     assert np.array_equal(t.sum(axes).numpy().view(np.uint32), t.sum(axes).numpy().view(np.uint32))
+
+
+INTERLEAVED_ROW_CASES = [  # (dtype, shape, axis): the middle axis of a contiguous [B, C, L], L a divisor of the 16-byte vector
+    (np.float32, (600, 2048, 2), 1), (np.float32, (700, 1000, 4), 1), (np.float32, (8000, 100, 2), 1), (np.float32, (3, 300, 1000, 2), 2),
+    (np.float32, (600, 8192, 2), 1), (np.float16, (900, 1000, 8), 1), (np.float16, (4000, 300, 4), 1), (np.float16, (800, 3000, 2), 1),
+    (np.float64, (600, 1000, 2), 1), (np.int32, (700, 1000, 4), 1), (np.int64, (600, 1000, 2), 1), (np.int16, (900, 1000, 8), 1),
+    (np.int8, (1200, 1000, 4), 1), (np.uint8, (300, 3000, 8), 1),
+]
+
+
+@pytest.mark.parametrize("npdt,shape,axis", INTERLEAVED_ROW_CASES, ids=lambda v: getattr(v, "__name__", str(v).replace(" ", "")))
+def test_reduction_over_the_middle_axis_with_an_inner_dim_that_divides_the_vector(hpt, orc, dev, npdt, shape, axis):
+    """The [C, L] slab runs as one row of C * L elements, a thread keeping L accumulators (one per place in the vector).
+    Inner positions get offsets far apart so that an accumulator fed from the wrong place shows; ties for the
+    arg-reductions sit at both ends of the axis (the lowest index wins)."""
+    rng = np.random.default_rng(733)
+    L, C = shape[-1], shape[axis]
+    if np.issubdtype(npdt, np.floating):
+        base = (rng.standard_normal(shape) + (np.arange(L) * 3.0 - 2.0)).astype(npdt)
+    else:
+        info = np.iinfo(npdt)
+        lo, hi = max(info.min, -100), min(info.max, 100)
+        base = (rng.integers(lo, hi + 1, shape) // 2 + (np.arange(L) % 3)).astype(npdt)
+    first = tuple(0 if i == axis else slice(None) for i in range(len(shape)))
+    last = tuple(C - 1 if i == axis else slice(None) for i in range(len(shape)))
+    top = np.asarray(base.max() + 1, dtype=np.float64).astype(npdt)
+    base[first] = top
+    base[last] = top
+    t, a = upload(hpt, base, dev=dev)
+    assert hpt.reduce_plan(t, hpt.SUM, [axis]).startswith("row-interleaved"), hpt.reduce_plan(t, hpt.SUM, [axis])
+    assert np.array_equal(t.max([axis]).numpy(), a.max(axis))
+    assert np.array_equal(t.min([axis]).numpy(), a.min(axis))
+    assert np.array_equal(t.argmax(axis).numpy(), orc.argreduce(True, a, axis))
+    assert np.array_equal(t.argmin(axis).numpy(), orc.argreduce(False, a, axis))
+    if npdt == np.float16:
+        want = orc.reduce(orc.SUM, a, [axis], acc=orc.ACC_F32).astype(np.float32)
+        assert_close(t.sum([axis]).numpy().astype(np.float32), want, HALF_RTOL, half_atol(want, 11), f"f16 sum {shape}")
+    elif np.issubdtype(npdt, np.floating):
+        rtol, atol = (F32_RTOL, F32_ATOL) if npdt == np.float32 else (1e-12, 1e-12)
+        assert_close(t.sum([axis]).numpy(), orc.reduce(orc.SUM, a, [axis], acc=orc.ACC_F64), rtol, atol, f"sum {shape}")
+        assert_close(t.mean([axis]).numpy(), orc.reduce(orc.MEAN, a, [axis], acc=orc.ACC_F64), rtol, atol, f"mean {shape}")
+        out = hpt.Tensor.from_numpy(np.ones(t.sum([axis]).shape, npdt)).to_hip(dev)
+        t.sum_([axis], False, False, out)
+        assert_close(out.numpy(), orc.reduce(orc.SUM, a, [axis], acc=orc.ACC_F64) + 1, rtol, atol, f"sum into out {shape}")
+    else:
+        assert np.array_equal(t.sum([axis]).numpy(), orc.reduce(orc.SUM, a, [axis]))
+        assert np.array_equal(t.prod([axis]).numpy(), orc.reduce(orc.PROD, a, [axis]))
