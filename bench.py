@@ -496,6 +496,7 @@ def cases_c8(P):
     nrm(ts, nb, "f32 [8192,2048,2] (slabs with an inner dim that divides the vector)", "softmax", 1, "softmax(axis=1)", 8192 * 2)
     del ts
     ts, nb = up([5592, 2000, 3])
+    red(ts, nb, "f32 [5592,2000,3] (slabs with a narrow inner dim)", "max", [1], "max(axis=1)", 5592 * 3)
     nrm(ts, nb, "f32 [5592,2000,3] (slabs with a narrow inner dim)", "softmax", 1, "softmax(axis=1)", 5592 * 3)
     del ts
     ts1, nb1 = up([33554403])

@@ -100,6 +100,7 @@ struct ReducePlan {
     bool ragged = false;        // Row (lean): rows of any length and alignment; aligned 128-bit loads over the body, the two ends element-wise
     bool unaligned = false;     // Col (lean): rows are not whole / aligned vectors; lanes still take VEC neighbours with unaligned 128-bit loads. Row: runs off the 16-byte grid read with unaligned 128-bit loads
     bool kept_swapped = false;  // Col (lean): the two kept dims are listed inner-most-in-memory last, not in output order
+    int mod_rows = 0;   // Row, > 0: a row is a contiguous [R, mod_rows] slab with mod_rows = 3, 5, 6 or 7 (no divisor of the vector) reduced over its first dim: threads in multiples of mod_rows keep an accumulator per vector place, rotated into outputs at the end
     int interleave = 1; // Row (lean), > 1: a row is a contiguous [R, interleave] slab reduced over its first dim (K counts the outputs, rows x interleave)
     int group_tile = 0; // Col, > 0: small contiguous [R, kin] groups staged through LDS, this many groups per workgroup
     int row_tile = 0;   // Row, > 0: short contiguous rows staged through LDS, this many rows per workgroup

@@ -267,6 +267,24 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
             std::swap(p.kept.stride[0], p.kept.stride[1]);
             p.kept_swapped = true;
         }
+        // The same slabs with an inner dim of 3, 5, 6 or 7 elements (points, colours): a row of the kernel whose
+        // lanes, in multiples of L, keep an accumulator per vector place. Mid-sized slabs, many of them: small
+        // groups go through LDS tiles, few long ones through the flat walk.
+        {
+            const int64_t full = elem_size <= 8 ? (int64_t)(16 / elem_size) : 1;
+            const int64_t L = nk == 2 ? p.kept.size[1] : 0;
+            if (nk == 2 && !p.kept_swapped && p.red.n == 1 && full > 1 && p.kept.stride[1] == 1 && L >= 3 && L <= 7 && full % L != 0 &&
+                p.red.stride[0] == L && p.kept.stride[0] == p.R * L && p.R * L * (int64_t)elem_size >= 4096 &&
+                p.R * L * (int64_t)elem_size <= (256 << 10) && p.kept.size[0] >= 512 &&
+                p.K * p.R * (int64_t)elem_size >= (4ll << 20) && ((uintptr_t)data % elem_size) == 0) {
+                p.kind = ReduceKind::Row;
+                p.mod_rows = (int)L;
+                p.vec = (int)full;
+                p.tpr = p.R * L / full >= 1024 ? 256 : 64;
+                p.rpb = 256 / p.tpr;
+                return p;
+            }
+        }
         int64_t kin = nk ? p.kept.size[nk - 1] : 1;
         p.vec = 1;
         if (nk && p.kept.stride[nk - 1] == 1)
@@ -485,7 +503,7 @@ std::string describe(const ReducePlan& p) {
         case ReduceKind::Identity: return "identity";
         case ReduceKind::Row:
             snprintf(buf, sizeof buf, "row%s%s vec=%d tpr=%d rpb=%d rows=%lld cols=%lld split=%d(%dx%d) ",
-                     p.row_tile ? "-tile" : p.ragged ? "-ragged" : p.lean ? "" : "-general", p.sstride == 2 ? "-step2" : p.unaligned ? "-unaligned" : p.interleave > 1 ? "-interleaved" : "", p.vec, p.tpr, p.rpb,
+                     p.row_tile ? "-tile" : p.ragged ? "-ragged" : (p.lean || p.mod_rows) ? "" : "-general", p.sstride == 2 ? "-step2" : p.unaligned ? "-unaligned" : p.interleave > 1 ? "-interleaved" : p.mod_rows ? "-modular" : "", p.vec, p.tpr, p.rpb,
                      (long long)p.K, (long long)p.R, p.split, p.split_q, p.split_i);
             break;
         case ReduceKind::Col:

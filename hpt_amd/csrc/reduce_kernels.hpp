@@ -176,6 +176,95 @@ __global__ void __launch_bounds__(1024) row_lean_kernel(const RowLeanArgs a) {
     }
 }
 
+// ---- rows that are [R, L] slabs, L no divisor of the vector -----------------------------------
+// out[row * L + k] = reduce over c of in[row * rin + c * L + k], rin = R * L elements per row, rows back to back
+// (a reduction over the middle axis of a contiguous [B, R, 3]: lanes along L idle, and the flat walk takes two
+// launches and a workgroup per period). A row's lanes walk it with 128-bit loads; only the first `act` = the largest
+// multiple of L lanes take part, so that a lane's vectors all start at the same place modulo L, (tx * VEC) % L: the
+// lane keeps one accumulator per vector place and rotates them into the L outputs once, at the end. Rows start
+// anywhere (unaligned loads); the elements after a row's last whole vector are folded one by one.
+struct RowModArgs {
+    const void* in;
+    void* out;
+    double count;
+    int K;    // rows
+    int rin;  // row length in elements, R * L
+    int tpr, tpr_log2, rpb, init_out;
+};
+
+template <class Op, int VEC, int L>
+__global__ void __launch_bounds__(256) row_mod_kernel(const RowModArgs a) {
+    static_assert(VEC > 1 && VEC % L != 0 && L >= 3 && L <= 7, "inner dims that divide the vector run as interleaved rows");
+    using T = typename Op::In;
+    using Acc = typename Op::Acc;
+    __shared__ Acc smem[4 * L];
+    const int tpr = a.tpr;
+    const int tx = threadIdx.x & (tpr - 1);
+    const int ty = threadIdx.x >> a.tpr_log2;
+    const int row = blockIdx.x * a.rpb + ty;
+    const bool valid = row < a.K;
+    const int act = tpr / L * L;
+    Acc acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = Op::identity();
+    Acc cls[L];
+#pragma unroll
+    for (int k = 0; k < L; ++k) cls[k] = Op::identity();
+    if (valid && tx < act) {
+        const T* p = (const T*)a.in + (int64_t)row * a.rin;
+        const int nvec = a.rin / VEC;
+        auto fold = [&](const Pack<T, VEC>& v, int i) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) fold_in<Op>(acc[j], v.v[j], (i * VEC + j) / L);
+        };
+        int iv = tx;
+        for (; iv + 3 * act < nvec; iv += 4 * act) {
+            Pack<T, VEC> v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = load_pack_unaligned<T, VEC>(p + (int64_t)(iv + u * act) * VEC);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) fold(v[u], iv + u * act);
+        }
+        for (; iv < nvec; iv += act) fold(load_pack_unaligned<T, VEC>(p + (int64_t)iv * VEC), iv);
+        // the lane's vector places as outputs: place j is output (tx * VEC + j) % L
+        const int r = tx * VEC % L;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            const int k = (r + j) % L;
+#pragma unroll
+            for (int kk = 0; kk < L; ++kk)
+                if (kk == k) cls[kk] = Op::comb(cls[kk], acc[j]);
+        }
+        // fewer than VEC elements after the last whole vector
+        const int e = nvec * VEC + tx;
+        if (e < a.rin) {
+            const T x = p[e];
+#pragma unroll
+            for (int kk = 0; kk < L; ++kk)
+                if (kk == e % L) fold_in<Op>(cls[kk], x, e / L);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < L; ++k) cls[k] = group_reduce<Op>(cls[k], tpr < 64 ? tpr : 64);
+    if (tpr > 64) {
+        const int wpr = tpr >> 6;  // wavefronts per row (<= 4)
+        if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+            for (int k = 0; k < L; ++k) smem[(threadIdx.x >> 6) * L + k] = cls[k];
+        }
+        __syncthreads();
+        if (tx == 0)
+            for (int w = 1; w < wpr; ++w) {
+#pragma unroll
+                for (int k = 0; k < L; ++k) cls[k] = Op::comb(cls[k], smem[(ty * wpr + w) * L + k]);
+            }
+    }
+    if (tx == 0 && valid) {
+#pragma unroll
+        for (int k = 0; k < L; ++k) write_out<Op>(a.out, (int64_t)row * L + k, cls[k], a.init_out, a.count);
+    }
+}
+
 // ---- general row kernel ---------------------------------------------------------
 struct RowArgs {
     const void* in;
@@ -1019,6 +1108,33 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             row_tile_kernel<Op, FULL><<<dim3((unsigned)((p.K + p.row_tile - 1) / p.row_tile)), dim3(256), 0, st>>>(a);
         }
         return;
+    }
+    if (p.kind == ReduceKind::Row && p.mod_rows > 0) {
+        if constexpr (FULL > 1) {
+            if (p.vec != FULL || p.split != 1 || p.K % p.mod_rows != 0 || p.tpr * p.rpb != 256 || p.tpr < 64 ||
+                p.R * p.mod_rows >= (1ll << 30))
+                fail(HPT_ERR_KERNEL, "rows of [R, L] slabs: 256-thread workgroups of whole rows");
+            const int64_t rows = p.K / p.mod_rows;
+            const dim3 grid((unsigned)((rows + p.rpb - 1) / p.rpb));
+            RowModArgs a{};
+            a.in = in;
+            a.out = out;
+            a.count = count;
+            a.K = (int)rows;
+            a.rin = (int)(p.R * p.mod_rows);
+            a.tpr = p.tpr;
+            a.tpr_log2 = ilog2(p.tpr);
+            a.rpb = p.rpb;
+            a.init_out = init_out;
+            switch (p.mod_rows) {
+                case 3: row_mod_kernel<Op, FULL, 3><<<grid, dim3(256), 0, st>>>(a); return;
+                case 5: row_mod_kernel<Op, FULL, 5><<<grid, dim3(256), 0, st>>>(a); return;
+                case 6: if constexpr (FULL != 2) { row_mod_kernel<Op, FULL, 6><<<grid, dim3(256), 0, st>>>(a); return; } break;
+                case 7: row_mod_kernel<Op, FULL, 7><<<grid, dim3(256), 0, st>>>(a); return;
+                default: break;
+            }
+        }
+        fail(HPT_ERR_KERNEL, "rows of [R, L] slabs: L = %d", p.mod_rows);
     }
     if (p.kind == ReduceKind::Row && p.interleave > 1) {
         // rows that are [R, interleave] slabs: the lean kernel over rows of R * interleave elements

@@ -141,6 +141,12 @@ static void fuzz_reduce() {
                       p.sstride == 1 && !p.row_tile && p.kept.n == 2 && p.kept.size[1] == p.interleave && p.kept.stride[1] == 1 &&
                       p.kept.stride[0] == p.R * p.interleave && v.base % 16 == 0,
                   "%s plan=%s", show(v).c_str(), d.c_str());
+        if (p.mod_rows > 0)  // rows that are [R, L] slabs, L = 3, 5, 6, 7: 256-thread workgroups of whole rows
+            CHECK(p.kind == ReduceKind::Row && p.split == 1 && (size_t)p.vec * elem == 16 && p.vec % p.mod_rows != 0 && p.mod_rows >= 3 &&
+                      p.mod_rows <= 7 && p.K % p.mod_rows == 0 && p.tpr * p.rpb == 256 && p.tpr >= 64 && p.kept.n == 2 &&
+                      p.kept.size[1] == p.mod_rows && p.kept.stride[1] == 1 && p.kept.stride[0] == p.R * p.mod_rows &&
+                      p.red.n == 1 && p.red.stride[0] == p.mod_rows && p.R * p.mod_rows < (1ll << 30) && p.interleave == 1,
+                  "%s plan=%s", show(v).c_str(), d.c_str());
         if (p.kind == ReduceKind::Row) {
             CHECK(pow2(p.tpr) && p.rpb >= 1 && (int64_t)p.tpr * p.rpb <= 1024, "%s plan=%s", show(v).c_str(),
                   d.c_str());

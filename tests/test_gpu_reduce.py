@@ -655,3 +655,50 @@ def test_reduction_over_the_middle_axis_with_an_inner_dim_that_divides_the_vecto
     else:
         assert np.array_equal(t.sum([axis]).numpy(), orc.reduce(orc.SUM, a, [axis]))
         assert np.array_equal(t.prod([axis]).numpy(), orc.reduce(orc.PROD, a, [axis]))
+
+
+MODULAR_ROW_CASES = [  # (dtype, shape, axis): the middle axis of a contiguous [B, C, L], L = 3, 5, 6, 7
+    (np.float32, (600, 2000, 3), 1), (np.float32, (2000, 1001, 3), 1), (np.float32, (1500, 401, 5), 1), (np.float32, (800, 3000, 7), 1),
+    (np.float32, (3, 400, 1000, 6), 2), (np.float32, (512, 20001, 3), 1), (np.float16, (900, 1000, 3), 1), (np.float16, (2000, 999, 5), 1),
+    (np.float16, (600, 2047, 7), 1), (np.float64, (600, 1001, 3), 1), (np.float64, (700, 333, 5), 1), (np.int32, (700, 1001, 3), 1),
+    (np.int64, (600, 1000, 7), 1), (np.int16, (900, 1001, 6), 1), (np.int8, (1200, 1501, 3), 1), (np.uint8, (600, 3001, 5), 1),
+]
+
+
+@pytest.mark.parametrize("npdt,shape,axis", MODULAR_ROW_CASES, ids=lambda v: getattr(v, "__name__", str(v).replace(" ", "")))
+def test_reduction_over_the_middle_axis_with_an_inner_dim_of_3_5_6_7(hpt, orc, dev, npdt, shape, axis):
+    """The [C, L] slab runs as one row; lanes in multiples of L keep an accumulator per vector place and rotate them into
+    the L outputs at the end; rows start off the 16-byte grid and end with a few single elements. Inner positions get
+    offsets far apart; ties for the arg-reductions sit at both ends of the axis (the lowest index wins)."""
+    rng = np.random.default_rng(734)
+    L, C = shape[-1], shape[axis]
+    if np.issubdtype(npdt, np.floating):
+        base = (rng.standard_normal(shape) + (np.arange(L) * 3.0 - 2.0)).astype(npdt)
+    else:
+        info = np.iinfo(npdt)
+        lo, hi = max(info.min, -100), min(info.max, 100)
+        base = (rng.integers(lo, hi + 1, shape) // 2 + (np.arange(L) % 3)).astype(npdt)
+    first = tuple(0 if i == axis else slice(None) for i in range(len(shape)))
+    last = tuple(C - 1 if i == axis else slice(None) for i in range(len(shape)))
+    top = np.asarray(base.max() + 1, dtype=np.float64).astype(npdt)
+    base[first] = top
+    base[last] = top
+    t, a = upload(hpt, base, dev=dev)
+    assert hpt.reduce_plan(t, hpt.SUM, [axis]).startswith("row-modular"), hpt.reduce_plan(t, hpt.SUM, [axis])
+    assert np.array_equal(t.max([axis]).numpy(), a.max(axis))
+    assert np.array_equal(t.min([axis]).numpy(), a.min(axis))
+    assert np.array_equal(t.argmax(axis).numpy(), orc.argreduce(True, a, axis))
+    assert np.array_equal(t.argmin(axis).numpy(), orc.argreduce(False, a, axis))
+    if npdt == np.float16:
+        want = orc.reduce(orc.SUM, a, [axis], acc=orc.ACC_F32).astype(np.float32)
+        assert_close(t.sum([axis]).numpy().astype(np.float32), want, HALF_RTOL, half_atol(want, 11), f"f16 sum {shape}")
+    elif np.issubdtype(npdt, np.floating):
+        rtol, atol = (F32_RTOL, F32_ATOL) if npdt == np.float32 else (1e-12, 1e-12)
+        assert_close(t.sum([axis]).numpy(), orc.reduce(orc.SUM, a, [axis], acc=orc.ACC_F64), rtol, atol, f"sum {shape}")
+        assert_close(t.mean([axis]).numpy(), orc.reduce(orc.MEAN, a, [axis], acc=orc.ACC_F64), rtol, atol, f"mean {shape}")
+        out = hpt.Tensor.from_numpy(np.ones(t.sum([axis]).shape, npdt)).to_hip(dev)
+        t.sum_([axis], False, False, out)
+        assert_close(out.numpy(), orc.reduce(orc.SUM, a, [axis], acc=orc.ACC_F64) + 1, rtol, atol, f"sum into out {shape}")
+    else:
+        assert np.array_equal(t.sum([axis]).numpy(), orc.reduce(orc.SUM, a, [axis]))
+        assert np.array_equal(t.prod([axis]).numpy(), orc.reduce(orc.PROD, a, [axis]))

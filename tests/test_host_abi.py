@@ -96,7 +96,9 @@ def test_plans_for_shapes_off_the_benchmark_list(hpt):
         ([65536, 512], [1], "row vec=4"), ([131584, 257], [1], "row-tile"),
         # the middle axis of [B, C, L] with L a divisor of the vector: the slab is a row, L accumulators per thread
         ([8192, 2048, 2], [1], "row-interleaved vec=4 tpr=256 rpb=1 rows=16384 cols=2048 split=1"), ([4000, 1000, 4], [1], "row-interleaved vec=4"),
-        ([5592, 2000, 3], [1], "col-flat "), ([300, 1000, 2], [1], "col vec=1"), ([2000, 1280, 8], [1], "col vec=4"),
+        ([300, 1000, 2], [1], "col vec=1"),
+        # ... with an inner dim of 3, 5, 6, 7: lanes in multiples of it, an accumulator per vector place
+        ([5592, 2000, 3], [1], "row-modular vec=4 tpr=256 rpb=1"), ([2000, 1001, 5], [1], "row-modular vec=4 tpr=256"), ([300, 2000, 3], [1], "col vec=1"), ([2000, 1280, 8], [1], "col vec=4"),
     ]
     for shape, axes, want in red:
         got = hpt.reduce_plan(view(shape), hpt.SUM, axes)
