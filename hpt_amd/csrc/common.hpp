@@ -148,7 +148,7 @@ struct NormPlan {
     int64_t inner = 1;  // Col: size of the contiguous inner dim the lanes walk
     int sstride = 1;    // RowReg: 2 = the row's elements sit at every second position of full vectors
     int flat_t = 0;     // ColSplit, > 0: a narrow inner dim; the slab is walked as a flat array by this many threads
-    int interleave = 1;  // RowReg softmax whose rows are contiguous [cols / interleave, interleave] slabs normalised over their first dim (2, 4 or 8: a divisor of the vector)
+    int interleave = 1;  // RowReg softmax whose rows are contiguous [cols / |interleave|, |interleave|] slabs normalised over their first dim: > 1, a divisor of the vector or two vectors; < 0, minus an inner dim of 3, 5, 6 or 7 (the largest multiple of it of a row's lanes take part)
     int slab_tile = 0;  // Col softmax over the middle axis of mid-sized contiguous [cols, L] slabs with a narrow L: one workgroup per slab through LDS (the value: lanes per column)
     int group_tile = 0; // Col softmax over a short middle axis of small contiguous [cols, L] groups: this many groups per workgroup through LDS
     int lds_rows = 0;   // RowReg softmax of 2- and 4-byte types: long rows held in the registers and the LDS of tpr = 256 or 512 threads (nchunk: vectors per thread in both together)

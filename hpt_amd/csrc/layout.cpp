@@ -983,7 +983,7 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
         // slab and the flat walk, f32 [1000, 2048, 8] 60.0 -> 31.1): a thread's vectors all hold the same places, and
         // only threads two apart are folded together.
         if (nk == 2 && max_vec > 1 && p.cols > 64 && sa > 1 && sa == p.kept_in.size[1] &&
-            (max_vec % sa == 0 || (sa == 2 * max_vec && p.cols > 1024)) &&
+            (max_vec % sa == 0 || (sa == 2 * max_vec && p.cols > 1024) || ((sa == 3 || sa == 5 || sa == 6 || sa == 7) && max_vec % sa != 0)) &&
             p.kept_in.stride[1] == 1 && p.kept_out.stride[1] == 1 && p.kept_in.size[1] == p.out_axis_stride &&
             p.kept_in.stride[0] == p.cols * sa && p.kept_out.stride[0] == p.cols * sa && (p.cols * sa) % max_vec == 0 &&
             p.cols * sa * (int64_t)elem_size <= (128 << 10) && p.kept_in.size[0] >= 256 &&
@@ -992,8 +992,20 @@ NormPlan plan_normalize(const void* in_data, const void* out_data, const int64_t
             NormPlan q = plan_normalize(in_data, out_data, shp, str, 2, 1, 0, elem_size, fused);
             if (q.kind == NormKind::RowReg && q.vec == max_vec && q.sstride == 1 && !q.shift && !q.tile_rows && !q.gb_lds &&
                 !q.lds_rows && !q.raw_rows && q.tpr * max_vec >= sa) {
-                q.interleave = (int)sa;
-                return q;
+                if (max_vec % sa == 0 || sa == 2 * max_vec) {
+                    q.interleave = (int)sa;
+                    return q;
+                }
+                // An inner dim of 3, 5, 6 or 7: the largest multiple of it of a row's lanes take part, so that all of a
+                // lane's vectors start at the same place modulo the inner dim; the lane keeps a (max, sum) per vector
+                // place and the places are rotated into softmaxes, folded, and rotated back.
+                const int64_t act = q.tpr / sa * sa, nvr = p.cols * sa / max_vec;
+                const int64_t nc = (nvr + act - 1) / act;
+                if (nc <= 8) {
+                    q.interleave = -(int)sa;
+                    q.nchunk = (int)nc;
+                    return q;
+                }
             }
         }
         // Mid-sized slabs with a very narrow inner dim ([B, 1000, 3], [B, 2048, 5]): one workgroup per slab through LDS.
@@ -1179,7 +1191,7 @@ std::string describe(const NormPlan& p) {
     static const char* names[] = {"empty", "rowreg", "rowstream", "rowsplit", "col", "col-split", "transposed", "transposed-tile", "col-reg", "generic"};
     char buf[256];
     snprintf(buf, sizeof buf, "%s%s%s rows=%lld cols=%lld vec=%d tpr=%d rpb=%d nchunk=%d ostride=%lld ",
-             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg || p.kind == NormKind::ColSplit) ? "-unaligned" : (p.lds_rows ? "-lds-shift" : "-shift")) : (p.gb_lds == 2 ? "-l2gb" : p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.interleave > 1 ? "-interleaved" : p.group_tile ? "-group-tile" : (p.slab_tile ? "-slab" : "")), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
+             names[(int)p.kind], p.sstride == 2 ? "-step2" : (p.flat_t ? (p.shift ? "-flat-unaligned" : "-flat") : (p.shift ? ((p.kind == NormKind::RowSplit || p.kind == NormKind::ColReg || p.kind == NormKind::ColSplit) ? "-unaligned" : (p.lds_rows ? "-lds-shift" : "-shift")) : (p.gb_lds == 2 ? "-l2gb" : p.gb_lds ? "-ldsgb" : (p.raw_rows ? "-raw" : (p.lds_rows ? "-lds" : ""))))), p.tile_rows ? "+tile" : (p.interleave > 1 ? "-interleaved" : p.interleave < 0 ? "-modular" : p.group_tile ? "-group-tile" : (p.slab_tile ? "-slab" : "")), (long long)p.rows, (long long)p.cols, p.vec, p.tpr, p.rpb,
              p.nchunk, (long long)p.out_axis_stride);
     std::string s = buf;
     if (p.kind == NormKind::RowReg) s += "max_blocks=" + std::to_string(p.max_blocks) + " ";  // (layernorm walks its rows)

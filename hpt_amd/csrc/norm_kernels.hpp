@@ -166,9 +166,12 @@ __device__ __forceinline__ void row_all_reduce_n(A (&v)[N], int tpr, int ty, A* 
 // [B, C, 2], [B, C, 4], [B, C, 8 heads]).
 template <int KIND, class T, int VEC, int NCHUNK, int SS = 1, bool SHIFT = false, bool PF = false, int GB = 0, int IL = 1>
 __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
-    static_assert(IL == 1 || (!norm_is_layer(KIND) && !norm_is_causal(KIND) && SS == 1 && !SHIFT && (VEC % IL == 0 || IL % VEC == 0)), "interleaved rows: a plain softmax of whole vectors");
-    constexpr int NS = IL < VEC ? IL : VEC;      // statistics a thread keeps
-    constexpr int IG = IL > VEC ? IL / VEC : 1;  // neighbouring threads that hold different ones
+    constexpr int ML = IL < 0 ? -IL : 0;  // interleaved softmaxes whose number is no divisor of the vector (3, 5, 6, 7)
+    static_assert(IL == 1 || (!norm_is_layer(KIND) && !norm_is_causal(KIND) && SS == 1 && !SHIFT && VEC > 1 &&
+                              (ML ? (ML >= 3 && ML <= 7 && VEC % ML != 0) : (VEC % IL == 0 || IL % VEC == 0))),
+                  "interleaved rows: a plain softmax of whole vectors");
+    constexpr int NS = ML ? VEC : (IL < VEC ? IL : VEC);  // statistics a thread keeps
+    constexpr int IG = IL > VEC ? IL / VEC : 1;            // neighbouring threads that hold different ones
     constexpr bool GBL = GB == 1;  // gamma / beta in LDS
     constexpr bool GBG = GB == 2;  // gamma / beta from global memory, every row
     static_assert(GB == 0 || (norm_is_layer(KIND) && VEC > 1 && SS == 1 && !SHIFT), "gamma / beta outside registers: an aligned layernorm form");
@@ -176,13 +179,20 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     constexpr int UV = VEC / SS;  // useful elements per vector
     using CT = typename Elem<T>::Wide;
     using ST = typename StatType<T>::type;
-    __shared__ __align__(8) unsigned char smem_stat[16 * IL * sizeof(double)];
+    __shared__ __align__(8) unsigned char smem_stat[16 * (ML ? ML : IL) * sizeof(double)];
     CT* smem = reinterpret_cast<CT*>(smem_stat);
     ST* ssmem = reinterpret_cast<ST*>(smem_stat);
     const int tpr = a.tpr;
     const int tx = threadIdx.x & (tpr - 1);
     const int ty = threadIdx.x >> a.tpr_log2;
     const int nv = SHIFT ? (int)((a.cols + 2 * (VEC - 1)) / VEC) : (int)(a.cols / UV);  // SHIFT: upper bound
+    // Vector c of this thread. ML: only the largest multiple of ML lanes of a row take part, so that all of a lane's
+    // vectors start at the same place modulo ML, (tx * VEC) % ML; the other lanes hold nothing.
+    const int tstep = ML ? tpr / (ML ? ML : 1) * ML : tpr;
+    auto vec_of = [&](int c) -> int {
+        if constexpr (ML > 0) return tx < tstep ? c * tstep + tx : nv;
+        else return c * tpr + tx;
+    };
     const int cols = (int)a.cols;
     // misalignment, in elements, of a row that starts at p
     auto shift_of = [](const T* p) -> int { return SHIFT ? (int)(((uintptr_t)p / sizeof(T)) % VEC) : 0; };
@@ -200,7 +210,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
     if constexpr (!kSoft && !GB) {
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
-            const int iv = c * tpr + tx;
+            const int iv = vec_of(c);
 #pragma unroll
             for (int j = 0; j < UV; ++j) {
                 gam[c].v[j] = Elem<T>::narrow((CT)1);
@@ -269,7 +279,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
         const int nv_row = (kCausal || SHIFT) ? (int)((row_limit(row) + m + UV - 1) / UV) : nv;
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
-            const int iv = c * tpr + tx;
+            const int iv = vec_of(c);
             if (iv < nv_row) {
                 if constexpr (VEC > 1) raw[c] = load_pack_stream<T, VEC>(in_row + (int64_t)iv * VEC);
                 else raw[c].v[0] = in_row[(int64_t)iv * a.sa];
@@ -314,7 +324,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
         CT x[NCHUNK][UV];
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
-            const int iv = c * tpr + tx;
+            const int iv = vec_of(c);
             if constexpr (kCausal && !SHIFT) {
                 // A chunk (the tpr vectors the row's lanes hold side by side) lies wholly below the diagonal, wholly
                 // above it, or across it. Only the one across it needs a test per element; the masked half of the
@@ -355,8 +365,28 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
             for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
                 for (int j = 0; j < UV; ++j) mv[j % NS] = MaxC<CT>::comb(mv[j % NS], x[c][j]);
-            if constexpr (IL == 1) mv[0] = row_all_reduce<MaxC<CT>>(mv[0], tpr, ty, smem);
-            else row_all_reduce_n<MaxC<CT>, CT, NS, IG>(mv, tpr, ty, smem);
+            // ML: place j of this lane's vectors belongs to softmax (tx * VEC + j) % ML
+            const int rot = ML ? tx * VEC % (ML ? ML : 1) : 0;
+            if constexpr (IL == 1) {
+                mv[0] = row_all_reduce<MaxC<CT>>(mv[0], tpr, ty, smem);
+            } else if constexpr (ML > 0) {
+                CT cm[ML];
+#pragma unroll
+                for (int k = 0; k < ML; ++k) cm[k] = neg_inf<CT>();
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+#pragma unroll
+                    for (int k = 0; k < ML; ++k)
+                        if (k == (rot + j) % ML) cm[k] = MaxC<CT>::comb(cm[k], mv[j]);
+                row_all_reduce_n<MaxC<CT>, CT, ML, 1>(cm, tpr, ty, smem);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+#pragma unroll
+                    for (int k = 0; k < ML; ++k)
+                        if (k == (rot + j) % ML) mv[j] = cm[k];
+            } else {
+                row_all_reduce_n<MaxC<CT>, CT, NS, IG>(mv, tpr, ty, smem);
+            }
             CT sv[NS];
 #pragma unroll
             for (int k = 0; k < NS; ++k) sv[k] = 0;
@@ -378,8 +408,26 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                     x[c][j] = kLog ? d : e;
                 }
             }
-            if constexpr (IL == 1) sv[0] = row_all_reduce<SumC<CT>>(sv[0], tpr, ty, smem);
-            else row_all_reduce_n<SumC<CT>, CT, NS, IG>(sv, tpr, ty, smem);
+            if constexpr (IL == 1) {
+                sv[0] = row_all_reduce<SumC<CT>>(sv[0], tpr, ty, smem);
+            } else if constexpr (ML > 0) {
+                CT cs[ML];
+#pragma unroll
+                for (int k = 0; k < ML; ++k) cs[k] = 0;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+#pragma unroll
+                    for (int k = 0; k < ML; ++k)
+                        if (k == (rot + j) % ML) cs[k] += sv[j];
+                row_all_reduce_n<SumC<CT>, CT, ML, 1>(cs, tpr, ty, smem);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+#pragma unroll
+                    for (int k = 0; k < ML; ++k)
+                        if (k == (rot + j) % ML) sv[j] = cs[k];
+            } else {
+                row_all_reduce_n<SumC<CT>, CT, NS, IG>(sv, tpr, ty, smem);
+            }
             CT kv[NS];
 #pragma unroll
             for (int k = 0; k < NS; ++k) kv[k] = kLog ? log_ct<T>(sv[k]) : (CT)1 / sv[k];
@@ -425,7 +473,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
                 asm volatile("" : "+s"(gp), "+s"(bp));
 #pragma unroll
                 for (int c = 0; c < NCHUNK; ++c) {
-                    const int iv = c * tpr + tx;
+                    const int iv = vec_of(c);
                     if (iv < nv) {
                         Pack<T, UV> g, b;
 #pragma unroll
@@ -443,7 +491,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
             } else if constexpr (GBL) {
 #pragma unroll
                 for (int c = 0; c < NCHUNK; ++c) {
-                    const int iv = c * tpr + tx;
+                    const int iv = vec_of(c);
                     if (iv < nv) {
                         const Pack<T, UV> g = load_pack<T, UV>(lds_gamma + (size_t)iv * UV);
                         const Pack<T, UV> b = load_pack<T, UV>(lds_beta + (size_t)iv * UV);
@@ -464,7 +512,7 @@ __global__ void __launch_bounds__(1024) row_reg_kernel(const NormArgs a) {
         if (valid) {
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c) {
-                const int iv = c * tpr + tx;
+                const int iv = vec_of(c);
                 if constexpr (SHIFT) {
                     const int e0 = iv * VEC - sh;
                     if (e0 + VEC > 0 && e0 < cols) {

@@ -187,7 +187,13 @@ static void fuzz_normalize() {
             return;
         }
         // (interleaved rows: a row is a whole [axis, inner] slab, the inner dim a divisor of the full vector)
-        CHECK(p.interleave >= 1 && p.cols == cols * p.interleave && p.rows * p.cols == total, "%s plan=%s", show(v).c_str(), d.c_str());
+        const int64_t il = p.interleave < 0 ? -p.interleave : p.interleave;
+        CHECK(il >= 1 && p.cols == cols * il && p.rows * p.cols == total, "%s plan=%s", show(v).c_str(), d.c_str());
+        if (p.interleave < 0)  // an inner dim of 3, 5, 6, 7: lanes in multiples of it hold the row
+            CHECK(p.kind == hpt::NormKind::RowReg && (size_t)p.vec * elem == 16 && il >= 3 && il <= 7 && p.vec % il != 0 && !p.shift &&
+                      p.sstride == 1 && !p.tile_rows && !p.gb_lds && !layernorm && p.cols % p.vec == 0 &&
+                      p.cols / p.vec <= (int64_t)(p.tpr / il * il) * p.nchunk && p.nchunk <= 8,
+                  "%s plan=%s", show(v).c_str(), d.c_str());
         if (p.interleave > 1)
             CHECK(p.kind == hpt::NormKind::RowReg && (size_t)p.vec * elem == 16 && (p.vec % p.interleave == 0 || (p.interleave == 2 * p.vec && p.tpr >= 2)) && !p.shift && p.sstride == 1 &&
                       !p.tile_rows && !p.gb_lds && !layernorm && p.cols % p.vec == 0 && p.cols / p.vec <= (int64_t)p.tpr * p.nchunk && p.nchunk <= 8,

@@ -675,16 +675,16 @@ GROUP_CASES = [
 
 
 SLAB_CASES = [
-    ("f16 [900, 1000, 3] axis 1", np.float16, [900, 1000, 3], 1),
-    ("f32 [300, 1092, 5] axis 1 (slabs off 16-byte boundaries)", np.float32, [300, 1092, 5], 1),
+    ("f16 [900, 1001, 3] axis 1", np.float16, [900, 1001, 3], 1),
+    ("f32 [300, 1093, 5] axis 1 (slabs off 16-byte boundaries)", np.float32, [300, 1093, 5], 1),
     ("bf16 [260, 2730, 12] axis 1 (64 KiB slabs)", "bf16", [260, 2730, 12], 1),
     ("f32 [1200, 501, 2] axis 1 (slabs of half vectors)", np.float32, [1200, 501, 2], 1),
-    ("f64 [300, 1100, 3] axis 1", np.float64, [300, 1100, 3], 1),
+    ("f64 [300, 1101, 3] axis 1", np.float64, [300, 1101, 3], 1),
     ("f16 [2, 300, 2049, 7] axis 2 (odd slab size)", np.float16, [2, 300, 2049, 7], 2),
     # four-byte inner dims up to 11 elements that are not whole vectors
-    ("f32 [600, 512, 7] axis 1", np.float32, [600, 512, 7], 1),
+    ("f32 [600, 513, 7] axis 1", np.float32, [600, 513, 7], 1),
     ("f32 [500, 300, 11] axis 1", np.float32, [500, 300, 11], 1),
-    ("f32 [8000, 100, 6] axis 1 (short axis)", np.float32, [8000, 100, 6], 1),
+    ("f32 [8000, 101, 6] axis 1 (short axis)", np.float32, [8000, 101, 6], 1),
 ]
 
 
@@ -697,8 +697,24 @@ INTERLEAVED_SLAB_CASES = [  # an inner dim that divides the vector: the slab is 
 ]
 
 
-@pytest.mark.parametrize("case", CHANNEL_CASES + GROUP_CASES + SLAB_CASES + INTERLEAVED_SLAB_CASES,
-                         ids=[c[0] for c in CHANNEL_CASES + GROUP_CASES + SLAB_CASES + INTERLEAVED_SLAB_CASES])
+MODULAR_SLAB_CASES = [  # an inner dim of 3, 5, 6, 7 and slabs of whole vectors: the slab is a row held by lanes in multiples of the inner dim
+    ("f16 [900, 1000, 3] axis 1", np.float16, [900, 1000, 3], 1),
+    ("f32 [300, 1092, 5] axis 1", np.float32, [300, 1092, 5], 1),
+    ("f64 [300, 1100, 3] axis 1", np.float64, [300, 1100, 3], 1),
+    ("f32 [600, 512, 7] axis 1", np.float32, [600, 512, 7], 1),
+    ("f32 [8000, 100, 6] axis 1 (short axis, 32 lanes per row)", np.float32, [8000, 100, 6], 1),
+    ("bf16 [2, 300, 1024, 7] axis 2", "bf16", [2, 300, 1024, 7], 2),
+    ("f32 [300, 8000, 3] axis 1 (rows of 1024 threads)", np.float32, [300, 8000, 3], 1),
+    ("f16 [700, 4000, 6] axis 1", np.float16, [700, 4000, 6], 1),
+    ("f32 [2000, 1000, 3] axis 1", np.float32, [2000, 1000, 3], 1),
+]
+
+
+ROW_SLAB_CASES = INTERLEAVED_SLAB_CASES + MODULAR_SLAB_CASES
+
+
+@pytest.mark.parametrize("case", CHANNEL_CASES + GROUP_CASES + SLAB_CASES + ROW_SLAB_CASES,
+                         ids=[c[0] for c in CHANNEL_CASES + GROUP_CASES + SLAB_CASES + ROW_SLAB_CASES])
 def test_softmax_over_a_short_strided_axis_in_registers(hpt, orc, dev, case):
     """softmax over the channels of [B, C, H, W], C <= 64: every thread keeps the whole axis of its
     inner positions in registers (one read, one write). Small [C, L] groups laid back to back go
@@ -719,7 +735,7 @@ def test_softmax_over_a_short_strided_axis_in_registers(hpt, orc, dev, case):
     a = cv(x)
     t = hpt.Tensor.from_numpy(a, dt).to_hip(dev)
     want_plan = ("col-group-tile" if case in GROUP_CASES else "col-slab" if case in SLAB_CASES else
-                 "rowreg-interleaved" if case in INTERLEAVED_SLAB_CASES else "col-reg")
+                 "rowreg-interleaved" if case in INTERLEAVED_SLAB_CASES else "rowreg-modular" if case in MODULAR_SLAB_CASES else "col-reg")
     assert hpt.normalize_plan(t, axis).startswith(want_plan), hpt.normalize_plan(t, axis)
     for log in (False, True):
         got = tof((t.log_softmax(axis) if log else t.softmax(axis)).numpy())
@@ -873,7 +889,7 @@ DOMINANT_CASES = [
     ([4096, 4096], 1, False, "rowreg"), ([8192, 1000], 1, False, "rowreg"), ([1000000, 8], 1, False, "rowreg+tile"),
     ([64, 65536], 1, False, "rowsplit"), ([8, 400000], 1, False, "rowsplit"),
     ([17310, 256, 2], 1, False, "col-group-tile"), ([100000, 16, 2], 1, False, "col-group-tile"),
-    ([2048, 2047, 2], 1, False, "col-slab"), ([512, 1000, 3], 1, False, "col-slab"), ([2048, 2048, 2], 1, False, "rowreg-interleaved"),
+    ([2048, 2047, 2], 1, False, "col-slab"), ([512, 1001, 3], 1, False, "col-slab"), ([512, 1000, 3], 1, False, "rowreg-modular"), ([2048, 2048, 2], 1, False, "rowreg-interleaved"),
     ([8, 512, 4096], 1, False, "col-reg"), ([4, 128, 3136], 1, False, "col-reg"), ([64, 64, 3000], 1, False, "col-reg"),
     ([200000, 3], 0, False, "col-split"), ([100000, 33], 0, False, "col-split-flat"), ([32768, 1024], 0, False, "col-split-flat"),
     ([4096, 4096], 1, True, "transposed-tile"),

@@ -138,7 +138,7 @@ def test_plans_for_shapes_off_the_benchmark_list(hpt):
         ([2000, 70], None, 0, 0, "col-split rows=70 cols=2000 vec=1"),
         # softmax over the middle axis, inner dim a divisor of the vector: rows of cols * L elements in registers
         ([8192, 2048, 2], None, 1, 0, "rowreg-interleaved rows=8192 cols=4096 vec=4 tpr=256 rpb=1 nchunk=4"), ([4000, 1000, 8], hpt.f16, 1, 0, "rowreg-interleaved rows=4000 cols=8000 vec=8"),
-        ([4000, 1000, 2], hpt.f64, 1, 0, "rowreg-interleaved rows=4000 cols=2000 vec=2"), ([4000, 1000, 3], None, 1, 0, "col-slab"), ([4000, 1001, 2], None, 1, 0, "col-slab"),
+        ([4000, 1000, 2], hpt.f64, 1, 0, "rowreg-interleaved rows=4000 cols=2000 vec=2"), ([4000, 1001, 3], None, 1, 0, "col-slab"), ([4000, 1000, 3], None, 1, 0, "rowreg-modular rows=4000 cols=3000 vec=4 tpr=256 rpb=1 nchunk=3"), ([4000, 1001, 2], None, 1, 0, "col-slab"),
     ]
     for shape, dt, axis, nn, want in norm:
         got = hpt.normalize_plan(view(shape, dt), axis, nn)
