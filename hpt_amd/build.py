@@ -39,12 +39,16 @@ N_NORM_KINDS = 6  # softmax, log_softmax, layernorm, add+layernorm, causal softm
 
 def units():
     """(object name, source, extra flags)"""
-    u = [("layout.o", CSRC / "layout.cpp", ["-x", "hip"]), ("api.o", CSRC / "api.hip", []),
-         ("elementwise.o", CSRC / "elementwise.hip", [])]
-    for e in range(N_REDUCE_ENTRIES):
-        u.append((f"reduce_op_{e}.o", CSRC / "reduce_op.hip", [f"-DHPT_REDUCE_ENTRY={e}"]))
+    # (the longest compilations first: the softmax kinds and their interleaved rows)
+    u = []
     for k in range(N_NORM_KINDS):
         u.append((f"norm_op_{k}.o", CSRC / "norm_op.hip", [f"-DHPT_NORM_KIND={k}"]))
+        if k < 2:
+            u.append((f"norm_interleaved_{k}.o", CSRC / "norm_interleaved.hip", [f"-DHPT_NORM_KIND={k}"]))
+    for e in range(N_REDUCE_ENTRIES):
+        u.append((f"reduce_op_{e}.o", CSRC / "reduce_op.hip", [f"-DHPT_REDUCE_ENTRY={e}"]))
+    u += [("layout.o", CSRC / "layout.cpp", ["-x", "hip"]), ("api.o", CSRC / "api.hip", []),
+          ("elementwise.o", CSRC / "elementwise.hip", [])]
     if (CSRC / "transpose_norm.hip").exists():
         u.append(("transpose_norm.o", CSRC / "transpose_norm.hip", []))
     return u
