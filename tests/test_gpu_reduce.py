@@ -702,3 +702,32 @@ def test_reduction_over_the_middle_axis_with_an_inner_dim_of_3_5_6_7(hpt, orc, d
     else:
         assert np.array_equal(t.sum([axis]).numpy(), orc.reduce(orc.SUM, a, [axis]))
         assert np.array_equal(t.prod([axis]).numpy(), orc.reduce(orc.PROD, a, [axis]))
+
+
+@pytest.mark.parametrize("shape,bool_shape,plan", [((700, 1000, 4), (1500, 1000, 4), "row-interleaved"), ((600, 2000, 3), (1500, 2000, 3), "row-modular")],
+                         ids=["interleaved", "modular"])
+def test_every_op_over_the_middle_axis_of_narrow_slabs(hpt, orc, dev, shape, bool_shape, plan):
+    """Every op family of the reductions through the row kernels that keep an accumulator per place in the vector."""
+    rng = np.random.default_rng(735)
+    base = (rng.standard_normal(shape) * 0.05 + 1.0).astype(np.float32)   # products of 1000 ... 2000 factors stay finite
+    t, a = upload(hpt, base, dev=dev)
+    assert hpt.reduce_plan(t, hpt.SUM, [1]).startswith(plan), hpt.reduce_plan(t, hpt.SUM, [1])
+    for op in ("sum", "prod", "mean", "reducel1", "reducel2", "reducel3", "sum_square", "logsumexp"):
+        got = getattr(t, op)([1]).numpy()
+        want = orc.reduce(getattr(orc, op.upper()), a, [1], acc=orc.ACC_F64)
+        assert_close(got, want, F32_RTOL, F32_ATOL * max(1.0, float(np.max(np.abs(want)))), f"{op} {shape}")
+    holes = base.copy()
+    holes.reshape(-1)[::7] = np.nan
+    th, ah = upload(hpt, holes, dev=dev)
+    for op in ("nansum", "nanprod"):
+        want = orc.reduce(getattr(orc, op.upper()), ah, [1], acc=orc.ACC_F64)
+        assert_close(getattr(th, op)([1]).numpy(), want, F32_RTOL, F32_ATOL * max(1.0, float(np.max(np.abs(want)))), f"{op} {shape}")
+    assert np.all(np.isnan(th.sum([1]).numpy()))          # every column meets a NaN
+    flags = rng.random(bool_shape) < 0.999
+    flags[3, :, 1] = True
+    flags[5, :, 0] = False
+    tb, ab = upload(hpt, flags, dev=dev)
+    assert hpt.reduce_plan(tb, hpt.SUM, [1]).startswith(plan), hpt.reduce_plan(tb, hpt.SUM, [1])
+    for op in ("sum", "max", "min", "all", "any"):
+        assert np.array_equal(getattr(tb, op)([1]).numpy(), orc.reduce(getattr(orc, op.upper()), ab, [1])), f"{op} bool {shape}"
+    assert np.array_equal(t.all([1]).numpy(), (a != 0).all(1))
