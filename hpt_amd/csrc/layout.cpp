@@ -268,13 +268,14 @@ ReducePlan plan_reduce(const void* data, const int64_t* shape, const int64_t* st
             p.kept_swapped = true;
         }
         // The same slabs with an inner dim of 3, 5, 6 or 7 elements (points, colours): a row of the kernel whose
-        // lanes, in multiples of L, keep an accumulator per vector place. Mid-sized slabs, many of them: small
-        // groups go through LDS tiles, few long ones through the flat walk.
+        // lanes, in multiples of L, keep an accumulator per vector place. Mid-sized slabs, many of them: groups up to
+        // 2 KiB go through LDS tiles (f32 [30000, 100, 3] 9.1 us there against 13.5 here; above, against the flat walk,
+        // [20000, 200, 3] 23.1 -> 12.4), few long ones through the flat walk.
         {
             const int64_t full = elem_size <= 8 ? (int64_t)(16 / elem_size) : 1;
             const int64_t L = nk == 2 ? p.kept.size[1] : 0;
             if (nk == 2 && !p.kept_swapped && p.red.n == 1 && full > 1 && p.kept.stride[1] == 1 && L >= 3 && L <= 7 && full % L != 0 &&
-                p.red.stride[0] == L && p.kept.stride[0] == p.R * L && p.R * L * (int64_t)elem_size >= 4096 &&
+                p.red.stride[0] == L && p.kept.stride[0] == p.R * L && p.R * L * (int64_t)elem_size > 2048 &&
                 p.R * L * (int64_t)elem_size <= (256 << 10) && p.kept.size[0] >= 512 &&
                 p.K * p.R * (int64_t)elem_size >= (4ll << 20) && ((uintptr_t)data % elem_size) == 0) {
                 p.kind = ReduceKind::Row;

@@ -1128,8 +1128,10 @@ void launch_reduce_t(const ReducePlan& p, const void* in, void* out, const Reduc
             a.init_out = init_out;
             switch (p.mod_rows) {
                 case 3: row_mod_kernel<Op, FULL, 3><<<grid, dim3(256), 0, st>>>(a); return;
+                // (eight-byte elements: four is no divisor of their two-element vector)
+                case 4: if constexpr (FULL == 2) { row_mod_kernel<Op, FULL, 4><<<grid, dim3(256), 0, st>>>(a); return; } break;
                 case 5: row_mod_kernel<Op, FULL, 5><<<grid, dim3(256), 0, st>>>(a); return;
-                case 6: if constexpr (FULL != 2) { row_mod_kernel<Op, FULL, 6><<<grid, dim3(256), 0, st>>>(a); return; } break;
+                case 6: row_mod_kernel<Op, FULL, 6><<<grid, dim3(256), 0, st>>>(a); return;
                 case 7: row_mod_kernel<Op, FULL, 7><<<grid, dim3(256), 0, st>>>(a); return;
                 default: break;
             }

@@ -707,6 +707,7 @@ MODULAR_SLAB_CASES = [  # an inner dim of 3, 5, 6, 7 and slabs of whole vectors:
     ("f32 [300, 8000, 3] axis 1 (rows of 1024 threads)", np.float32, [300, 8000, 3], 1),
     ("f16 [700, 4000, 6] axis 1", np.float16, [700, 4000, 6], 1),
     ("f32 [2000, 1000, 3] axis 1", np.float32, [2000, 1000, 3], 1),
+    ("f64 [400, 1000, 6] axis 1 (three two-element vectors per inner row)", np.float64, [400, 1000, 6], 1),
 ]
 
 

@@ -29,7 +29,7 @@ def rand_case(rng):
     return npdt, (B, C, L), 1
 
 
-@pytest.mark.parametrize("seed", [7001, 7002, 7003, 7004])
+@pytest.mark.parametrize("seed", [7001, 7002, 7003, 7004, 7005, 7006])
 def test_random_slabs(hpt, orc, dev, seed):
     rng = np.random.default_rng(seed)
     plans = set()

@@ -662,6 +662,10 @@ MODULAR_ROW_CASES = [  # (dtype, shape, axis): the middle axis of a contiguous [
     (np.float32, (3, 400, 1000, 6), 2), (np.float32, (512, 20001, 3), 1), (np.float16, (900, 1000, 3), 1), (np.float16, (2000, 999, 5), 1),
     (np.float16, (600, 2047, 7), 1), (np.float64, (600, 1001, 3), 1), (np.float64, (700, 333, 5), 1), (np.int32, (700, 1001, 3), 1),
     (np.int64, (600, 1000, 7), 1), (np.int16, (900, 1001, 6), 1), (np.int8, (1200, 1501, 3), 1), (np.uint8, (600, 3001, 5), 1),
+    # slabs just above the 2 KiB that the LDS group tiles take
+    (np.float32, (6000, 200, 3), 1), (np.float16, (5000, 500, 3), 1), (np.float32, (9000, 90, 7), 1),
+    # eight-byte elements: inner dims of 4 and 6 are no divisors of the two-element vector either
+    (np.float64, (6633, 80, 4), 1), (np.int64, (700, 1001, 4), 1), (np.float64, (900, 333, 6), 1),
 ]
 
 
